@@ -1,0 +1,657 @@
+"""CPU restatement (numpy) of LuxLib's fused-operator forward + pullback path.
+
+TEST INFRASTRUCTURE ONLY.  This module is the checker that the HIP path is compared
+against; it is never the thing measured or shipped.  Only tests, the smoke check and the
+`cpu_baseline` leg of the benchmark may import it.
+
+Arrays carry Julia's *logical* shapes (e.g. WHCN for images, features x batch for
+matrices); numpy memory order is irrelevant here.  Every function computes in the dtype
+it is handed (pass float64 inputs for the fp64 arbiter, float32 for the fp32 restatement).
+
+Each function cites the reference file:line it follows (paths relative to
+lib/LuxLib/src/ of the reference unless stated otherwise).
+
+Pinning status (what independent evidence each function is checked against, see
+tests/test_oracle_*.py):
+  * activations / derivatives ......... textbook closed forms, torch library routines,
+                                        fp64 central finite differences
+  * bias_activation (+pullback) ....... closed form, torch autograd, finite differences
+  * fused_dense (+pullback) ........... reference known answers (Dense 10->1/2 with ones),
+                                        torch F.linear autograd, finite differences
+  * batchnorm (+running stats, bwd) ... reference known-answer test (x=[1 3 5;2 4 6]),
+                                        torch F.batch_norm autograd, finite differences
+  * groupnorm (+bwd) .................. torch F.group_norm autograd, finite differences
+  * layernorm (+bwd) .................. mean~0/std~1 invariant, torch F.layer_norm autograd
+  * conv / dgrad / wgrad .............. reference known answers (impulse response,
+                                        asymmetric-pad counts), brute-force 7-loop direct
+                                        convolution, torch conv2d with flipped kernel
+  * NNlib's `tanh_fast`/`sigmoid_fast` rational approximations, exact `gelu` constants and
+    Julia's summation order are NOT reproducible without Julia: parity for those is pinned
+    to tolerance only (few-ulp effects), not bit-for-bit.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+# --------------------------------------------------------------------------------------
+# Activation table.  Values: NNlib (third party, compat 0.9.33, not vendored in the
+# reference tree); derivative forms: ChainRulesCore.derivatives_given_output as used by
+# `only_derivative` (utils.jl:81-84) and `∇activation` (impl/activation.jl:135-154).
+# swish / sigmoid / tanh derivative forms are visible in ext/SLEEFPiratesExt.jl:20-35;
+# gelu is the tanh approximation (ext/CUDAExt/cublaslt.jl:308-315 maps it to
+# CUBLASLT_EPILOGUE_GELU).
+# --------------------------------------------------------------------------------------
+ACTIVATIONS = (
+    "identity", "relu", "tanh", "sigmoid", "swish", "gelu", "softplus", "logsigmoid", "lisht",
+    "tanh_fast", "sigmoid_fast",
+)
+_ALIASES = {"tanh_fast": "tanh", "sigmoid_fast": "sigmoid", "gelu_tanh": "gelu"}
+
+_SQRT_2_OVER_PI = math.sqrt(2.0 / math.pi)
+_GELU_C = 0.044715
+
+
+def canonical_act(name: str) -> str:
+    name = _ALIASES.get(name, name)
+    if name not in ACTIVATIONS:
+        raise ValueError(f"unknown activation {name!r}")
+    return name
+
+
+def _sigmoid(x):
+    # numerically stable logistic
+    t = np.exp(-np.abs(x))
+    return np.where(x >= 0, 1 / (1 + t), t / (1 + t)).astype(x.dtype, copy=False)
+
+
+def act_value(name: str, x: np.ndarray) -> np.ndarray:
+    """σ.(x) for the named activation."""
+    name = canonical_act(name)
+    x = np.asarray(x)
+    T = x.dtype.type
+    if name == "identity":
+        return x.copy()
+    if name == "relu":
+        return np.maximum(x, T(0))
+    if name == "tanh":
+        return np.tanh(x)
+    if name == "sigmoid":
+        return _sigmoid(x)
+    if name == "swish":
+        return x * _sigmoid(x)
+    if name == "gelu":
+        u = T(_SQRT_2_OVER_PI) * (x + T(_GELU_C) * x * x * x)
+        return T(0.5) * x * (T(1) + np.tanh(u))
+    if name == "softplus":
+        return np.log1p(np.exp(-np.abs(x))) + np.maximum(x, T(0))
+    if name == "logsigmoid":
+        return -(np.log1p(np.exp(-np.abs(x))) + np.maximum(-x, T(0)))
+    if name == "lisht":
+        return x * np.tanh(x)
+    raise AssertionError(name)
+
+
+# Which saved quantity the derivative is computed from (impl/dense.jl:83-112,
+# traits.jl:59-70): "out" -> derivative needs only the output Ω (rrule branch 1);
+# "pre" -> needs the pre-activation x as well (branch 2).
+ACT_NEEDS = {
+    "identity": "none", "relu": "out", "tanh": "out", "sigmoid": "out",
+    "swish": "pre", "gelu": "pre", "softplus": "pre", "logsigmoid": "pre", "lisht": "pre",
+}
+
+
+def act_derivative(name: str, out: np.ndarray, x: np.ndarray | None) -> np.ndarray:
+    """dσ(Ω, x) as LuxLib multiplies Δ by (impl/activation.jl:139-154).
+
+    `out` = Ω = σ(x).  `x` may be None for activations whose derivative needs only Ω
+    (the reference passes NotaNumber() there).
+    """
+    name = canonical_act(name)
+    out = np.asarray(out)
+    T = out.dtype.type
+    if name == "identity":
+        return np.ones_like(out)
+    if name == "relu":
+        return (out > 0).astype(out.dtype)
+    if name == "tanh":
+        return T(1) - out * out
+    if name == "sigmoid":
+        return out * (T(1) - out)
+    if x is None:
+        raise ValueError(f"activation {name} needs the pre-activation for its derivative")
+    x = np.asarray(x)
+    if name == "swish":
+        return out + _sigmoid(x) * (T(1) - out)
+    if name == "gelu":
+        x2 = x * x
+        u = T(_SQRT_2_OVER_PI) * (x + T(_GELU_C) * x2 * x)
+        t = np.tanh(u)
+        du = T(_SQRT_2_OVER_PI) * (T(1) + T(3 * _GELU_C) * x2)
+        return T(0.5) * (T(1) + t) + T(0.5) * x * (T(1) - t * t) * du
+    if name == "softplus":
+        return _sigmoid(x)
+    if name == "logsigmoid":
+        return _sigmoid(-x)
+    if name == "lisht":
+        t = np.tanh(x)
+        return t + x * (T(1) - t * t)
+    raise AssertionError(name)
+
+
+def grad_activation(delta, out, name, x=None):
+    """∇activation(Δ, out, act, x) = Δ .* only_derivative(out, act, x) (impl/activation.jl:135-141)."""
+    if canonical_act(name) == "identity":
+        return np.asarray(delta).copy()
+    return np.asarray(delta) * act_derivative(name, out, x)
+
+
+# --------------------------------------------------------------------------------------
+# bias_activation  (api/bias_activation.jl:16-45, impl/bias_activation.jl:2-62,
+# impl/common_ops.jl:1-38)
+# --------------------------------------------------------------------------------------
+def _bias_shape(x: np.ndarray, n: int):
+    # reshaped_bias_dims (impl/common_ops.jl:1-3): bias lies along dim N-1 (vectors: dim 1)
+    if x.ndim == 1:
+        return (n,)
+    return tuple(n if i == x.ndim - 2 else 1 for i in range(x.ndim))
+
+
+def bias_add(x, bias):
+    x = np.asarray(x)
+    if bias is None:
+        return x.copy()
+    bias = np.asarray(bias)
+    want = x.shape[0] if x.ndim == 1 else x.shape[-2]
+    if bias.ndim != 1 or bias.shape[0] != want:
+        # api/bias_activation.jl:38-45 (@assert length(bias) == size(x, N-1))
+        raise AssertionError("length(bias) must equal size(x, ndims(x)-1)")
+    return x + bias.reshape(_bias_shape(x, bias.shape[0]))
+
+
+def bias_activation(act: str, x, bias):
+    """y[i,c,n] = σ(x[i,c,n] + b[c])  (impl/bias_activation.jl:207-220,253-270)."""
+    return act_value(act, bias_add(x, bias))
+
+
+def grad_bias_add(bias, delta):
+    """∂b = sum of Δ over every dim except N-1 (impl/common_ops.jl:25-38)."""
+    if bias is None:
+        return None
+    delta = np.asarray(delta)
+    if delta.ndim == 1:
+        return delta.copy()
+    axes = tuple(i for i in range(delta.ndim) if i != delta.ndim - 2)
+    return delta.sum(axis=axes)
+
+
+def bias_activation_pullback(act: str, x, bias, delta):
+    """rrule of bias_activation (impl/bias_activation.jl:64-104): returns (y, ∂x, ∂b)."""
+    pre = bias_add(x, bias)
+    y = act_value(act, pre)
+    dx = grad_activation(delta, y, act, pre)
+    return y, dx, grad_bias_add(bias, dx)
+
+
+# --------------------------------------------------------------------------------------
+# fused_dense_bias_activation  (api/dense.jl:33-37, impl/dense.jl:4-113,290-291,
+# impl/matmul.jl:2-129)
+# --------------------------------------------------------------------------------------
+class DimensionMismatch(ValueError):
+    """Mirror of Julia's DimensionMismatch (impl/matmul.jl:21-34)."""
+
+
+def matmuladd(W, x, b):
+    W, x = np.asarray(W), np.asarray(x)
+    if W.shape[1] != x.shape[0]:
+        raise DimensionMismatch(f"A has shape {W.shape} but B has shape {x.shape}")
+    if b is not None and np.asarray(b).shape[0] != W.shape[0]:
+        raise DimensionMismatch("bias length does not match rows of A")
+    y = W @ x
+    if b is not None:
+        y = y + np.asarray(b)[:, None]
+    return y
+
+
+def fused_dense_bias_activation(act: str, W, x, b):
+    """y = σ.(W*x .+ b), W (out x in), x (in x batch)  (impl/dense.jl:29-57)."""
+    return act_value(act, matmuladd(W, x, b))
+
+
+def fused_dense_pullback(act: str, W, x, b, delta):
+    """rrule (impl/dense.jl:71-113) + ∇matmul_bias (:290-291): (y, ∂W, ∂x, ∂b)."""
+    pre = matmuladd(W, x, b)
+    y = act_value(act, pre)
+    dz = grad_activation(delta, y, act, pre)
+    db = None if b is None else dz.sum(axis=1)
+    dW = dz @ np.asarray(x).T
+    dx = np.asarray(W).T @ dz
+    return y, dW, dx, db
+
+
+# --------------------------------------------------------------------------------------
+# mean_var and its rrule (impl/common_ops.jl:40-61)
+# --------------------------------------------------------------------------------------
+def mean_var(x, axes, corrected=False):
+    x = np.asarray(x)
+    mu = x.mean(axis=axes, keepdims=True)
+    n = int(np.prod([x.shape[a] for a in axes]))
+    var = ((x - mu) ** 2).sum(axis=axes, keepdims=True) / x.dtype.type(n - (1 if corrected else 0))
+    return mu, var
+
+
+def mean_var_pullback(x, mu, axes, dmu, dvar, corrected=False):
+    """∂x = ∂μ/n + (2/(n - corrected)) ∂σ² (x - μ)  (impl/common_ops.jl:45-61)."""
+    x = np.asarray(x)
+    T = x.dtype.type
+    n = int(np.prod([x.shape[a] for a in axes]))
+    return dmu / T(n) + T(2.0 / (n - (1 if corrected else 0))) * dvar * (x - mu)
+
+
+def default_epsilon(dtype) -> float:
+    """eps(T)^(5/7)  (utils.jl:130)."""
+    return float(np.finfo(dtype).eps) ** (5.0 / 7.0)
+
+
+# --------------------------------------------------------------------------------------
+# batchnorm  (api/batchnorm.jl:31-55, impl/batchnorm.jl:29-147, impl/normalization.jl:20-143)
+# --------------------------------------------------------------------------------------
+def _bn_axes(x):
+    # batchnorm_reduce_dims (impl/batchnorm.jl:4-6): all dims except N-1
+    return tuple(i for i in range(x.ndim) if i != x.ndim - 2)
+
+
+def _chan_shape(x, C):
+    return tuple(C if i == x.ndim - 2 else 1 for i in range(x.ndim))
+
+
+def batchnorm(x, gamma, beta, rmean, rvar, training: bool, act: str = "identity",
+              momentum=0.1, eps=None):
+    """Returns (y, running_mean', running_var')  (impl/batchnorm.jl:29-49).
+
+    training: batch statistics (biased variance); running stats, when given, become
+    (1-m)·r + m·μ and (1-m)·r + m·n/(n-1)·σ² (impl/normalization.jl:95-110, 20-37).
+    inference: the running stats are the statistics (batch statistics when none are given,
+    impl/normalization.jl:116-127).
+    """
+    x = np.asarray(x)
+    T = x.dtype.type
+    if eps is None:
+        eps = default_epsilon(x.dtype)
+    C = x.shape[-2]
+    axes = _bn_axes(x)
+    cs = _chan_shape(x, C)
+    if training or rmean is None:
+        mu, var = mean_var(x, axes, corrected=False)
+        if training and rmean is not None:
+            n = T(np.prod([x.shape[a] for a in axes]))
+            m = T(momentum)
+            rmean_new = (T(1) - m) * np.asarray(rmean) + m * mu.reshape(C)
+            rvar_new = (T(1) - m) * np.asarray(rvar) + (m * n / (n - T(1))) * var.reshape(C)
+        else:
+            rmean_new, rvar_new = rmean, rvar
+    else:
+        mu, var = np.asarray(rmean).reshape(cs), np.asarray(rvar).reshape(cs)
+        rmean_new, rvar_new = rmean, rvar
+    y = _affine_normalize(act, x, mu, var, gamma, beta, T(eps), cs)
+    return y, rmean_new, rvar_new
+
+
+def _affine_normalize(act, x, mu, var, gamma, beta, eps, pshape):
+    """act(x·γ′ + β′), γ′ = γ/√(σ²+ϵ), β′ = β - μγ′  (impl/normalization.jl:3-17,
+    impl/batchnorm.jl:149-176)."""
+    T = x.dtype.type
+    if gamma is None:
+        gp = T(1) / np.sqrt(var + eps)
+        bp = -mu * gp
+    else:
+        gp = np.asarray(gamma).reshape(pshape) / np.sqrt(var + eps)
+        bp = np.asarray(beta).reshape(pshape) - mu * gp
+    return act_value(act, x * gp + bp)
+
+
+def batchnorm_pullback(x, gamma, beta, act: str, eps, delta, *, training=True,
+                       rmean=None, rvar=None):
+    """Pullback of batchnorm w.r.t. (x, γ, β): (∂x, ∂γ, ∂β).
+
+    Follows ∇batchnorm_affine_normalize_cpu! (impl/batchnorm.jl:517-570) completed, in
+    training mode, by the mean_var rrule (impl/common_ops.jl:45-61).  In inference mode the
+    statistics are constants (impl/normalization.jl:39,114 are non-differentiable) so only
+    the ∂x̃ = ∂y·γ′ term survives.
+    """
+    x = np.asarray(x)
+    T = x.dtype.type
+    C = x.shape[-2]
+    axes = _bn_axes(x)
+    cs = _chan_shape(x, C)
+    if training or rmean is None:
+        mu, var = mean_var(x, axes)
+        stats_depend_on_x = True
+    else:
+        mu, var = np.asarray(rmean).reshape(cs), np.asarray(rvar).reshape(cs)
+        stats_depend_on_x = False
+    eps = T(eps)
+    idenom = T(1) / np.sqrt(var + eps)
+    g = np.ones(cs, x.dtype) if gamma is None else np.asarray(gamma).reshape(cs)
+    b = np.zeros(cs, x.dtype) if beta is None else np.asarray(beta).reshape(cs)
+    gp = g * idenom
+    pre = x * gp + (b - mu * gp)
+    out = act_value(act, pre)
+    dy = grad_activation(delta, out, act, pre)
+    xmu = x - mu
+    dbeta = dy.sum(axis=axes)
+    dgamma = (dy * xmu * idenom).sum(axis=axes)
+    dxt = dy * gp
+    dx = dxt
+    if stats_depend_on_x:
+        dmu = -dxt.sum(axis=axes, keepdims=True)
+        dvar = -(dxt * xmu).sum(axis=axes, keepdims=True) * T(0.5) * idenom * idenom
+        dx = dxt + mean_var_pullback(x, mu, axes, dmu, dvar)
+    return dx, (None if gamma is None else dgamma), (None if beta is None else dbeta)
+
+
+# --------------------------------------------------------------------------------------
+# groupnorm  (api/groupnorm.jl:26-64, impl/groupnorm.jl:5-85, 477-533)
+# --------------------------------------------------------------------------------------
+class ArgumentError(ValueError):
+    """Mirror of Julia's ArgumentError (api/groupnorm.jl:40-64)."""
+
+
+def _gn_view(x, groups):
+    # x (..., C, N) -> (..., C/G, G, N) in *Julia column-major* order: channel c (0-based)
+    # maps to j = c mod C/G, k = c div C/G (impl/groupnorm.jl:13-15).  With numpy logical
+    # indices that is x5[..., j, k, n] = x[..., k*Cg + j, n].
+    C, N = x.shape[-2], x.shape[-1]
+    Cg = C // groups
+    lead = x.shape[:-2]
+    x5 = x.reshape(lead + (groups, Cg, N))          # [..., k, j, n]
+    return np.swapaxes(x5, -3, -2), Cg              # [..., j, k, n]
+
+
+def groupnorm(x, gamma, beta, groups: int, act: str = "identity", eps=None):
+    x = np.asarray(x)
+    T = x.dtype.type
+    C = x.shape[-2]
+    if gamma is not None and (len(gamma) != len(beta) or len(beta) != C):
+        raise ArgumentError("Length of `scale` and `bias` must be equal to the number of channels")
+    if C % groups != 0:
+        raise ArgumentError(f"Number of channels {C} must be divisible by the number of groups {groups}")
+    if eps is None:
+        eps = default_epsilon(x.dtype)
+    xv, Cg = _gn_view(x, groups)
+    axes = tuple(range(xv.ndim - 2))                # all but (G, N)  (impl/groupnorm.jl:1)
+    mu, var = mean_var(xv, axes)
+    pshape = (1,) * (xv.ndim - 3) + (Cg, groups, 1)
+    gv = None if gamma is None else np.asarray(gamma).reshape(groups, Cg).T.reshape(pshape)
+    bv = None if beta is None else np.asarray(beta).reshape(groups, Cg).T.reshape(pshape)
+    yv = _affine_normalize_arr(act, xv, mu, var, gv, bv, T(eps))
+    return np.swapaxes(yv, -3, -2).reshape(x.shape)
+
+
+def _affine_normalize_arr(act, x, mu, var, g, b, eps):
+    T = x.dtype.type
+    if g is None:
+        gp = T(1) / np.sqrt(var + eps)
+        bp = -mu * gp
+    else:
+        gp = g / np.sqrt(var + eps)
+        bp = b - mu * gp
+    return act_value(act, x * gp + bp)
+
+
+def groupnorm_pullback(x, gamma, beta, groups: int, act: str, eps, delta):
+    """(∂x, ∂γ, ∂β): ∇groupnorm_affine_normalize_cpu! (impl/groupnorm.jl:477-533) completed
+    by the mean_var rrule with n = W·H·C/G."""
+    x = np.asarray(x)
+    T = x.dtype.type
+    C = x.shape[-2]
+    xv, Cg = _gn_view(x, groups)
+    dv, _ = _gn_view(np.asarray(delta), groups)
+    axes = tuple(range(xv.ndim - 2))
+    mu, var = mean_var(xv, axes)
+    eps = T(eps)
+    idenom = T(1) / np.sqrt(var + eps)
+    pshape = (1,) * (xv.ndim - 3) + (Cg, groups, 1)
+    g = np.ones(pshape, x.dtype) if gamma is None else np.asarray(gamma).reshape(groups, Cg).T.reshape(pshape)
+    b = np.zeros(pshape, x.dtype) if beta is None else np.asarray(beta).reshape(groups, Cg).T.reshape(pshape)
+    gp = g * idenom
+    pre = xv * gp + (b - mu * gp)
+    out = act_value(act, pre)
+    dy = grad_activation(dv, out, act, pre)
+    xmu = xv - mu
+    par_axes = tuple(range(xv.ndim - 3)) + (xv.ndim - 1,)       # over (i..., n)
+    dbeta = dy.sum(axis=par_axes).T.reshape(C)                   # [j,k] -> c = k*Cg + j
+    dgamma = (dy * xmu * idenom).sum(axis=par_axes).T.reshape(C)
+    dxt = dy * gp
+    dmu = -dxt.sum(axis=axes, keepdims=True)
+    dvar = -(dxt * xmu).sum(axis=axes, keepdims=True) * T(0.5) * idenom * idenom
+    dxv = dxt + mean_var_pullback(xv, mu, axes, dmu, dvar)
+    dx = np.swapaxes(dxv, -3, -2).reshape(x.shape)
+    return dx, (None if gamma is None else dgamma), (None if beta is None else dbeta)
+
+
+# --------------------------------------------------------------------------------------
+# layernorm  (api/layernorm.jl:32-43, impl/layernorm.jl:3-51, impl/normalization.jl:3-17)
+# --------------------------------------------------------------------------------------
+def layernorm(x, gamma, beta, act: str = "identity", dims=None, eps=None):
+    """`dims` are 0-based numpy axes here (Julia's 1:(N-1) default = all but the last).
+    γ, β must broadcast against x (the reference requires ndims(γ) == ndims(x) when dims is
+    given, impl/layernorm.jl:47-51)."""
+    x = np.asarray(x)
+    T = x.dtype.type
+    if dims is None:
+        dims = tuple(range(x.ndim - 1))
+    if eps is None:
+        eps = default_epsilon(x.dtype)
+    mu, var = mean_var(x, tuple(dims))
+    g = None if gamma is None else np.asarray(gamma)
+    b = None if beta is None else np.asarray(beta)
+    return _affine_normalize_arr(act, x, mu, var, g, b, T(eps))
+
+
+def _sum_to_shape(a, shape):
+    axes = tuple(i for i, (s, t) in enumerate(zip(a.shape, shape)) if t == 1 and s != 1)
+    return a.sum(axis=axes, keepdims=True).reshape(shape)
+
+
+def layernorm_pullback(x, gamma, beta, act: str, dims, eps, delta):
+    """(∂x, ∂γ, ∂β).  The reference has no custom rrule: AD differentiates the broadcasts
+    of impl/normalization.jl:11-17 and chains into the mean_var rrule
+    (impl/common_ops.jl:45-61).  This is that chain written out."""
+    x = np.asarray(x)
+    T = x.dtype.type
+    if dims is None:
+        dims = tuple(range(x.ndim - 1))
+    dims = tuple(dims)
+    eps = T(eps)
+    mu, var = mean_var(x, dims)
+    idenom = T(1) / np.sqrt(var + eps)
+    g = np.ones((1,) * x.ndim, x.dtype) if gamma is None else np.asarray(gamma)
+    b = np.zeros((1,) * x.ndim, x.dtype) if beta is None else np.asarray(beta)
+    gp = g * idenom
+    bp = b - mu * gp
+    pre = x * gp + bp
+    out = act_value(act, pre)
+    dy = grad_activation(np.asarray(delta), out, act, pre)
+    # y = x·γ′ + β′ ;  γ′ = γ·idenom ; β′ = β - μ γ′
+    dgp = _sum_to_shape(dy * x, np.broadcast_shapes(g.shape, idenom.shape))   # ∂γ′ (direct)
+    dbp = _sum_to_shape(dy, np.broadcast_shapes(b.shape, mu.shape))           # ∂β′
+    dgp = dgp - dbp * mu                                                     # via β′ = β - μγ′
+    dmu = _sum_to_shape(-dbp * gp, mu.shape)
+    dgamma = _sum_to_shape(dgp * idenom, g.shape)
+    dbeta = _sum_to_shape(dbp, b.shape)
+    didenom = _sum_to_shape(dgp * g, idenom.shape)
+    dvar = didenom * (T(-0.5) * idenom * idenom * idenom)
+    dx = dy * gp + mean_var_pullback(x, mu, dims, dmu, dvar)
+    return dx, (None if gamma is None else dgamma), (None if beta is None else dbeta)
+
+
+# --------------------------------------------------------------------------------------
+# fused_conv_bias_activation  (api/conv.jl:30-38, impl/conv.jl:138-275).  The arithmetic
+# lives in NNlib (third party, compat 0.9.33, not vendored): its published algorithm is the
+# direct / im2col convolution over WHCN tensors; orientation and padding order are anchored
+# on the reference's own known-answer tests (test/core_layers/conv_tests.jl:54-69,145-190).
+# --------------------------------------------------------------------------------------
+class ConvDims:
+    """The fields of NNlib.DenseConvDims that the path consumes (2 spatial dims)."""
+
+    def __init__(self, x_shape, w_shape, stride=(1, 1), padding=(0, 0, 0, 0), dilation=(1, 1),
+                 groups=1, flipkernel=False):
+        if isinstance(stride, int):
+            stride = (stride, stride)
+        if isinstance(dilation, int):
+            dilation = (dilation, dilation)
+        if isinstance(padding, int):
+            padding = (padding,) * 4
+        elif len(padding) == 2:
+            padding = (padding[0], padding[0], padding[1], padding[1])
+        self.x_shape = tuple(x_shape)
+        self.w_shape = tuple(w_shape)
+        self.stride = tuple(stride)
+        self.padding = tuple(padding)          # (w_lo, w_hi, h_lo, h_hi)
+        self.dilation = tuple(dilation)
+        self.groups = int(groups)
+        self.flipkernel = bool(flipkernel)
+        W, H, Cin, _ = self.x_shape
+        kW, kH, Cin_g, Cout = self.w_shape
+        if Cin_g * self.groups != Cin:
+            raise DimensionMismatch("input channels do not match weight channels x groups")
+        if Cout % self.groups != 0:
+            raise DimensionMismatch("output channels must be divisible by groups")
+
+    @property
+    def out_spatial(self):
+        W, H = self.x_shape[:2]
+        kW, kH = self.w_shape[:2]
+        ow = (W + self.padding[0] + self.padding[1] - self.dilation[0] * (kW - 1) - 1) // self.stride[0] + 1
+        oh = (H + self.padding[2] + self.padding[3] - self.dilation[1] * (kH - 1) - 1) // self.stride[1] + 1
+        return ow, oh
+
+    def y_shape(self, N=None):
+        ow, oh = self.out_spatial
+        return (ow, oh, self.w_shape[3], self.x_shape[3] if N is None else N)
+
+
+def _tap_slices(cd: ConvDims, a, b):
+    """For kernel tap (a, b) (0-based): the output index range and the matching input
+    index range per spatial dim.  Input position for output o and tap a is
+    o·stride + koff·dil - pad_lo with koff = K-1-a (true convolution, flipkernel=false)
+    or a (cross-correlation, flipkernel=true)."""
+    W, H = cd.x_shape[:2]
+    kW, kH = cd.w_shape[:2]
+    OW, OH = cd.out_spatial
+    res = []
+    for (L, K, O, s, d, plo, t) in ((W, kW, OW, cd.stride[0], cd.dilation[0], cd.padding[0], a),
+                                     (H, kH, OH, cd.stride[1], cd.dilation[1], cd.padding[2], b)):
+        koff = t if cd.flipkernel else (K - 1 - t)
+        base = koff * d - plo                   # input index at o = 0
+        o_lo = 0 if base >= 0 else (-base + s - 1) // s
+        o_hi = min(O - 1, (L - 1 - base) // s) if (L - 1 - base) >= 0 else -1
+        if o_hi < o_lo:
+            res.append(None)
+        else:
+            res.append((slice(o_lo, o_hi + 1), slice(base + o_lo * s, base + o_hi * s + 1, s)))
+    return res
+
+
+def conv(x, w, cd: ConvDims):
+    """NNlib.conv(x, w, cdims) over WHCN (call site impl/conv.jl:39,56)."""
+    x, w = np.asarray(x), np.asarray(w)
+    N = x.shape[3]
+    OW, OH = cd.out_spatial
+    kW, kH, Cin_g, Cout = w.shape
+    G = cd.groups
+    Cout_g = Cout // G
+    y = np.zeros((OW, OH, Cout, N), dtype=np.result_type(x, w))
+    for a in range(kW):
+        for b in range(kH):
+            sl = _tap_slices(cd, a, b)
+            if sl[0] is None or sl[1] is None:
+                continue
+            (ow, iw), (oh, ih) = sl
+            for g in range(G):
+                xs = x[iw, ih, g * Cin_g:(g + 1) * Cin_g, :]            # (ow, oh, Cin_g, N)
+                wk = w[a, b, :, g * Cout_g:(g + 1) * Cout_g]            # (Cin_g, Cout_g)
+                y[ow, oh, g * Cout_g:(g + 1) * Cout_g, :] += np.einsum("whcn,co->whon", xs, wk)
+    return y
+
+
+def conv_data_grad(dy, w, cd: ConvDims):
+    """NNlib.∇conv_data(∂y, w, cdims) (call site impl/conv.jl:130): adjoint of conv in x."""
+    dy, w = np.asarray(dy), np.asarray(w)
+    kW, kH, Cin_g, Cout = w.shape
+    G = cd.groups
+    Cout_g = Cout // G
+    dx = np.zeros(cd.x_shape[:3] + (dy.shape[3],), dtype=np.result_type(dy, w))
+    for a in range(kW):
+        for b in range(kH):
+            sl = _tap_slices(cd, a, b)
+            if sl[0] is None or sl[1] is None:
+                continue
+            (ow, iw), (oh, ih) = sl
+            for g in range(G):
+                d = dy[ow, oh, g * Cout_g:(g + 1) * Cout_g, :]
+                wk = w[a, b, :, g * Cout_g:(g + 1) * Cout_g]
+                dx[iw, ih, g * Cin_g:(g + 1) * Cin_g, :] += np.einsum("whon,co->whcn", d, wk)
+    return dx
+
+
+def conv_filter_grad(x, dy, cd: ConvDims):
+    """NNlib.∇conv_filter(x, ∂y, cdims) (call site impl/conv.jl:135): adjoint of conv in w."""
+    x, dy = np.asarray(x), np.asarray(dy)
+    kW, kH, Cin_g, Cout = cd.w_shape
+    G = cd.groups
+    Cout_g = Cout // G
+    dw = np.zeros(cd.w_shape, dtype=np.result_type(x, dy))
+    for a in range(kW):
+        for b in range(kH):
+            sl = _tap_slices(cd, a, b)
+            if sl[0] is None or sl[1] is None:
+                continue
+            (ow, iw), (oh, ih) = sl
+            for g in range(G):
+                xs = x[iw, ih, g * Cin_g:(g + 1) * Cin_g, :]
+                d = dy[ow, oh, g * Cout_g:(g + 1) * Cout_g, :]
+                dw[a, b, :, g * Cout_g:(g + 1) * Cout_g] = np.einsum("whcn,whon->co", xs, d)
+    return dw
+
+
+def fused_conv_bias_activation(act: str, w, x, b, cd: ConvDims):
+    """y = σ(conv(x, w) .+ b[cout])  (impl/conv.jl:138-155)."""
+    return bias_activation(act, conv(x, w, cd), b)
+
+
+def fused_conv_pullback(act: str, w, x, b, cd: ConvDims, delta):
+    """rrule (impl/conv.jl:204-248) + ∇fused_conv (:261-275): (y, ∂w, ∂x, ∂b)."""
+    pre = bias_add(conv(x, w, cd), b)
+    y = act_value(act, pre)
+    dy = grad_activation(delta, y, act, pre)
+    db = grad_bias_add(b, dy)
+    return y, conv_filter_grad(x, dy, cd), conv_data_grad(dy, w, cd), db
+
+
+# --------------------------------------------------------------------------------------
+# helpers shared by the tests
+# --------------------------------------------------------------------------------------
+def generate_fixed_array(dtype, shape):
+    """reshape(T.((1:n)./n), sz) in Julia column-major order
+    (lib/LuxLib/test/shared_testsetup.jl:69-73)."""
+    n = int(np.prod(shape))
+    return (np.arange(1, n + 1, dtype=np.float64) / n).astype(dtype).reshape(shape, order="F")
+
+
+def to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    """float32 -> bfloat16 bit patterns (uint16), round-to-nearest-even."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    rounded = u + (np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1)))
+    return (rounded >> np.uint32(16)).astype(np.uint16)
+
+
+def from_bf16_bits(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def round_to_bf16(a: np.ndarray) -> np.ndarray:
+    """float32 array whose values are exactly representable in bfloat16."""
+    return from_bf16_bits(to_bf16_bits(a)).reshape(np.shape(a))

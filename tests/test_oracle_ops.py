@@ -1,0 +1,380 @@
+"""Pins the oracle's operators against the reference's own known-answer tests, independent
+library routines (torch CPU + autograd), closed forms and fp64 finite differences."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import luxlib_oracle as O
+
+RNG = np.random.default_rng(20240)
+
+
+def fd_grad(f, x, h=1e-6):
+    """Central finite differences of scalar f at x (fp64), as LuxTestUtils.test_gradients does
+    (lib/LuxTestUtils/src/autodiff.jl:147-294)."""
+    g = np.zeros_like(x)
+    it = np.nditer(x, flags=["multi_index"])
+    for _ in it:
+        i = it.multi_index
+        xp, xm = x.copy(), x.copy()
+        xp[i] += h
+        xm[i] -= h
+        g[i] = (f(xp) - f(xm)) / (2 * h)
+    return g
+
+
+# ----------------------------------------------------------------------------- bias_activation
+@pytest.mark.parametrize("act", ["identity", "relu", "sigmoid", "softplus", "logsigmoid", "gelu",
+                                 "swish", "lisht", "tanh"])
+@pytest.mark.parametrize("shape", [(2, 2, 3, 4), (4, 5)])
+def test_bias_activation_closed_form_and_grad(act, shape):
+    # lib/LuxLib/test/common_ops/bias_act_tests.jl:6,16-99
+    x = RNG.random(shape)
+    b = RNG.random(shape[-2])
+    bshape = [1] * len(shape)
+    bshape[-2] = shape[-2]
+    want = O.act_value(act, x + b.reshape(bshape))
+    np.testing.assert_allclose(O.bias_activation(act, x, b), want, rtol=0, atol=0)
+    delta = RNG.normal(size=shape)
+    y, dx, db = O.bias_activation_pullback(act, x, b, delta)
+    np.testing.assert_allclose(dx, fd_grad(lambda v: (O.bias_activation(act, v, b) * delta).sum(), x),
+                               rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(db, fd_grad(lambda v: (O.bias_activation(act, x, v) * delta).sum(), b),
+                               rtol=1e-6, atol=1e-8)
+
+
+def test_bias_activation_edge_cases():
+    # zero-sized arrays (bias_act_tests.jl:119-131), vectors, missing bias, wrong bias length
+    x = np.zeros((4, 3, 2, 0))
+    assert O.bias_activation("relu", x, np.ones(2)).shape == (4, 3, 2, 0)
+    v = np.array([1.0, -2.0, 3.0])
+    np.testing.assert_array_equal(O.bias_activation("relu", v, np.array([0.5, 0.5, 0.5])), [1.5, 0, 3.5])
+    np.testing.assert_array_equal(O.bias_activation("relu", v, None), [1, 0, 3])
+    with pytest.raises(AssertionError):
+        O.bias_activation("relu", np.ones((3, 4)), np.ones(4))
+
+
+# ----------------------------------------------------------------------------- dense
+def test_dense_reference_known_answers():
+    # test/core_layers/basic_tests.jl:151-194: Dense(10 => 1/2) with ones -> 10, [10 20; 10 20]
+    y = O.fused_dense_bias_activation("identity", np.ones((1, 10)), np.ones((10, 1)), None)
+    assert y.tolist() == [[10.0]]
+    y = O.fused_dense_bias_activation("identity", np.ones((2, 10)), np.ones((10, 1)), np.ones(2))
+    assert y.tolist() == [[11.0], [11.0]]
+    y = O.fused_dense_bias_activation("identity", np.ones((2, 10)), np.array([np.ones(10), 2 * np.ones(10)]).T, None)
+    assert y.tolist() == [[10.0, 20.0], [10.0, 20.0]]
+    y = O.fused_dense_bias_activation("relu", -np.ones((1, 10)), np.ones((10, 1)), None)
+    assert y.tolist() == [[0.0]]
+
+
+@pytest.mark.parametrize("act", ["identity", "tanh", "sigmoid_fast", "relu", "gelu", "swish"])
+@pytest.mark.parametrize("M,N,bias", [(4, 32, True), (32, 4, False)])
+def test_dense_vs_torch_autograd(act, M, N, bias):
+    # lib/LuxLib/test/common_ops/dense_tests.jl:13-76: sizes 4/32, batch 3, bias on/off
+    W = RNG.normal(size=(M, N))
+    x = RNG.normal(size=(N, 3))
+    b = RNG.normal(size=M) if bias else None
+    delta = RNG.normal(size=(M, 3))
+    y, dW, dx, db = O.fused_dense_pullback(act, W, x, b, delta)
+    from tests.test_oracle_activations import TORCH
+    tW, tx = torch.tensor(W, requires_grad=True), torch.tensor(x, requires_grad=True)
+    tb = torch.tensor(b, requires_grad=True) if bias else None
+    ty = TORCH[act](F.linear(tx.T, tW, tb)).T          # torch: rows = batch
+    ty.backward(torch.tensor(delta))
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dW, tW.grad.numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-10, atol=1e-12)
+    if bias:
+        np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-10, atol=1e-12)
+    else:
+        assert db is None
+
+
+def test_dense_dimension_mismatch():
+    # impl/matmul.jl:21-34
+    with pytest.raises(O.DimensionMismatch):
+        O.fused_dense_bias_activation("relu", np.ones((3, 4)), np.ones((5, 2)), None)
+    with pytest.raises(O.DimensionMismatch):
+        O.fused_dense_bias_activation("relu", np.ones((3, 4)), np.ones((4, 2)), np.ones(4))
+
+
+# ----------------------------------------------------------------------------- batchnorm
+def test_batchnorm_reference_known_answer():
+    # test/core_layers/normalize_tests.jl:10-49: x = [1 3 5; 2 4 6] (2 channels x 3 samples)
+    x = np.array([[1.0, 3.0, 5.0], [2.0, 4.0, 6.0]], dtype=np.float32)
+    y, rm, rv = O.batchnorm(x, np.ones(2, np.float32), np.zeros(2, np.float32),
+                            np.zeros(2, np.float32), np.ones(2, np.float32), True, "identity",
+                            0.1, 1e-5)
+    np.testing.assert_allclose(y, [[-1.22474, 0, 1.22474], [-1.22474, 0, 1.22474]], atol=1e-5)
+    np.testing.assert_allclose(rm, [0.3, 0.4], rtol=1e-6)
+    # 0.1 * var(corrected) + 0.9 = 0.1 * (8/3 * 3/2) + 0.9 = 1.3
+    np.testing.assert_allclose(rv, [1.3, 1.3], rtol=1e-6)
+    yi, rm2, rv2 = O.batchnorm(x, np.ones(2, np.float32), np.zeros(2, np.float32), rm, rv, False,
+                               "identity", 0.1, 1e-5)
+    np.testing.assert_allclose(yi[0, 0], (1 - 0.3) / np.sqrt(1.3 + 1e-5), rtol=1e-6)
+    assert rm2 is rm and rv2 is rv
+
+
+@pytest.mark.parametrize("shape", [(4, 4, 6, 2), (8, 2), (3, 5, 4)])
+@pytest.mark.parametrize("act", ["identity", "sigmoid_fast", "relu", "swish"])
+@pytest.mark.parametrize("affine", [True, False])
+def test_batchnorm_vs_torch(shape, act, affine):
+    # lib/LuxLib/test/normalization/batchnorm_tests.jl:58-145 shapes; inputs from generate_fixed_array
+    from tests.test_oracle_activations import TORCH
+    x = O.generate_fixed_array(np.float64, shape) + 0.1 * RNG.normal(size=shape)
+    C = shape[-2]
+    g = RNG.uniform(0.5, 1.5, C) if affine else None
+    b = RNG.normal(size=C) if affine else None
+    rm, rv = RNG.normal(size=C), RNG.uniform(0.5, 2, C)
+    delta = RNG.normal(size=shape)
+    eps = 1e-5
+    y, rm_n, rv_n = O.batchnorm(x, g, b, rm, rv, True, act, 0.1, eps)
+    dx, dg, db = O.batchnorm_pullback(x, g, b, act, eps, delta)
+    perm = (len(shape) - 1, len(shape) - 2) + tuple(range(len(shape) - 2))   # -> N, C, spatial...
+    inv = np.argsort(perm)
+    tx = torch.tensor(np.transpose(x, perm).copy(), requires_grad=True)
+    tg = torch.tensor(g, requires_grad=True) if affine else None
+    tb = torch.tensor(b, requires_grad=True) if affine else None
+    trm, trv = torch.tensor(rm), torch.tensor(rv)
+    ty = TORCH[act](F.batch_norm(tx, trm, trv, tg, tb, True, 0.1, eps))
+    ty.backward(torch.tensor(np.transpose(delta, perm).copy()))
+    np.testing.assert_allclose(y, np.transpose(ty.detach().numpy(), inv), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(rm_n, trm.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(rv_n, trv.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(dx, np.transpose(tx.grad.numpy(), inv), rtol=1e-8, atol=1e-10)
+    if affine:
+        np.testing.assert_allclose(dg, tg.grad.numpy(), rtol=1e-9, atol=1e-11)
+        np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-9, atol=1e-11)
+    # inference mode
+    yi, _, _ = O.batchnorm(x, g, b, rm, rv, False, act, 0.1, eps)
+    tyi = TORCH[act](F.batch_norm(tx.detach(), torch.tensor(rm), torch.tensor(rv), None if not affine else tg.detach(),
+                                  None if not affine else tb.detach(), False, 0.1, eps))
+    np.testing.assert_allclose(yi, np.transpose(tyi.numpy(), inv), rtol=1e-10, atol=1e-11)
+
+
+def test_batchnorm_pullback_finite_differences():
+    shape = (3, 2, 4, 3)
+    x = RNG.normal(size=shape)
+    g, b = RNG.uniform(0.5, 1.5, 4), RNG.normal(size=4)
+    delta = RNG.normal(size=shape)
+    dx, dg, db = O.batchnorm_pullback(x, g, b, "gelu", 1e-5, delta)
+    loss = lambda xx, gg, bb: (O.batchnorm(xx, gg, bb, None, None, True, "gelu", 0.1, 1e-5)[0] * delta).sum()
+    np.testing.assert_allclose(dx, fd_grad(lambda v: loss(v, g, b), x), rtol=2e-6, atol=1e-8)
+    np.testing.assert_allclose(dg, fd_grad(lambda v: loss(x, v, b), g), rtol=2e-6, atol=1e-8)
+    np.testing.assert_allclose(db, fd_grad(lambda v: loss(x, g, v), b), rtol=2e-6, atol=1e-8)
+    # inference-mode pullback: statistics are constants
+    rm, rv = RNG.normal(size=4), RNG.uniform(0.5, 2, 4)
+    dxi, _, _ = O.batchnorm_pullback(x, g, b, "gelu", 1e-5, delta, training=False, rmean=rm, rvar=rv)
+    lossi = lambda xx: (O.batchnorm(xx, g, b, rm, rv, False, "gelu", 0.1, 1e-5)[0] * delta).sum()
+    np.testing.assert_allclose(dxi, fd_grad(lossi, x), rtol=2e-6, atol=1e-8)
+
+
+# ----------------------------------------------------------------------------- groupnorm
+@pytest.mark.parametrize("shape,groups", [((6, 2), 2), ((4, 4, 6, 2), 3), ((2, 2, 6, 2), 2), ((5, 12, 3), 4)])
+@pytest.mark.parametrize("act", ["identity", "swish", "relu"])
+@pytest.mark.parametrize("affine", [True, False])
+def test_groupnorm_vs_torch(shape, groups, act, affine):
+    # lib/LuxLib/test/normalization/groupnorm_tests.jl:48-115 shapes and groups
+    from tests.test_oracle_activations import TORCH
+    x = RNG.normal(size=shape)
+    C = shape[-2]
+    g = RNG.uniform(0.8, 1.2, C) if affine else None
+    b = RNG.normal(size=C) if affine else None
+    delta = RNG.normal(size=shape)
+    eps = 1e-5
+    y = O.groupnorm(x, g, b, groups, act, eps)
+    dx, dg, db = O.groupnorm_pullback(x, g, b, groups, act, eps, delta)
+    perm = (len(shape) - 1, len(shape) - 2) + tuple(range(len(shape) - 2))
+    inv = np.argsort(perm)
+    tx = torch.tensor(np.transpose(x, perm).copy(), requires_grad=True)
+    tg = torch.tensor(g, requires_grad=True) if affine else None
+    tb = torch.tensor(b, requires_grad=True) if affine else None
+    ty = TORCH[act](F.group_norm(tx, groups, tg, tb, eps))
+    ty.backward(torch.tensor(np.transpose(delta, perm).copy()))
+    np.testing.assert_allclose(y, np.transpose(ty.detach().numpy(), inv), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(dx, np.transpose(tx.grad.numpy(), inv), rtol=1e-8, atol=1e-10)
+    if affine:
+        np.testing.assert_allclose(dg, tg.grad.numpy(), rtol=1e-9, atol=1e-11)
+        np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-9, atol=1e-11)
+
+
+def test_groupnorm_argument_errors():
+    # api/groupnorm.jl:40-64
+    with pytest.raises(O.ArgumentError):
+        O.groupnorm(np.ones((4, 6, 2)), np.ones(6), np.ones(6), 4)
+    with pytest.raises(O.ArgumentError):
+        O.groupnorm(np.ones((4, 6, 2)), np.ones(5), np.ones(5), 2)
+
+
+def test_groupnorm_equals_instance_stats_when_groups_eq_channels():
+    # G == C  =>  per-(channel, sample) statistics (instancenorm, impl/normalization.jl:191-208)
+    x = RNG.normal(size=(5, 4, 3))
+    y = O.groupnorm(x, None, None, 4, "identity", 0.0)
+    np.testing.assert_allclose(y.mean(axis=0), 0, atol=1e-14)
+    np.testing.assert_allclose(y.std(axis=0), 1, rtol=1e-12)
+
+
+# ----------------------------------------------------------------------------- layernorm
+def test_layernorm_invariants():
+    # lib/LuxLib/test/normalization/layernorm_tests.jl:54-57: mean ~ 0, std ~ 1 without affine
+    x = O.generate_fixed_array(np.float32, (4, 4, 6, 2))
+    y = O.layernorm(x, None, None, "identity", (0, 1, 2), None)
+    assert abs(y.mean(axis=(0, 1, 2))).max() < 1e-5
+    # epsilon in the denominator biases the std slightly below 1
+    np.testing.assert_allclose(y.std(axis=(0, 1, 2)), 1, atol=1e-3)
+
+
+@pytest.mark.parametrize("shape,nd", [((4, 4, 6, 2), 3), ((6, 3), 1), ((16, 5), 1), ((3, 4, 5), 1)])
+@pytest.mark.parametrize("act", ["identity", "relu", "gelu"])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layernorm_vs_torch(shape, nd, act, affine):
+    from tests.test_oracle_activations import TORCH
+    x = RNG.normal(size=shape)
+    dims = tuple(range(nd))
+    pshape = shape[:nd] + (1,) * (len(shape) - nd)
+    g = RNG.uniform(0.5, 1.5, pshape) if affine else None
+    b = RNG.normal(size=pshape) if affine else None
+    delta = RNG.normal(size=shape)
+    eps = 1e-5
+    y = O.layernorm(x, g, b, act, dims, eps)
+    dx, dg, db = O.layernorm_pullback(x, g, b, act, dims, eps, delta)
+    # torch normalises trailing dims: reverse the axes
+    rev = tuple(reversed(range(len(shape))))
+    tx = torch.tensor(np.transpose(x, rev).copy(), requires_grad=True)
+    nshape = tuple(reversed(shape[:nd]))
+    tg = torch.tensor(np.transpose(g, rev).reshape(nshape).copy(), requires_grad=True) if affine else None
+    tb = torch.tensor(np.transpose(b, rev).reshape(nshape).copy(), requires_grad=True) if affine else None
+    ty = TORCH[act](F.layer_norm(tx, nshape, tg, tb, eps))
+    ty.backward(torch.tensor(np.transpose(delta, rev).copy()))
+    np.testing.assert_allclose(y, np.transpose(ty.detach().numpy(), rev), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(dx, np.transpose(tx.grad.numpy(), rev), rtol=1e-8, atol=1e-10)
+    if affine:
+        np.testing.assert_allclose(dg, np.transpose(tg.grad.numpy().reshape(tuple(reversed(pshape))), rev), rtol=1e-9, atol=1e-11)
+        np.testing.assert_allclose(db, np.transpose(tb.grad.numpy().reshape(tuple(reversed(pshape))), rev), rtol=1e-9, atol=1e-11)
+
+
+# ----------------------------------------------------------------------------- conv
+def brute_conv(x, w, cd):
+    """7-loop direct convolution straight from the index formula
+    y[o] = sum_k w[k] x[(o)*s + (K-1-k)*d - pad_lo] (0-based), grouped."""
+    W, H, Cin, N = x.shape
+    kW, kH, Cg, Cout = w.shape
+    OW, OH = cd.out_spatial
+    G = cd.groups
+    y = np.zeros((OW, OH, Cout, N))
+    for n in range(N):
+        for co in range(Cout):
+            g = co // (Cout // G)
+            for oh in range(OH):
+                for ow in range(OW):
+                    acc = 0.0
+                    for b in range(kH):
+                        for a in range(kW):
+                            ka = a if cd.flipkernel else kW - 1 - a
+                            kb = b if cd.flipkernel else kH - 1 - b
+                            iw = ow * cd.stride[0] + ka * cd.dilation[0] - cd.padding[0]
+                            ih = oh * cd.stride[1] + kb * cd.dilation[1] - cd.padding[2]
+                            if 0 <= iw < W and 0 <= ih < H:
+                                for c in range(Cg):
+                                    acc += w[a, b, c, co] * x[iw, ih, g * Cg + c, n]
+                    y[ow, oh, co, n] = acc
+    return y
+
+
+def test_conv_reference_impulse_known_answer():
+    # test/core_layers/conv_tests.jl:145-190: delta at the centre of 7x7, 3x3 kernel
+    #   => y[2:4, 2:4] == w  (true convolution orientation)
+    x = np.zeros((7, 7, 1, 1))
+    x[3, 3, 0, 0] = 1
+    w = RNG.normal(size=(3, 3, 1, 1))
+    y = O.conv(x, w, O.ConvDims(x.shape, w.shape))
+    assert y.shape == (5, 5, 1, 1)
+    np.testing.assert_array_equal(y[1:4, 1:4, 0, 0], w[:, :, 0, 0])
+    # cross-correlation flips it
+    yc = O.conv(x, w, O.ConvDims(x.shape, w.shape, flipkernel=True))
+    np.testing.assert_array_equal(yc[1:4, 1:4, 0, 0], w[::-1, ::-1, 0, 0])
+
+
+def test_conv_reference_asymmetric_padding_known_answer():
+    # test/core_layers/conv_tests.jl:54-69: ones(28,28,1,1), 3x3 ones kernel, pad=(0, 1, 1, 2):
+    # the reference checks size (27, 29) and the counts 6, 9, 4, 3, 6, 2 at fixed positions.
+    x = np.ones((28, 28, 1, 1))
+    w = np.ones((3, 3, 1, 1))
+    y = O.conv(x, w, O.ConvDims(x.shape, w.shape, padding=(0, 1, 1, 2)))
+    assert y.shape == (27, 29, 1, 1)
+    y = y[:, :, 0, 0]
+    assert y[0, 0] == 6.0            # (1, 1)
+    assert y[1, 1] == 9.0            # (2, 2)
+    assert y[26, 0] == 4.0           # (end, 1)
+    assert y[0, 28] == 3.0           # (1, end)
+    assert y[0, 27] == 6.0           # (1, end-1)
+    assert y[26, 28] == 2.0          # (end, end)
+
+
+CONV_CASES = [
+    # (x shape, w shape, stride, pad, dilation, groups, flip)
+    ((6, 5, 4, 2), (2, 2, 4, 6), 1, 0, 1, 1, False),
+    ((6, 5, 4, 2), (2, 2, 4, 6), 2, 1, 1, 1, False),
+    ((6, 5, 4, 2), (2, 2, 2, 6), 1, 1, 1, 2, False),      # groups=2 (conv_tests.jl:87-92)
+    ((7, 8, 3, 2), (3, 3, 3, 5), (2, 1), (0, 1, 2, 1), (1, 2), 1, False),
+    ((7, 8, 3, 2), (3, 2, 3, 5), 1, 1, 1, 1, True),
+]
+
+
+@pytest.mark.parametrize("xs,ws,stride,pad,dil,groups,flip", CONV_CASES)
+def test_conv_vs_bruteforce_and_torch(xs, ws, stride, pad, dil, groups, flip):
+    x, w = RNG.normal(size=xs), RNG.normal(size=ws)
+    cd = O.ConvDims(xs, ws, stride=stride, padding=pad, dilation=dil, groups=groups, flipkernel=flip)
+    y = O.conv(x, w, cd)
+    np.testing.assert_allclose(y, brute_conv(x, w, cd), rtol=1e-12, atol=1e-12)
+    # torch conv2d is cross-correlation over NCHW; flip the kernel spatially unless flipkernel
+    tx = torch.tensor(np.transpose(x, (3, 2, 1, 0)).copy(), requires_grad=True)      # N C H W
+    wk = w if flip else w[::-1, ::-1]
+    tw = torch.tensor(np.transpose(wk, (3, 2, 1, 0)).copy(), requires_grad=True)     # Cout Cin kH kW
+    p = cd.padding
+    txp = F.pad(tx, (p[0], p[1], p[2], p[3]))
+    ty = F.conv2d(txp, tw, None, stride=(cd.stride[1], cd.stride[0]), dilation=(cd.dilation[1], cd.dilation[0]),
+                  groups=groups)
+    np.testing.assert_allclose(y, np.transpose(ty.detach().numpy(), (3, 2, 1, 0)), rtol=1e-11, atol=1e-11)
+    delta = RNG.normal(size=y.shape)
+    ty.backward(torch.tensor(np.transpose(delta, (3, 2, 1, 0)).copy()))
+    dx = O.conv_data_grad(delta, w, cd)
+    dw = O.conv_filter_grad(x, delta, cd)
+    np.testing.assert_allclose(dx, np.transpose(tx.grad.numpy(), (3, 2, 1, 0)), rtol=1e-10, atol=1e-11)
+    twg = np.transpose(tw.grad.numpy(), (3, 2, 1, 0))
+    np.testing.assert_allclose(dw, twg if flip else twg[::-1, ::-1], rtol=1e-10, atol=1e-11)
+
+
+def test_fused_conv_pullback_finite_differences():
+    xs, ws = (5, 4, 2, 2), (3, 3, 2, 3)
+    x, w, b = RNG.normal(size=xs), RNG.normal(size=ws), RNG.normal(size=3)
+    cd = O.ConvDims(xs, ws, padding=1)
+    delta = RNG.normal(size=cd.y_shape())
+    y, dw, dx, db = O.fused_conv_pullback("gelu", w, x, b, cd, delta)
+    loss = lambda ww, xx, bb: (O.fused_conv_bias_activation("gelu", ww, xx, bb, cd) * delta).sum()
+    np.testing.assert_allclose(dw, fd_grad(lambda v: loss(v, x, b), w), rtol=2e-6, atol=1e-8)
+    np.testing.assert_allclose(dx, fd_grad(lambda v: loss(w, v, b), x), rtol=2e-6, atol=1e-8)
+    np.testing.assert_allclose(db, fd_grad(lambda v: loss(w, x, v), b), rtol=2e-6, atol=1e-8)
+
+
+# ----------------------------------------------------------------------------- helpers
+def test_generate_fixed_array_is_column_major():
+    a = O.generate_fixed_array(np.float32, (2, 3))
+    np.testing.assert_allclose(a, np.array([[1, 3, 5], [2, 4, 6]], np.float32) / 6)
+
+
+def test_bf16_round_trip_is_rne():
+    a = np.array([1.0, 1.00390625, 1.005859375, 3.140625, -2.5], np.float32)
+    r = O.round_to_bf16(a)
+    # 1 + 2^-8 is a tie between 1.0 and 1+2^-7 -> rounds to even (1.0)
+    assert r[0] == 1.0 and r[1] == 1.0 and r[2] == 1.0078125
+    t = torch.tensor(a).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(r, t)
+    big = RNG.normal(size=1000).astype(np.float32)
+    np.testing.assert_array_equal(O.round_to_bf16(big), torch.tensor(big).to(torch.bfloat16).float().numpy())
+
+
+def test_default_epsilon():
+    # utils.jl:130: eps(T)^(5/7)
+    assert abs(O.default_epsilon(np.float32) - (2.0 ** -23) ** (5 / 7)) < 1e-12
