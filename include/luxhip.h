@@ -1,0 +1,234 @@
+/*
+ * libluxhip -- C ABI of the MI355X (gfx950) backend for LuxLib's fused operators.
+ *
+ * The reference (LuxDL/Lux.jl, lib/LuxLib) has no C interface: a backend plugs in by adding
+ * Julia methods on LuxLib.Impl's device-dispatch points.  Every entry point below names the
+ * reference function(s) it stands behind (paths relative to lib/LuxLib/ of the reference).
+ *
+ * Conventions (modelled on the reference's vendor wrappers, ext/CUDAExt/cublaslt.jl:185-293
+ * and ext/cuDNNExt/batchnorm.jl:81-118,221-241):
+ *   - all tensors are dense, column-major (Julia order), passed as raw device pointers that
+ *     the library only borrows for the duration of the call;
+ *   - sizes are int64_t; leading dimensions are in elements;
+ *   - every op is enqueued on the given stream and returns without synchronising the host;
+ *   - return value: LUXHIP_OK, or a negative status.  LUXHIP_UNSUPPORTED (-1) means "this
+ *     dtype / activation / shape is not handled" and the caller falls back to its generic
+ *     path, exactly like cublaslt.jl:359-402; shape errors are expected to be raised by the
+ *     host *before* the call (impl/matmul.jl:21-34, api/groupnorm.jl:40-64) and come back as
+ *     LUXHIP_INVALID if they are not;
+ *   - no exception crosses the ABI; luxhip_last_error() returns the message of the last
+ *     failure on the calling thread;
+ *   - optional tensors are passed as NULL (Julia `nothing`);
+ *   - dtype selects the storage type of every tensor argument; arithmetic and reductions
+ *     are carried in fp32 for both storage types.  Saved statistics are always fp32.
+ */
+#ifndef LUXHIP_H
+#define LUXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LUXHIP_OK 0
+#define LUXHIP_UNSUPPORTED (-1)
+#define LUXHIP_INVALID (-2)
+#define LUXHIP_HIP_ERROR (-3)
+#define LUXHIP_NOT_INITIALIZED (-4)
+
+/* storage types */
+#define LUXHIP_F32 0
+#define LUXHIP_BF16 1
+
+/* activation ids.  tanh_fast / sigmoid_fast (NNlib.fast_act, src/layers/basic.jl:366-371 of
+ * the reference) map to TANH / SIGMOID on the host side. */
+#define LUXHIP_ACT_IDENTITY 0
+#define LUXHIP_ACT_RELU 1
+#define LUXHIP_ACT_TANH 2
+#define LUXHIP_ACT_SIGMOID 3
+#define LUXHIP_ACT_SWISH 4
+#define LUXHIP_ACT_GELU 5 /* tanh approximation (NNlib.gelu) */
+#define LUXHIP_ACT_SOFTPLUS 6
+#define LUXHIP_ACT_LOGSIGMOID 7
+#define LUXHIP_ACT_LISHT 8
+#define LUXHIP_ACT_COUNT 9
+
+typedef void* luxhip_stream_t; /* a hipStream_t; NULL is the null stream */
+typedef void* luxhip_event_t;  /* a hipEvent_t */
+
+/* ---------------------------------------------------------------- runtime ------------
+ * The reference leaves device buffers and streams to CUDA.jl / AMDGPU.jl (task-local
+ * handles, ext/CUDAExt/cublaslt.jl:80-82,156-178; CUDA.stream() :287).  This library owns
+ * them instead. */
+int luxhip_init(int device);
+int luxhip_shutdown(void);
+const char* luxhip_last_error(void);
+int luxhip_device_info(char* name, size_t name_len, int* compute_units, int64_t* total_mem);
+
+int luxhip_stream_create(luxhip_stream_t* out);
+int luxhip_stream_synchronize(luxhip_stream_t s);
+int luxhip_stream_destroy(luxhip_stream_t s);
+
+int luxhip_event_create(luxhip_event_t* out);
+int luxhip_event_record(luxhip_event_t e, luxhip_stream_t s);
+int luxhip_event_elapsed_ms(float* ms, luxhip_event_t start, luxhip_event_t stop); /* waits for stop */
+int luxhip_event_destroy(luxhip_event_t e);
+
+/* Pooled device allocator (size-bucketed free lists; luxhip_free returns the block to the
+ * pool, luxhip_trim releases the pool to the driver). */
+int luxhip_malloc(void** out, size_t bytes);
+int luxhip_free(void* p);
+int luxhip_trim(void);
+int luxhip_memcpy_h2d(void* dst, const void* src, size_t bytes, luxhip_stream_t s); /* synchronous w.r.t. host */
+int luxhip_memcpy_d2h(void* dst, const void* src, size_t bytes, luxhip_stream_t s); /* synchronous w.r.t. host */
+int luxhip_memcpy_d2d(void* dst, const void* src, size_t bytes, luxhip_stream_t s); /* asynchronous */
+int luxhip_fill_zero(void* dst, size_t bytes, luxhip_stream_t s);                   /* fill kernel, capturable */
+
+/* ---------------------------------------------------------------- bias_activation ----
+ * x, y, pre, delta, out, dx: (I, C, N) column-major, I = product of the leading dims,
+ * C = size(x, ndims-1), N = size(x, ndims).  bias, dbias: length C. */
+
+/* y = act.(x .+ bias).  Stands behind Impl.bias_activation!(y, ::GPUBroadcastOp, act, x, bias)
+ * (src/impl/bias_activation.jl:207-220) and Impl.activation! (src/impl/activation.jl:113-124)
+ * when bias == NULL.  y may alias x (bias_activation!!, :143-152).  If pre != NULL it
+ * receives x .+ bias (the `tmp` kept by the rrule, :86-95, and by bias_activation_cached!!,
+ * :312-351). */
+int luxhip_bias_activation_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                               const void* x, const void* bias, void* y, void* pre);
+
+/* dx = delta .* act'(out, pre);  dbias[c] = sum_{i,n} dx[i,c,n].  Stands behind
+ * Impl.∇activation(::GPUBroadcastOp, Δ, out, act, x) (src/impl/activation.jl:139-141) fused
+ * with Impl.∇bias_add / reduce_sum (src/impl/common_ops.jl:25-38), i.e. the pullbacks at
+ * src/impl/bias_activation.jl:76-95.  out may be NULL for IDENTITY; pre may be NULL for
+ * activations whose derivative needs only the output (identity, relu, tanh, sigmoid);
+ * dbias may be NULL; dx may alias delta. */
+int luxhip_bias_activation_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                               const void* delta, const void* out, const void* pre, void* dx, void* dbias);
+
+/* ---------------------------------------------------------------- batchnorm ----------
+ * x, y, delta, dx: (I, C, N); gamma, beta, rmean, rvar, rmean_out, rvar_out, dgamma, dbeta:
+ * length C in `dtype`; save_mean, save_invstd: length C, fp32. */
+
+/* Whole-op override of Impl.batchnorm (src/impl/batchnorm.jl:29-49; precedent
+ * ext/cuDNNExt/cuDNNExt.jl:26-54): statistics (compute_batch_statistics,
+ * src/impl/normalization.jl:116-143), running-stat update (:20-110,
+ * update_running_statistics_kernel! :78-93), and y = act(x*γ' + β')
+ * (batchnorm_affine_normalize_internal_kernel!, src/impl/batchnorm.jl:333-403).
+ * training != 0: batch statistics (biased variance); when rmean/rvar are given,
+ *   rmean_out = (1-m) rmean + m μ and rvar_out = (1-m) rvar + m n/(n-1) σ² are written
+ *   (new arrays; the inputs are not modified).
+ * training == 0: rmean/rvar are the statistics (batch statistics if they are NULL).
+ * gamma and beta are given together or both NULL.  save_mean / save_invstd (optional)
+ * receive μ and 1/sqrt(σ²+eps) for the pullback. */
+int luxhip_batchnorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                         const void* x, const void* gamma, const void* beta, const void* rmean,
+                         const void* rvar, int training, double momentum, double eps, void* y,
+                         void* rmean_out, void* rvar_out, float* save_mean, float* save_invstd);
+
+/* Complete pullback w.r.t. (x, γ, β): ∇activation, ∇batchnorm_affine_normalize
+ * (src/impl/batchnorm.jl:445-663) and the mean_var rrule (src/impl/common_ops.jl:45-61)
+ * in two passes over (delta, x).  The pre-activation is recomputed from x and the saved
+ * statistics, so no activation intermediate is needed.  stats_from_batch == 0 treats the
+ * statistics as constants (inference: only dx = ∂y γ').  dgamma / dbeta may be NULL. */
+int luxhip_batchnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                         const void* delta, const void* x, const void* gamma, const void* beta,
+                         const float* save_mean, const float* save_invstd, int stats_from_batch,
+                         void* dx, void* dgamma, void* dbeta);
+
+/* ---------------------------------------------------------------- groupnorm ----------
+ * x viewed as (I, C/G, G, N) (src/impl/groupnorm.jl:13-15,76): channel c = j + (C/G) k.
+ * gamma, beta, dgamma, dbeta: length C; save_mean, save_invstd: (G, N) fp32. */
+
+/* Impl.groupnorm (src/impl/groupnorm.jl:5-22) = statistics per (group, sample) +
+ * groupnorm_affine_normalize_kernel! (:315-347). */
+int luxhip_groupnorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t G, int64_t N,
+                         const void* x, const void* gamma, const void* beta, double eps, void* y,
+                         float* save_mean, float* save_invstd);
+
+/* Pullback: ∇groupnorm_affine_normalize (src/impl/groupnorm.jl:383-598) + mean_var rrule. */
+int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t G, int64_t N,
+                         const void* delta, const void* x, const void* gamma, const void* beta,
+                         const float* save_mean, const float* save_invstd, void* dx, void* dgamma,
+                         void* dbeta);
+
+/* ---------------------------------------------------------------- layernorm ----------
+ * x, y, delta, dx: (L, R): statistics over the L leading (contiguous) elements of each of
+ * the R columns.  gamma, beta, dgamma, dbeta: length L (elementwise affine over the
+ * normalised dims) or NULL; save_mean, save_invstd: length R, fp32.
+ * The reference has no device hook for layernorm (src/impl/layernorm.jl:3-14 is generic
+ * broadcasts); the host adds an Impl.layernorm method + rrule that call these. */
+int luxhip_layernorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t L, int64_t R, const void* x,
+                         const void* gamma, const void* beta, double eps, void* y, float* save_mean,
+                         float* save_invstd);
+int luxhip_layernorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t L, int64_t R, const void* delta,
+                         const void* x, const void* gamma, const void* beta, const float* save_mean,
+                         const float* save_invstd, void* dx, void* dgamma, void* dbeta);
+
+/* ---------------------------------------------------------------- dense --------------*/
+
+/* C (M x N) = op(A) * op(B) (+ bias broadcast down the columns).  Stands behind
+ * Impl.matmul!(C, ::GPUBroadcastOp, A, B) and Impl.matmuladd!(C, ::GPUBroadcastOp, A, B, bias)
+ * (src/impl/matmul.jl:85-94,120-125) including Adjoint/Transpose operands (transX != 0:
+ * the stored matrix is the transpose of the operand, as unwrapped by prepare_transposed,
+ * ext/CUDAExt/cublaslt.jl:15-33). */
+int luxhip_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                  const void* A, int64_t lda, const void* B, int64_t ldb, const void* bias, void* C,
+                  int64_t ldc);
+
+/* y (M x N) = act.(W (M x K) * x (K x N) .+ bias).  Stands behind
+ * Impl.fused_dense!(y, ::GPUBroadcastOp, act, W, x, b) (src/impl/dense.jl:46-69; precedent
+ * cublasLt_fused_dense!, ext/CUDAExt/cublaslt.jl:351-403).  If pre != NULL (M x N, ld =
+ * ldy) it receives the pre-activation W*x .+ bias (the cuBLASLt AUX output used by the gelu
+ * rrule, src/impl/dense.jl:116-134). */
+int luxhip_fused_dense_fwd(luxhip_stream_t s, int dtype, int act, int64_t M, int64_t K, int64_t N,
+                           const void* W, int64_t ldw, const void* x, int64_t ldx, const void* bias,
+                           void* y, int64_t ldy, void* pre);
+
+/* Pullback of fused_dense (src/impl/dense.jl:71-113, ∇matmul_bias :290-291):
+ * dz = delta .* act'(y, pre); dbias = sum over the batch of dz; dW = dz * x'; dx = W' * dz.
+ * delta, y, pre, dz: M x N contiguous; dW: M x K; dx: K x N contiguous.  dz is caller-
+ * provided scratch of M*N elements (may alias delta when delta may be overwritten; may be
+ * NULL for IDENTITY).  dbias, dW, dx may each be NULL to skip that output. */
+int luxhip_fused_dense_bwd(luxhip_stream_t s, int dtype, int act, int64_t M, int64_t K, int64_t N,
+                           const void* delta, const void* y, const void* pre, const void* W, int64_t ldw,
+                           const void* x, int64_t ldx, void* dz, void* dW, void* dx, void* dbias);
+
+/* ---------------------------------------------------------------- conv ---------------
+ * The fields of NNlib.DenseConvDims the path consumes (2 spatial dims, WHCN tensors):
+ * x (W, H, Cin, N); w (kW, kH, Cin/groups, Cout); y (OW, OH, Cout, N).
+ * flipkernel == 0 is true convolution (the DenseConvDims default used by Lux.Conv,
+ * src/layers/conv.jl:97-98 of the reference); != 0 is cross-correlation. */
+typedef struct luxhip_conv_dims {
+    int64_t W, H, Cin, N;
+    int64_t kW, kH, Cout;
+    int64_t stride_w, stride_h;
+    int64_t pad_w_lo, pad_w_hi, pad_h_lo, pad_h_hi;
+    int64_t dil_w, dil_h;
+    int64_t groups;
+    int64_t flipkernel;
+} luxhip_conv_dims_t;
+
+/* y = act.(conv(x, w) .+ bias[cout]).  Stands behind Impl.conv!(y, ::Type{Dev}, x, w, cdims)
+ * (bias == NULL, act identity) and Impl.conv_bias_act(::Type{Dev}, x, w, cdims, bias, act)
+ * (src/impl/conv.jl:29-60,138-166).  pre (optional) receives conv .+ bias. */
+int luxhip_conv_fwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d, const void* x,
+                    const void* w, const void* bias, void* y, void* pre);
+/* dx = ∇conv_data(dy, w, cdims) (src/impl/conv.jl:128-131). */
+int luxhip_conv_bwd_data(luxhip_stream_t s, int dtype, const luxhip_conv_dims_t* d, const void* dy,
+                         const void* w, void* dx);
+/* dw = ∇conv_filter(x, dy, cdims) (src/impl/conv.jl:133-136). */
+int luxhip_conv_bwd_filter(luxhip_stream_t s, int dtype, const luxhip_conv_dims_t* d, const void* x,
+                           const void* dy, void* dw);
+/* ∇fused_conv (src/impl/conv.jl:261-275): dz = delta .* act'(y, pre); dbias = sum_{w,h,n} dz;
+ * dw = ∇conv_filter(x, dz); dx = ∇conv_data(dz, w).  dz: caller scratch like
+ * luxhip_fused_dense_bwd. */
+int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d,
+                          const void* delta, const void* y, const void* pre, const void* x, const void* w,
+                          void* dz, void* dw, void* dx, void* dbias);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LUXHIP_H */

@@ -1,0 +1,276 @@
+// Shared host + device helpers of libluxhip (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/luxhip.h"
+
+namespace luxhip {
+
+// ----------------------------------------------------------------------------- host side
+int set_error(int status, const char* fmt, ...);
+bool initialized();
+int num_cus();
+
+// Per-stream scratch owned by the library.  Layout: [counters | data].  The counter region
+// (kCounterBytes, zero on creation) backs the "last workgroup finishes the reduction"
+// pattern; every kernel that uses a counter resets it to zero before it exits, so the
+// region is all-zero between launches.  get_workspace grows the data region on demand.
+constexpr size_t kCounterBytes = 64 * 1024;
+struct Workspace {
+    unsigned int* counters;  // kCounterBytes / 4 entries, zero between launches
+    char* data;              // >= the requested number of bytes, 256-byte aligned
+};
+int get_workspace(hipStream_t s, size_t bytes, Workspace* out);
+
+#define LUX_CHECK_HIP(expr)                                                                     \
+    do {                                                                                        \
+        hipError_t _e = (expr);                                                                 \
+        if (_e != hipSuccess)                                                                   \
+            return ::luxhip::set_error(LUXHIP_HIP_ERROR, "%s failed: %s (%s:%d)", #expr,        \
+                                       hipGetErrorString(_e), __FILE__, __LINE__);              \
+    } while (0)
+
+#define LUX_CHECK_LAUNCH()                                                                      \
+    do {                                                                                        \
+        hipError_t _e = hipGetLastError();                                                      \
+        if (_e != hipSuccess)                                                                   \
+            return ::luxhip::set_error(LUXHIP_HIP_ERROR, "kernel launch failed: %s (%s:%d)",    \
+                                       hipGetErrorString(_e), __FILE__, __LINE__);              \
+    } while (0)
+
+#define LUX_REQUIRE_INIT()                                                                      \
+    do {                                                                                        \
+        if (!::luxhip::initialized())                                                           \
+            return ::luxhip::set_error(LUXHIP_NOT_INITIALIZED, "luxhip_init has not been called"); \
+    } while (0)
+
+#define LUX_INVALID_IF(cond, ...)                                                               \
+    do {                                                                                        \
+        if (cond) return ::luxhip::set_error(LUXHIP_INVALID, __VA_ARGS__);                      \
+    } while (0)
+
+#define LUX_UNSUPPORTED_IF(cond, ...)                                                           \
+    do {                                                                                        \
+        if (cond) return ::luxhip::set_error(LUXHIP_UNSUPPORTED, __VA_ARGS__);                  \
+    } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Division of a 31-bit numerator by a fixed divisor with one multiply-high and a shift
+// (round-up method of Granlund & Montgomery).  Valid for 0 <= n < 2^31, 1 <= d < 2^31.
+struct FastDiv {
+    uint32_t d, m, l;
+    FastDiv() : d(1), m(0), l(0) {}
+    explicit FastDiv(uint32_t div) : d(div) {
+        l = 0;
+        while ((1ull << l) < div) ++l;
+        m = (uint32_t)(((1ull << 32) * ((1ull << l) - div)) / div + 1);
+    }
+    __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        uint32_t t = __umulhi(n, m);
+#else
+        uint32_t t = (uint32_t)(((uint64_t)n * m) >> 32);
+#endif
+        return (t + n) >> l;
+    }
+};
+
+// ----------------------------------------------------------------------------- storage types
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    // round to nearest even; NaN stays NaN
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+template <typename T>
+struct Vec;  // 16-byte vector access
+template <>
+struct Vec<float> {
+    static constexpr int N = 4;
+    __device__ __forceinline__ static void load(const float* p, float (&v)[4]) {
+        float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    __device__ __forceinline__ static void store(float* p, const float (&v)[4]) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+};
+template <>
+struct Vec<bf16_t> {
+    static constexpr int N = 8;
+    __device__ __forceinline__ static void load(const bf16_t* p, float (&v)[8]) {
+        uint4 t = *reinterpret_cast<const uint4*>(p);
+        uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    __device__ __forceinline__ static void store(bf16_t* p, const float (&v)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+        *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ float ld(const T* p);
+template <>
+__device__ __forceinline__ float ld<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float ld<bf16_t>(const bf16_t* p) { return bf16_to_f32(*p); }
+template <typename T>
+__device__ __forceinline__ void st(T* p, float v);
+template <>
+__device__ __forceinline__ void st<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void st<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// ----------------------------------------------------------------------------- activations
+// value f(x) and the derivative LuxLib multiplies the cotangent by, given the output `o`
+// and the pre-activation `x`.
+template <int ACT>
+struct Act;
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+template <>
+struct Act<LUXHIP_ACT_IDENTITY> {
+    static constexpr bool needs_pre = false;
+    __device__ __forceinline__ static float f(float x) { return x; }
+    __device__ __forceinline__ static float d(float, float) { return 1.0f; }
+};
+template <>
+struct Act<LUXHIP_ACT_RELU> {
+    static constexpr bool needs_pre = false;
+    __device__ __forceinline__ static float f(float x) { return fmaxf(x, 0.0f); }
+    __device__ __forceinline__ static float d(float o, float) { return o > 0.0f ? 1.0f : 0.0f; }
+};
+template <>
+struct Act<LUXHIP_ACT_TANH> {
+    static constexpr bool needs_pre = false;
+    __device__ __forceinline__ static float f(float x) { return tanhf(x); }
+    __device__ __forceinline__ static float d(float o, float) { return 1.0f - o * o; }
+};
+template <>
+struct Act<LUXHIP_ACT_SIGMOID> {
+    static constexpr bool needs_pre = false;
+    __device__ __forceinline__ static float f(float x) { return sigmoidf_(x); }
+    __device__ __forceinline__ static float d(float o, float) { return o * (1.0f - o); }
+};
+template <>
+struct Act<LUXHIP_ACT_SWISH> {
+    static constexpr bool needs_pre = true;
+    __device__ __forceinline__ static float f(float x) { return x * sigmoidf_(x); }
+    __device__ __forceinline__ static float d(float o, float x) { return o + sigmoidf_(x) * (1.0f - o); }
+};
+template <>
+struct Act<LUXHIP_ACT_GELU> {
+    static constexpr bool needs_pre = true;
+    __device__ __forceinline__ static float f(float x) {
+        float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+        return 0.5f * x * (1.0f + tanhf(u));
+    }
+    __device__ __forceinline__ static float d(float, float x) {
+        float x2 = x * x;
+        float u = 0.7978845608028654f * (x + 0.044715f * x2 * x);
+        float t = tanhf(u);
+        float du = 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x2);
+        return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * du;
+    }
+};
+template <>
+struct Act<LUXHIP_ACT_SOFTPLUS> {
+    static constexpr bool needs_pre = true;
+    __device__ __forceinline__ static float f(float x) { return log1pf(expf(-fabsf(x))) + fmaxf(x, 0.0f); }
+    __device__ __forceinline__ static float d(float, float x) { return sigmoidf_(x); }
+};
+template <>
+struct Act<LUXHIP_ACT_LOGSIGMOID> {
+    static constexpr bool needs_pre = true;
+    __device__ __forceinline__ static float f(float x) { return -(log1pf(expf(-fabsf(x))) + fmaxf(-x, 0.0f)); }
+    __device__ __forceinline__ static float d(float, float x) { return sigmoidf_(-x); }
+};
+template <>
+struct Act<LUXHIP_ACT_LISHT> {
+    static constexpr bool needs_pre = true;
+    __device__ __forceinline__ static float f(float x) { return x * tanhf(x); }
+    __device__ __forceinline__ static float d(float, float x) {
+        float t = tanhf(x);
+        return t + x * (1.0f - t * t);
+    }
+};
+
+inline bool act_needs_pre(int act) {
+    return act == LUXHIP_ACT_SWISH || act == LUXHIP_ACT_GELU || act == LUXHIP_ACT_SOFTPLUS ||
+           act == LUXHIP_ACT_LOGSIGMOID || act == LUXHIP_ACT_LISHT;
+}
+
+// Expands `CALL(ActId)` for the runtime activation id.
+#define LUX_DISPATCH_ACT(act, CALL)                                      \
+    switch (act) {                                                       \
+        case LUXHIP_ACT_IDENTITY: CALL(LUXHIP_ACT_IDENTITY); break;      \
+        case LUXHIP_ACT_RELU: CALL(LUXHIP_ACT_RELU); break;              \
+        case LUXHIP_ACT_TANH: CALL(LUXHIP_ACT_TANH); break;              \
+        case LUXHIP_ACT_SIGMOID: CALL(LUXHIP_ACT_SIGMOID); break;        \
+        case LUXHIP_ACT_SWISH: CALL(LUXHIP_ACT_SWISH); break;            \
+        case LUXHIP_ACT_GELU: CALL(LUXHIP_ACT_GELU); break;              \
+        case LUXHIP_ACT_SOFTPLUS: CALL(LUXHIP_ACT_SOFTPLUS); break;      \
+        case LUXHIP_ACT_LOGSIGMOID: CALL(LUXHIP_ACT_LOGSIGMOID); break;  \
+        case LUXHIP_ACT_LISHT: CALL(LUXHIP_ACT_LISHT); break;            \
+        default: break;                                                  \
+    }
+
+// ----------------------------------------------------------------------------- reductions
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Sum over the workgroup; every thread receives the total.  `smem` needs blockDim.x/64
+// floats; contains a trailing barrier so it can be reused immediately.
+__device__ __forceinline__ float block_sum(float v, float* smem) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    if (nw == 1) return v;
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int i = 0; i < nw; ++i) t += smem[i];
+    __syncthreads();
+    return t;
+}
+
+// Marks this workgroup as finished with its partial result and tells whether it is the
+// last of `total` workgroups sharing `counter` (which it then resets).  All threads of the
+// workgroup must call it; partial results must be written to global memory before the call
+// and may be read (by the last workgroup) after it.
+__device__ __forceinline__ bool last_block_done(unsigned int* counter, unsigned int total) {
+    __shared__ bool is_last;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned int prev = atomicAdd(counter, 1u);
+        is_last = (prev == total - 1);
+        if (is_last) *counter = 0u;
+    }
+    __syncthreads();
+    bool r = is_last;
+    if (r) __threadfence();
+    return r;
+}
+
+}  // namespace luxhip

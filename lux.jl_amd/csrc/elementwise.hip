@@ -1,0 +1,396 @@
+// bias_activation forward / pullback: HBM-bound streaming kernels.
+//
+// Tensor view: (I, C, N) column-major; element (i, c, n) lives at (n*C + c)*I + i.
+// Two reduction layouts for dbias[c] = sum_{i,n} dx[i,c,n]:
+//   "channel": workgroup (s, c) streams a slice of channel c's I*N elements (rows of I
+//              contiguous elements) -- used when rows are long enough to coalesce;
+//   "plane":   the I*C elements of one n are contiguous; a thread owns VEC consecutive plane
+//              positions and walks over n -- used when I is small (dense layers: I == 1).
+// Reductions are deterministic: per-workgroup partials are combined in a fixed order.
+#include <algorithm>
+
+#include "common.h"
+
+namespace luxhip {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 1;  // one 16-byte vector per thread and a huge grid streams fastest on MI355X
+
+// ------------------------------------------------------------------------------- forward
+template <typename T, int ACT, int VEC, bool HAS_BIAS, bool WRITE_PRE>
+__global__ __launch_bounds__(kThreads) void bias_act_fwd_kernel(const T* __restrict__ x, const T* __restrict__ bias,
+                                                                T* y, T* pre, uint32_t total_vec, FastDiv rowdiv,
+                                                                FastDiv cdiv, uint32_t C) {
+    // rowdiv divides a vector index by the number of vectors per row (I / VEC)
+    for (uint32_t base = blockIdx.x * (kThreads * kUnroll); base < total_vec; base += gridDim.x * (kThreads * kUnroll)) {
+        float v[kUnroll][VEC];
+        uint32_t idx[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            idx[u] = base + u * kThreads + threadIdx.x;
+            if (idx[u] < total_vec) {
+                if constexpr (VEC == 1) v[u][0] = ld(x + idx[u]);
+                else Vec<T>::load(x + (size_t)idx[u] * VEC, v[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (idx[u] < total_vec) {
+                float b = 0.0f;
+                if constexpr (HAS_BIAS) {
+                    uint32_t row = rowdiv.div(idx[u]);
+                    uint32_t c = row - cdiv.div(row) * C;
+                    b = ld(bias + c);
+                }
+                float p[VEC], o[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    p[k] = v[u][k] + b;
+                    o[k] = Act<ACT>::f(p[k]);
+                }
+                if constexpr (VEC == 1) {
+                    if constexpr (WRITE_PRE) st(pre + idx[u], p[0]);
+                    st(y + idx[u], o[0]);
+                } else {
+                    if constexpr (WRITE_PRE) Vec<T>::store(pre + (size_t)idx[u] * VEC, p);
+                    Vec<T>::store(y + (size_t)idx[u] * VEC, o);
+                }
+            }
+        }
+    }
+}
+
+// Plane layout with the bias varying inside a vector (I < VEC, e.g. dense layers where
+// I == 1): element e of the flat tensor belongs to channel (e / I) % C.
+template <typename T, int ACT, int VEC, bool WRITE_PRE>
+__global__ __launch_bounds__(kThreads) void bias_act_fwd_smallI_kernel(const T* __restrict__ x,
+                                                                       const T* __restrict__ bias, T* y, T* pre,
+                                                                       uint32_t total_vec, FastDiv idiv, FastDiv cdiv,
+                                                                       uint32_t C) {
+    for (uint32_t base = blockIdx.x * (kThreads * kUnroll); base < total_vec; base += gridDim.x * (kThreads * kUnroll)) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            uint32_t idx = base + u * kThreads + threadIdx.x;
+            if (idx < total_vec) {
+                float v[VEC], p[VEC], o[VEC];
+                Vec<T>::load(x + (size_t)idx * VEC, v);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    uint32_t row = idiv.div(idx * VEC + k);
+                    uint32_t c = row - cdiv.div(row) * C;
+                    p[k] = v[k] + ld(bias + c);
+                    o[k] = Act<ACT>::f(p[k]);
+                }
+                if constexpr (WRITE_PRE) Vec<T>::store(pre + (size_t)idx * VEC, p);
+                Vec<T>::store(y + (size_t)idx * VEC, o);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------- pullback
+template <typename T, int ACT, int VEC>
+__device__ __forceinline__ void dx_vec(const T* delta, const T* out, const T* pre, size_t off, float (&dx)[VEC]) {
+    float d[VEC], o[VEC], p[VEC];
+    if constexpr (VEC == 1) {
+        d[0] = ld(delta + off);
+        if constexpr (ACT != LUXHIP_ACT_IDENTITY && !Act<ACT>::needs_pre) o[0] = ld(out + off);
+        if constexpr (Act<ACT>::needs_pre) p[0] = ld(pre + off);
+    } else {
+        Vec<T>::load(delta + off, d);
+        if constexpr (ACT != LUXHIP_ACT_IDENTITY && !Act<ACT>::needs_pre) Vec<T>::load(out + off, o);
+        if constexpr (Act<ACT>::needs_pre) Vec<T>::load(pre + off, p);
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        if constexpr (ACT == LUXHIP_ACT_IDENTITY) dx[k] = d[k];
+        else if constexpr (Act<ACT>::needs_pre) dx[k] = d[k] * Act<ACT>::d(Act<ACT>::f(p[k]), p[k]);
+        else dx[k] = d[k] * Act<ACT>::d(o[k], 0.0f);
+    }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(T* p, size_t off, const float (&v)[VEC]) {
+    if constexpr (VEC == 1) st(p + off, v[0]);
+    else Vec<T>::store(p + off, v);
+}
+
+// dx only (no bias gradient): flat streaming.
+template <typename T, int ACT, int VEC>
+__global__ __launch_bounds__(kThreads) void act_bwd_kernel(const T* __restrict__ delta, const T* __restrict__ out,
+                                                           const T* __restrict__ pre, T* dx, uint32_t total_vec) {
+    for (uint32_t base = blockIdx.x * (kThreads * kUnroll); base < total_vec; base += gridDim.x * (kThreads * kUnroll)) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            uint32_t idx = base + u * kThreads + threadIdx.x;
+            if (idx < total_vec) {
+                float r[VEC];
+                dx_vec<T, ACT, VEC>(delta, out, pre, (size_t)idx * VEC, r);
+                store_vec<T, VEC>(dx, (size_t)idx * VEC, r);
+            }
+        }
+    }
+}
+
+// "channel" layout: grid (S, C).  Workgroup (s, c) handles vectors [s*chunk, (s+1)*chunk) of
+// the nq = I*N/VEC vectors of channel c, writes its partial sum and the last workgroup of
+// the channel adds the S partials in order.
+template <typename T, int ACT, int VEC>
+__global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T* __restrict__ delta,
+                                                                        const T* __restrict__ out,
+                                                                        const T* __restrict__ pre, T* dx, T* dbias,
+                                                                        float* partial, unsigned int* counters,
+                                                                        uint32_t nq, uint32_t chunk, FastDiv rowdiv,
+                                                                        uint32_t vec_per_row, uint32_t C) {
+    __shared__ float smem[kThreads / 64];
+    const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
+    const uint32_t q0 = s * chunk;
+    const uint32_t q1 = min(q0 + chunk, nq);
+    float acc = 0.0f;
+    for (uint32_t q = q0 + threadIdx.x; q < q1; q += kThreads) {
+        const uint32_t n = rowdiv.div(q);
+        const size_t off = ((size_t)q + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
+        float r[VEC];
+        dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
+        store_vec<T, VEC>(dx, off, r);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc += r[k];
+    }
+    acc = block_sum(acc, smem);
+    if (threadIdx.x == 0) partial[(size_t)c * S + s] = acc;
+    if (last_block_done(counters + c, S)) {
+        float t = threadIdx.x < S ? partial[(size_t)c * S + threadIdx.x] : 0.0f;   // S <= kThreads
+        t = block_sum(t, smem);
+        if (threadIdx.x == 0) st(dbias + c, t);
+    }
+}
+
+// "plane" layout: P = I*C contiguous elements per n.  grid (ceil(P/(T*VEC)), S); a thread
+// owns VEC consecutive plane positions and sums over the n of its slice.
+template <typename T, int ACT, int VEC>
+__global__ __launch_bounds__(kThreads) void bias_act_bwd_plane_kernel(const T* __restrict__ delta,
+                                                                      const T* __restrict__ out,
+                                                                      const T* __restrict__ pre, T* dx, float* partial,
+                                                                      uint32_t P, uint32_t N, uint32_t n_per_slice) {
+    const uint32_t p = (blockIdx.x * kThreads + threadIdx.x) * VEC;
+    if (p >= P) return;
+    const uint32_t n0 = blockIdx.y * n_per_slice, n1 = min(n0 + n_per_slice, N);
+    float acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+    for (uint32_t n = n0; n < n1; ++n) {
+        const size_t off = (size_t)n * P + p;
+        float r[VEC];
+        dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
+        store_vec<T, VEC>(dx, off, r);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] += r[k];
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) partial[(size_t)blockIdx.y * P + p + k] = acc[k];
+}
+
+// dbias[c] = sum_s sum_{i<I} partial[s][c*I + i]; one wave per channel.
+template <typename T>
+__global__ __launch_bounds__(64) void plane_finalize_kernel(const float* __restrict__ partial, T* dbias, uint32_t P,
+                                                            uint32_t I, uint32_t S) {
+    const uint32_t c = blockIdx.x;
+    float acc = 0.0f;
+    const uint32_t cnt = S * I;
+    for (uint32_t t = threadIdx.x; t < cnt; t += 64) {
+        const uint32_t s = t / I, i = t - s * I;
+        acc += partial[(size_t)s * P + (size_t)c * I + i];
+    }
+    acc = wave_sum(acc);
+    if (threadIdx.x == 0) st(dbias + c, acc);
+}
+
+static inline unsigned grid_for(uint32_t total_vec) {
+    return (unsigned)ceil_div(total_vec, kThreads * kUnroll);
+}
+
+template <typename T>
+static int bias_act_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, const T* x, const T* bias, T* y,
+                             T* pre) {
+    constexpr int V = Vec<T>::N;
+    const int64_t total = I * C * N;
+    const bool ptr_ok = aligned16(x) && aligned16(y) && (pre == nullptr || aligned16(pre));
+    const FastDiv cdiv((uint32_t)C);
+#define LAUNCH_FWD(A)                                                                                              \
+    do {                                                                                                           \
+        if (ptr_ok && I % V == 0) {                                                                                \
+            const uint32_t tv = (uint32_t)(total / V);                                                             \
+            const FastDiv rowdiv((uint32_t)(I / V));                                                               \
+            if (bias && pre)                                                                                       \
+                bias_act_fwd_kernel<T, A, V, true, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+            else if (bias)                                                                                         \
+                bias_act_fwd_kernel<T, A, V, true, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+            else if (pre)                                                                                          \
+                bias_act_fwd_kernel<T, A, V, false, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+            else                                                                                                   \
+                bias_act_fwd_kernel<T, A, V, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+        } else if (ptr_ok && bias && total % V == 0) {                                                             \
+            const uint32_t tv = (uint32_t)(total / V);                                                             \
+            const FastDiv idiv((uint32_t)I);                                                                       \
+            if (pre)                                                                                               \
+                bias_act_fwd_smallI_kernel<T, A, V, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, idiv, cdiv, (uint32_t)C); \
+            else                                                                                                   \
+                bias_act_fwd_smallI_kernel<T, A, V, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, idiv, cdiv, (uint32_t)C); \
+        } else if (ptr_ok && !bias && total % V == 0) {                                                            \
+            const uint32_t tv = (uint32_t)(total / V);                                                             \
+            if (pre)                                                                                               \
+                bias_act_fwd_kernel<T, A, V, false, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, cdiv, cdiv, (uint32_t)C); \
+            else                                                                                                   \
+                bias_act_fwd_kernel<T, A, V, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, cdiv, cdiv, (uint32_t)C); \
+        } else {                                                                                                   \
+            const uint32_t tv = (uint32_t)total;                                                                   \
+            const FastDiv rowdiv((uint32_t)I);                                                                     \
+            if (bias && pre)                                                                                       \
+                bias_act_fwd_kernel<T, A, 1, true, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+            else if (bias)                                                                                         \
+                bias_act_fwd_kernel<T, A, 1, true, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+            else if (pre)                                                                                          \
+                bias_act_fwd_kernel<T, A, 1, false, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+            else                                                                                                   \
+                bias_act_fwd_kernel<T, A, 1, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+        }                                                                                                          \
+    } while (0)
+    LUX_DISPATCH_ACT(act, LAUNCH_FWD);
+#undef LAUNCH_FWD
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, const T* delta, const T* out,
+                             const T* pre, T* dx, T* dbias) {
+    constexpr int V = Vec<T>::N;
+    const int64_t total = I * C * N;
+    const bool ptr_ok = aligned16(delta) && aligned16(dx) && (out == nullptr || aligned16(out)) &&
+                        (pre == nullptr || aligned16(pre));
+    if (dbias == nullptr) {
+#define LAUNCH_ACT_BWD(A)                                                                                   \
+    do {                                                                                                    \
+        if (ptr_ok && total % V == 0) {                                                                     \
+            const uint32_t tv = (uint32_t)(total / V);                                                      \
+            act_bwd_kernel<T, A, V><<<grid_for(tv), kThreads, 0, s>>>(delta, out, pre, dx, tv);             \
+        } else {                                                                                            \
+            act_bwd_kernel<T, A, 1><<<grid_for((uint32_t)total), kThreads, 0, s>>>(delta, out, pre, dx, (uint32_t)total); \
+        }                                                                                                   \
+    } while (0)
+        LUX_DISPATCH_ACT(act, LAUNCH_ACT_BWD);
+#undef LAUNCH_ACT_BWD
+        LUX_CHECK_LAUNCH();
+        return LUXHIP_OK;
+    }
+
+    const bool channel_layout = I >= 64 && C <= (int64_t)(kCounterBytes / sizeof(unsigned int));
+    if (channel_layout) {
+        const bool vec = ptr_ok && I % V == 0;
+        const int vv = vec ? V : 1;
+        const uint32_t nq = (uint32_t)(I * N / vv);
+        int64_t S = ceil_div(nq, kThreads);
+        const int64_t smax = std::min<int64_t>(kThreads, std::max<int64_t>(1, 16384 / C));
+        if (S > smax) S = smax;
+        if (S < 1) S = 1;
+        const uint32_t chunk = (uint32_t)ceil_div(nq, S);
+        S = ceil_div(nq, chunk);
+        Workspace ws;
+        int rc = get_workspace(s, (size_t)C * S * sizeof(float), &ws);
+        if (rc != LUXHIP_OK) return rc;
+        float* partial = reinterpret_cast<float*>(ws.data);
+        const FastDiv rowdiv((uint32_t)(I / vv));
+        dim3 grid((unsigned)S, (unsigned)C);
+#define LAUNCH_CH(A)                                                                                               \
+    do {                                                                                                           \
+        if (vec)                                                                                                   \
+            bias_act_bwd_channel_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, ws.counters, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+        else                                                                                                       \
+            bias_act_bwd_channel_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, ws.counters, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+    } while (0)
+        LUX_DISPATCH_ACT(act, LAUNCH_CH);
+#undef LAUNCH_CH
+        LUX_CHECK_LAUNCH();
+        return LUXHIP_OK;
+    }
+
+    // plane layout
+    const int64_t P = I * C;
+    const bool vec = ptr_ok && P % V == 0;
+    const int vv = vec ? V : 1;
+    const int64_t gx = ceil_div(P, (int64_t)kThreads * vv);
+    int64_t S = std::max<int64_t>(1, std::min<int64_t>(ceil_div(N, 8), ceil_div(2048, gx)));
+    const uint32_t n_per_slice = (uint32_t)ceil_div(N, S);
+    S = ceil_div(N, n_per_slice);
+    LUX_UNSUPPORTED_IF(S > 65535, "bias_activation_bwd: batch split too large");
+    Workspace ws;
+    int rc = get_workspace(s, (size_t)P * S * sizeof(float), &ws);
+    if (rc != LUXHIP_OK) return rc;
+    float* partial = reinterpret_cast<float*>(ws.data);
+    dim3 grid((unsigned)gx, (unsigned)S);
+#define LAUNCH_PL(A)                                                                                               \
+    do {                                                                                                           \
+        if (vec)                                                                                                   \
+            bias_act_bwd_plane_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, (uint32_t)P, (uint32_t)N, n_per_slice); \
+        else                                                                                                       \
+            bias_act_bwd_plane_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, (uint32_t)P, (uint32_t)N, n_per_slice); \
+    } while (0)
+    LUX_DISPATCH_ACT(act, LAUNCH_PL);
+#undef LAUNCH_PL
+    LUX_CHECK_LAUNCH();
+    plane_finalize_kernel<T><<<(unsigned)C, 64, 0, s>>>(partial, dbias, (uint32_t)P, (uint32_t)I, (uint32_t)S);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+static int check_common(int dtype, int act, int64_t I, int64_t C, int64_t N) {
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_UNSUPPORTED_IF(act < 0 || act >= LUXHIP_ACT_COUNT, "unsupported activation id %d", act);
+    LUX_INVALID_IF(I < 0 || C < 0 || N < 0, "negative dimension (%lld, %lld, %lld)", (long long)I, (long long)C, (long long)N);
+    // 31-bit element indexing inside the kernels
+    if (I > 0 && C > 0 && N > 0) {
+        const long double tot = (long double)I * (long double)C * (long double)N;
+        LUX_UNSUPPORTED_IF(tot >= 2147483648.0L, "tensors of 2^31 or more elements are not supported");
+    }
+    return LUXHIP_OK;
+}
+
+}  // namespace luxhip
+
+using namespace luxhip;
+
+extern "C" {
+
+int luxhip_bias_activation_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* x,
+                               const void* bias, void* y, void* pre) {
+    LUX_REQUIRE_INIT();
+    int rc = check_common(dtype, act, I, C, N);
+    if (rc != LUXHIP_OK) return rc;
+    if (I * C * N == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(x == nullptr || y == nullptr, "bias_activation_fwd: x and y must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return bias_act_fwd_impl<float>((hipStream_t)s, act, I, C, N, (const float*)x, (const float*)bias, (float*)y, (float*)pre);
+    return bias_act_fwd_impl<bf16_t>((hipStream_t)s, act, I, C, N, (const bf16_t*)x, (const bf16_t*)bias, (bf16_t*)y, (bf16_t*)pre);
+}
+
+int luxhip_bias_activation_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                               const void* delta, const void* out, const void* pre, void* dx, void* dbias) {
+    LUX_REQUIRE_INIT();
+    int rc = check_common(dtype, act, I, C, N);
+    if (rc != LUXHIP_OK) return rc;
+    if (I * C * N == 0) {
+        if (dbias != nullptr && C > 0) return luxhip_fill_zero(dbias, (size_t)C * (dtype == LUXHIP_F32 ? 4 : 2), s);
+        return LUXHIP_OK;
+    }
+    LUX_INVALID_IF(delta == nullptr || dx == nullptr, "bias_activation_bwd: delta and dx must not be NULL");
+    LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && !act_needs_pre(act) && out == nullptr,
+                   "bias_activation_bwd: activation %d needs `out`", act);
+    LUX_INVALID_IF(act_needs_pre(act) && pre == nullptr, "bias_activation_bwd: activation %d needs `pre`", act);
+    if (dtype == LUXHIP_F32)
+        return bias_act_bwd_impl<float>((hipStream_t)s, act, I, C, N, (const float*)delta, (const float*)out,
+                                        (const float*)pre, (float*)dx, (float*)dbias);
+    return bias_act_bwd_impl<bf16_t>((hipStream_t)s, act, I, C, N, (const bf16_t*)delta, (const bf16_t*)out,
+                                     (const bf16_t*)pre, (bf16_t*)dx, (bf16_t*)dbias);
+}
+
+}  // extern "C"

@@ -1,0 +1,279 @@
+// libluxhip runtime: context, error reporting, streams, events, pooled device memory and
+// the per-stream workspace used by the reduction kernels.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace luxhip {
+
+namespace {
+thread_local char g_err[512] = "";
+std::mutex g_mu;
+bool g_init = false;
+int g_device = -1;
+int g_cus = 0;
+
+struct Pool {
+    std::multimap<size_t, void*> free_blocks;       // rounded size -> block
+    std::unordered_map<void*, size_t> live;         // block -> rounded size
+} g_pool;
+
+struct WsEntry {
+    void* base = nullptr;
+    size_t data_bytes = 0;
+};
+std::map<hipStream_t, WsEntry> g_ws;
+
+size_t round_size(size_t b) {
+    if (b == 0) b = 1;
+    if (b <= (1u << 20)) return (b + 511) & ~size_t(511);               // 512 B granules
+    return (b + (size_t(2) << 20) - 1) & ~((size_t(2) << 20) - 1);      // 2 MiB granules
+}
+}  // namespace
+
+int set_error(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+bool initialized() { return g_init; }
+int num_cus() { return g_cus; }
+
+int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    WsEntry& e = g_ws[s];
+    if (e.base == nullptr || e.data_bytes < bytes) {
+        size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : round_size(bytes);
+        if (e.base != nullptr) {
+            // the old block may still be in use by kernels queued on this stream
+            LUX_CHECK_HIP(hipStreamSynchronize(s));
+            LUX_CHECK_HIP(hipFree(e.base));
+            e.base = nullptr;
+        }
+        void* p = nullptr;
+        LUX_CHECK_HIP(hipMalloc(&p, kCounterBytes + want));
+        LUX_CHECK_HIP(hipMemset(p, 0, kCounterBytes));
+        LUX_CHECK_HIP(hipDeviceSynchronize());
+        e.base = p;
+        e.data_bytes = want;
+    }
+    out->counters = reinterpret_cast<unsigned int*>(e.base);
+    out->data = reinterpret_cast<char*>(e.base) + kCounterBytes;
+    return LUXHIP_OK;
+}
+
+__global__ void fill_zero_kernel(uint32_t* p, size_t nwords) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < nwords; i += stride) p[i] = 0u;
+}
+__global__ void fill_zero_bytes_kernel(uint8_t* p, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+}  // namespace luxhip
+
+using namespace luxhip;
+
+extern "C" {
+
+int luxhip_init(int device) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int n = 0;
+    LUX_CHECK_HIP(hipGetDeviceCount(&n));
+    if (n <= 0) return set_error(LUXHIP_HIP_ERROR, "no HIP device visible");
+    if (device < 0 || device >= n) return set_error(LUXHIP_INVALID, "device %d out of range (0..%d)", device, n - 1);
+    if (g_init && device == g_device) return LUXHIP_OK;
+    if (g_init) return set_error(LUXHIP_INVALID, "already initialised on device %d", g_device);
+    LUX_CHECK_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    LUX_CHECK_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(LUXHIP_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
+                         prop.gcnArchName);
+    g_cus = prop.multiProcessorCount;
+    g_device = device;
+    g_init = true;
+    return LUXHIP_OK;
+}
+
+int luxhip_shutdown(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_init) return LUXHIP_OK;
+    (void)hipDeviceSynchronize();
+    for (auto& kv : g_ws)
+        if (kv.second.base) (void)hipFree(kv.second.base);
+    g_ws.clear();
+    for (auto& kv : g_pool.free_blocks) (void)hipFree(kv.second);
+    g_pool.free_blocks.clear();
+    for (auto& kv : g_pool.live) (void)hipFree(kv.first);
+    g_pool.live.clear();
+    g_init = false;
+    g_device = -1;
+    return LUXHIP_OK;
+}
+
+const char* luxhip_last_error(void) { return g_err; }
+
+int luxhip_device_info(char* name, size_t name_len, int* compute_units, int64_t* total_mem) {
+    LUX_REQUIRE_INIT();
+    hipDeviceProp_t prop;
+    LUX_CHECK_HIP(hipGetDeviceProperties(&prop, g_device));
+    if (name && name_len) snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (total_mem) *total_mem = (int64_t)prop.totalGlobalMem;
+    return LUXHIP_OK;
+}
+
+int luxhip_stream_create(luxhip_stream_t* out) {
+    LUX_REQUIRE_INIT();
+    LUX_INVALID_IF(out == nullptr, "null output pointer");
+    hipStream_t s;
+    LUX_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+    *out = s;
+    return LUXHIP_OK;
+}
+int luxhip_stream_synchronize(luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    LUX_CHECK_HIP(hipStreamSynchronize((hipStream_t)s));
+    return LUXHIP_OK;
+}
+int luxhip_stream_destroy(luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    if (s == nullptr) return LUXHIP_OK;
+    LUX_CHECK_HIP(hipStreamSynchronize((hipStream_t)s));
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        auto it = g_ws.find((hipStream_t)s);
+        if (it != g_ws.end()) {
+            if (it->second.base) (void)hipFree(it->second.base);
+            g_ws.erase(it);
+        }
+    }
+    LUX_CHECK_HIP(hipStreamDestroy((hipStream_t)s));
+    return LUXHIP_OK;
+}
+
+int luxhip_event_create(luxhip_event_t* out) {
+    LUX_REQUIRE_INIT();
+    LUX_INVALID_IF(out == nullptr, "null output pointer");
+    hipEvent_t e;
+    LUX_CHECK_HIP(hipEventCreate(&e));
+    *out = e;
+    return LUXHIP_OK;
+}
+int luxhip_event_record(luxhip_event_t e, luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    LUX_CHECK_HIP(hipEventRecord((hipEvent_t)e, (hipStream_t)s));
+    return LUXHIP_OK;
+}
+int luxhip_event_elapsed_ms(float* ms, luxhip_event_t start, luxhip_event_t stop) {
+    LUX_REQUIRE_INIT();
+    LUX_INVALID_IF(ms == nullptr, "null output pointer");
+    LUX_CHECK_HIP(hipEventSynchronize((hipEvent_t)stop));
+    LUX_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return LUXHIP_OK;
+}
+int luxhip_event_destroy(luxhip_event_t e) {
+    LUX_REQUIRE_INIT();
+    LUX_CHECK_HIP(hipEventDestroy((hipEvent_t)e));
+    return LUXHIP_OK;
+}
+
+int luxhip_malloc(void** out, size_t bytes) {
+    LUX_REQUIRE_INIT();
+    LUX_INVALID_IF(out == nullptr, "null output pointer");
+    const size_t r = round_size(bytes);
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_pool.free_blocks.find(r);
+    if (it != g_pool.free_blocks.end()) {
+        *out = it->second;
+        g_pool.free_blocks.erase(it);
+        g_pool.live[*out] = r;
+        return LUXHIP_OK;
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, r);
+    if (e != hipSuccess) {
+        // give the pool back to the driver and retry once
+        for (auto& kv : g_pool.free_blocks) (void)hipFree(kv.second);
+        g_pool.free_blocks.clear();
+        e = hipMalloc(&p, r);
+        if (e != hipSuccess)
+            return set_error(LUXHIP_HIP_ERROR, "hipMalloc(%zu) failed: %s", r, hipGetErrorString(e));
+    }
+    g_pool.live[p] = r;
+    *out = p;
+    return LUXHIP_OK;
+}
+
+int luxhip_free(void* p) {
+    LUX_REQUIRE_INIT();
+    if (p == nullptr) return LUXHIP_OK;
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_pool.live.find(p);
+    LUX_INVALID_IF(it == g_pool.live.end(), "luxhip_free: %p was not allocated by luxhip_malloc", p);
+    g_pool.free_blocks.emplace(it->second, p);
+    g_pool.live.erase(it);
+    return LUXHIP_OK;
+}
+
+int luxhip_trim(void) {
+    LUX_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lk(g_mu);
+    LUX_CHECK_HIP(hipDeviceSynchronize());
+    for (auto& kv : g_pool.free_blocks) (void)hipFree(kv.second);
+    g_pool.free_blocks.clear();
+    return LUXHIP_OK;
+}
+
+int luxhip_memcpy_h2d(void* dst, const void* src, size_t bytes, luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    if (bytes == 0) return LUXHIP_OK;
+    LUX_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)s));
+    LUX_CHECK_HIP(hipStreamSynchronize((hipStream_t)s));
+    return LUXHIP_OK;
+}
+int luxhip_memcpy_d2h(void* dst, const void* src, size_t bytes, luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    if (bytes == 0) return LUXHIP_OK;
+    LUX_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)s));
+    LUX_CHECK_HIP(hipStreamSynchronize((hipStream_t)s));
+    return LUXHIP_OK;
+}
+int luxhip_memcpy_d2d(void* dst, const void* src, size_t bytes, luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    if (bytes == 0) return LUXHIP_OK;
+    LUX_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)s));
+    return LUXHIP_OK;
+}
+int luxhip_fill_zero(void* dst, size_t bytes, luxhip_stream_t s) {
+    LUX_REQUIRE_INIT();
+    if (bytes == 0) return LUXHIP_OK;
+    LUX_INVALID_IF((reinterpret_cast<uintptr_t>(dst) & 3u) != 0, "luxhip_fill_zero: destination must be 4-byte aligned");
+    const size_t nwords = bytes / 4, tail = bytes % 4;
+    if (nwords) {
+        size_t blocks = (nwords + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        fill_zero_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)s>>>(reinterpret_cast<uint32_t*>(dst), nwords);
+        LUX_CHECK_LAUNCH();
+    }
+    if (tail) {
+        fill_zero_bytes_kernel<<<dim3(1), dim3(64), 0, (hipStream_t)s>>>(reinterpret_cast<uint8_t*>(dst) + nwords * 4, tail);
+        LUX_CHECK_LAUNCH();
+    }
+    return LUXHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,482 @@
+"""Host-side mirror of LuxLib's public fused-operator API on top of libluxhip.
+
+Same names, argument order and error behaviour as lib/LuxLib/src/api/*.jl of the reference
+(Julia is not available where this runs, so this module plays the role the Julia glue in
+`julia/LuxHIP.jl` plays inside LuxLib): arguments are checked on the host before anything is
+launched (DimensionMismatch / ArgumentError / AssertionError), the device work goes through
+the C ABI, and every operator has an `rrule` that returns `(y, pullback)` like its
+ChainRulesCore counterpart.  `pullback(f, *args)` is the `Zygote.pullback` analogue.
+
+Activations are passed by name ("relu", "tanh", "gelu", ...).  Tensors are `DeviceArray`s in
+Julia's column-major layout and logical shapes (W, H, C, N) / (features, batch).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _lib
+from .array import DeviceArray, StatArray, current_stream
+
+
+# ------------------------------------------------------------------------------- errors
+class DimensionMismatch(ValueError):
+    """Julia's DimensionMismatch (impl/matmul.jl:21-34 of the reference)."""
+
+
+class ArgumentError(ValueError):
+    """Julia's ArgumentError (api/groupnorm.jl:40-64 of the reference)."""
+
+
+def _act_id(act: str) -> int:
+    try:
+        return _lib.ACT_IDS[act]
+    except KeyError:
+        # arbitrary closures are differentiated by host-side AD in the reference
+        # (impl/dense.jl:104-112); the device backend reports "unsupported" for them.
+        raise _lib.Unsupported(_lib.UNSUPPORTED, f"activation {act!r} has no device kernel") from None
+
+
+_NEEDS_PRE = {4, 5, 6, 7, 8}   # swish, gelu, softplus, logsigmoid, lisht (rrule branch 2)
+
+
+def _p(a) -> Optional[int]:
+    return None if a is None else a.ptr
+
+
+def _same_dtype(*arrs):
+    dts = {a.dtype for a in arrs if a is not None}
+    if len(dts) > 1:
+        # the reference promotes mixed inputs with a one-time warning (impl/conv.jl:11-19,
+        # ext/CUDAExt/cublaslt.jl:46-63); the device kernels want one storage type
+        raise _lib.Unsupported(_lib.UNSUPPORTED, f"mixed storage types {sorted(dts)}")
+    return dts.pop()
+
+
+def default_epsilon(dtype: str) -> float:
+    """eps(T)^(5/7) (utils.jl:130); eps(BFloat16) = 2^-7."""
+    eps = 2.0 ** -23 if dtype == "f32" else 2.0 ** -7
+    return eps ** (5.0 / 7.0)
+
+
+def _icn(x: DeviceArray) -> Tuple[int, int, int]:
+    """(I, C, N) view of an array whose channel dim is ndims-1 (vectors: (len, 1))."""
+    if x.ndim == 1:
+        return 1, x.shape[0], 1
+    I = 1
+    for s in x.shape[:-2]:
+        I *= s
+    return I, x.shape[-2], x.shape[-1]
+
+
+# ------------------------------------------------------------------------------- bias_activation
+def _check_bias(x: DeviceArray, bias: Optional[DeviceArray]):
+    if bias is None:
+        return
+    want = x.shape[0] if x.ndim == 1 else x.shape[-2]
+    # api/bias_activation.jl:38-45
+    assert bias.ndim == 1 and bias.shape[0] == want, "length(bias) must equal size(x, ndims(x) - 1)"
+
+
+def bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray]) -> DeviceArray:
+    """`bias_activation(σ, x, bias)` (api/bias_activation.jl:16-21)."""
+    _check_bias(x, bias)
+    y = DeviceArray(x.shape, _same_dtype(x, bias))
+    I, Cc, N = _icn(x)
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, _act_id(act), I, Cc, N, x.ptr, _p(bias), y.ptr, None)
+    return y
+
+
+def bias_activation_inplace(act: str, x: DeviceArray, bias: Optional[DeviceArray]) -> DeviceArray:
+    """`bias_activation!!(σ, x, bias)` (api/bias_activation.jl:31-36): overwrites and returns x."""
+    _check_bias(x, bias)
+    _same_dtype(x, bias)
+    I, Cc, N = _icn(x)
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, _act_id(act), I, Cc, N, x.ptr, _p(bias), x.ptr, None)
+    return x
+
+
+def rrule_bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray]):
+    """CRC.rrule(bias_activation) (impl/bias_activation.jl:64-104): (y, Δ -> (∂x, ∂b))."""
+    _check_bias(x, bias)
+    aid = _act_id(act)
+    dt = _same_dtype(x, bias)
+    I, Cc, N = _icn(x)
+    y = DeviceArray(x.shape, dt)
+    pre = DeviceArray(x.shape, dt) if aid in _NEEDS_PRE else None
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, aid, I, Cc, N, x.ptr, _p(bias), y.ptr, _p(pre))
+
+    def back(delta: DeviceArray):
+        dx = DeviceArray(x.shape, dt)
+        db = None if bias is None else DeviceArray(bias.shape, dt)
+        _lib.call("luxhip_bias_activation_bwd", current_stream(), x.code, aid, I, Cc, N, delta.ptr, y.ptr, _p(pre),
+                  dx.ptr, _p(db))
+        return dx, db
+
+    return y, back
+
+
+# ------------------------------------------------------------------------------- dense
+def _check_dense(weight, x, b):
+    if weight.ndim != 2 or x.ndim != 2:
+        raise DimensionMismatch("weight and x must be matrices")
+    if weight.shape[1] != x.shape[0]:
+        raise DimensionMismatch(f"A has shape {weight.shape} but B has shape {x.shape}")
+    if b is not None and (b.ndim != 1 or b.shape[0] != weight.shape[0]):
+        raise DimensionMismatch(f"bias has length {b.shape} but the output has {weight.shape[0]} rows")
+
+
+def fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b: Optional[DeviceArray]) -> DeviceArray:
+    """`fused_dense_bias_activation(σ, weight, x, b)` (api/dense.jl:33-37): σ.(weight * x .+ b)."""
+    _check_dense(weight, x, b)
+    dt = _same_dtype(weight, x, b)
+    M, K = weight.shape
+    N = x.shape[1]
+    y = DeviceArray((M, N), dt)
+    _lib.call("luxhip_fused_dense_fwd", current_stream(), y.code, _act_id(act), M, K, N, weight.ptr, max(M, 1), x.ptr,
+              max(K, 1), _p(b), y.ptr, max(M, 1), None)
+    return y
+
+
+def rrule_fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b: Optional[DeviceArray]):
+    """CRC.rrule(fused_dense) (impl/dense.jl:71-134): (y, Δ -> (∂W, ∂x, ∂b))."""
+    _check_dense(weight, x, b)
+    aid = _act_id(act)
+    dt = _same_dtype(weight, x, b)
+    M, K = weight.shape
+    N = x.shape[1]
+    y = DeviceArray((M, N), dt)
+    pre = DeviceArray((M, N), dt) if aid in _NEEDS_PRE else None
+    _lib.call("luxhip_fused_dense_fwd", current_stream(), y.code, aid, M, K, N, weight.ptr, max(M, 1), x.ptr, max(K, 1),
+              _p(b), y.ptr, max(M, 1), _p(pre))
+
+    def back(delta: DeviceArray):
+        dW = DeviceArray((M, K), dt)
+        dx = DeviceArray((K, N), dt)
+        db = None if b is None else DeviceArray((M,), dt)
+        dz = None if aid == 0 else DeviceArray((M, N), dt)
+        _lib.call("luxhip_fused_dense_bwd", current_stream(), y.code, aid, M, K, N, delta.ptr, y.ptr, _p(pre), weight.ptr,
+                  max(M, 1), x.ptr, max(K, 1), _p(dz), dW.ptr, dx.ptr, _p(db))
+        return dW, dx, db
+
+    return y, back
+
+
+def matmul(A: DeviceArray, B: DeviceArray, bias: Optional[DeviceArray] = None, transA=False, transB=False) -> DeviceArray:
+    """`matmul` / `matmuladd` (impl/matmul.jl:2-94) with optionally transposed operands."""
+    am, ak = (A.shape[1], A.shape[0]) if transA else A.shape
+    bk, bn = (B.shape[1], B.shape[0]) if transB else B.shape
+    if ak != bk:
+        raise DimensionMismatch(f"A has shape {(am, ak)} but B has shape {(bk, bn)}")
+    if bias is not None and bias.shape[0] != am:
+        raise DimensionMismatch("bias length does not match rows of A")
+    dt = _same_dtype(A, B, bias)
+    out = DeviceArray((am, bn), dt)
+    _lib.call("luxhip_matmul", current_stream(), out.code, int(transA), int(transB), am, bn, ak, A.ptr, max(A.shape[0], 1),
+              B.ptr, max(B.shape[0], 1), _p(bias), out.ptr, max(am, 1))
+    return out
+
+
+# ------------------------------------------------------------------------------- batchnorm
+def batchnorm(x: DeviceArray, scale, bias, running_mean, running_var, training, act: str = "identity",
+              momentum: float = 0.1, epsilon: Optional[float] = None):
+    """`batchnorm(x, scale, bias, running_mean, running_var, training, σ, momentum, epsilon)`
+    (api/batchnorm.jl:31-55): returns `(y, {"running_mean": .., "running_var": ..})`."""
+    y, stats, _ = _batchnorm_fwd(x, scale, bias, running_mean, running_var, bool(training), act, momentum, epsilon, False)
+    return y, stats
+
+
+def _batchnorm_fwd(x, scale, bias, rmean, rvar, training, act, momentum, epsilon, save):
+    dt = _same_dtype(x, scale, bias, rmean, rvar)
+    I, Cc, N = _icn(x)
+    for v in (scale, bias, rmean, rvar):
+        if v is not None and (v.ndim != 1 or v.shape[0] != Cc):
+            raise ArgumentError("Invalid Dimensions!")      # get_norm_reshape_dims, impl/normalization.jl:178-185
+    if (scale is None) != (bias is None):
+        raise ArgumentError("scale and bias must be given together")
+    if epsilon is None:
+        epsilon = default_epsilon(dt)
+    y = DeviceArray(x.shape, dt)
+    upd = training and rmean is not None
+    rm_out = DeviceArray((Cc,), dt) if upd else None
+    rv_out = DeviceArray((Cc,), dt) if upd else None
+    sm = StatArray(Cc) if save else None
+    si = StatArray(Cc) if save else None
+    _lib.call("luxhip_batchnorm_fwd", current_stream(), x.code, _act_id(act), I, Cc, N, x.ptr, _p(scale), _p(bias),
+              _p(rmean), _p(rvar), int(training), float(momentum), float(epsilon), y.ptr, _p(rm_out), _p(rv_out),
+              _p(sm), _p(si))
+    stats = {"running_mean": rm_out if upd else rmean, "running_var": rv_out if upd else rvar}
+    return y, stats, (sm, si, float(epsilon))
+
+
+def rrule_batchnorm(x, scale, bias, running_mean, running_var, training, act="identity", momentum=0.1, epsilon=None):
+    """Whole-op rrule (precedent: ext/cuDNNExt/cuDNNExt.jl:26-54): ((y, stats), Δ -> (∂x, ∂γ, ∂β))."""
+    training = bool(training)
+    y, stats, (sm, si, eps) = _batchnorm_fwd(x, scale, bias, running_mean, running_var, training, act, momentum, epsilon, True)
+    I, Cc, N = _icn(x)
+    from_batch = training or running_mean is None
+    aid = _act_id(act)
+
+    def back(delta: DeviceArray):
+        dx = DeviceArray(x.shape, x.dtype)
+        dg = None if scale is None else DeviceArray((Cc,), x.dtype)
+        db = None if bias is None else DeviceArray((Cc,), x.dtype)
+        _lib.call("luxhip_batchnorm_bwd", current_stream(), x.code, aid, I, Cc, N, delta.ptr, x.ptr, _p(scale), _p(bias),
+                  sm.ptr, si.ptr, int(from_batch), dx.ptr, _p(dg), _p(db))
+        return dx, dg, db
+
+    return (y, stats), back
+
+
+# ------------------------------------------------------------------------------- groupnorm
+def _check_groupnorm(x, scale, bias, groups):
+    Cc = x.shape[-2]
+    if scale is not None or bias is not None:
+        if scale is None or bias is None or scale.shape[0] != bias.shape[0] or bias.shape[0] != Cc:
+            raise ArgumentError("Length of `scale` and `bias` must be equal to the number of channels "
+                                "((N - 1) dim of the input array).")
+    if Cc % groups != 0:
+        raise ArgumentError(f"Number of channels {Cc} must be divisible by the number of groups {groups}.")
+
+
+def groupnorm(x: DeviceArray, scale, bias, groups: int, act: str = "identity", epsilon: Optional[float] = None):
+    """`groupnorm(x, scale, bias, groups, σ, epsilon)` (api/groupnorm.jl:26-39)."""
+    return _groupnorm_fwd(x, scale, bias, groups, act, epsilon, False)[0]
+
+
+def _groupnorm_fwd(x, scale, bias, groups, act, epsilon, save):
+    if x.ndim < 2:
+        raise ArgumentError("groupnorm needs at least 2 dimensions")
+    _check_groupnorm(x, scale, bias, groups)
+    dt = _same_dtype(x, scale, bias)
+    if epsilon is None:
+        epsilon = default_epsilon(dt)
+    I, Cc, N = _icn(x)
+    y = DeviceArray(x.shape, dt)
+    sm = StatArray(groups * N) if save else None
+    si = StatArray(groups * N) if save else None
+    _lib.call("luxhip_groupnorm_fwd", current_stream(), x.code, _act_id(act), I, Cc, groups, N, x.ptr, _p(scale), _p(bias),
+              float(epsilon), y.ptr, _p(sm), _p(si))
+    return y, (sm, si)
+
+
+def rrule_groupnorm(x, scale, bias, groups, act="identity", epsilon=None):
+    """CRC.rrule(groupnorm_affine_normalize_internal) + mean_var rrule (impl/groupnorm.jl:349-404,
+    impl/common_ops.jl:45-61): (y, Δ -> (∂x, ∂γ, ∂β))."""
+    y, (sm, si) = _groupnorm_fwd(x, scale, bias, groups, act, epsilon, True)
+    I, Cc, N = _icn(x)
+    aid = _act_id(act)
+
+    def back(delta):
+        dx = DeviceArray(x.shape, x.dtype)
+        dg = None if scale is None else DeviceArray((Cc,), x.dtype)
+        db = None if bias is None else DeviceArray((Cc,), x.dtype)
+        _lib.call("luxhip_groupnorm_bwd", current_stream(), x.code, aid, I, Cc, groups, N, delta.ptr, x.ptr, _p(scale),
+                  _p(bias), sm.ptr, si.ptr, dx.ptr, _p(dg), _p(db))
+        return dx, dg, db
+
+    return y, back
+
+
+# ------------------------------------------------------------------------------- layernorm
+def _layernorm_geometry(x, scale, bias, dims):
+    """Returns (L, R) when the normalised dims are the leading ones and scale/bias (if any)
+    span exactly those dims; raises Unsupported otherwise (the host would fall back to the
+    generic broadcast path, impl/layernorm.jl:3-14)."""
+    if scale is None and bias is None and dims is None:
+        raise ArgumentError("`dims` must be passed explicitly if `scale` and `bias` are `nothing`")
+    if (scale is None) != (bias is None):
+        raise ArgumentError("scale and bias must be given together")
+    nd = x.ndim
+    if dims is None:
+        # compute_layernorm_dims (impl/layernorm.jl:21-28): 1:(N - M)
+        assert nd > scale.ndim, "`x` must have more dimensions than `scale` and `bias` when `dims` is `nothing`"
+        dims = tuple(range(1, nd - scale.ndim + 1))
+        raise _lib.Unsupported(_lib.UNSUPPORTED, "layernorm with dims=nothing and trailing-dim affine parameters")
+    if isinstance(dims, int):
+        dims = (dims,)
+    dims = tuple(sorted(dims))
+    if dims != tuple(range(1, len(dims) + 1)):
+        raise _lib.Unsupported(_lib.UNSUPPORTED, f"layernorm over non-leading dims {dims}")
+    L = 1
+    for d in dims:
+        L *= x.shape[d - 1]
+    R = x.size // max(L, 1)
+    if scale is not None:
+        want = tuple(x.shape[:len(dims)]) + (1,) * (nd - len(dims))
+        if scale.ndim != nd or bias.ndim != nd:
+            raise ArgumentError("scale and bias must have the same number of dimensions as x when dims is given")
+        if tuple(scale.shape) != want or tuple(bias.shape) != want:
+            raise _lib.Unsupported(_lib.UNSUPPORTED, f"layernorm affine parameters of shape {scale.shape} (want {want})")
+    return L, R
+
+
+DEFAULT_DIMS = "1:(N-1)"
+
+
+def layernorm(x: DeviceArray, scale, bias, act: str = "identity", dims=DEFAULT_DIMS, epsilon: Optional[float] = None):
+    """`layernorm(x, scale, bias, σ, dims, epsilon)` (api/layernorm.jl:32-43).  `dims` uses
+    Julia's 1-based numbering; the default is 1:(N-1); `None` is Julia's `nothing`."""
+    return _layernorm_fwd(x, scale, bias, act, dims, epsilon, False)[0]
+
+
+def _layernorm_fwd(x, scale, bias, act, dims, epsilon, save):
+    if isinstance(dims, str) and dims == DEFAULT_DIMS:
+        dims = tuple(range(1, x.ndim))
+    L, R = _layernorm_geometry(x, scale, bias, dims)
+    dt = _same_dtype(x, scale, bias)
+    if epsilon is None:
+        epsilon = default_epsilon(dt)
+    y = DeviceArray(x.shape, dt)
+    sm = StatArray(R) if save else None
+    si = StatArray(R) if save else None
+    _lib.call("luxhip_layernorm_fwd", current_stream(), x.code, _act_id(act), L, R, x.ptr, _p(scale), _p(bias),
+              float(epsilon), y.ptr, _p(sm), _p(si))
+    return y, (sm, si, L, R)
+
+
+def rrule_layernorm(x, scale, bias, act="identity", dims=DEFAULT_DIMS, epsilon=None):
+    """Pullback of layernorm: the chain AD derives from impl/normalization.jl:11-17 and the
+    mean_var rrule (impl/common_ops.jl:45-61), as one fused device pass."""
+    y, (sm, si, L, R) = _layernorm_fwd(x, scale, bias, act, dims, epsilon, True)
+    aid = _act_id(act)
+
+    def back(delta):
+        dx = DeviceArray(x.shape, x.dtype)
+        dg = None if scale is None else DeviceArray(scale.shape, x.dtype)
+        db = None if bias is None else DeviceArray(bias.shape, x.dtype)
+        _lib.call("luxhip_layernorm_bwd", current_stream(), x.code, aid, L, R, delta.ptr, x.ptr, _p(scale), _p(bias),
+                  sm.ptr, si.ptr, dx.ptr, _p(dg), _p(db))
+        return dx, dg, db
+
+    return y, back
+
+
+# ------------------------------------------------------------------------------- conv
+@dataclass
+class DenseConvDims:
+    """The fields of NNlib.DenseConvDims this path consumes (2 spatial dims).
+    padding = (w_lo, w_hi, h_lo, h_hi); flipkernel=False is true convolution."""
+    x_shape: Tuple[int, int, int, int]
+    w_shape: Tuple[int, int, int, int]
+    stride: Tuple[int, int] = (1, 1)
+    padding: Tuple[int, int, int, int] = (0, 0, 0, 0)
+    dilation: Tuple[int, int] = (1, 1)
+    groups: int = 1
+    flipkernel: bool = False
+    _c: Optional[_lib.ConvDimsStruct] = field(default=None, repr=False, compare=False)
+
+    def __post_init__(self):
+        if isinstance(self.stride, int):
+            self.stride = (self.stride,) * 2
+        if isinstance(self.dilation, int):
+            self.dilation = (self.dilation,) * 2
+        if isinstance(self.padding, int):
+            self.padding = (self.padding,) * 4
+        elif len(self.padding) == 2:
+            self.padding = (self.padding[0], self.padding[0], self.padding[1], self.padding[1])
+        self.x_shape, self.w_shape = tuple(self.x_shape), tuple(self.w_shape)
+        if len(self.x_shape) != 4 or len(self.w_shape) != 4:
+            raise _lib.Unsupported(_lib.UNSUPPORTED, "only 2 spatial dimensions are handled on the device")
+        W, H, Cin, N = self.x_shape
+        kW, kH, Cg, Cout = self.w_shape
+        if Cg * self.groups != Cin:
+            raise DimensionMismatch(f"input channels {Cin} != weight channels {Cg} x groups {self.groups}")
+        if Cout % self.groups != 0:
+            raise DimensionMismatch("output channels must be divisible by groups")
+        self._c = _lib.ConvDimsStruct(W, H, Cin, N, kW, kH, Cout, self.stride[0], self.stride[1], *self.padding,
+                                      self.dilation[0], self.dilation[1], self.groups, int(self.flipkernel))
+
+    @property
+    def out_spatial(self):
+        W, H = self.x_shape[:2]
+        kW, kH = self.w_shape[:2]
+        ow = (W + self.padding[0] + self.padding[1] - self.dilation[0] * (kW - 1) - 1) // self.stride[0] + 1
+        oh = (H + self.padding[2] + self.padding[3] - self.dilation[1] * (kH - 1) - 1) // self.stride[1] + 1
+        return ow, oh
+
+    @property
+    def y_shape(self):
+        ow, oh = self.out_spatial
+        return (ow, oh, self.w_shape[3], self.x_shape[3])
+
+
+def _check_conv(weight, x, b, cdims):
+    if tuple(x.shape) != cdims.x_shape or tuple(weight.shape) != cdims.w_shape:
+        raise DimensionMismatch(f"x {x.shape} / weight {weight.shape} do not match cdims {cdims.x_shape} / {cdims.w_shape}")
+    if b is not None:
+        assert b.ndim == 1 and b.shape[0] == cdims.w_shape[3], "length(bias) must equal the number of output channels"
+
+
+def fused_conv_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b, cdims: DenseConvDims) -> DeviceArray:
+    """`fused_conv_bias_activation(σ, weight, x, b, cdims)` (api/conv.jl:30-38)."""
+    _check_conv(weight, x, b, cdims)
+    dt = _same_dtype(weight, x, b)
+    y = DeviceArray(cdims.y_shape, dt)
+    _lib.call("luxhip_conv_fwd", current_stream(), y.code, _act_id(act), C.byref(cdims._c), x.ptr, weight.ptr, _p(b),
+              y.ptr, None)
+    return y
+
+
+def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDims):
+    """CRC.rrule(fused_conv) + ∇fused_conv (impl/conv.jl:204-275): (y, Δ -> (∂w, ∂x, ∂b))."""
+    _check_conv(weight, x, b, cdims)
+    aid = _act_id(act)
+    dt = _same_dtype(weight, x, b)
+    y = DeviceArray(cdims.y_shape, dt)
+    pre = DeviceArray(cdims.y_shape, dt) if aid in _NEEDS_PRE else None
+    _lib.call("luxhip_conv_fwd", current_stream(), y.code, aid, C.byref(cdims._c), x.ptr, weight.ptr, _p(b), y.ptr, _p(pre))
+
+    def back(delta):
+        dw = DeviceArray(weight.shape, dt)
+        dx = DeviceArray(x.shape, dt)
+        db = None if b is None else DeviceArray(b.shape, dt)
+        dz = None if aid == 0 else DeviceArray(cdims.y_shape, dt)
+        _lib.call("luxhip_fused_conv_bwd", current_stream(), y.code, aid, C.byref(cdims._c), delta.ptr, y.ptr, _p(pre),
+                  x.ptr, weight.ptr, _p(dz), dw.ptr, dx.ptr, _p(db))
+        return dw, dx, db
+
+    return y, back
+
+
+def conv(x, weight, cdims):
+    """`Impl.conv(x, weight, cdims)` (impl/conv.jl:62-72)."""
+    return fused_conv_bias_activation("identity", weight, x, None, cdims)
+
+
+def conv_data_grad(dy, weight, cdims):
+    """`Impl.∇conv_data` (impl/conv.jl:128-131)."""
+    dx = DeviceArray(cdims.x_shape, dy.dtype)
+    _lib.call("luxhip_conv_bwd_data", current_stream(), dy.code, C.byref(cdims._c), dy.ptr, weight.ptr, dx.ptr)
+    return dx
+
+
+def conv_filter_grad(x, dy, cdims):
+    """`Impl.∇conv_filter` (impl/conv.jl:133-136)."""
+    dw = DeviceArray(cdims.w_shape, x.dtype)
+    _lib.call("luxhip_conv_bwd_filter", current_stream(), x.code, C.byref(cdims._c), x.ptr, dy.ptr, dw.ptr)
+    return dw
+
+
+# ------------------------------------------------------------------------------- Zygote.pullback analogue
+_RRULES = {
+    bias_activation: rrule_bias_activation,
+    fused_dense_bias_activation: rrule_fused_dense_bias_activation,
+    batchnorm: rrule_batchnorm,
+    groupnorm: rrule_groupnorm,
+    layernorm: rrule_layernorm,
+    fused_conv_bias_activation: rrule_fused_conv_bias_activation,
+}
+
+
+def pullback(f, *args, **kwargs):
+    """`y, back = pullback(f, args...)`; `back(Δ)` returns the tangents of the array
+    arguments in the order the rrule lists them."""
+    try:
+        rule = _RRULES[f]
+    except KeyError:
+        raise TypeError(f"no rrule registered for {f}") from None
+    return rule(*args, **kwargs)

@@ -1,0 +1,56 @@
+"""Shared helpers of the GPU parity tests."""
+import numpy as np
+
+from oracle import luxlib_oracle as O
+
+# Parity bars stated by the benchmark definition: fp32 within rel 1e-5, bf16 within rel 1e-2
+# of the CPU restatement on identical inputs.  "rel" is applied per element against
+# |want| + rms(want): a pure per-element relative bound is meaningless where the exact
+# result crosses zero.
+REL = {"f32": 1e-5, "bf16": 1e-2}
+
+
+def assert_close(got, want, dtype, what="", rel=None, scale=0.0):
+    """`scale`: magnitude of the terms the result is a sum of, for results that are small
+    through cancellation (gradients of normalisations); the absolute floor is
+    rel * max(rms(want), scale)."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, f"{what}: shape {got.shape} != {want.shape}"
+    if want.size == 0:
+        return
+    rel = REL[dtype] if rel is None else rel
+    rms = max(float(np.sqrt(np.mean(want * want))), float(scale))
+    bound = rel * (np.abs(want) + rms) + 1e-30
+    err = np.abs(got - want)
+    bad = ~(err <= bound)
+    if bad.any():
+        i = np.unravel_index(np.argmax(err / bound), err.shape)
+        raise AssertionError(
+            f"{what}: {bad.sum()}/{bad.size} elements outside rel {rel:g}; worst at {i}: got {got[i]!r} want {want[i]!r} "
+            f"(err {err[i]:.3e}, bound {bound[i]:.3e})")
+
+
+def host_inputs(dtype, *arrays):
+    """fp32 host arrays as the device will see them (bf16: rounded to representable values)."""
+    out = []
+    for a in arrays:
+        if a is None:
+            out.append(None)
+            continue
+        a = np.asarray(a, dtype=np.float32)
+        out.append(O.round_to_bf16(a) if dtype == "bf16" else a)
+    return out
+
+
+def dev(lux, a, dtype):
+    return None if a is None else lux.DeviceArray.from_numpy(a, dtype)
+
+
+def f64(a):
+    return None if a is None else np.asarray(a, dtype=np.float64)
+
+
+def rms(a):
+    a = np.asarray(a, dtype=np.float64)
+    return float(np.sqrt(np.mean(a * a))) if a.size else 0.0
