@@ -1,0 +1,283 @@
+#!/usr/bin/env python3
+"""Benchmark of the LuxLib fused-operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2]
+
+A "step" is one forward + pullback pass of the workload's operator chain over one batch of
+synthetic input that is already resident in HBM.  Prints ONE JSON line (see the README of the
+benchmark contract): whole-job throughput in the workload's roofline unit, the roofline of
+the dominant kernel (per-kernel durations measured with HIP events on the launch stream) and
+a CPU baseline (the C restatement of LuxLib's CPU loops, timed on this host).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from __graft_entry__ import load_package  # noqa: E402
+
+PEAK_HBM_GBS = 8000.0                 # MI355X HBM3E
+PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+METRIC = "fwd+bwd TFLOP/s & HBM GB/s (% MI355X roofline) per LuxLib fused op, 1 GPU"
+
+
+# ----------------------------------------------------------------------------- workloads
+class Workload:
+    name = ""
+    dtype = "f32"
+    bound = "hbm"            # "hbm" -> GB/s, "mfma" -> TFLOP/s
+    description = ""
+
+    def setup(self, lux):
+        raise NotImplementedError
+
+    def step(self):
+        raise NotImplementedError
+
+    def work_per_step(self) -> float:
+        """Algorithmic bytes (hbm) or flops (mfma) of one step."""
+        raise NotImplementedError
+
+    def kernel_work(self) -> dict:
+        """kernel name -> algorithmic bytes/flops of ONE launch."""
+        return {}
+
+    def cpu_baseline(self, budget_s: float):
+        return None
+
+
+class C2BatchnormBiasAct(Workload):
+    """BASELINE config 2: batchnorm (training, running stats updated) then bias_activation(relu),
+    forward and pullback, fp32, x 32x32x64x128."""
+    name = "C2"
+    dtype = "f32"
+    bound = "hbm"
+    description = "batchnorm(train)+bias_activation(relu) fwd+bwd, x 32x32x64x128 fp32"
+    shape = (32, 32, 64, 128)
+
+    def host_inputs(self):
+        rng = np.random.default_rng(1001)
+        W, H, Cc, N = self.shape
+        return dict(
+            x=(0.5 + 2.0 * rng.standard_normal(size=self.shape, dtype=np.float32)),
+            gamma=rng.uniform(0.5, 1.5, Cc).astype(np.float32),
+            beta=(0.1 * rng.standard_normal(Cc)).astype(np.float32),
+            rmean=np.zeros(Cc, np.float32), rvar=np.ones(Cc, np.float32),
+            bias2=(0.1 * rng.standard_normal(Cc)).astype(np.float32),
+            delta=rng.standard_normal(size=self.shape, dtype=np.float32),
+        )
+
+    def setup(self, lux):
+        self.lux = lux
+        lib = lux._lib.load()
+        W, H, Cc, N = self.shape
+        self.I, self.C, self.N = W * H, Cc, N
+        h = self.host_inputs()
+        d = lux.DeviceArray.from_numpy
+        self.t = {k: d(v) for k, v in h.items()}
+        for k in ("y1", "y2", "dy1", "dx"):
+            self.t[k] = lux.DeviceArray(self.shape, "f32")
+        for k in ("rmean_out", "rvar_out", "dgamma", "dbeta", "dbias2"):
+            self.t[k] = lux.DeviceArray((Cc,), "f32")
+        self.sm, self.si = lux.StatArray(Cc), lux.StatArray(Cc)
+        t, s = self.t, lux.current_stream()
+        vp = C.c_void_p
+        p = lambda k: vp(t[k].ptr)
+        I, Cc_, N_ = C.c_int64(self.I), C.c_int64(self.C), C.c_int64(self.N)
+        f32, ident, relu = 0, 0, 1
+        self.calls = [
+            (lib.luxhip_batchnorm_fwd, (s, f32, ident, I, Cc_, N_, p("x"), p("gamma"), p("beta"), p("rmean"), p("rvar"), 1,
+                                        C.c_double(0.1), C.c_double(1e-5), p("y1"), p("rmean_out"), p("rvar_out"),
+                                        vp(self.sm.ptr), vp(self.si.ptr))),
+            (lib.luxhip_bias_activation_fwd, (s, f32, relu, I, Cc_, N_, p("y1"), p("bias2"), p("y2"), None)),
+            (lib.luxhip_bias_activation_bwd, (s, f32, relu, I, Cc_, N_, p("delta"), p("y2"), None, p("dy1"), p("dbias2"))),
+            (lib.luxhip_batchnorm_bwd, (s, f32, ident, I, Cc_, N_, p("dy1"), p("x"), p("gamma"), p("beta"), vp(self.sm.ptr),
+                                        vp(self.si.ptr), 1, p("dx"), p("dgamma"), p("dbeta"))),
+        ]
+        # fused variant: batchnorm(..., relu) forward + pullback
+        self.fused_calls = [
+            (lib.luxhip_batchnorm_fwd, (s, f32, relu, I, Cc_, N_, p("x"), p("gamma"), p("beta"), p("rmean"), p("rvar"), 1,
+                                        C.c_double(0.1), C.c_double(1e-5), p("y2"), p("rmean_out"), p("rvar_out"),
+                                        vp(self.sm.ptr), vp(self.si.ptr))),
+            (lib.luxhip_batchnorm_bwd, (s, f32, relu, I, Cc_, N_, p("delta"), p("x"), p("gamma"), p("beta"), vp(self.sm.ptr),
+                                        vp(self.si.ptr), 1, p("dx"), p("dgamma"), p("dbeta"))),
+        ]
+
+    def step(self):
+        for fn, args in self.calls:
+            rc = fn(*args)
+            if rc != 0:
+                raise RuntimeError(self.lux._lib.last_error())
+
+    def step_fused(self):
+        for fn, args in self.fused_calls:
+            rc = fn(*args)
+            if rc != 0:
+                raise RuntimeError(self.lux._lib.last_error())
+
+    @property
+    def E(self):
+        return int(np.prod(self.shape)) * 4
+
+    def work_per_step(self):
+        # bn fwd 2E + relu fwd 2E + relu bwd 3E + bn bwd 3E (each API-level tensor read/written once)
+        return 10 * self.E
+
+    def work_per_step_fused(self):
+        return 5 * self.E        # fwd: x in, y out; bwd: delta, x in, dx out
+
+    def kernel_work(self):
+        E = self.E
+        return {"bn_stats_kernel": 1 * E, "bn_apply_kernel": 2 * E, "bias_act_fwd_kernel": 2 * E,
+                "bias_act_bwd_channel_kernel": 3 * E, "bn_bwd_reduce_kernel": 2 * E, "bn_bwd_apply_kernel": 3 * E}
+
+    def cpu_baseline(self, budget_s: float):
+        path = os.path.join(ROOT, "oracle", "libluxcpu.so")
+        if not os.path.exists(path):
+            return None
+        cpu = C.CDLL(path)
+        cpu.luxcpu_num_threads.restype = C.c_int
+        h = self.host_inputs()
+        W, H, Cc, N = self.shape
+        I = W * H
+        fa = lambda a: np.asfortranarray(a, dtype=np.float32)
+        x, delta = fa(h["x"]), fa(h["delta"])
+        y1, y2, dy1, dx = (np.empty(self.shape, np.float32, order="F") for _ in range(4))
+        mean, var, rmo, rvo, dg, db, db2 = (np.empty(Cc, np.float32) for _ in range(7))
+        ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+        i64 = C.c_int64
+
+        def cpu_step():
+            cpu.luxcpu_batchnorm_train_fwd(0, i64(I), i64(Cc), i64(N), ptr(x), ptr(h["gamma"]), ptr(h["beta"]), ptr(h["rmean"]),
+                                           ptr(h["rvar"]), C.c_float(0.1), C.c_float(1e-5), ptr(y1), ptr(rmo), ptr(rvo),
+                                           ptr(mean), ptr(var))
+            cpu.luxcpu_bias_activation_fwd(1, i64(I), i64(Cc), i64(N), ptr(y1), ptr(h["bias2"]), ptr(y2))
+            cpu.luxcpu_bias_activation_bwd(1, i64(I), i64(Cc), i64(N), ptr(delta), ptr(y2), None, ptr(dy1), ptr(db2))
+            cpu.luxcpu_batchnorm_train_bwd(i64(I), i64(Cc), i64(N), ptr(dy1), ptr(x), ptr(h["gamma"]), ptr(mean), ptr(var),
+                                           C.c_float(1e-5), ptr(dx), ptr(dg), ptr(db))
+
+        cpu_step()                      # warm-up / page-in
+        t0 = time.perf_counter()
+        n = 0
+        while True:
+            cpu_step()
+            n += 1
+            if time.perf_counter() - t0 > budget_s or n >= 200:
+                break
+        dt = (time.perf_counter() - t0) / n
+        threads = int(cpu.luxcpu_num_threads())
+        return {"value": self.work_per_step() / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "ms_per_step": dt * 1e3,
+                "sample": f"{n} full-size steps of the same chain (C port of LuxLib's CPU loops; like LuxLib, only the "
+                          f"normalise loop is threaded: {threads} OpenMP threads; all other passes are serial SIMD loops)"}
+
+
+WORKLOADS = {"C2": C2BatchnormBiasAct}
+
+
+# ----------------------------------------------------------------------------- timing
+def timed(lux, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    lux.synchronize()
+    e0, e1 = lux.Event(), lux.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    ms_gpu = e0.elapsed_ms(e1)          # waits for e1
+    lux.synchronize()
+    ms_wall = (time.perf_counter() - t0) * 1e3
+    return ms_gpu / steps, ms_wall / steps
+
+
+def kernel_profile(lux, fn, steps):
+    """Per-kernel average duration: every launch bracketed by HIP events on its stream."""
+    lux._lib.call("luxhip_profile_enable", 1)
+    for _ in range(steps):
+        fn()
+    buf = C.create_string_buffer(1 << 16)
+    lux._lib.call("luxhip_profile_report", buf, len(buf))
+    lux._lib.call("luxhip_profile_enable", 0)
+    return json.loads(buf.value.decode())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline (0 disables it)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path is single-GPU; no collective is part of it); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    lux = load_package()
+    lux.init(0)
+    wl = WORKLOADS[args.workload]()
+    wl.setup(lux)
+
+    ms_gpu, ms_wall = timed(lux, wl.step, args.steps, args.warmup)
+    ms = max(ms_gpu, ms_wall)           # whole-job time: the slower of the device and host clocks
+    work = wl.work_per_step()
+    if wl.bound == "hbm":
+        value, unit, peak = work / (ms * 1e-3) / 1e9, "GB/s", PEAK_HBM_GBS
+    else:
+        value, unit, peak = work / (ms * 1e-3) / 1e12, "TFLOP/s", PEAK_MFMA_TFLOPS[wl.dtype]
+
+    prof = kernel_profile(lux, wl.step, min(args.steps, 100))
+    kw = wl.kernel_work()
+    kernels = []
+    for k in prof:
+        avg_ms = k["total_ms"] / max(k["count"], 1)
+        w = kw.get(k["kernel"])
+        ent = {"kernel": k["kernel"], "avg_us": round(avg_ms * 1e3, 3), "launches": k["count"]}
+        if w:
+            ach = w / (avg_ms * 1e-3) / (1e9 if wl.bound == "hbm" else 1e12)
+            ent.update({"algorithmic": w, "achieved": round(ach, 1), "frac": round(ach / peak, 4)})
+        kernels.append(ent)
+    kernels.sort(key=lambda e: -e["avg_us"])
+    dom = next((e for e in kernels if "achieved" in e), None)
+    roofline = None
+    if dom is not None:
+        roofline = {"bound": wl.bound, "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": peak, "unit": unit,
+                    "frac": dom["frac"], "traffic": None, "avg_us": dom["avg_us"],
+                    "algorithmic_per_launch": dom["algorithmic"]}
+
+    out = {
+        "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype,
+        "data": "synthetic", "config": {"workload": f"{wl.name}: {wl.description}"},
+        "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
+        "ms_per_step_host_clock": round(ms_wall, 5), "roofline": roofline, "kernels": kernels,
+    }
+    if hasattr(wl, "step_fused"):
+        fg, fw = timed(lux, wl.step_fused, args.steps, args.warmup)
+        fms = max(fg, fw)
+        out["fused_variant"] = {"workload": "batchnorm(..., relu) fwd+bwd (activation fused into batchnorm)",
+                                "ms_per_step": round(fms, 5), "value": round(wl.work_per_step_fused() / (fms * 1e-3) / 1e9, 2),
+                                "unit": "GB/s", "algorithmic_bytes": wl.work_per_step_fused()}
+    if args.cpu_seconds > 0:
+        cb = wl.cpu_baseline(args.cpu_seconds)
+        if cb is not None:
+            cb["value"] = round(cb["value"], 3)
+            cb["ms_per_step"] = round(cb["ms_per_step"], 3)
+            out["cpu_baseline"] = cb
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -76,6 +76,13 @@ int luxhip_event_record(luxhip_event_t e, luxhip_stream_t s);
 int luxhip_event_elapsed_ms(float* ms, luxhip_event_t start, luxhip_event_t stop); /* waits for stop */
 int luxhip_event_destroy(luxhip_event_t e);
 
+/* Per-kernel timing (no counterpart in the reference, which has no tracing for its native GPU
+ * path): while enabled, every kernel launch is bracketed by HIP events on its own stream.
+ * luxhip_profile_report synchronises, writes a JSON array of {kernel, count, total_ms, min_ms,
+ * max_ms} into buf and clears the log. */
+int luxhip_profile_enable(int on);
+int luxhip_profile_report(char* buf, size_t len);
+
 /* Pooled device allocator (size-bucketed free lists; luxhip_free returns the block to the
  * pool, luxhip_trim releases the pool to the driver). */
 int luxhip_malloc(void** out, size_t bytes);

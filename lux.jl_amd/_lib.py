@@ -50,6 +50,8 @@ SIGNATURES = {
     "luxhip_event_record": [_vp, _vp],
     "luxhip_event_elapsed_ms": [C.POINTER(C.c_float), _vp, _vp],
     "luxhip_event_destroy": [_vp],
+    "luxhip_profile_enable": [_i],
+    "luxhip_profile_report": [C.c_char_p, _sz],
     "luxhip_malloc": [C.POINTER(_vp), _sz],
     "luxhip_free": [_vp],
     "luxhip_trim": [],

@@ -2,15 +2,19 @@
 // pullback, as HBM-bound streaming kernels over the (I, C, N) view.
 //
 // Channel c owns the rows (n*C + c)*I .. +I for every n.  Reduction kernels use a (S, C)
-// grid: workgroup (s, c) streams a contiguous slice of channel c's I*N elements and the last
-// workgroup of a channel to finish combines the S partials in a fixed order (deterministic,
-// no floating-point atomics) and writes the per-channel results.
+// grid: workgroup (s, c) streams a contiguous slice of channel c's I*N elements and writes one
+// partial; a one-wave-per-channel finalize kernel combines the S partials in a fixed order
+// (deterministic, no floating-point atomics, no device-wide fences inside the streaming
+// kernels: an agent-scope fence per workgroup writes back the L2 and costs far more than the
+// extra launch) and writes the per-channel results.
 //
-//   forward, training : bn_stats_kernel  (read x)           -> mean, invstd, scale, shift, running stats
+//   forward, training : bn_stats_kernel (read x) -> partials
+//                       bn_stats_finalize_kernel -> mean, invstd, scale, shift, running stats
 //                       bn_apply_kernel  (read x, write y)
-//   forward, inference: bn_infer_prep_kernel (C threads)    -> scale, shift
+//   forward, inference: bn_infer_prep_kernel (C threads) -> scale, shift
 //                       bn_apply_kernel
-//   pullback          : bn_bwd_reduce_kernel (read delta, x) -> dgamma, dbeta, per-channel coefficients
+//   pullback          : bn_bwd_reduce_kernel (read delta, x) -> partials
+//                       bn_bwd_finalize_kernel -> dgamma, dbeta, per-channel coefficients
 //                       bn_bwd_apply_kernel  (read delta, x, write dx)
 #include <algorithm>
 
@@ -56,81 +60,85 @@ __device__ __forceinline__ void chan_merge(float& n, float& mean, float& m2, flo
 }
 
 // ------------------------------------------------------------------------------- statistics
+// Partial (count, mean, M2) of slice s of channel c -> partial[(c*S + s)*3 ..].  A workgroup
+// keeps its slice (up to kStatVecs vectors per thread) in registers and makes two passes over
+// the registers: workgroup mean, then the sum of squared deviations from it (exact two-pass
+// statistics per slice; slices are combined with Chan's formula by the finalize kernel).
+constexpr int kStatVecs = 4;
 template <typename T, int VEC>
-__global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(
-    const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, const T* __restrict__ rmean,
-    const T* __restrict__ rvar, T* rmean_out, T* rvar_out, float* save_mean, float* save_invstd, float* scale,
-    float* shift, float* partial, unsigned int* counters, ChanGeom g, float count, float momentum, float eps) {
-    __shared__ float sm[3][kBnThreads / 64];
+__global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(const T* __restrict__ x, float* partial, ChanGeom g) {
+    __shared__ float sm[kBnThreads / 64];
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     const uint32_t q0 = s * g.chunk, q1 = min(q0 + g.chunk, g.nq);
-    float n = 0.0f, mean = 0.0f, m2 = 0.0f;
-    for (uint32_t q = q0 + threadIdx.x; q < q1; q += kBnThreads) {
-        float v[VEC];
-        load_vec<T, VEC>(x, g.offset(q, c, VEC), v);
-        if constexpr (VEC == 1) {
-            // Welford
-            n += 1.0f;
-            const float d = v[0] - mean;
-            mean += d / n;
-            m2 += d * (v[0] - mean);
-        } else {
-            float sum = 0.0f;
+    const float cnt = (float)((q1 - q0) * VEC);
+    float n = 0.0f, mean = 0.0f, m2 = 0.0f;   // running (count, mean, M2) over the passes of the outer loop
+    for (uint32_t base = q0; base < q1; base += kBnThreads * kStatVecs) {
+        float v[kStatVecs][VEC];
+        bool ok[kStatVecs];
+        float sum = 0.0f;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) sum += v[k];
-            const float mb = sum * (1.0f / VEC);
-            float m2b = 0.0f;
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) m2b += (v[k] - mb) * (v[k] - mb);
-            chan_merge(n, mean, m2, (float)VEC, mb, m2b);
+        for (int u = 0; u < kStatVecs; ++u) {
+            const uint32_t q = base + u * kBnThreads + threadIdx.x;
+            ok[u] = q < q1;
+            if (ok[u]) load_vec<T, VEC>(x, g.offset(q, c, VEC), v[u]);
         }
+#pragma unroll
+        for (int u = 0; u < kStatVecs; ++u)
+            if (ok[u]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) sum += v[u][k];
+            }
+        const uint32_t nvec = min(q1 - base, (uint32_t)(kBnThreads * kStatVecs));
+        const float nb = (float)(nvec * VEC);
+        const float mb = block_sum(sum, sm) / nb;
+        float dev = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kStatVecs; ++u)
+            if (ok[u]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) dev = fmaf(v[u][k] - mb, v[u][k] - mb, dev);
+            }
+        const float m2b = block_sum(dev, sm);
+        chan_merge(n, mean, m2, nb, mb, m2b);
     }
-    // wave, then workgroup
+    (void)cnt;
+    if (threadIdx.x == 0) {
+        float* p = partial + ((size_t)c * S + s) * 3;
+        p[0] = n; p[1] = mean; p[2] = m2;
+    }
+}
+
+// One wave per channel merges the S partials (fixed tree order) and writes every per-channel
+// result of the forward pass.  S <= kBnThreads.
+template <typename T>
+__global__ __launch_bounds__(kWave) void bn_stats_finalize_kernel(
+    const float* __restrict__ partial, uint32_t S, const T* __restrict__ gamma, const T* __restrict__ beta,
+    const T* __restrict__ rmean, const T* __restrict__ rvar, T* rmean_out, T* rvar_out, float* save_mean,
+    float* save_invstd, float* scale, float* shift, float count, float momentum, float eps) {
+    const uint32_t c = blockIdx.x;
+    const float* p = partial + (size_t)c * S * 3;
+    float n = 0.0f, mean = 0.0f, m2 = 0.0f;
+    for (uint32_t i = threadIdx.x; i < S; i += kWave) chan_merge(n, mean, m2, p[3 * i], p[3 * i + 1], p[3 * i + 2]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         const float nb = __shfl_xor(n, off, kWave), mb = __shfl_xor(mean, off, kWave), qb = __shfl_xor(m2, off, kWave);
         chan_merge(n, mean, m2, nb, mb, qb);
     }
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    if (lane == 0) { sm[0][w] = n; sm[1][w] = mean; sm[2][w] = m2; }
-    __syncthreads();
     if (threadIdx.x == 0) {
-        n = sm[0][0]; mean = sm[1][0]; m2 = sm[2][0];
-        for (int i = 1; i < kBnThreads / 64; ++i) chan_merge(n, mean, m2, sm[0][i], sm[1][i], sm[2][i]);
-        float* p = partial + ((size_t)c * S + s) * 3;
-        p[0] = n; p[1] = mean; p[2] = m2;
-    }
-    if (last_block_done(counters + c, S)) {
-        // all threads combine the S partials (S <= kBnThreads) in a fixed tree order
-        const float* p = partial + (size_t)c * S * 3;
-        n = 0.0f; mean = 0.0f; m2 = 0.0f;
-        if (threadIdx.x < S) { n = p[3 * threadIdx.x]; mean = p[3 * threadIdx.x + 1]; m2 = p[3 * threadIdx.x + 2]; }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float nb = __shfl_xor(n, off, kWave), mb = __shfl_xor(mean, off, kWave), qb = __shfl_xor(m2, off, kWave);
-            chan_merge(n, mean, m2, nb, mb, qb);
-        }
-        __syncthreads();
-        if (lane == 0) { sm[0][w] = n; sm[1][w] = mean; sm[2][w] = m2; }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            n = sm[0][0]; mean = sm[1][0]; m2 = sm[2][0];
-            for (int i = 1; i < kBnThreads / 64; ++i) chan_merge(n, mean, m2, sm[0][i], sm[1][i], sm[2][i]);
-            const float var = m2 / count;
-            const float invstd = 1.0f / sqrtf(var + eps);
-            const float gm = gamma ? ld(gamma + c) : 1.0f;
-            const float bt = beta ? ld(beta + c) : 0.0f;
-            const float sc = gm * invstd;
-            scale[c] = sc;
-            shift[c] = fmaf(-mean, sc, bt);
-            if (save_mean) save_mean[c] = mean;
-            if (save_invstd) save_invstd[c] = invstd;
-            if (rmean_out) {
-                const float m1 = momentum, m3 = 1.0f - momentum;
-                const float m2c = momentum * count / (count - 1.0f);
-                st(rmean_out + c, m3 * ld(rmean + c) + m1 * mean);
-                st(rvar_out + c, m3 * ld(rvar + c) + m2c * var);
-            }
+        const float var = m2 / count;
+        const float invstd = 1.0f / sqrtf(var + eps);
+        const float gm = gamma ? ld(gamma + c) : 1.0f;
+        const float bt = beta ? ld(beta + c) : 0.0f;
+        const float sc = gm * invstd;
+        scale[c] = sc;
+        shift[c] = fmaf(-mean, sc, bt);
+        if (save_mean) save_mean[c] = mean;
+        if (save_invstd) save_invstd[c] = invstd;
+        if (rmean_out) {
+            const float m1 = momentum, m3 = 1.0f - momentum;
+            const float m2c = momentum * count / (count - 1.0f);
+            st(rmean_out + c, m3 * ld(rmean + c) + m1 * mean);
+            st(rvar_out + c, m3 * ld(rvar + c) + m2c * var);
         }
     }
 }
@@ -181,12 +189,11 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const T* __restric
 }
 
 // ------------------------------------------------------------------------------- pullback
-// s1 = sum dy, s2 = sum dy * (x - mean) * invstd with dy = delta * act'(recomputed).
+// Partials of s1 = sum dy and s2 = sum dy * (x - mean) * invstd, dy = delta * act'(recomputed).
 template <typename T, int ACT, int VEC>
 __global__ __launch_bounds__(kBnThreads) void bn_bwd_reduce_kernel(
     const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
-    const float* __restrict__ save_mean, const float* __restrict__ save_invstd, T* dgamma, T* dbeta, float* coef,
-    float* partial, unsigned int* counters, ChanGeom g, float inv_count, int stats_from_batch) {
+    const float* __restrict__ save_mean, const float* __restrict__ save_invstd, float* partial, ChanGeom g) {
     __shared__ float sm[kBnThreads / 64];
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     const uint32_t q0 = s * g.chunk, q1 = min(q0 + g.chunk, g.nq);
@@ -194,21 +201,33 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_reduce_kernel(
     const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
     const float sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
     float s1 = 0.0f, s2 = 0.0f;
-    for (uint32_t q = q0 + threadIdx.x; q < q1; q += kBnThreads) {
-        const size_t off = g.offset(q, c, VEC);
-        float d[VEC], v[VEC];
-        load_vec<T, VEC>(delta, off, d);
-        load_vec<T, VEC>(x, off, v);
+    for (uint32_t base = q0; base < q1; base += kBnThreads * kStatVecs) {
+        float d[kStatVecs][VEC], v[kStatVecs][VEC];
+        bool ok[kStatVecs];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-            float dy = d[k];
-            if constexpr (ACT != LUXHIP_ACT_IDENTITY) {
-                const float pre = fmaf(v[k], sc, sh);
-                dy *= Act<ACT>::d(Act<ACT>::f(pre), pre);
+        for (int u = 0; u < kStatVecs; ++u) {
+            const uint32_t q = base + u * kBnThreads + threadIdx.x;
+            ok[u] = q < q1;
+            if (ok[u]) {
+                const size_t off = g.offset(q, c, VEC);
+                load_vec<T, VEC>(delta, off, d[u]);
+                load_vec<T, VEC>(x, off, v[u]);
             }
-            s1 += dy;
-            s2 = fmaf(dy, (v[k] - mean) * invstd, s2);
         }
+#pragma unroll
+        for (int u = 0; u < kStatVecs; ++u)
+            if (ok[u]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float dy = d[u][k];
+                    if constexpr (ACT != LUXHIP_ACT_IDENTITY) {
+                        const float pre = fmaf(v[u][k], sc, sh);
+                        dy *= Act<ACT>::d(Act<ACT>::f(pre), pre);
+                    }
+                    s1 += dy;
+                    s2 = fmaf(dy, (v[u][k] - mean) * invstd, s2);
+                }
+            }
     }
     s1 = block_sum(s1, sm);
     s2 = block_sum(s2, sm);
@@ -216,20 +235,29 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_reduce_kernel(
         partial[((size_t)c * S + s) * 2] = s1;
         partial[((size_t)c * S + s) * 2 + 1] = s2;
     }
-    if (last_block_done(counters + c, S)) {
-        const float* p = partial + (size_t)c * S * 2;
-        float t1 = 0.0f, t2 = 0.0f;
-        if (threadIdx.x < S) { t1 = p[2 * threadIdx.x]; t2 = p[2 * threadIdx.x + 1]; }
-        t1 = block_sum(t1, sm);
-        t2 = block_sum(t2, sm);
-        if (threadIdx.x == 0) {
-            if (dgamma) st(dgamma + c, t2);
-            if (dbeta) st(dbeta + c, t1);
-            // dx = A*dy + B*(x - mean) + D
-            coef[c] = sc;
-            coef[g.C + c] = stats_from_batch ? -sc * invstd * t2 * inv_count : 0.0f;
-            coef[2 * g.C + c] = stats_from_batch ? -sc * t1 * inv_count : 0.0f;
-        }
+}
+
+// One wave per channel: dgamma, dbeta and the coefficients of dx = A*dy + B*(x - mean) + D.
+template <typename T>
+__global__ __launch_bounds__(kWave) void bn_bwd_finalize_kernel(const float* __restrict__ partial, uint32_t S,
+                                                                const T* __restrict__ gamma,
+                                                                const float* __restrict__ save_invstd, T* dgamma,
+                                                                T* dbeta, float* coef, uint32_t C, float inv_count,
+                                                                int stats_from_batch) {
+    const uint32_t c = blockIdx.x;
+    const float* p = partial + (size_t)c * S * 2;
+    float t1 = 0.0f, t2 = 0.0f;
+    for (uint32_t i = threadIdx.x; i < S; i += kWave) { t1 += p[2 * i]; t2 += p[2 * i + 1]; }
+    t1 = wave_sum(t1);
+    t2 = wave_sum(t2);
+    if (threadIdx.x == 0) {
+        const float invstd = save_invstd[c];
+        const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
+        if (dgamma) st(dgamma + c, t2);
+        if (dbeta) st(dbeta + c, t1);
+        coef[c] = sc;
+        coef[C + c] = stats_from_batch ? -sc * invstd * t2 * inv_count : 0.0f;
+        coef[2 * C + c] = stats_from_batch ? -sc * t1 * inv_count : 0.0f;
     }
 }
 
@@ -283,10 +311,10 @@ static ChanGeom make_geom(int64_t I, int64_t C, int64_t N, int vec, int64_t* S_o
     g.vec_per_row = (uint32_t)(I / vec);
     g.C = (uint32_t)C;
     g.rowdiv = FastDiv(g.vec_per_row);
-    // one vector per thread where possible; at most kBnThreads slices per channel (the last
-    // workgroup combines them with one partial per thread) and about 16K workgroups in all
-    int64_t S = ceil_div(g.nq, kBnThreads);
-    const int64_t smax = std::min<int64_t>(kBnThreads, std::max<int64_t>(1, 16384 / C));
+    // kStatVecs vectors per thread where possible (amortises the workgroup reduction), at most
+    // 256 slices per channel and about 16K workgroups in all
+    int64_t S = ceil_div(g.nq, kBnThreads * kStatVecs);
+    const int64_t smax = std::min<int64_t>(256, std::max<int64_t>(1, 16384 / C));
     S = std::max<int64_t>(1, std::min(S, smax));
     g.chunk = (uint32_t)ceil_div(g.nq, S);
     *S_out = ceil_div(g.nq, g.chunk);
@@ -301,8 +329,7 @@ static int bn_check(int dtype, int act, int64_t I, int64_t C, int64_t N) {
         const long double tot = (long double)I * (long double)C * (long double)N;
         LUX_UNSUPPORTED_IF(tot >= 2147483648.0L, "tensors of 2^31 or more elements are not supported");
     }
-    LUX_UNSUPPORTED_IF(C > (int64_t)(kCounterBytes / sizeof(unsigned int)), "more than %zu channels are not supported",
-                       kCounterBytes / sizeof(unsigned int));
+    LUX_UNSUPPORTED_IF(C > 65535, "more than 65535 channels are not supported");
     return LUXHIP_OK;
 }
 
@@ -319,7 +346,7 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     int64_t S = 1;
     ChanGeom g = make_geom(I, C, N, vv, &S);
     Workspace ws;
-    int rc = get_workspace(s, (size_t)C * (2 + 3 * S) * sizeof(float), &ws);
+    int rc = get_workspace(s, (size_t)C * (2 + 3 * S) * sizeof(float), &ws);  // scale, shift, partials
     if (rc != LUXHIP_OK) return rc;
     float* scale = reinterpret_cast<float*>(ws.data);
     float* shift = scale + C;
@@ -327,15 +354,19 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     if (batch_stats) {
         const bool upd = training && rmean != nullptr;
         dim3 grid((unsigned)S, (unsigned)C);
-        if (vec)
-            bn_stats_kernel<T, V><<<grid, kBnThreads, 0, s>>>(x, gamma, beta, rmean, rvar, upd ? rmean_out : nullptr,
-                                                              upd ? rvar_out : nullptr, save_mean, save_invstd, scale,
-                                                              shift, partial, ws.counters, g, (float)(I * N), momentum, eps);
-        else
-            bn_stats_kernel<T, 1><<<grid, kBnThreads, 0, s>>>(x, gamma, beta, rmean, rvar, upd ? rmean_out : nullptr,
-                                                              upd ? rvar_out : nullptr, save_mean, save_invstd, scale,
-                                                              shift, partial, ws.counters, g, (float)(I * N), momentum, eps);
+        {
+            ProfScope ps("bn_stats_kernel", s);
+            if (vec) bn_stats_kernel<T, V><<<grid, kBnThreads, 0, s>>>(x, partial, g);
+            else bn_stats_kernel<T, 1><<<grid, kBnThreads, 0, s>>>(x, partial, g);
+        }
+        LUX_CHECK_LAUNCH();
+        ProfScope ps("bn_stats_finalize_kernel", s);
+        bn_stats_finalize_kernel<T><<<(unsigned)C, kWave, 0, s>>>(partial, (uint32_t)S, gamma, beta, rmean, rvar,
+                                                                 upd ? rmean_out : nullptr, upd ? rvar_out : nullptr,
+                                                                 save_mean, save_invstd, scale, shift, (float)(I * N),
+                                                                 momentum, eps);
     } else {
+        ProfScope ps("bn_infer_prep_kernel", s);
         bn_infer_prep_kernel<T><<<(unsigned)ceil_div(C, 256), 256, 0, s>>>(gamma, beta, rmean, rvar, save_mean,
                                                                            save_invstd, scale, shift, (uint32_t)C, eps);
     }
@@ -347,7 +378,10 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         if (vec) bn_apply_kernel<T, A, V><<<flat_grid(tv), kBnThreads, 0, s>>>(x, scale, shift, y, tv, rowdiv, cdiv, (uint32_t)C); \
         else bn_apply_kernel<T, A, 1><<<flat_grid(tv), kBnThreads, 0, s>>>(x, scale, shift, y, tv, rowdiv, cdiv, (uint32_t)C);     \
     } while (0)
-    LUX_DISPATCH_ACT(act, LAUNCH_APPLY);
+    {
+        ProfScope ps("bn_apply_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_APPLY);
+    }
 #undef LAUNCH_APPLY
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
@@ -371,18 +405,33 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     dim3 grid((unsigned)S, (unsigned)C);
     const uint32_t tv = (uint32_t)(I * C * N / vv);
     const FastDiv rowdiv((uint32_t)(I / vv)), cdiv((uint32_t)C);
-#define LAUNCH_BWD(A)                                                                                               \
+#define LAUNCH_REDUCE(A)                                                                                            \
     do {                                                                                                            \
-        if (vec) {                                                                                                  \
-            bn_bwd_reduce_kernel<T, A, V><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dgamma, dbeta, coef, partial, ws.counters, g, inv_count, stats_from_batch); \
-            bn_bwd_apply_kernel<T, A, V><<<flat_grid(tv), kBnThreads, 0, s>>>(delta, x, beta, save_mean, coef, dx, tv, rowdiv, cdiv, (uint32_t)C); \
-        } else {                                                                                                    \
-            bn_bwd_reduce_kernel<T, A, 1><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dgamma, dbeta, coef, partial, ws.counters, g, inv_count, stats_from_batch); \
-            bn_bwd_apply_kernel<T, A, 1><<<flat_grid(tv), kBnThreads, 0, s>>>(delta, x, beta, save_mean, coef, dx, tv, rowdiv, cdiv, (uint32_t)C); \
-        }                                                                                                           \
+        if (vec) bn_bwd_reduce_kernel<T, A, V><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, partial, g); \
+        else bn_bwd_reduce_kernel<T, A, 1><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, partial, g);     \
     } while (0)
-    LUX_DISPATCH_ACT(act, LAUNCH_BWD);
-#undef LAUNCH_BWD
+#define LAUNCH_BWD_APPLY(A)                                                                                         \
+    do {                                                                                                            \
+        if (vec) bn_bwd_apply_kernel<T, A, V><<<flat_grid(tv), kBnThreads, 0, s>>>(delta, x, beta, save_mean, coef, dx, tv, rowdiv, cdiv, (uint32_t)C); \
+        else bn_bwd_apply_kernel<T, A, 1><<<flat_grid(tv), kBnThreads, 0, s>>>(delta, x, beta, save_mean, coef, dx, tv, rowdiv, cdiv, (uint32_t)C);     \
+    } while (0)
+    {
+        ProfScope ps("bn_bwd_reduce_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_REDUCE);
+    }
+    LUX_CHECK_LAUNCH();
+    {
+        ProfScope ps("bn_bwd_finalize_kernel", s);
+        bn_bwd_finalize_kernel<T><<<(unsigned)C, kWave, 0, s>>>(partial, (uint32_t)S, gamma, save_invstd, dgamma, dbeta, coef,
+                                                               (uint32_t)C, inv_count, stats_from_batch);
+    }
+    LUX_CHECK_LAUNCH();
+    {
+        ProfScope ps("bn_bwd_apply_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_BWD_APPLY);
+    }
+#undef LAUNCH_REDUCE
+#undef LAUNCH_BWD_APPLY
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

@@ -13,16 +13,22 @@ int set_error(int status, const char* fmt, ...);
 bool initialized();
 int num_cus();
 
-// Per-stream scratch owned by the library.  Layout: [counters | data].  The counter region
-// (kCounterBytes, zero on creation) backs the "last workgroup finishes the reduction"
-// pattern; every kernel that uses a counter resets it to zero before it exits, so the
-// region is all-zero between launches.  get_workspace grows the data region on demand.
-constexpr size_t kCounterBytes = 64 * 1024;
+// Per-stream scratch owned by the library (partial results of the reduction kernels,
+// per-channel coefficients).  get_workspace grows it on demand; kernels on one stream are
+// ordered, so consecutive operators may share it.
 struct Workspace {
-    unsigned int* counters;  // kCounterBytes / 4 entries, zero between launches
-    char* data;              // >= the requested number of bytes, 256-byte aligned
+    char* data;  // >= the requested number of bytes, 256-byte aligned
 };
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out);
+
+// Optional per-kernel timing with HIP events on the launch stream (luxhip_profile_enable).
+struct ProfScope {
+    const char* name;
+    hipStream_t stream;
+    bool active;
+    ProfScope(const char* n, hipStream_t s);
+    ~ProfScope();
+};
 
 #define LUX_CHECK_HIP(expr)                                                                     \
     do {                                                                                        \
@@ -252,25 +258,6 @@ __device__ __forceinline__ float block_sum(float v, float* smem) {
     for (int i = 0; i < nw; ++i) t += smem[i];
     __syncthreads();
     return t;
-}
-
-// Marks this workgroup as finished with its partial result and tells whether it is the
-// last of `total` workgroups sharing `counter` (which it then resets).  All threads of the
-// workgroup must call it; partial results must be written to global memory before the call
-// and may be read (by the last workgroup) after it.
-__device__ __forceinline__ bool last_block_done(unsigned int* counter, unsigned int total) {
-    __shared__ bool is_last;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned int prev = atomicAdd(counter, 1u);
-        is_last = (prev == total - 1);
-        if (is_last) *counter = 0u;
-    }
-    __syncthreads();
-    bool r = is_last;
-    if (r) __threadfence();
-    return r;
 }
 
 }  // namespace luxhip

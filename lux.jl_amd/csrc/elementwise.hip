@@ -6,7 +6,8 @@
 //              contiguous elements) -- used when rows are long enough to coalesce;
 //   "plane":   the I*C elements of one n are contiguous; a thread owns VEC consecutive plane
 //              positions and walks over n -- used when I is small (dense layers: I == 1).
-// Reductions are deterministic: per-workgroup partials are combined in a fixed order.
+// Reductions are deterministic: per-workgroup partials are combined in a fixed order by a
+// small finalize kernel.
 #include <algorithm>
 
 #include "common.h"
@@ -133,14 +134,12 @@ __global__ __launch_bounds__(kThreads) void act_bwd_kernel(const T* __restrict__
 }
 
 // "channel" layout: grid (S, C).  Workgroup (s, c) handles vectors [s*chunk, (s+1)*chunk) of
-// the nq = I*N/VEC vectors of channel c, writes its partial sum and the last workgroup of
-// the channel adds the S partials in order.
+// the nq = I*N/VEC vectors of channel c and writes its partial sum.
 template <typename T, int ACT, int VEC>
 __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T* __restrict__ delta,
                                                                         const T* __restrict__ out,
-                                                                        const T* __restrict__ pre, T* dx, T* dbias,
-                                                                        float* partial, unsigned int* counters,
-                                                                        uint32_t nq, uint32_t chunk, FastDiv rowdiv,
+                                                                        const T* __restrict__ pre, T* dx,
+                                                                        float* partial, uint32_t nq, uint32_t chunk, FastDiv rowdiv,
                                                                         uint32_t vec_per_row, uint32_t C) {
     __shared__ float smem[kThreads / 64];
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
@@ -158,11 +157,16 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T*
     }
     acc = block_sum(acc, smem);
     if (threadIdx.x == 0) partial[(size_t)c * S + s] = acc;
-    if (last_block_done(counters + c, S)) {
-        float t = threadIdx.x < S ? partial[(size_t)c * S + threadIdx.x] : 0.0f;   // S <= kThreads
-        t = block_sum(t, smem);
-        if (threadIdx.x == 0) st(dbias + c, t);
-    }
+}
+
+// dbias[c] = sum_s partial[c][s]; one wave per channel, fixed order.
+template <typename T>
+__global__ __launch_bounds__(64) void channel_finalize_kernel(const float* __restrict__ partial, T* dbias, uint32_t S) {
+    const uint32_t c = blockIdx.x;
+    float t = 0.0f;
+    for (uint32_t i = threadIdx.x; i < S; i += 64) t += partial[(size_t)c * S + i];
+    t = wave_sum(t);
+    if (threadIdx.x == 0) st(dbias + c, t);
 }
 
 // "plane" layout: P = I*C contiguous elements per n.  grid (ceil(P/(T*VEC)), S); a thread
@@ -255,7 +259,10 @@ static int bias_act_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
                 bias_act_fwd_kernel<T, A, 1, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
         }                                                                                                          \
     } while (0)
-    LUX_DISPATCH_ACT(act, LAUNCH_FWD);
+    {
+        ProfScope ps("bias_act_fwd_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_FWD);
+    }
 #undef LAUNCH_FWD
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
@@ -278,13 +285,16 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
             act_bwd_kernel<T, A, 1><<<grid_for((uint32_t)total), kThreads, 0, s>>>(delta, out, pre, dx, (uint32_t)total); \
         }                                                                                                   \
     } while (0)
-        LUX_DISPATCH_ACT(act, LAUNCH_ACT_BWD);
+        {
+            ProfScope ps("act_bwd_kernel", s);
+            LUX_DISPATCH_ACT(act, LAUNCH_ACT_BWD);
+        }
 #undef LAUNCH_ACT_BWD
         LUX_CHECK_LAUNCH();
         return LUXHIP_OK;
     }
 
-    const bool channel_layout = I >= 64 && C <= (int64_t)(kCounterBytes / sizeof(unsigned int));
+    const bool channel_layout = I >= 64 && C <= 65535;
     if (channel_layout) {
         const bool vec = ptr_ok && I % V == 0;
         const int vv = vec ? V : 1;
@@ -304,12 +314,18 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
 #define LAUNCH_CH(A)                                                                                               \
     do {                                                                                                           \
         if (vec)                                                                                                   \
-            bias_act_bwd_channel_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, ws.counters, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+            bias_act_bwd_channel_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
         else                                                                                                       \
-            bias_act_bwd_channel_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, ws.counters, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+            bias_act_bwd_channel_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
     } while (0)
-        LUX_DISPATCH_ACT(act, LAUNCH_CH);
+        {
+            ProfScope ps("bias_act_bwd_channel_kernel", s);
+            LUX_DISPATCH_ACT(act, LAUNCH_CH);
+        }
 #undef LAUNCH_CH
+        LUX_CHECK_LAUNCH();
+        ProfScope ps2("channel_finalize_kernel", s);
+        channel_finalize_kernel<T><<<(unsigned)C, 64, 0, s>>>(partial, dbias, (uint32_t)S);
         LUX_CHECK_LAUNCH();
         return LUXHIP_OK;
     }
@@ -335,9 +351,13 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
         else                                                                                                       \
             bias_act_bwd_plane_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, (uint32_t)P, (uint32_t)N, n_per_slice); \
     } while (0)
-    LUX_DISPATCH_ACT(act, LAUNCH_PL);
+    {
+        ProfScope ps("bias_act_bwd_plane_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_PL);
+    }
 #undef LAUNCH_PL
     LUX_CHECK_LAUNCH();
+    ProfScope ps2("plane_finalize_kernel", s);
     plane_finalize_kernel<T><<<(unsigned)C, 64, 0, s>>>(partial, dbias, (uint32_t)P, (uint32_t)I, (uint32_t)S);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;

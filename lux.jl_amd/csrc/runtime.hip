@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <map>
+#include <string>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -31,12 +32,35 @@ struct WsEntry {
 };
 std::map<hipStream_t, WsEntry> g_ws;
 
+struct ProfEntry {
+    const char* name;
+    hipEvent_t a, b;
+};
+bool g_prof = false;
+std::vector<ProfEntry> g_prof_entries;
+
 size_t round_size(size_t b) {
     if (b == 0) b = 1;
     if (b <= (1u << 20)) return (b + 511) & ~size_t(511);               // 512 B granules
     return (b + (size_t(2) << 20) - 1) & ~((size_t(2) << 20) - 1);      // 2 MiB granules
 }
 }  // namespace
+
+ProfScope::ProfScope(const char* n, hipStream_t s) : name(n), stream(s), active(g_prof) {
+    if (!active) return;
+    ProfEntry e{n, nullptr, nullptr};
+    if (hipEventCreate(&e.a) != hipSuccess || hipEventCreate(&e.b) != hipSuccess) { active = false; return; }
+    (void)hipEventRecord(e.a, s);
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_prof_entries.push_back(e);
+}
+ProfScope::~ProfScope() {
+    if (!active) return;
+    std::lock_guard<std::mutex> lk(g_mu);
+    // the matching entry is the last one with this name and stream still open
+    for (auto it = g_prof_entries.rbegin(); it != g_prof_entries.rend(); ++it)
+        if (it->name == name) { (void)hipEventRecord(it->b, stream); break; }
+}
 
 int set_error(int status, const char* fmt, ...) {
     va_list ap;
@@ -61,14 +85,11 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
             e.base = nullptr;
         }
         void* p = nullptr;
-        LUX_CHECK_HIP(hipMalloc(&p, kCounterBytes + want));
-        LUX_CHECK_HIP(hipMemset(p, 0, kCounterBytes));
-        LUX_CHECK_HIP(hipDeviceSynchronize());
+        LUX_CHECK_HIP(hipMalloc(&p, want));
         e.base = p;
         e.data_bytes = want;
     }
-    out->counters = reinterpret_cast<unsigned int*>(e.base);
-    out->data = reinterpret_cast<char*>(e.base) + kCounterBytes;
+    out->data = reinterpret_cast<char*>(e.base);
     return LUXHIP_OK;
 }
 
@@ -188,6 +209,45 @@ int luxhip_event_elapsed_ms(float* ms, luxhip_event_t start, luxhip_event_t stop
 int luxhip_event_destroy(luxhip_event_t e) {
     LUX_REQUIRE_INIT();
     LUX_CHECK_HIP(hipEventDestroy((hipEvent_t)e));
+    return LUXHIP_OK;
+}
+
+int luxhip_profile_enable(int on) {
+    LUX_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_prof = on != 0;
+    return LUXHIP_OK;
+}
+
+int luxhip_profile_report(char* buf, size_t len) {
+    LUX_REQUIRE_INIT();
+    LUX_INVALID_IF(buf == nullptr || len < 3, "profile_report: buffer too small");
+    LUX_CHECK_HIP(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lk(g_mu);
+    struct Agg { int count = 0; double total = 0, mn = 1e30, mx = 0; };
+    std::map<std::string, Agg> agg;
+    for (auto& e : g_prof_entries) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, e.a, e.b) == hipSuccess) {
+            Agg& a = agg[e.name];
+            a.count++; a.total += ms;
+            if (ms < a.mn) a.mn = ms;
+            if (ms > a.mx) a.mx = ms;
+        }
+        (void)hipEventDestroy(e.a);
+        (void)hipEventDestroy(e.b);
+    }
+    g_prof_entries.clear();
+    size_t off = 0;
+    off += snprintf(buf + off, len - off, "[");
+    bool first = true;
+    for (auto& kv : agg) {
+        if (off + 200 >= len) break;
+        off += snprintf(buf + off, len - off, "%s{\"kernel\": \"%s\", \"count\": %d, \"total_ms\": %.6f, \"min_ms\": %.6f, \"max_ms\": %.6f}",
+                        first ? "" : ", ", kv.first.c_str(), kv.second.count, kv.second.total, kv.second.mn, kv.second.mx);
+        first = false;
+    }
+    snprintf(buf + off, len - off, "]");
     return LUXHIP_OK;
 }
 

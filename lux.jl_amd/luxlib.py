@@ -84,9 +84,10 @@ def _check_bias(x: DeviceArray, bias: Optional[DeviceArray]):
 def bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray]) -> DeviceArray:
     """`bias_activation(σ, x, bias)` (api/bias_activation.jl:16-21)."""
     _check_bias(x, bias)
+    aid = _act_id(act)
     y = DeviceArray(x.shape, _same_dtype(x, bias))
     I, Cc, N = _icn(x)
-    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, _act_id(act), I, Cc, N, x.ptr, _p(bias), y.ptr, None)
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, aid, I, Cc, N, x.ptr, _p(bias), y.ptr, None)
     return y
 
 

@@ -55,8 +55,9 @@ def test_training_forward_and_pullback(gpu, dtype, act, affine, track):
         args = [dev(gpu, a, dtype) for a in (x, g, b, rm, rv)]
         (y, st), back = gpu.pullback(gpu.batchnorm, *args, True, act, 0.1, eps)
         wy, wrm, wrv = O.batchnorm(f64(x), f64(g), f64(b), f64(rm), f64(rv), True, act, 0.1, eps)
+        wy32 = O.batchnorm(x, g, b, rm, rv, True, act, 0.1, eps)[0]
         tag = f"{dtype} {act} {shape} affine={affine} track={track}"
-        assert_close(y.to_numpy(), wy, dtype, tag + " y")
+        assert_close(y.to_numpy(), wy, dtype, tag + " y", want32=wy32)
         if track:
             assert_close(st["running_mean"].to_numpy(), wrm, dtype, tag + " running_mean")
             assert_close(st["running_var"].to_numpy(), wrv, dtype, tag + " running_var")
@@ -66,11 +67,12 @@ def test_training_forward_and_pullback(gpu, dtype, act, affine, track):
             assert st["running_mean"] is None and st["running_var"] is None
         gx, gg, gb = back(dev(gpu, delta, dtype))
         wdx, wdg, wdb = O.batchnorm_pullback(f64(x), f64(g), f64(b), act, eps, f64(delta))
+        w32 = O.batchnorm_pullback(x, g, b, act, np.float32(eps), delta)
         rel = None if dtype == "f32" else 3e-2
-        assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=dx_scale(x, g, eps, delta))
+        assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=dx_scale(x, g, eps, delta), want32=w32[0])
         if affine:
-            assert_close(gg.to_numpy(), wdg, dtype, tag + " dgamma", rel=rel, scale=rms(delta))
-            assert_close(gb.to_numpy(), wdb, dtype, tag + " dbeta", rel=rel, scale=rms(delta))
+            assert_close(gg.to_numpy(), wdg, dtype, tag + " dgamma", rel=rel, scale=rms(delta), want32=w32[1])
+            assert_close(gb.to_numpy(), wdb, dtype, tag + " dbeta", rel=rel, scale=rms(delta), want32=w32[2])
         else:
             assert gg is None and gb is None
 

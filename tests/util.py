@@ -10,10 +10,13 @@ from oracle import luxlib_oracle as O
 REL = {"f32": 1e-5, "bf16": 1e-2}
 
 
-def assert_close(got, want, dtype, what="", rel=None, scale=0.0):
+def assert_close(got, want, dtype, what="", rel=None, scale=0.0, want32=None):
     """`scale`: magnitude of the terms the result is a sum of, for results that are small
     through cancellation (gradients of normalisations); the absolute floor is
-    rel * max(rms(want), scale)."""
+    rel * max(rms(want), scale).
+    `want32`: the same oracle evaluated in float32 arithmetic (what a CPU run of the reference
+    produces); where the problem is so ill-conditioned that fp32 arithmetic itself misses the
+    exact answer by more than the bar, the allowance grows to 4x that fp32 error."""
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, f"{what}: shape {got.shape} != {want.shape}"
@@ -22,6 +25,8 @@ def assert_close(got, want, dtype, what="", rel=None, scale=0.0):
     rel = REL[dtype] if rel is None else rel
     rms = max(float(np.sqrt(np.mean(want * want))), float(scale))
     bound = rel * (np.abs(want) + rms) + 1e-30
+    if want32 is not None:
+        bound = np.maximum(bound, 4.0 * np.abs(np.asarray(want32, dtype=np.float64) - want))
     err = np.abs(got - want)
     bad = ~(err <= bound)
     if bad.any():
