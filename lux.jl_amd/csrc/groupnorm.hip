@@ -1,0 +1,444 @@
+// groupnorm forward and pullback.
+//
+// x is viewed as (I, C/G, G, N): the slice of group k and sample n is the contiguous run of
+// m = I*C/G elements at ((n*G + k)*C/G)*I.  One workgroup owns one slice.
+//   * cached kernels keep the slice (forward: x; pullback: delta and x) in registers, so HBM
+//     sees every tensor once: statistics, normalisation and the input gradient all come from
+//     the registers (slices of up to kGnCache vectors per thread x 1024 threads);
+//   * streaming kernels handle larger slices with a second read of the slice.
+// Per-channel gradients (dgamma, dbeta) are accumulated per wave in LDS in program order,
+// combined across waves in a fixed order, written as [N][C] partials and reduced over N by a
+// finalize kernel: deterministic, no floating-point atomics.
+#include <algorithm>
+
+#include "common.h"
+
+namespace luxhip {
+
+constexpr int kGnCache = 8;  // vectors per thread kept in registers
+
+struct GnGeom {
+    uint32_t I, Cg, G, C;
+    uint32_t nvec;         // vectors per slice = I*Cg / VEC
+    FastDiv chdiv;         // vector index -> channel within group: / (I / VEC)   (VEC == 1: / I)
+    float inv_m;           // 1 / (I*Cg)
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ void gn_load(const T* p, size_t off, float (&v)[VEC]) {
+    if constexpr (VEC == 1) v[0] = ld(p + off);
+    else Vec<T>::load(p + off, v);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void gn_store(T* p, size_t off, const float (&v)[VEC]) {
+    if constexpr (VEC == 1) st(p + off, v[0]);
+    else Vec<T>::store(p + off, v);
+}
+
+// ------------------------------------------------------------------------------- forward
+template <typename T, int ACT, int VEC, bool CACHED>
+__global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, T* y,
+                              float* save_mean, float* save_invstd, GnGeom g, float eps) {
+    __shared__ float sm[16];
+    const uint32_t slice = blockIdx.x;              // = n*G + k
+    const uint32_t k = slice % g.G;
+    const size_t base = (size_t)slice * g.nvec * VEC;
+    const uint32_t T_ = blockDim.x;
+    float v[CACHED ? kGnCache : 1][VEC];
+
+    // pass 1: mean
+    float sum = 0.0f;
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            if (q < g.nvec) gn_load<T, VEC>(x, base + (size_t)q * VEC, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            if (q < g.nvec) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) sum += v[u][e];
+            }
+        }
+    } else {
+        for (uint32_t q = threadIdx.x; q < g.nvec; q += T_) {
+            gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) sum += v[0][e];
+        }
+    }
+    const float mean = block_sum(sum, sm) * g.inv_m;
+    // pass 2: variance about the mean
+    float dev = 0.0f;
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            if (q < g.nvec) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) dev = fmaf(v[u][e] - mean, v[u][e] - mean, dev);
+            }
+        }
+    } else {
+        for (uint32_t q = threadIdx.x; q < g.nvec; q += T_) {
+            gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) dev = fmaf(v[0][e] - mean, v[0][e] - mean, dev);
+        }
+    }
+    const float var = block_sum(dev, sm) * g.inv_m;
+    const float invstd = 1.0f / sqrtf(var + eps);
+    if (threadIdx.x == 0) {
+        if (save_mean) save_mean[slice] = mean;
+        if (save_invstd) save_invstd[slice] = invstd;
+    }
+    // pass 3: normalise
+    auto emit = [&](uint32_t q, const float (&xv)[VEC]) {
+        const uint32_t c = k * g.Cg + g.chdiv.div(q);
+        const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
+        const float sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+        float o[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = Act<ACT>::f(fmaf(xv[e], sc, sh));
+        gn_store<T, VEC>(y, base + (size_t)q * VEC, o);
+    };
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            if (q < g.nvec) emit(q, v[u]);
+        }
+    } else {
+        for (uint32_t q = threadIdx.x; q < g.nvec; q += T_) {
+            gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+            emit(q, v[0]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------- pullback
+// Adds the per-lane contributions (a, b) of channel j to this wave's LDS accumulators.
+// Lanes of a wave usually share j (rows are longer than a wave); otherwise the distinct
+// channels present in the wave are handled one after the other.
+__device__ __forceinline__ void wave_channel_accumulate(float* accg, float* accb, uint32_t j, float a, float b,
+                                                        bool active) {
+    const int lane = threadIdx.x & 63;
+    unsigned long long todo = __ballot(active);
+    while (todo) {
+        const int first = __ffsll((long long)todo) - 1;
+        const uint32_t j0 = __shfl(j, first, kWave);
+        const bool sel = active && j == j0;
+        const float ta = wave_sum(sel ? a : 0.0f);
+        const float tb = wave_sum(sel ? b : 0.0f);
+        if (lane == 0) {
+            accg[j0] += ta;
+            accb[j0] += tb;
+        }
+        todo &= ~__ballot(sel);
+    }
+}
+
+template <typename T, int ACT, int VEC, bool CACHED, bool AFFINE>
+__global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma,
+                              const T* __restrict__ beta, const float* __restrict__ save_mean,
+                              const float* __restrict__ save_invstd, T* dx, float* pdg, float* pdb, GnGeom g) {
+    extern __shared__ float lds[];                  // [16] reduction scratch, then [nw][Cg] x 2
+    float* sm = lds;
+    const uint32_t T_ = blockDim.x, nw = T_ >> 6, w = threadIdx.x >> 6;
+    float* accg = lds + 16 + (size_t)w * g.Cg;
+    float* accb = lds + 16 + (size_t)(nw + w) * g.Cg;
+    const uint32_t slice = blockIdx.x, k = slice % g.G, n = slice / g.G;
+    const size_t base = (size_t)slice * g.nvec * VEC;
+    const float mean = save_mean[slice], invstd = save_invstd[slice];
+    if constexpr (AFFINE) {
+        for (uint32_t i = threadIdx.x; i < 2 * nw * g.Cg; i += T_) lds[16 + i] = 0.0f;
+        __syncthreads();
+    }
+    float d[CACHED ? kGnCache : 1][VEC], v[CACHED ? kGnCache : 1][VEC];
+    float s1 = 0.0f, s2 = 0.0f;
+
+    // dy and g = dy * gamma for one vector; also returns the channel's parameters
+    auto grad_terms = [&](uint32_t q, const float (&dv)[VEC], const float (&xv)[VEC], float (&gv)[VEC], float& a, float& b) {
+        const uint32_t c = k * g.Cg + g.chdiv.div(q);
+        const float gm = gamma ? ld(gamma + c) : 1.0f;
+        const float sc = gm * invstd;
+        const float sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+        a = 0.0f;
+        b = 0.0f;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float dy = dv[e];
+            if constexpr (ACT != LUXHIP_ACT_IDENTITY) {
+                const float pre = fmaf(xv[e], sc, sh);
+                dy *= Act<ACT>::d(Act<ACT>::f(pre), pre);
+            }
+            const float xh = (xv[e] - mean) * invstd;
+            gv[e] = dy * gm;
+            a = fmaf(dy, xh, a);
+            b += dy;
+        }
+    };
+
+    const uint32_t iters = (g.nvec + T_ - 1) / T_;
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            if (q < g.nvec) {
+                gn_load<T, VEC>(delta, base + (size_t)q * VEC, d[u]);
+                gn_load<T, VEC>(x, base + (size_t)q * VEC, v[u]);
+            }
+        }
+    }
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            if ((uint32_t)u < iters) {              // uniform
+                const uint32_t q = u * T_ + threadIdx.x;
+                const bool active = q < g.nvec;
+                float gv[VEC], a = 0.0f, b = 0.0f;
+                if (active) {
+                    grad_terms(q, d[u], v[u], gv, a, b);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float xh = (v[u][e] - mean) * invstd;
+                        s1 += gv[e];
+                        s2 = fmaf(gv[e], xh, s2);
+                    }
+                }
+                if constexpr (AFFINE) {
+                    // the first lane of the wave decides whether the wave has work this round
+                    if (u * T_ + (w << 6) < g.nvec)
+                        wave_channel_accumulate(accg, accb, active ? g.chdiv.div(q) : 0u, a, b, active);
+                }
+            }
+        }
+    } else {
+        for (uint32_t u = 0; u < iters; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            const bool active = q < g.nvec;
+            float gv[VEC], a = 0.0f, b = 0.0f;
+            if (active) {
+                gn_load<T, VEC>(delta, base + (size_t)q * VEC, d[0]);
+                gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+                grad_terms(q, d[0], v[0], gv, a, b);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float xh = (v[0][e] - mean) * invstd;
+                    s1 += gv[e];
+                    s2 = fmaf(gv[e], xh, s2);
+                }
+            }
+            if constexpr (AFFINE) {
+                if (u * T_ + (w << 6) < g.nvec)
+                    wave_channel_accumulate(accg, accb, active ? g.chdiv.div(q) : 0u, a, b, active);
+            }
+        }
+    }
+    s1 = block_sum(s1, sm) * g.inv_m;
+    s2 = block_sum(s2, sm) * g.inv_m;
+
+    auto emit = [&](uint32_t q, const float (&dv)[VEC], const float (&xv)[VEC]) {
+        float gv[VEC], a, b, o[VEC];
+        grad_terms(q, dv, xv, gv, a, b);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float xh = (xv[e] - mean) * invstd;
+            o[e] = invstd * (gv[e] - s1 - xh * s2);
+        }
+        gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
+    };
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kGnCache; ++u) {
+            const uint32_t q = u * T_ + threadIdx.x;
+            if (q < g.nvec) emit(q, d[u], v[u]);
+        }
+    } else {
+        for (uint32_t q = threadIdx.x; q < g.nvec; q += T_) {
+            gn_load<T, VEC>(delta, base + (size_t)q * VEC, d[0]);
+            gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+            emit(q, d[0], v[0]);
+        }
+    }
+    if constexpr (AFFINE) {
+        __syncthreads();
+        for (uint32_t j = threadIdx.x; j < g.Cg; j += T_) {
+            float tg = 0.0f, tb = 0.0f;
+            for (uint32_t ww = 0; ww < nw; ++ww) {
+                tg += lds[16 + (size_t)ww * g.Cg + j];
+                tb += lds[16 + (size_t)(nw + ww) * g.Cg + j];
+            }
+            pdg[(size_t)n * g.C + k * g.Cg + j] = tg;
+            pdb[(size_t)n * g.C + k * g.Cg + j] = tb;
+        }
+    }
+}
+
+// dgamma[c] = sum_n pdg[n][c], dbeta[c] = sum_n pdb[n][c]
+template <typename T>
+__global__ void gn_param_finalize_kernel(const float* __restrict__ pdg, const float* __restrict__ pdb, T* dgamma,
+                                         T* dbeta, uint32_t C, uint32_t N) {
+    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float tg = 0.0f, tb = 0.0f;
+    for (uint32_t n = 0; n < N; ++n) {
+        tg += pdg[(size_t)n * C + c];
+        tb += pdb[(size_t)n * C + c];
+    }
+    if (dgamma) st(dgamma + c, tg);
+    if (dbeta) st(dbeta + c, tb);
+}
+
+// ------------------------------------------------------------------------------- host side
+static int gn_check(int dtype, int act, int64_t I, int64_t C, int64_t G, int64_t N) {
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_UNSUPPORTED_IF(act < 0 || act >= LUXHIP_ACT_COUNT, "unsupported activation id %d", act);
+    LUX_INVALID_IF(I < 0 || C < 0 || N < 0 || G <= 0, "invalid dimension");
+    LUX_INVALID_IF(C % G != 0, "number of channels %lld must be divisible by the number of groups %lld", (long long)C,
+                   (long long)G);
+    if (I > 0 && C > 0 && N > 0) {
+        const long double tot = (long double)I * (long double)C * (long double)N;
+        LUX_UNSUPPORTED_IF(tot >= 2147483648.0L, "tensors of 2^31 or more elements are not supported");
+    }
+    return LUXHIP_OK;
+}
+
+struct GnLaunch {
+    GnGeom g;
+    bool vec, cached;
+    unsigned threads, blocks;
+};
+
+template <typename T>
+static GnLaunch gn_plan(int64_t I, int64_t C, int64_t G, int64_t N, bool ptr_ok) {
+    constexpr int V = Vec<T>::N;
+    GnLaunch L;
+    const int64_t Cg = C / G, m = I * Cg;
+    L.vec = ptr_ok && I % V == 0;
+    const int vv = L.vec ? V : 1;
+    L.g.I = (uint32_t)I; L.g.Cg = (uint32_t)Cg; L.g.G = (uint32_t)G; L.g.C = (uint32_t)C;
+    L.g.nvec = (uint32_t)(m / vv);
+    L.g.chdiv = FastDiv((uint32_t)(I / vv));
+    L.g.inv_m = 1.0f / (float)m;
+    int64_t t = 64;
+    while (t < 1024 && t * kGnCache < L.g.nvec) t <<= 1;
+    L.threads = (unsigned)t;
+    L.cached = (int64_t)L.g.nvec <= t * kGnCache;
+    L.blocks = (unsigned)(G * N);
+    return L;
+}
+
+template <typename T>
+static int gn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, int64_t N, const T* x, const T* gamma,
+                       const T* beta, float eps, T* y, float* save_mean, float* save_invstd) {
+    constexpr int V = Vec<T>::N;
+    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(y));
+    ProfScope ps("gn_fwd_kernel", s);
+#define GN_FWD(A)                                                                                                     \
+    do {                                                                                                              \
+        if (L.vec && L.cached) gn_fwd_kernel<T, A, V, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);   \
+        else if (L.vec) gn_fwd_kernel<T, A, V, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);        \
+        else if (L.cached) gn_fwd_kernel<T, A, 1, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);      \
+        else gn_fwd_kernel<T, A, 1, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);                   \
+    } while (0)
+    LUX_DISPATCH_ACT(act, GN_FWD);
+#undef GN_FWD
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, int64_t N, const T* delta, const T* x,
+                       const T* gamma, const T* beta, const float* save_mean, const float* save_invstd, T* dx,
+                       T* dgamma, T* dbeta) {
+    constexpr int V = Vec<T>::N;
+    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(delta) && aligned16(dx));
+    const bool affine = gamma != nullptr && (dgamma != nullptr || dbeta != nullptr);
+    // LDS: 16 floats of reduction scratch + 2 * nw * Cg accumulators
+    size_t lds_bytes = 64;
+    if (affine) {
+        while (L.threads > 64 && (16 + 2 * (size_t)(L.threads / 64) * L.g.Cg) * 4 > 60 * 1024) {
+            L.threads >>= 1;
+            L.cached = (int64_t)L.g.nvec <= (int64_t)L.threads * kGnCache;
+        }
+        lds_bytes = (16 + 2 * (size_t)(L.threads / 64) * L.g.Cg) * 4;
+        LUX_UNSUPPORTED_IF(lds_bytes > 60 * 1024, "groupnorm_bwd: %u channels per group exceed the LDS accumulators", L.g.Cg);
+    }
+    float *pdg = nullptr, *pdb = nullptr;
+    if (affine) {
+        Workspace ws;
+        int rc = get_workspace(s, (size_t)2 * N * C * sizeof(float), &ws);
+        if (rc != LUXHIP_OK) return rc;
+        pdg = reinterpret_cast<float*>(ws.data);
+        pdb = pdg + (size_t)N * C;
+    }
+    {
+        ProfScope ps("gn_bwd_kernel", s);
+#define GN_BWD_A(A, VV, CA)                                                                                           \
+    do {                                                                                                              \
+        if (affine) gn_bwd_kernel<T, A, VV, CA, true><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, L.g); \
+        else gn_bwd_kernel<T, A, VV, CA, false><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, L.g);       \
+    } while (0)
+#define GN_BWD(A)                                                                                                     \
+    do {                                                                                                              \
+        if (L.vec && L.cached) GN_BWD_A(A, V, true);                                                                  \
+        else if (L.vec) GN_BWD_A(A, V, false);                                                                        \
+        else if (L.cached) GN_BWD_A(A, 1, true);                                                                      \
+        else GN_BWD_A(A, 1, false);                                                                                   \
+    } while (0)
+        LUX_DISPATCH_ACT(act, GN_BWD);
+#undef GN_BWD
+#undef GN_BWD_A
+    }
+    LUX_CHECK_LAUNCH();
+    if (affine) {
+        ProfScope ps("gn_param_finalize_kernel", s);
+        gn_param_finalize_kernel<T><<<(unsigned)ceil_div(C, 128), 128, 0, s>>>(pdg, pdb, dgamma, dbeta, (uint32_t)C, (uint32_t)N);
+        LUX_CHECK_LAUNCH();
+    }
+    return LUXHIP_OK;
+}
+
+}  // namespace luxhip
+
+using namespace luxhip;
+
+extern "C" {
+
+int luxhip_groupnorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t G, int64_t N, const void* x,
+                         const void* gamma, const void* beta, double eps, void* y, float* save_mean,
+                         float* save_invstd) {
+    LUX_REQUIRE_INIT();
+    int rc = gn_check(dtype, act, I, C, G, N);
+    if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF((gamma == nullptr) != (beta == nullptr), "groupnorm_fwd: gamma and beta must be given together");
+    if (I * C * N == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(x == nullptr || y == nullptr, "groupnorm_fwd: x and y must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return gn_fwd_impl<float>((hipStream_t)s, act, I, C, G, N, (const float*)x, (const float*)gamma, (const float*)beta,
+                                  (float)eps, (float*)y, save_mean, save_invstd);
+    return gn_fwd_impl<bf16_t>((hipStream_t)s, act, I, C, G, N, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta,
+                               (float)eps, (bf16_t*)y, save_mean, save_invstd);
+}
+
+int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t G, int64_t N,
+                         const void* delta, const void* x, const void* gamma, const void* beta, const float* save_mean,
+                         const float* save_invstd, void* dx, void* dgamma, void* dbeta) {
+    LUX_REQUIRE_INIT();
+    int rc = gn_check(dtype, act, I, C, G, N);
+    if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF((gamma == nullptr) != (beta == nullptr), "groupnorm_bwd: gamma and beta must be given together");
+    if (I * C * N == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(delta == nullptr || x == nullptr || dx == nullptr || save_mean == nullptr || save_invstd == nullptr,
+                   "groupnorm_bwd: delta, x, dx, save_mean and save_invstd must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return gn_bwd_impl<float>((hipStream_t)s, act, I, C, G, N, (const float*)delta, (const float*)x, (const float*)gamma,
+                                  (const float*)beta, save_mean, save_invstd, (float*)dx, (float*)dgamma, (float*)dbeta);
+    return gn_bwd_impl<bf16_t>((hipStream_t)s, act, I, C, G, N, (const bf16_t*)delta, (const bf16_t*)x, (const bf16_t*)gamma,
+                               (const bf16_t*)beta, save_mean, save_invstd, (bf16_t*)dx, (bf16_t*)dgamma, (bf16_t*)dbeta);
+}
+
+}  // extern "C"

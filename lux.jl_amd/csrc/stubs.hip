@@ -3,10 +3,6 @@
 using namespace luxhip;
 extern "C" {
 #define NOT_YET(name) return set_error(LUXHIP_UNSUPPORTED, name ": not implemented yet")
-int luxhip_groupnorm_fwd(luxhip_stream_t, int, int, int64_t, int64_t, int64_t, int64_t, const void*, const void*, const void*, double, void*, float*, float*) { NOT_YET("groupnorm_fwd"); }
-int luxhip_groupnorm_bwd(luxhip_stream_t, int, int, int64_t, int64_t, int64_t, int64_t, const void*, const void*, const void*, const void*, const float*, const float*, void*, void*, void*) { NOT_YET("groupnorm_bwd"); }
-int luxhip_layernorm_fwd(luxhip_stream_t, int, int, int64_t, int64_t, const void*, const void*, const void*, double, void*, float*, float*) { NOT_YET("layernorm_fwd"); }
-int luxhip_layernorm_bwd(luxhip_stream_t, int, int, int64_t, int64_t, const void*, const void*, const void*, const void*, const float*, const float*, void*, void*, void*) { NOT_YET("layernorm_bwd"); }
 int luxhip_matmul(luxhip_stream_t, int, int, int, int64_t, int64_t, int64_t, const void*, int64_t, const void*, int64_t, const void*, void*, int64_t) { NOT_YET("matmul"); }
 int luxhip_fused_dense_fwd(luxhip_stream_t, int, int, int64_t, int64_t, int64_t, const void*, int64_t, const void*, int64_t, const void*, void*, int64_t, void*) { NOT_YET("fused_dense_fwd"); }
 int luxhip_fused_dense_bwd(luxhip_stream_t, int, int, int64_t, int64_t, int64_t, const void*, const void*, const void*, const void*, int64_t, const void*, int64_t, void*, void*, void*, void*) { NOT_YET("fused_dense_bwd"); }

@@ -1,0 +1,91 @@
+"""groupnorm forward + pullback on the GPU against the oracle
+(mirrors lib/LuxLib/test/normalization/groupnorm_tests.jl:48-115 of the reference)."""
+import numpy as np
+import pytest
+
+from oracle import luxlib_oracle as O
+from tests.util import assert_close, dev, f64, host_inputs, rms
+
+pytestmark = pytest.mark.gpu
+
+CASES = [((6, 2), 2), ((4, 4, 6, 2), 3), ((2, 2, 6, 2), 2), ((5, 12, 3), 4), ((16, 16, 8, 3), 2), ((64, 6, 2), 3),
+         ((32, 32, 12, 2), 1), ((8, 8, 16, 2), 16), ((96, 96, 4, 2), 1)]
+
+
+def dx_scale(x, g, groups, eps, delta):
+    xv, Cg = O._gn_view(f64(x), groups)
+    axes = tuple(range(xv.ndim - 2))
+    var = xv.var(axis=axes, keepdims=True)
+    gg = 1.0 if g is None else np.abs(f64(g)).max()
+    return rms(f64(delta)) * gg / float(np.sqrt(var.min() + eps))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("act", ["identity", "relu", "sigmoid_fast", "swish", "gelu"])
+@pytest.mark.parametrize("affine", [True, False])
+def test_forward_and_pullback(gpu, dtype, act, affine):
+    rng = np.random.default_rng(abs(hash((dtype, act, affine))) % 2 ** 31)
+    for shape, groups in CASES:
+        Cc = shape[-2]
+        x, g, b, delta = host_inputs(dtype, rng.normal(size=shape), rng.uniform(0.8, 1.2, Cc) if affine else None,
+                                     rng.normal(size=Cc) * 0.05 if affine else None, rng.normal(size=shape))
+        eps = 1e-5 if dtype == "f32" else 1e-3
+        tag = f"{dtype} {act} {shape} G={groups} affine={affine}"
+        y, back = gpu.pullback(gpu.groupnorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), groups, act, eps)
+        wy = O.groupnorm(f64(x), f64(g), f64(b), groups, act, eps)
+        assert_close(y.to_numpy(), wy, dtype, tag + " y", want32=O.groupnorm(x, g, b, groups, act, np.float32(eps)))
+        y2 = gpu.groupnorm(dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), groups, act, eps)
+        np.testing.assert_array_equal(y2.to_numpy(), y.to_numpy())
+        gx, gg, gb = back(dev(gpu, delta, dtype))
+        wdx, wdg, wdb = O.groupnorm_pullback(f64(x), f64(g), f64(b), groups, act, eps, f64(delta))
+        w32 = O.groupnorm_pullback(x, g, b, groups, act, np.float32(eps), delta)
+        rel = None if dtype == "f32" else 3e-2
+        assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=dx_scale(x, g, groups, eps, delta), want32=w32[0])
+        if affine:
+            assert_close(gg.to_numpy(), wdg, dtype, tag + " dgamma", rel=rel, scale=rms(delta), want32=w32[1])
+            assert_close(gb.to_numpy(), wdb, dtype, tag + " dbeta", rel=rel, scale=rms(delta), want32=w32[2])
+        else:
+            assert gg is None and gb is None
+
+
+def test_argument_errors(gpu):
+    d = lambda *s: gpu.DeviceArray.from_numpy(np.ones(s, np.float32))
+    with pytest.raises(gpu.ArgumentError):
+        gpu.groupnorm(d(4, 6, 2), d(6), d(6), 4)
+    with pytest.raises(gpu.ArgumentError):
+        gpu.groupnorm(d(4, 6, 2), d(5), d(5), 2)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_config3_full_size(gpu, dtype):
+    """BASELINE config 3 at full size: x 64x64x256x16, 32 groups, swish.  Oracle comparison on
+    two samples; whole-tensor invariants: per-(group, sample) slices of dx sum to zero and are
+    orthogonal to xhat (the two conservation laws of the normalisation pullback)."""
+    rng = np.random.default_rng(1002)
+    shape, G = (64, 64, 256, 16), 32
+    x = rng.standard_normal(size=shape, dtype=np.float32)
+    g = rng.uniform(0.8, 1.2, 256).astype(np.float32)
+    b = (0.05 * rng.standard_normal(256)).astype(np.float32)
+    delta = rng.standard_normal(size=shape, dtype=np.float32)
+    x, g, b, delta = host_inputs(dtype, x, g, b, delta)
+    eps = 1e-5
+    y, back = gpu.pullback(gpu.groupnorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), G, "swish", eps)
+    gx, gg, gb = back(dev(gpu, delta, dtype))
+    yh, gxh = y.to_numpy(), gx.to_numpy().astype(np.float64)
+    sub = [0, 11]
+    wy = O.groupnorm(f64(x[..., sub]), f64(g), f64(b), G, "swish", eps)
+    assert_close(yh[..., sub], wy, dtype, "config3 y")
+    wdx, _, _ = O.groupnorm_pullback(f64(x[..., sub]), f64(g), f64(b), G, "swish", eps, f64(delta[..., sub]))
+    assert_close(gxh[..., sub], wdx, dtype, "config3 dx", rel=None if dtype == "f32" else 3e-2)
+    # conservation laws on every slice
+    xs = f64(x).reshape(64 * 64 * 8, 32, 16, order="F")
+    ds = gxh.reshape(64 * 64 * 8, 32, 16, order="F")
+    xh = (xs - xs.mean(axis=0)) / np.sqrt(xs.var(axis=0) + eps)
+    tol = 1e-2 if dtype == "f32" else 3.0
+    assert np.abs(ds.sum(axis=0)).max() < tol
+    assert np.abs((ds * xh).sum(axis=0)).max() < tol
+    # parameter gradients against an fp64 reduction of the full tensors
+    _, wdg, wdb = O.groupnorm_pullback(f64(x), f64(g), f64(b), G, "swish", eps, f64(delta))
+    rel = None if dtype == "f32" else 3e-2
+    assert_close(gg.to_numpy(), wdg, dtype, "config3 dgamma", rel=rel, scale=rms(delta) * 10)
+    assert_close(gb.to_numpy(), wdb, dtype, "config3 dbeta", rel=rel, scale=rms(delta) * 10)

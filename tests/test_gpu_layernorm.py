@@ -1,0 +1,94 @@
+"""layernorm forward + pullback on the GPU against the oracle
+(mirrors lib/LuxLib/test/normalization/layernorm_tests.jl:22-113 of the reference)."""
+import numpy as np
+import pytest
+
+from oracle import luxlib_oracle as O
+from tests.util import assert_close, dev, f64, host_inputs, rms
+
+pytestmark = pytest.mark.gpu
+
+# (shape, number of leading normalised dims)
+CASES = [((4, 4, 6, 2), 3), ((6, 3), 1), ((16, 5), 1), ((3, 4, 5), 1), ((3, 4, 5), 2), ((512, 9), 1), ((1000, 7), 1),
+         ((4096, 6), 1), ((20000, 3), 1), ((24, 24, 8, 5), 3)]
+
+
+def test_invariants_without_affine(gpu):
+    # layernorm_tests.jl:54-57: mean(y) ~ 0, std(y) ~ 1
+    x = O.generate_fixed_array(np.float32, (4, 4, 6, 2))
+    y = gpu.layernorm(gpu.DeviceArray.from_numpy(x), None, None, "identity", (1, 2, 3)).to_numpy()
+    assert abs(y.mean(axis=(0, 1, 2))).max() < 1e-5
+    np.testing.assert_allclose(y.std(axis=(0, 1, 2)), 1, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("act", ["identity", "relu", "gelu", "tanh"])
+@pytest.mark.parametrize("affine", [True, False])
+def test_forward_and_pullback(gpu, dtype, act, affine):
+    rng = np.random.default_rng(abs(hash((dtype, act, affine))) % 2 ** 31)
+    for shape, nd in CASES:
+        pshape = shape[:nd] + (1,) * (len(shape) - nd)
+        x, g, b, delta = host_inputs(dtype, rng.normal(size=shape), rng.uniform(0.5, 1.5, pshape) if affine else None,
+                                     rng.normal(size=pshape) if affine else None, rng.normal(size=shape))
+        eps = 1e-5 if dtype == "f32" else 1e-3
+        dims_np, dims_jl = tuple(range(nd)), tuple(range(1, nd + 1))
+        tag = f"{dtype} {act} {shape} nd={nd} affine={affine}"
+        y, back = gpu.pullback(gpu.layernorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), act, dims_jl, eps)
+        wy = O.layernorm(f64(x), f64(g), f64(b), act, dims_np, eps)
+        assert_close(y.to_numpy(), wy, dtype, tag + " y", want32=O.layernorm(x, g, b, act, dims_np, np.float32(eps)))
+        gx, gg, gb = back(dev(gpu, delta, dtype))
+        wdx, wdg, wdb = O.layernorm_pullback(f64(x), f64(g), f64(b), act, dims_np, eps, f64(delta))
+        w32 = O.layernorm_pullback(x, g, b, act, dims_np, np.float32(eps), delta)
+        rel = None if dtype == "f32" else 3e-2
+        var = f64(x).var(axis=dims_np)
+        scale = rms(delta) * (1.5 if affine else 1.0) / float(np.sqrt(var.min() + eps))
+        assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=scale, want32=w32[0])
+        if affine:
+            assert gg.shape == pshape and gb.shape == pshape
+            assert_close(gg.to_numpy(), wdg, dtype, tag + " dgamma", rel=rel, scale=rms(delta), want32=w32[1])
+            assert_close(gb.to_numpy(), wdb, dtype, tag + " dbeta", rel=rel, scale=rms(delta), want32=w32[2])
+        else:
+            assert gg is None and gb is None
+
+
+def test_default_dims_and_errors(gpu):
+    rng = np.random.default_rng(2)
+    x = rng.normal(size=(6, 5, 4)).astype(np.float32)
+    g = rng.normal(size=(6, 5, 1)).astype(np.float32)
+    b = rng.normal(size=(6, 5, 1)).astype(np.float32)
+    d = gpu.DeviceArray.from_numpy
+    y = gpu.layernorm(d(x), d(g), d(b))                      # dims default 1:(N-1)
+    assert_close(y.to_numpy(), O.layernorm(f64(x), f64(g), f64(b), "identity", (0, 1), O.default_epsilon(np.float32)),
+                 "f32", "default dims")
+    with pytest.raises(gpu.ArgumentError):                   # layernorm_tests.jl:100-113
+        gpu.layernorm(d(x), None, None, "identity", None)
+    with pytest.raises(gpu.Unsupported):                     # non-leading dims: generic host path
+        gpu.layernorm(d(x), None, None, "identity", (2,))
+
+
+def test_config4_layernorm_full_size(gpu):
+    """BASELINE config 4's layernorm: 4096 features x 8192 tokens, bf16, affine.  Oracle on a
+    token subset; invariants on all tokens (normalised rows have zero mean / unit variance;
+    dx rows sum to zero and are orthogonal to xhat)."""
+    rng = np.random.default_rng(1003)
+    L, R = 4096, 8192
+    x = rng.standard_normal(size=(L, R), dtype=np.float32)
+    g = rng.uniform(0.5, 1.5, (L, 1)).astype(np.float32)
+    b = (0.1 * rng.standard_normal((L, 1))).astype(np.float32)
+    delta = (0.02 * rng.standard_normal(size=(L, R), dtype=np.float32))
+    x, g, b, delta = host_inputs("bf16", x, g, b, delta)
+    eps = 1e-5
+    y, back = gpu.pullback(gpu.layernorm, dev(gpu, x, "bf16"), dev(gpu, g, "bf16"), dev(gpu, b, "bf16"), "identity", (1,), eps)
+    gx, gg, gb = back(dev(gpu, delta, "bf16"))
+    yh, gxh = y.to_numpy(), gx.to_numpy().astype(np.float64)
+    sub = slice(0, R, 257)
+    assert_close(yh[:, sub], O.layernorm(f64(x[:, sub]), f64(g), f64(b), "identity", (0,), eps), "bf16", "config4 LN y")
+    wdx, _, _ = O.layernorm_pullback(f64(x[:, sub]), f64(g), f64(b), "identity", (0,), eps, f64(delta[:, sub]))
+    assert_close(gxh[:, sub], wdx, "bf16", "config4 LN dx", rel=3e-2)
+    xh = (yh.astype(np.float64) - f64(b)) / f64(g)
+    assert np.abs(xh.mean(axis=0)).max() < 2e-2
+    assert np.abs(xh.var(axis=0) - 1).max() < 3e-2
+    assert np.abs(gxh.sum(axis=0)).max() < 0.5            # 4096 bf16-rounded terms of size ~0.02
+    _, wdg, wdb = O.layernorm_pullback(f64(x), f64(g), f64(b), "identity", (0,), eps, f64(delta))
+    assert_close(gg.to_numpy(), wdg, "bf16", "config4 LN dgamma", rel=3e-2, scale=rms(delta) * 90)
+    assert_close(gb.to_numpy(), wdb, "bf16", "config4 LN dbeta", rel=3e-2, scale=rms(delta) * 90)
