@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T*
         const size_t off = ((size_t)q + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
         float r[VEC];
         dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
-        store_vec<T, VEC>(dx, off, r);
+        if (dx) store_vec<T, VEC>(dx, off, r);
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc += r[k];
     }
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_plane_kernel(const T* _
         const size_t off = (size_t)n * P + p;
         float r[VEC];
         dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
-        store_vec<T, VEC>(dx, off, r);
+        if (dx) store_vec<T, VEC>(dx, off, r);
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] += r[k];
     }
@@ -373,6 +373,23 @@ static int check_common(int dtype, int act, int64_t I, int64_t C, int64_t N) {
         LUX_UNSUPPORTED_IF(tot >= 2147483648.0L, "tensors of 2^31 or more elements are not supported");
     }
     return LUXHIP_OK;
+}
+
+// Shared with the dense and convolution pullbacks: dx may be NULL (bias gradient only).
+int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* delta,
+                          const void* out, const void* pre, void* dx, void* dbias) {
+    int rc = check_common(dtype, act, I, C, N);
+    if (rc != LUXHIP_OK) return rc;
+    if (I * C * N == 0) {
+        if (dbias != nullptr && C > 0) return luxhip_fill_zero(dbias, (size_t)C * (dtype == LUXHIP_F32 ? 4 : 2), s);
+        return LUXHIP_OK;
+    }
+    if (dx == nullptr && dbias == nullptr) return LUXHIP_OK;
+    if (dtype == LUXHIP_F32)
+        return bias_act_bwd_impl<float>(s, act, I, C, N, (const float*)delta, (const float*)out, (const float*)pre,
+                                        (float*)dx, (float*)dbias);
+    return bias_act_bwd_impl<bf16_t>(s, act, I, C, N, (const bf16_t*)delta, (const bf16_t*)out, (const bf16_t*)pre,
+                                     (bf16_t*)dx, (bf16_t*)dbias);
 }
 
 }  // namespace luxhip

@@ -1,0 +1,278 @@
+// LDS-staged MFMA GEMM mainloop for gfx950, shared by the dense and convolution kernels.
+//
+//   C(m, n) = sum_k A(m, k) * B(k, n),  fp32 accumulation.
+//
+// A workgroup of 4 waves (2 along m x 2 along n) owns a (2*WM*32) x (2*WN*32) tile of C; each
+// wave owns WM x WN MFMA tiles of 32 x 32.  The MFMA "row" dimension is mapped to n and the
+// "column" dimension (one column per lane) to m, so that the 32 lanes of a half-wave hold 32
+// consecutive m: stores to the column-major C are contiguous and a per-m bias is one value per
+// lane.
+//
+// Storage types:  bf16 -> v_mfma_f32_32x32x16_bf16 (BK = 64 per stage),
+//                 fp32 -> v_mfma_f32_32x32x2_f32   (BK = 16 per stage).
+//
+// Each operand tile is staged global -> registers -> LDS (double buffered, one barrier per
+// stage) in the layout that matches how it lies in memory:
+//   K-major operand  (k contiguous): LDS [row][BK]; bf16 rows are 128 B with an XOR swizzle of
+//       the 16-byte chunk index so that the ds_read_b128 fragment reads of 8 consecutive rows
+//       fall into different banks; fp32 rows are padded by 4 floats.
+//   MN-major operand (m or n contiguous, k strided): LDS [k][rows + pad]; bf16 fragments are
+//       read with ds_read_b64_tr_b16 (the LDS transpose read of gfx950), which hands each lane
+//       the 4 consecutive k of its own row out of a 4(k) x 16(rows) block; fp32 fragments are
+//       plain ds_read_b32.
+// The same (lane group, slot) -> k assignment is used for both operands of an MFMA, which is
+// all the instruction needs.
+#pragma once
+
+#include "common.h"
+
+namespace luxhip {
+
+typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
+typedef float f32x16_v __attribute__((ext_vector_type(16)));
+typedef short s16x4_v __attribute__((ext_vector_type(4)));
+typedef short s16x8_v __attribute__((ext_vector_type(8)));
+
+constexpr int kGemmThreads = 256;
+
+template <typename T>
+struct GemmTraits;
+template <>
+struct GemmTraits<bf16_t> {
+    static constexpr int BK = 64, VEC = 8, KSTEP = 16;   // KSTEP: k consumed per fragment load
+    static constexpr int PAD_MN = 16;
+    __host__ __device__ static constexpr int kmajor_stride() { return BK; }
+};
+template <>
+struct GemmTraits<float> {
+    static constexpr int BK = 16, VEC = 4, KSTEP = 8;
+    static constexpr int PAD_MN = 4;
+    __host__ __device__ static constexpr int kmajor_stride() { return BK + 4; }
+};
+
+// elements of one LDS stage of an operand tile with `rows` rows
+template <typename T, bool KMAJOR>
+__host__ __device__ constexpr int lds_tile_elems(int rows) {
+    return KMAJOR ? rows * GemmTraits<T>::kmajor_stride() : GemmTraits<T>::BK * (rows + GemmTraits<T>::PAD_MN);
+}
+
+// An operand seen as rows x K: element (r, k) at p[r*sr + k*sk]; one of sr, sk is 1.
+template <typename T>
+struct Operand {
+    const T* p;
+    int64_t sr, sk;
+    int rows;      // valid rows (M or N)
+    int vec_ok;    // 16-byte loads along the contiguous dimension are aligned
+};
+
+// ----------------------------------------------------------------------------- global -> registers
+template <typename T, bool KMAJOR, int ROWS>
+struct TileLoader {
+    using Tr = GemmTraits<T>;
+    static constexpr int CHUNKS = ROWS * Tr::BK / Tr::VEC;
+    static constexpr int PER_THREAD = CHUNKS / kGemmThreads;
+    static_assert(CHUNKS % kGemmThreads == 0, "tile must split evenly over the workgroup");
+    uint4 reg[PER_THREAD];
+
+    __device__ __forceinline__ static void coords(int id, int& r, int& k) {
+        if constexpr (KMAJOR) {
+            r = id / (Tr::BK / Tr::VEC);
+            k = (id % (Tr::BK / Tr::VEC)) * Tr::VEC;
+        } else {
+            k = id / (ROWS / Tr::VEC);
+            r = (id % (ROWS / Tr::VEC)) * Tr::VEC;
+        }
+    }
+
+    __device__ __forceinline__ void load(const Operand<T>& op, int r0, int k0, int K) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            int r, k;
+            coords(threadIdx.x + i * kGemmThreads, r, k);
+            r += r0;
+            k += k0;
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            const int rem = KMAJOR ? (K - k) : (op.rows - r);     // valid elements along the chunk
+            const bool in = KMAJOR ? (r < op.rows) : (k < K);
+            if (in && rem > 0) {
+                const T* src = op.p + (int64_t)r * op.sr + (int64_t)k * op.sk;
+                if (op.vec_ok && rem >= Tr::VEC) {
+                    v = *reinterpret_cast<const uint4*>(src);
+                } else {
+                    T tmp[Tr::VEC];
+#pragma unroll
+                    for (int e = 0; e < Tr::VEC; ++e) tmp[e] = e < rem ? src[e] : T(0);
+                    v = *reinterpret_cast<const uint4*>(tmp);
+                }
+            }
+            reg[i] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(T* lds) const {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            int r, k;
+            coords(threadIdx.x + i * kGemmThreads, r, k);
+            int off;
+            if constexpr (KMAJOR) {
+                if constexpr (sizeof(T) == 2) off = r * Tr::BK + (((k >> 3) ^ (r & 7)) << 3);
+                else off = r * Tr::kmajor_stride() + k;
+            } else {
+                off = k * (ROWS + Tr::PAD_MN) + r;
+            }
+            *reinterpret_cast<uint4*>(lds + off) = reg[i];
+        }
+    }
+};
+
+// ----------------------------------------------------------------------------- LDS -> fragments
+// bf16: fragment of 32 rows x 16 k (one k-step `kk` of the stage) for rows rbase..rbase+31
+template <bool KMAJOR, int ROWS>
+__device__ __forceinline__ bf16x8_v load_frag_bf16(const bf16_t* lds, int rbase, int kk) {
+    const int l = threadIdx.x & 63;
+    if constexpr (KMAJOR) {
+        const int r = rbase + (l & 31);
+        const int chunk = 2 * kk + (l >> 5);
+        const uint4 v = *reinterpret_cast<const uint4*>(lds + r * 64 + ((chunk ^ (r & 7)) << 3));
+        return __builtin_bit_cast(bf16x8_v, v);
+    } else {
+        constexpr int STRIDE = ROWS + GemmTraits<bf16_t>::PAD_MN;
+        const int b = l >> 4, s = l & 15;
+        const int r = rbase + ((b & 1) << 4) + ((s & 3) << 2);
+        const int k = kk * 16 + ((b >> 1) << 3) + (s >> 2);
+        typedef __attribute__((address_space(3))) s16x4_v* lds_ptr;
+        const bf16_t* p0 = lds + k * STRIDE + r;
+        const s16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+        const s16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 4 * STRIDE));
+        s16x8_v v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(bf16x8_v, v);
+    }
+}
+
+// fp32: 4 floats per lane covering one 8-k window `kw`: slot s <-> k = kw*8 + 4*(lane/32) + s
+template <bool KMAJOR, int ROWS>
+__device__ __forceinline__ void load_frag_f32(const float* lds, int rbase, int kw, float (&f)[4]) {
+    const int l = threadIdx.x & 63;
+    const int r = rbase + (l & 31), kb = kw * 8 + ((l >> 5) << 2);
+    if constexpr (KMAJOR) {
+        const float4 v = *reinterpret_cast<const float4*>(lds + r * GemmTraits<float>::kmajor_stride() + kb);
+        f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+    } else {
+        constexpr int STRIDE = ROWS + GemmTraits<float>::PAD_MN;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) f[s] = lds[(kb + s) * STRIDE + r];
+    }
+}
+
+// ----------------------------------------------------------------------------- tile -> C coordinates
+// XCD-aware ordering: consecutive workgroup ids land on different XCDs (8 of them, each with
+// its own L2), so ids are first regrouped per XCD and then walked in groups of 8 tiles along m.
+__device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int nb = gridDim.x, bid = blockIdx.x;
+    const int per = nb >> 3;
+    const int lid = bid < (per << 3) ? (bid & 7) * per + (bid >> 3) : bid;
+    constexpr int GROUP = 8;
+    const int in_group = GROUP * tiles_n;
+    const int first_m = (lid / in_group) * GROUP;
+    const int gsize = min(tiles_m - first_m, GROUP);
+    tm = first_m + (lid % in_group) % gsize;
+    tn = (lid % in_group) / gsize;
+}
+
+// ----------------------------------------------------------------------------- mainloop
+// Accumulates the (2*WM*32) x (2*WN*32) tile at (m0, n0).  acc[wm][wn][r] of lane l belongs to
+//   m = m0 + wave_m*WM*32 + wm*32 + l%32,   n = n0 + wave_n*WN*32 + wn*32 + 8*(r/4) + 4*(l/32) + r%4.
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+struct GemmMainloop {
+    using Tr = GemmTraits<T>;
+    static constexpr int TILE_M = 2 * WM * 32, TILE_N = 2 * WN * 32;
+    static constexpr int A_ELEMS = lds_tile_elems<T, A_KMAJOR>(TILE_M);
+    static constexpr int B_ELEMS = lds_tile_elems<T, B_KMAJOR>(TILE_N);
+    static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
+    static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * sizeof(T);
+
+    __device__ __forceinline__ static void run(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0, T* lds,
+                                               f32x16_v (&acc)[WM][WN]) {
+        const int w = threadIdx.x >> 6;
+        const int wave_m = (w & 1) * (WM * 32), wave_n = (w >> 1) * (WN * 32);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+        TileLoader<T, A_KMAJOR, TILE_M> la;
+        TileLoader<T, B_KMAJOR, TILE_N> lb;
+        const int KT = (K + Tr::BK - 1) / Tr::BK;
+        la.load(A, m0, 0, K);
+        lb.load(B, n0, 0, K);
+        la.store(lds);
+        lb.store(lds + A_ELEMS);
+        __syncthreads();
+        for (int kt = 0; kt < KT; ++kt) {
+            T* cur = lds + (kt & 1) * STAGE_ELEMS;
+            T* nxt = lds + ((kt + 1) & 1) * STAGE_ELEMS;
+            const bool more = kt + 1 < KT;
+            if (more) {
+                la.load(A, m0, (kt + 1) * Tr::BK, K);
+                lb.load(B, n0, (kt + 1) * Tr::BK, K);
+            }
+            const T* As = cur;
+            const T* Bs = cur + A_ELEMS;
+            if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                for (int kk = 0; kk < Tr::BK / 16; ++kk) {
+                    bf16x8_v fa[WM], fb[WN];
+#pragma unroll
+                    for (int i = 0; i < WM; ++i) fa[i] = load_frag_bf16<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kk);
+#pragma unroll
+                    for (int j = 0; j < WN; ++j) fb[j] = load_frag_bf16<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kk);
+#pragma unroll
+                    for (int i = 0; i < WM; ++i)
+#pragma unroll
+                        for (int j = 0; j < WN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int kw = 0; kw < Tr::BK / 8; ++kw) {
+                    float fa[WM][4], fb[WN][4];
+#pragma unroll
+                    for (int i = 0; i < WM; ++i) load_frag_f32<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kw, fa[i]);
+#pragma unroll
+                    for (int j = 0; j < WN; ++j) load_frag_f32<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kw, fb[j]);
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+#pragma unroll
+                        for (int i = 0; i < WM; ++i)
+#pragma unroll
+                            for (int j = 0; j < WN; ++j)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][s], fa[i][s], acc[i][j], 0, 0, 0);
+                }
+            }
+            if (more) {
+                la.store(nxt);
+                lb.store(nxt + A_ELEMS);
+            }
+            __syncthreads();
+        }
+    }
+
+    // Calls f(m, n, value) for every element of the tile owned by this lane.
+    template <typename F>
+    __device__ __forceinline__ static void for_each(const f32x16_v (&acc)[WM][WN], int m0, int n0, F&& f) {
+        const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
+        const int mb = m0 + (w & 1) * (WM * 32) + (l & 31);
+        const int nb = n0 + (w >> 1) * (WN * 32) + ((l >> 5) << 2);
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) f(mb + i * 32, nb + j * 32 + ((r >> 2) << 3) + (r & 3), acc[i][j][r]);
+    }
+};
+
+}  // namespace luxhip

@@ -1,0 +1,79 @@
+// Dense GEMM kernel (MFMA mainloop of gemm_core.h + bias / activation / pre-activation
+// epilogue) and its tile-size selection.  launch_layout<T, A_KMAJOR, B_KMAJOR> is explicitly
+// instantiated in gemm_inst_*.hip, one translation unit per storage type and layout pair, so
+// that the heavy kernels compile in parallel.
+#pragma once
+
+#include <algorithm>
+
+#include "common.h"
+#include "gemm_core.h"
+#include "gemm_dense_decl.h"
+
+namespace luxhip {
+
+__device__ __forceinline__ float apply_act(int act, float x) {
+    switch (act) {
+        case LUXHIP_ACT_RELU: return Act<LUXHIP_ACT_RELU>::f(x);
+        case LUXHIP_ACT_TANH: return Act<LUXHIP_ACT_TANH>::f(x);
+        case LUXHIP_ACT_SIGMOID: return Act<LUXHIP_ACT_SIGMOID>::f(x);
+        case LUXHIP_ACT_SWISH: return Act<LUXHIP_ACT_SWISH>::f(x);
+        case LUXHIP_ACT_GELU: return Act<LUXHIP_ACT_GELU>::f(x);
+        case LUXHIP_ACT_SOFTPLUS: return Act<LUXHIP_ACT_SOFTPLUS>::f(x);
+        case LUXHIP_ACT_LOGSIGMOID: return Act<LUXHIP_ACT_LOGSIGMOID>::f(x);
+        case LUXHIP_ACT_LISHT: return Act<LUXHIP_ACT_LISHT>::f(x);
+        default: return x;
+    }
+}
+
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(kGemmThreads) void dense_gemm_kernel(DenseArgs<T> a) {
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR>;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    int tm, tn;
+    tile_coords(a.tiles_m, a.tiles_n, tm, tn);
+    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+    f32x16_v acc[WM][WN];
+    ML::run(a.A, a.B, a.K, m0, n0, lds, acc);
+    const int act = a.act;
+    ML::for_each(acc, m0, n0, [&](int m, int n, float v) {
+        if (m < a.M && n < a.N) {
+            if (a.bias) v += ld(a.bias + m);
+            const int64_t off = m + (int64_t)n * a.ldc;
+            if (a.pre) st(a.pre + off, v);
+            st(a.C + off, apply_act(act, v));
+        }
+    });
+}
+
+template <typename T, int WM, int WN, bool AK, bool BKM>
+int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
+    using ML = GemmMainloop<T, WM, WN, AK, BKM>;
+    a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
+    a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
+    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)ML::LDS_BYTES));
+        attr_set = true;
+    }
+    ProfScope ps(sizeof(T) == 2 ? "dense_gemm_kernel<bf16>" : "dense_gemm_kernel<f32>", s);
+    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(kGemmThreads), ML::LDS_BYTES, s>>>(a);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T, bool AK, bool BKM>
+int launch_layout(hipStream_t s, DenseArgs<T>& a) {
+    // largest tile that still yields at least ~one workgroup per compute unit
+    const int64_t cus = std::max(1, num_cus());
+    const int64_t t256 = ceil_div(a.M, 256) * ceil_div(a.N, 256);
+    const int64_t t128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
+    if (t256 >= cus) return launch_cfg<T, 4, 4, AK, BKM>(s, a);
+    if (t128 >= cus / 2 || (a.M > 64 && a.N > 64 && t128 >= 4)) return launch_cfg<T, 2, 2, AK, BKM>(s, a);
+    return launch_cfg<T, 1, 1, AK, BKM>(s, a);
+}
+
+}  // namespace luxhip

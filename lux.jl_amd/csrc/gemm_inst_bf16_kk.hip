@@ -1,0 +1,5 @@
+// Explicit instantiation: storage bf16, A K-major, B K-major.
+#include "gemm_dense.h"
+namespace luxhip {
+template int launch_layout<bf16_t, true, true>(hipStream_t, DenseArgs<bf16_t>&);
+}

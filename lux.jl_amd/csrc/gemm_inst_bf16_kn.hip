@@ -1,0 +1,5 @@
+// Explicit instantiation: storage bf16, A K-major, B N-major.
+#include "gemm_dense.h"
+namespace luxhip {
+template int launch_layout<bf16_t, true, false>(hipStream_t, DenseArgs<bf16_t>&);
+}

@@ -1,0 +1,5 @@
+// Explicit instantiation: storage f32, A K-major, B N-major.
+#include "gemm_dense.h"
+namespace luxhip {
+template int launch_layout<float, true, false>(hipStream_t, DenseArgs<float>&);
+}

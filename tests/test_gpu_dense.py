@@ -1,0 +1,164 @@
+"""matmul / fused_dense_bias_activation forward + pullback on the GPU against the oracle
+(mirrors lib/LuxLib/test/common_ops/dense_tests.jl:13-93 and the Dense known answers of
+test/core_layers/basic_tests.jl:151-194 of the reference)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import luxlib_oracle as O
+from tests.util import assert_close, dev, f64, host_inputs, rms
+
+pytestmark = pytest.mark.gpu
+
+
+def test_reference_known_answers(gpu):
+    d = lambda a: gpu.DeviceArray.from_numpy(np.asarray(a, np.float32))
+    y = gpu.fused_dense_bias_activation("identity", d(np.ones((1, 10))), d(np.ones((10, 1))), None)
+    assert y.to_numpy().tolist() == [[10.0]]
+    y = gpu.fused_dense_bias_activation("identity", d(np.ones((2, 10))), d(np.array([np.ones(10), 2 * np.ones(10)]).T), None)
+    assert y.to_numpy().tolist() == [[10.0, 20.0], [10.0, 20.0]]
+    y = gpu.fused_dense_bias_activation("identity", d(np.ones((2, 10))), d(np.ones((10, 1))), d(np.ones(2)))
+    assert y.to_numpy().tolist() == [[11.0], [11.0]]
+    y = gpu.fused_dense_bias_activation("relu", d(-np.ones((1, 10))), d(np.ones((10, 1))), None)
+    assert y.to_numpy().tolist() == [[0.0]]
+
+
+MNK = [(4, 3, 32), (32, 3, 4), (33, 17, 65), (128, 128, 128), (130, 70, 257), (256, 64, 128), (300, 520, 96), (64, 64, 8)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("transA", [False, True])
+@pytest.mark.parametrize("transB", [False, True])
+def test_matmul_all_layouts(gpu, dtype, transA, transB):
+    rng = np.random.default_rng(17)
+    for (M, N, K) in MNK:
+        for with_bias in (False, True):
+            A = rng.normal(size=(K, M) if transA else (M, K))
+            B = rng.normal(size=(N, K) if transB else (K, N))
+            bias = rng.normal(size=M) if with_bias else None
+            A, B, bias = host_inputs(dtype, A, B, bias)
+            got = gpu.matmul(dev(gpu, A, dtype), dev(gpu, B, dtype), dev(gpu, bias, dtype), transA, transB).to_numpy()
+            want = (f64(A).T if transA else f64(A)) @ (f64(B).T if transB else f64(B))
+            if with_bias:
+                want = want + f64(bias)[:, None]
+            assert_close(got, want, dtype, f"{dtype} matmul {M}x{N}x{K} tA={transA} tB={transB} bias={with_bias}")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("act", ["identity", "tanh", "sigmoid_fast", "relu", "gelu", "swish"])
+def test_fused_dense_forward_and_pullback(gpu, dtype, act):
+    rng = np.random.default_rng(abs(hash((dtype, act))) % 2 ** 31)
+    for (M, K, N, with_bias) in [(4, 4, 3, True), (4, 32, 3, False), (32, 4, 3, True), (32, 32, 3, True), (200, 136, 72, True),
+                                 (96, 264, 130, False)]:
+        W = rng.normal(size=(M, K)) / np.sqrt(K)
+        x = rng.normal(size=(K, N))
+        b = rng.normal(size=M) * 0.1 if with_bias else None
+        delta = rng.normal(size=(M, N))
+        W, x, b, delta = host_inputs(dtype, W, x, b, delta)
+        tag = f"{dtype} {act} dense {M}x{K}x{N} bias={with_bias}"
+        y = gpu.fused_dense_bias_activation(act, dev(gpu, W, dtype), dev(gpu, x, dtype), dev(gpu, b, dtype))
+        wy, wdW, wdx, wdb = O.fused_dense_pullback(act, f64(W), f64(x), f64(b), f64(delta))
+        assert_close(y.to_numpy(), wy, dtype, tag + " y")
+        y2, back = gpu.pullback(gpu.fused_dense_bias_activation, act, dev(gpu, W, dtype), dev(gpu, x, dtype), dev(gpu, b, dtype))
+        np.testing.assert_array_equal(y2.to_numpy(), y.to_numpy())
+        gW, gx, gb = back(dev(gpu, delta, dtype))
+        if dtype == "bf16":
+            # the rrule keeps y (and the pre-activation) in bf16 and the activation gradient dz is
+            # stored in bf16 before the two gradient GEMMs (impl/dense.jl:83-103): restate that
+            pre = O.matmuladd(f64(W), f64(x), f64(b))
+            yq = f64(O.round_to_bf16(wy.astype(np.float32)))
+            preq = f64(O.round_to_bf16(pre.astype(np.float32)))
+            dz = f64(O.round_to_bf16(O.grad_activation(f64(delta), yq, act, preq).astype(np.float32)))
+            wdW, wdx = dz @ f64(x).T, f64(W).T @ dz
+            wdb = None if b is None else O.grad_activation(f64(delta), yq, act, preq).sum(axis=1)
+        assert_close(gW.to_numpy(), wdW, dtype, tag + " dW")
+        assert_close(gx.to_numpy(), wdx, dtype, tag + " dx")
+        if with_bias:
+            assert_close(gb.to_numpy(), wdb, dtype, tag + " db", rel=None if dtype == "f32" else 2e-2)
+        else:
+            assert gb is None
+
+
+def test_dimension_mismatch(gpu):
+    d = lambda *s: gpu.DeviceArray.from_numpy(np.ones(s, np.float32))
+    with pytest.raises(gpu.DimensionMismatch):
+        gpu.fused_dense_bias_activation("relu", d(3, 4), d(5, 2), None)
+    with pytest.raises(gpu.DimensionMismatch):
+        gpu.fused_dense_bias_activation("relu", d(3, 4), d(4, 2), d(4))
+    with pytest.raises(gpu.DimensionMismatch):
+        gpu.matmul(d(3, 4), d(5, 2))
+
+
+def test_views_with_leading_dimension(gpu):
+    """Operands that are views of larger arrays (leading dimension > rows), through the C ABI."""
+    rng = np.random.default_rng(23)
+    M, K, N, ldw, ldx, ldy = 37, 29, 21, 48, 40, 64
+    Wb = rng.normal(size=(ldw, K)).astype(np.float32)
+    xb = rng.normal(size=(ldx, N)).astype(np.float32)
+    b = rng.normal(size=M).astype(np.float32)
+    d = gpu.DeviceArray.from_numpy
+    dW, dx_, db = d(Wb), d(xb), d(b)
+    y = d(np.full((ldy, N), 7.0, np.float32))
+    gpu._lib.call("luxhip_fused_dense_fwd", gpu.current_stream(), 0, gpu._lib.ACT_IDS["tanh"], M, K, N, dW.ptr, ldw, dx_.ptr, ldx,
+                  db.ptr, y.ptr, ldy, None)
+    got = y.to_numpy()
+    want = np.tanh(f64(Wb[:M]) @ f64(xb[:K]) + f64(b)[:, None])
+    assert_close(got[:M], want, "f32", "view y")
+    np.testing.assert_array_equal(got[M:], 7.0)          # rows outside the view are untouched
+
+
+def test_config1(gpu):
+    """BASELINE config 1: W 256x128 Glorot-uniform, x 128x64, bias 256, tanh, fp32."""
+    rng = np.random.default_rng(1000)
+    lim = np.sqrt(6.0 / 384.0)
+    W = rng.uniform(-lim, lim, size=(256, 128)).astype(np.float32)
+    x = rng.standard_normal(size=(128, 64)).astype(np.float32)
+    b = (0.01 * rng.standard_normal(256)).astype(np.float32)
+    delta = rng.standard_normal(size=(256, 64)).astype(np.float32)
+    d = gpu.DeviceArray.from_numpy
+    y, back = gpu.pullback(gpu.fused_dense_bias_activation, "tanh", d(W), d(x), d(b))
+    gW, gx, gb = back(d(delta))
+    wy, wdW, wdx, wdb = O.fused_dense_pullback("tanh", f64(W), f64(x), f64(b), f64(delta))
+    w32 = O.fused_dense_pullback("tanh", W, x, b, delta)
+    assert_close(y.to_numpy(), wy, "f32", "config1 y", want32=w32[0])
+    assert_close(gW.to_numpy(), wdW, "f32", "config1 dW", want32=w32[1])
+    assert_close(gx.to_numpy(), wdx, "f32", "config1 dx", want32=w32[2])
+    assert_close(gb.to_numpy(), wdb, "f32", "config1 db", want32=w32[3])
+
+
+def test_config4_dense_full_size(gpu):
+    """BASELINE config 4's first dense layer at full size (4096 -> 11008, 8192 tokens, gelu,
+    bf16 storage / fp32 accumulation): output rows, weight-gradient rows and input-gradient
+    columns are spot-checked against the fp64 oracle; linearity of the pullback in the
+    cotangent is checked on the whole tensors."""
+    rng = np.random.default_rng(1003)
+    K, M, N = 4096, 11008, 8192
+    std = np.sqrt(2.0 / (K + M))
+    W = (std * rng.standard_normal(size=(M, K), dtype=np.float32))
+    x = rng.standard_normal(size=(K, N), dtype=np.float32)
+    b = np.zeros(M, np.float32)
+    delta = (0.02 * rng.standard_normal(size=(M, N), dtype=np.float32))
+    W, x, b, delta = host_inputs("bf16", W, x, b, delta)
+    dW_, dx_, db_, dd_ = (dev(gpu, a, "bf16") for a in (W, x, b, delta))
+    y, back = gpu.pullback(gpu.fused_dense_bias_activation, "gelu", dW_, dx_, db_)
+    gW, gx, gb = back(dd_)
+    rows = rng.choice(M, 24, replace=False)
+    cols = rng.choice(N, 24, replace=False)
+    yh = y.to_numpy()
+    pre_rows = f64(W[rows]) @ f64(x)
+    assert_close(yh[rows], O.act_value("gelu", pre_rows), "bf16", "config4 y rows")
+    # dz as the device computes it: from the bf16-stored pre-activation and bf16-rounded
+    pre_q = f64(O.round_to_bf16(pre_rows.astype(np.float32)))
+    dz_rows = f64(O.round_to_bf16((f64(delta[rows]) * O.act_derivative("gelu", O.act_value("gelu", pre_q), pre_q)).astype(np.float32)))
+    assert_close(gW.to_numpy()[rows], dz_rows @ f64(x).T, "bf16", "config4 dW rows")
+    pre_cols = f64(W) @ f64(x[:, cols])
+    pre_cq = f64(O.round_to_bf16(pre_cols.astype(np.float32)))
+    dz_cols = f64(O.round_to_bf16((f64(delta[:, cols]) * O.act_derivative("gelu", O.act_value("gelu", pre_cq), pre_cq)).astype(np.float32)))
+    assert_close(gx.to_numpy()[:, cols], f64(W).T @ dz_cols, "bf16", "config4 dx cols")
+    assert_close(gb.to_numpy()[rows], (f64(delta[rows]) * O.act_derivative("gelu", O.act_value("gelu", pre_q), pre_q)).sum(axis=1),
+                 "bf16", "config4 db rows", rel=3e-2, scale=rms(delta) * 90)
+    # linearity: pullback(2 * delta) == 2 * pullback(delta) (exact: scaling by 2 commutes with rounding)
+    gW2, gx2, _ = back(dev(gpu, 2 * delta, "bf16"))
+    np.testing.assert_array_equal(gW2.to_numpy()[rows], 2 * gW.to_numpy()[rows])
+    np.testing.assert_array_equal(gx2.to_numpy()[:, cols], 2 * gx.to_numpy()[:, cols])
