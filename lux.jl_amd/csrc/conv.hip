@@ -1,0 +1,378 @@
+// Convolution entry points: layout transforms, filter repacking, launch logic of the
+// implicit-GEMM kernels (conv_kernels.h) and the split-K reduction of the filter gradient.
+#include <algorithm>
+
+#include "common.h"
+#include "conv_kernels.h"
+
+namespace luxhip {
+
+int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* delta,
+                          const void* out, const void* pre, void* dx, void* dbias);   // elementwise.hip
+
+// ----------------------------------------------------------------------------- layout transforms
+// in (P, C, N) with p contiguous  ->  out (C, P, N) with c contiguous
+template <typename T>
+__global__ __launch_bounds__(256) void whcn_to_cwhn_kernel(const T* __restrict__ in, T* __restrict__ out, int P, int C) {
+    __shared__ T tile[32][33];
+    const int n = blockIdx.z;
+    const int p0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;       // 32 x 8
+    const T* src = in + (size_t)n * C * P;
+    T* dst = out + (size_t)n * C * P;
+#pragma unroll
+    for (int j = 0; j < 32; j += 8) {
+        const int c = c0 + ty + j, p = p0 + tx;
+        if (c < C && p < P) tile[ty + j][tx] = src[(size_t)c * P + p];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 32; j += 8) {
+        const int p = p0 + ty + j, c = c0 + tx;
+        if (c < C && p < P) dst[(size_t)p * C + c] = tile[tx][ty + j];
+    }
+}
+
+// wF[(co*T + t)*Cin_g + ci] (fprop, K = T*Cin_g) or wD[((g*Cin_g + ci)*T + t)*Cout_g + col]
+// (dgrad, K = T*Cout_g) from w[a + kW*(b + kH*(ci + Cin_g*co))]; tap t = ka + kW*kb with
+// a = flip ? ka : kW-1-ka (same for b).
+template <typename T>
+__global__ void pack_filter_kernel(const T* __restrict__ w, T* __restrict__ out, ConvGeom g, int for_dgrad) {
+    const int total = g.kW * g.kH * g.Cin_g * g.Cout;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int Tt = g.kW * g.kH;
+    int co, t, ci;
+    if (!for_dgrad) {
+        ci = idx % g.Cin_g;
+        t = (idx / g.Cin_g) % Tt;
+        co = idx / (g.Cin_g * Tt);
+    } else {
+        const int col = idx % g.Cout_g;
+        t = (idx / g.Cout_g) % Tt;
+        const int cig = idx / (g.Cout_g * Tt);       // g*Cin_g + ci
+        const int grp = cig / g.Cin_g;
+        ci = cig - grp * g.Cin_g;
+        co = grp * g.Cout_g + col;
+    }
+    const int ka = t % g.kW, kb = t / g.kW;
+    const int a = g.flip ? ka : g.kW - 1 - ka, b = g.flip ? kb : g.kH - 1 - kb;
+    out[idx] = w[a + g.kW * (b + g.kH * (ci + g.Cin_g * co))];
+}
+
+// dw[a, b, ci, g*Cout_g + col] = sum over slices of partial[slice][m' = t*Cin_g + ci][col]
+template <typename T>
+__global__ void wgrad_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw, ConvGeom g, int grp, int slices) {
+    const int Mrows = g.kW * g.kH * g.Cin_g;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= Mrows * g.Cout_g) return;
+    const int m = idx % Mrows, col = idx / Mrows;
+    float acc = 0.0f;
+    for (int sl = 0; sl < slices; ++sl) acc += partial[(size_t)sl * Mrows * g.Cout_g + idx];
+    const int t = m / g.Cin_g, ci = m - t * g.Cin_g;
+    const int ka = t % g.kW, kb = t / g.kW;
+    const int a = g.flip ? ka : g.kW - 1 - ka, b = g.flip ? kb : g.kH - 1 - kb;
+    st(dw + a + g.kW * (b + g.kH * (ci + g.Cin_g * (grp * g.Cout_g + col))), acc);
+}
+
+// ----------------------------------------------------------------------------- host helpers
+static int make_geom(const luxhip_conv_dims_t* d, ConvGeom* g) {
+    LUX_INVALID_IF(d == nullptr, "conv: dims must not be NULL");
+    LUX_INVALID_IF(d->W <= 0 || d->H <= 0 || d->Cin <= 0 || d->N < 0 || d->kW <= 0 || d->kH <= 0 || d->Cout <= 0,
+                   "conv: non-positive dimension");
+    LUX_INVALID_IF(d->stride_w <= 0 || d->stride_h <= 0 || d->dil_w <= 0 || d->dil_h <= 0 || d->groups <= 0,
+                   "conv: stride, dilation and groups must be positive");
+    LUX_INVALID_IF(d->pad_w_lo < 0 || d->pad_w_hi < 0 || d->pad_h_lo < 0 || d->pad_h_hi < 0, "conv: negative padding");
+    LUX_INVALID_IF(d->Cin % d->groups != 0 || d->Cout % d->groups != 0, "conv: channels must be divisible by groups");
+    const int64_t ow = (d->W + d->pad_w_lo + d->pad_w_hi - d->dil_w * (d->kW - 1) - 1) / d->stride_w + 1;
+    const int64_t oh = (d->H + d->pad_h_lo + d->pad_h_hi - d->dil_h * (d->kH - 1) - 1) / d->stride_h + 1;
+    LUX_INVALID_IF(ow <= 0 || oh <= 0, "conv: empty output");
+    const long double big = 2147483648.0L;
+    LUX_UNSUPPORTED_IF((long double)d->W * d->H * d->Cin * std::max<int64_t>(d->N, 1) >= big ||
+                           (long double)ow * oh * d->Cout * std::max<int64_t>(d->N, 1) >= big,
+                       "conv: tensors of 2^31 or more elements are not supported");
+    g->W = (int)d->W; g->H = (int)d->H; g->Cin = (int)d->Cin; g->N = (int)d->N; g->kW = (int)d->kW; g->kH = (int)d->kH;
+    g->Cout = (int)d->Cout; g->OW = (int)ow; g->OH = (int)oh; g->sw = (int)d->stride_w; g->sh = (int)d->stride_h;
+    g->pw = (int)d->pad_w_lo; g->ph = (int)d->pad_h_lo; g->dw = (int)d->dil_w; g->dh = (int)d->dil_h;
+    g->groups = (int)d->groups; g->Cin_g = (int)(d->Cin / d->groups); g->Cout_g = (int)(d->Cout / d->groups);
+    g->flip = d->flipkernel != 0;
+    return LUXHIP_OK;
+}
+
+static inline size_t align256(size_t b) { return (b + 255) & ~size_t(255); }
+
+template <typename T>
+static int transpose_to_cwhn(hipStream_t s, const T* in, T* out, int P, int C, int N) {
+    ProfScope ps("whcn_to_cwhn_kernel", s);
+    dim3 grid((unsigned)ceil_div(P, 32), (unsigned)ceil_div(C, 32), (unsigned)N);
+    LUX_UNSUPPORTED_IF(grid.y > 65535 || grid.z > 65535, "conv: too many channels or images for the layout transform");
+    whcn_to_cwhn_kernel<T><<<grid, 256, 0, s>>>(in, out, P, C);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static int pack_filter(hipStream_t s, const T* w, T* out, const ConvGeom& g, int for_dgrad) {
+    ProfScope ps("pack_filter_kernel", s);
+    const int total = g.kW * g.kH * g.Cin_g * g.Cout;
+    pack_filter_kernel<T><<<(unsigned)ceil_div(total, 256), 256, 0, s>>>(w, out, g, for_dgrad);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static void fill_gather(GatherK<T>& q, const ConvGeom& g, bool dgrad) {
+    constexpr int V = GemmTraits<T>::VEC;
+    q.kW = g.kW; q.sw = g.sw; q.sh = g.sh; q.pw = g.pw; q.ph = g.ph; q.dw = g.dw; q.dh = g.dh;
+    q.dgrad = dgrad;
+    if (!dgrad) {            // rows: output positions; source: xT
+        q.Ctot = g.Cin; q.Cg = g.Cin_g; q.P = g.OW; q.PQ = g.OW * g.OH; q.SP = g.W; q.SQ = g.H;
+    } else {                 // rows: input positions; source: dyT
+        q.Ctot = g.Cout; q.Cg = g.Cout_g; q.P = g.W; q.PQ = g.W * g.H; q.SP = g.OW; q.SQ = g.OH;
+    }
+    q.M = q.PQ * g.N;
+    q.divP = FastDiv((uint32_t)q.P); q.divPQ = FastDiv((uint32_t)q.PQ); q.divCg = FastDiv((uint32_t)q.Cg);
+    q.divkW = FastDiv((uint32_t)g.kW); q.divsw = FastDiv((uint32_t)g.sw); q.divsh = FastDiv((uint32_t)g.sh);
+    q.vec_ok = (q.Cg % V == 0) && (q.Ctot % V == 0);
+}
+
+// fprop (dgrad == false): out = y; dgrad: out = dx.  src is the channel-contiguous activation,
+// wm the packed filter (all groups).
+template <typename T>
+static int run_conv_gemm(hipStream_t s, const ConvGeom& g, bool dgrad, const T* src, const T* wm, const T* bias, T* out,
+                         T* pre, int act) {
+    const int Tt = g.kW * g.kH;
+    for (int grp = 0; grp < g.groups; ++grp) {
+        ConvGemmArgs<T> a;
+        fill_gather(a.gather, g, dgrad);
+        a.gather.src = src;
+        a.gather.c_off = grp * a.gather.Cg;
+        a.gather.vec_ok = a.gather.vec_ok && aligned16(src);
+        a.K = Tt * a.gather.Cg;
+        a.Ncols = dgrad ? g.Cin_g : g.Cout_g;
+        a.Wm.p = wm + (size_t)grp * a.Ncols * a.K;
+        a.Wm.sr = a.K; a.Wm.sk = 1; a.Wm.rows = a.Ncols;
+        a.Wm.vec_ok = aligned16(a.Wm.p) && ((size_t)a.K * sizeof(T)) % 16 == 0;
+        a.out = out; a.pre = pre; a.bias = bias;
+        a.Ctot_out = dgrad ? g.Cin : g.Cout;
+        a.col_off = grp * a.Ncols;
+        a.act = act;
+        int rc = launch_conv_gemm_any<T>(s, a);
+        if (rc != LUXHIP_OK) return rc;
+    }
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static int wgrad_plan(const ConvGeom& g, int* slices, int* kslice, bool* small) {
+    constexpr int BK = GemmTraits<T>::BK;
+    const int Mrows = g.kW * g.kH * g.Cin_g;
+    *small = Mrows <= 64 || g.Cout_g <= 64;
+    const int tile = *small ? 64 : 128;
+    const int64_t tiles = ceil_div(Mrows, tile) * ceil_div(g.Cout_g, tile);
+    const int64_t Ktotal = (int64_t)g.OW * g.OH * g.N;
+    int64_t want = std::max<int64_t>(1, ceil_div(2 * (int64_t)std::max(1, num_cus()), tiles * g.groups));
+    int64_t ks = ceil_div(ceil_div(Ktotal, want), BK) * BK;
+    ks = std::max<int64_t>(ks, 4 * BK);
+    *kslice = (int)ks;
+    *slices = (int)ceil_div(Ktotal, ks);
+    LUX_UNSUPPORTED_IF(*slices > 65535, "conv wgrad: too many k slices");
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static size_t wgrad_partial_bytes(const ConvGeom& g) {
+    int slices = 1, kslice = 0;
+    bool small = false;
+    if (wgrad_plan<T>(g, &slices, &kslice, &small) != LUXHIP_OK) return 0;
+    return align256((size_t)slices * g.kW * g.kH * g.Cin_g * g.Cout_g * sizeof(float));
+}
+
+template <typename T>
+static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dyT, float* partial, T* dw) {
+    constexpr int V = GemmTraits<T>::VEC;
+    int slices, kslice;
+    bool small;
+    int rc = wgrad_plan<T>(g, &slices, &kslice, &small);
+    if (rc != LUXHIP_OK) return rc;
+    for (int grp = 0; grp < g.groups; ++grp) {
+        ConvWgradArgs<T> a;
+        GatherMN<T>& q = a.gather;
+        q.src = xT; q.Ctot = g.Cin; q.c_off = grp * g.Cin_g; q.Cg = g.Cin_g; q.Mrows = g.kW * g.kH * g.Cin_g;
+        q.OW = g.OW; q.OWOH = g.OW * g.OH; q.SP = g.W; q.SQ = g.H; q.kW = g.kW; q.sw = g.sw; q.sh = g.sh; q.pw = g.pw;
+        q.ph = g.ph; q.dw = g.dw; q.dh = g.dh;
+        q.vec_ok = (g.Cin_g % V == 0) && (g.Cin % V == 0) && aligned16(xT);
+        q.divOW = FastDiv((uint32_t)q.OW); q.divOWOH = FastDiv((uint32_t)q.OWOH); q.divCg = FastDiv((uint32_t)q.Cg);
+        q.divkW = FastDiv((uint32_t)g.kW);
+        a.dyT = dyT; a.Cout = g.Cout; a.co_off = grp * g.Cout_g; a.Cout_g = g.Cout_g;
+        a.Ktotal = g.OW * g.OH * g.N; a.kslice = kslice; a.partial = partial;
+        a.dy_vec_ok = (g.Cout % V == 0) && (g.Cout_g % V == 0) && aligned16(dyT);
+        rc = launch_conv_wgrad_any<T>(s, a, slices, small);
+        if (rc != LUXHIP_OK) return rc;
+        ProfScope ps("wgrad_reduce_kernel", s);
+        const int total = q.Mrows * g.Cout_g;
+        wgrad_reduce_kernel<T><<<(unsigned)ceil_div(total, 256), 256, 0, s>>>(partial, dw, g, grp, slices);
+        LUX_CHECK_LAUNCH();
+    }
+    return LUXHIP_OK;
+}
+
+// ----------------------------------------------------------------------------- typed entry points
+template <typename T>
+static int conv_fwd_t(hipStream_t s, int act, const ConvGeom& g, const T* x, const T* w, const T* bias, T* y, T* pre) {
+    const size_t xb = align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
+    const size_t wb = align256((size_t)g.kW * g.kH * g.Cin_g * g.Cout * sizeof(T));
+    Workspace ws;
+    int rc = get_workspace(s, xb + wb, &ws);
+    if (rc != LUXHIP_OK) return rc;
+    T* xT = reinterpret_cast<T*>(ws.data);
+    T* wF = reinterpret_cast<T*>(ws.data + xb);
+    if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
+    if ((rc = pack_filter<T>(s, w, wF, g, 0)) != LUXHIP_OK) return rc;
+    return run_conv_gemm<T>(s, g, false, xT, wF, bias, y, pre, act);
+}
+
+template <typename T>
+static int conv_bwd_data_t(hipStream_t s, const ConvGeom& g, const T* dy, const T* w, T* dx) {
+    const size_t yb = align256((size_t)g.OW * g.OH * g.Cout * g.N * sizeof(T));
+    const size_t wb = align256((size_t)g.kW * g.kH * g.Cin_g * g.Cout * sizeof(T));
+    Workspace ws;
+    int rc = get_workspace(s, yb + wb, &ws);
+    if (rc != LUXHIP_OK) return rc;
+    T* dyT = reinterpret_cast<T*>(ws.data);
+    T* wD = reinterpret_cast<T*>(ws.data + yb);
+    if ((rc = transpose_to_cwhn<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
+    if ((rc = pack_filter<T>(s, w, wD, g, 1)) != LUXHIP_OK) return rc;
+    return run_conv_gemm<T>(s, g, true, dyT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY);
+}
+
+template <typename T>
+static int conv_bwd_filter_t(hipStream_t s, const ConvGeom& g, const T* x, const T* dy, T* dw) {
+    const size_t xb = align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
+    const size_t yb = align256((size_t)g.OW * g.OH * g.Cout * g.N * sizeof(T));
+    const size_t pb = wgrad_partial_bytes<T>(g);
+    Workspace ws;
+    int rc = get_workspace(s, xb + yb + pb, &ws);
+    if (rc != LUXHIP_OK) return rc;
+    T* xT = reinterpret_cast<T*>(ws.data);
+    T* dyT = reinterpret_cast<T*>(ws.data + xb);
+    float* partial = reinterpret_cast<float*>(ws.data + xb + yb);
+    if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
+    if ((rc = transpose_to_cwhn<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
+    return run_wgrad<T>(s, g, xT, dyT, partial, dw);
+}
+
+template <typename T>
+static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g, const T* delta, const T* y,
+                            const T* pre, const T* x, const T* w, T* dz, T* dw, T* dx, T* dbias) {
+    const size_t xb = align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
+    const size_t yb = align256((size_t)g.OW * g.OH * g.Cout * g.N * sizeof(T));
+    const size_t wb = align256((size_t)g.kW * g.kH * g.Cin_g * g.Cout * sizeof(T));
+    const size_t pb = wgrad_partial_bytes<T>(g);
+    // reserve everything up front: the bias-gradient pass below uses the start of the same
+    // workspace, and the buffer must not be reallocated while pointers into it are live
+    Workspace ws;
+    int rc = get_workspace(s, xb + yb + wb + pb, &ws);
+    if (rc != LUXHIP_OK) return rc;
+    const T* dzp = delta;
+    if (act != LUXHIP_ACT_IDENTITY || dbias != nullptr) {
+        T* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : dz;
+        rc = bias_act_bwd_dispatch(s, dtype, act, (int64_t)g.OW * g.OH, g.Cout, g.N, delta, y, pre, dz_out, dbias);
+        if (rc != LUXHIP_OK) return rc;
+        if (dz_out) dzp = dz_out;
+    }
+    if (dw == nullptr && dx == nullptr) return LUXHIP_OK;
+    T* xT = reinterpret_cast<T*>(ws.data);
+    T* dzT = reinterpret_cast<T*>(ws.data + xb);
+    T* wD = reinterpret_cast<T*>(ws.data + xb + yb);
+    float* partial = reinterpret_cast<float*>(ws.data + xb + yb + wb);
+    if ((rc = transpose_to_cwhn<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
+    if (dx != nullptr) {
+        if ((rc = pack_filter<T>(s, w, wD, g, 1)) != LUXHIP_OK) return rc;
+        if ((rc = run_conv_gemm<T>(s, g, true, dzT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY)) != LUXHIP_OK) return rc;
+    }
+    if (dw != nullptr) {
+        if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
+        if ((rc = run_wgrad<T>(s, g, xT, dzT, partial, dw)) != LUXHIP_OK) return rc;
+    }
+    return LUXHIP_OK;
+}
+
+static int conv_check(int dtype, int act) {
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_UNSUPPORTED_IF(act < 0 || act >= LUXHIP_ACT_COUNT, "unsupported activation id %d", act);
+    return LUXHIP_OK;
+}
+
+}  // namespace luxhip
+
+using namespace luxhip;
+
+extern "C" {
+
+int luxhip_conv_fwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d, const void* x, const void* w,
+                    const void* bias, void* y, void* pre) {
+    LUX_REQUIRE_INIT();
+    int rc = conv_check(dtype, act);
+    if (rc != LUXHIP_OK) return rc;
+    ConvGeom g;
+    if ((rc = make_geom(d, &g)) != LUXHIP_OK) return rc;
+    if (g.N == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(x == nullptr || w == nullptr || y == nullptr, "conv_fwd: x, w and y must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return conv_fwd_t<float>((hipStream_t)s, act, g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, (float*)pre);
+    return conv_fwd_t<bf16_t>((hipStream_t)s, act, g, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, (bf16_t*)pre);
+}
+
+int luxhip_conv_bwd_data(luxhip_stream_t s, int dtype, const luxhip_conv_dims_t* d, const void* dy, const void* w, void* dx) {
+    LUX_REQUIRE_INIT();
+    int rc = conv_check(dtype, 0);
+    if (rc != LUXHIP_OK) return rc;
+    ConvGeom g;
+    if ((rc = make_geom(d, &g)) != LUXHIP_OK) return rc;
+    if (g.N == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(dy == nullptr || w == nullptr || dx == nullptr, "conv_bwd_data: dy, w and dx must not be NULL");
+    if (dtype == LUXHIP_F32) return conv_bwd_data_t<float>((hipStream_t)s, g, (const float*)dy, (const float*)w, (float*)dx);
+    return conv_bwd_data_t<bf16_t>((hipStream_t)s, g, (const bf16_t*)dy, (const bf16_t*)w, (bf16_t*)dx);
+}
+
+int luxhip_conv_bwd_filter(luxhip_stream_t s, int dtype, const luxhip_conv_dims_t* d, const void* x, const void* dy, void* dw) {
+    LUX_REQUIRE_INIT();
+    int rc = conv_check(dtype, 0);
+    if (rc != LUXHIP_OK) return rc;
+    ConvGeom g;
+    if ((rc = make_geom(d, &g)) != LUXHIP_OK) return rc;
+    LUX_INVALID_IF(dw == nullptr, "conv_bwd_filter: dw must not be NULL");
+    if (g.N == 0) return luxhip_fill_zero(dw, (size_t)g.kW * g.kH * g.Cin_g * g.Cout * (dtype == LUXHIP_F32 ? 4 : 2), s);
+    LUX_INVALID_IF(x == nullptr || dy == nullptr, "conv_bwd_filter: x and dy must not be NULL");
+    if (dtype == LUXHIP_F32) return conv_bwd_filter_t<float>((hipStream_t)s, g, (const float*)x, (const float*)dy, (float*)dw);
+    return conv_bwd_filter_t<bf16_t>((hipStream_t)s, g, (const bf16_t*)x, (const bf16_t*)dy, (bf16_t*)dw);
+}
+
+int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d, const void* delta,
+                          const void* y, const void* pre, const void* x, const void* w, void* dz, void* dw, void* dx,
+                          void* dbias) {
+    LUX_REQUIRE_INIT();
+    int rc = conv_check(dtype, act);
+    if (rc != LUXHIP_OK) return rc;
+    ConvGeom g;
+    if ((rc = make_geom(d, &g)) != LUXHIP_OK) return rc;
+    const size_t esz = dtype == LUXHIP_F32 ? 4 : 2;
+    if (g.N == 0) {
+        if (dw) { rc = luxhip_fill_zero(dw, (size_t)g.kW * g.kH * g.Cin_g * g.Cout * esz, s); if (rc) return rc; }
+        if (dbias) { rc = luxhip_fill_zero(dbias, (size_t)g.Cout * esz, s); if (rc) return rc; }
+        return LUXHIP_OK;
+    }
+    LUX_INVALID_IF(delta == nullptr, "fused_conv_bwd: delta must not be NULL");
+    LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && dz == nullptr, "fused_conv_bwd: dz scratch is required");
+    LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && !act_needs_pre(act) && y == nullptr, "fused_conv_bwd: activation %d needs y", act);
+    LUX_INVALID_IF(act_needs_pre(act) && pre == nullptr, "fused_conv_bwd: activation %d needs the pre-activation", act);
+    LUX_INVALID_IF((dw != nullptr && x == nullptr) || (dx != nullptr && w == nullptr), "fused_conv_bwd: x / w must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return fused_conv_bwd_t<float>((hipStream_t)s, dtype, act, g, (const float*)delta, (const float*)y, (const float*)pre,
+                                       (const float*)x, (const float*)w, (float*)dz, (float*)dw, (float*)dx, (float*)dbias);
+    return fused_conv_bwd_t<bf16_t>((hipStream_t)s, dtype, act, g, (const bf16_t*)delta, (const bf16_t*)y, (const bf16_t*)pre,
+                                    (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)dz, (bf16_t*)dw, (bf16_t*)dx, (bf16_t*)dbias);
+}
+
+}  // extern "C"

@@ -1,0 +1,11 @@
+// fprop / dgrad implicit-GEMM kernels, storage type bf16: tile selection + instantiation.
+#include "conv_kernels.h"
+namespace luxhip {
+template <>
+int launch_conv_gemm_any<bf16_t>(hipStream_t s, ConvGemmArgs<bf16_t>& a) {
+    const int64_t cus = num_cus() > 0 ? num_cus() : 256;
+    if (a.Ncols > 64 && ceil_div(a.gather.M, 256) * ceil_div(a.Ncols, 128) >= cus) return launch_conv_gemm<bf16_t, 4, 2>(s, a);
+    if (a.Ncols > 64 && a.gather.M > 64) return launch_conv_gemm<bf16_t, 2, 2>(s, a);
+    return launch_conv_gemm<bf16_t, 1, 1>(s, a);
+}
+}  // namespace luxhip

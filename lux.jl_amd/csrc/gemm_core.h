@@ -66,13 +66,32 @@ struct Operand {
 };
 
 // ----------------------------------------------------------------------------- global -> registers
+// LDS offset (in elements) of the 16-byte chunk that starts at (row r, column k) of a tile.
 template <typename T, bool KMAJOR, int ROWS>
+__device__ __forceinline__ int lds_chunk_offset(int r, int k) {
+    using Tr = GemmTraits<T>;
+    if constexpr (KMAJOR) {
+        if constexpr (sizeof(T) == 2) return r * Tr::BK + (((k >> 3) ^ (r & 7)) << 3);
+        else return r * Tr::kmajor_stride() + k;
+    } else {
+        return k * (ROWS + Tr::PAD_MN) + r;
+    }
+}
+
+// Loader policy of the mainloop: load(k0) fetches this thread's share of the stage that starts
+// at k0 into registers, store(lds) writes it to the stage buffer.  TileLoader reads a plain
+// strided matrix; the convolution kernels provide gathering loaders with the same interface.
+template <typename T, bool KMAJOR_, int ROWS>
 struct TileLoader {
     using Tr = GemmTraits<T>;
+    static constexpr bool KMAJOR = KMAJOR_;
     static constexpr int CHUNKS = ROWS * Tr::BK / Tr::VEC;
     static constexpr int PER_THREAD = CHUNKS / kGemmThreads;
     static_assert(CHUNKS % kGemmThreads == 0, "tile must split evenly over the workgroup");
     uint4 reg[PER_THREAD];
+    Operand<T> op;
+    int r0, K;
+    __device__ __forceinline__ TileLoader(const Operand<T>& o, int row0, int k_total) : op(o), r0(row0), K(k_total) {}
 
     __device__ __forceinline__ static void coords(int id, int& r, int& k) {
         if constexpr (KMAJOR) {
@@ -84,7 +103,7 @@ struct TileLoader {
         }
     }
 
-    __device__ __forceinline__ void load(const Operand<T>& op, int r0, int k0, int K) {
+    __device__ __forceinline__ void load(int k0) {
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
             int r, k;
@@ -114,14 +133,7 @@ struct TileLoader {
         for (int i = 0; i < PER_THREAD; ++i) {
             int r, k;
             coords(threadIdx.x + i * kGemmThreads, r, k);
-            int off;
-            if constexpr (KMAJOR) {
-                if constexpr (sizeof(T) == 2) off = r * Tr::BK + (((k >> 3) ^ (r & 7)) << 3);
-                else off = r * Tr::kmajor_stride() + k;
-            } else {
-                off = k * (ROWS + Tr::PAD_MN) + r;
-            }
-            *reinterpret_cast<uint4*>(lds + off) = reg[i];
+            *reinterpret_cast<uint4*>(lds + lds_chunk_offset<T, KMAJOR, ROWS>(r, k)) = reg[i];
         }
     }
 };
@@ -187,6 +199,8 @@ template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
 struct GemmMainloop {
     using Tr = GemmTraits<T>;
     static constexpr int TILE_M = 2 * WM * 32, TILE_N = 2 * WN * 32;
+    using PlainLoaderA = TileLoader<T, A_KMAJOR, TILE_M>;
+    using PlainLoaderB = TileLoader<T, B_KMAJOR, TILE_N>;
     static constexpr int A_ELEMS = lds_tile_elems<T, A_KMAJOR>(TILE_M);
     static constexpr int B_ELEMS = lds_tile_elems<T, B_KMAJOR>(TILE_N);
     static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
@@ -194,6 +208,15 @@ struct GemmMainloop {
 
     __device__ __forceinline__ static void run(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0, T* lds,
                                                f32x16_v (&acc)[WM][WN]) {
+        PlainLoaderA la(A, m0, K);
+        PlainLoaderB lb(B, n0, K);
+        run(la, lb, K, lds, acc);
+    }
+
+    // k range [0, K) in stages of BK; the loaders decide what a stage contains
+    template <class LoaderA, class LoaderB>
+    __device__ __forceinline__ static void run(LoaderA& la, LoaderB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
+        static_assert(LoaderA::KMAJOR == A_KMAJOR && LoaderB::KMAJOR == B_KMAJOR, "loader layout mismatch");
         const int w = threadIdx.x >> 6;
         const int wave_m = (w & 1) * (WM * 32), wave_n = (w >> 1) * (WN * 32);
 #pragma unroll
@@ -203,11 +226,9 @@ struct GemmMainloop {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-        TileLoader<T, A_KMAJOR, TILE_M> la;
-        TileLoader<T, B_KMAJOR, TILE_N> lb;
         const int KT = (K + Tr::BK - 1) / Tr::BK;
-        la.load(A, m0, 0, K);
-        lb.load(B, n0, 0, K);
+        la.load(0);
+        lb.load(0);
         la.store(lds);
         lb.store(lds + A_ELEMS);
         __syncthreads();
@@ -216,8 +237,8 @@ struct GemmMainloop {
             T* nxt = lds + ((kt + 1) & 1) * STAGE_ELEMS;
             const bool more = kt + 1 < KT;
             if (more) {
-                la.load(A, m0, (kt + 1) * Tr::BK, K);
-                lb.load(B, n0, (kt + 1) * Tr::BK, K);
+                la.load((kt + 1) * Tr::BK);
+                lb.load((kt + 1) * Tr::BK);
             }
             const T* As = cur;
             const T* Bs = cur + A_ELEMS;

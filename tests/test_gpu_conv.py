@@ -1,0 +1,150 @@
+"""fused_conv_bias_activation forward + pullback (fprop, dgrad, wgrad) on the GPU against the
+oracle (mirrors lib/LuxLib/test/common_ops/conv_tests.jl:25-117 and the known answers of
+test/core_layers/conv_tests.jl:54-69,145-190 of the reference)."""
+import numpy as np
+import pytest
+
+from oracle import luxlib_oracle as O
+from tests.util import assert_close, dev, f64, host_inputs, rms
+
+pytestmark = pytest.mark.gpu
+
+
+def cdims(gpu, xs, ws, **kw):
+    return gpu.DenseConvDims(xs, ws, **kw), O.ConvDims(xs, ws, **kw)
+
+
+def test_reference_known_answers(gpu):
+    d = lambda a: gpu.DeviceArray.from_numpy(np.asarray(a, np.float32))
+    # impulse response => true convolution orientation
+    x = np.zeros((7, 7, 1, 1), np.float32)
+    x[3, 3, 0, 0] = 1
+    w = np.random.default_rng(1).normal(size=(3, 3, 1, 1)).astype(np.float32)
+    gd, _ = cdims(gpu, x.shape, w.shape)
+    y = gpu.fused_conv_bias_activation("identity", d(w), d(x), None, gd).to_numpy()
+    assert y.shape == (5, 5, 1, 1)
+    np.testing.assert_array_equal(y[1:4, 1:4, 0, 0], w[:, :, 0, 0])
+    gd, _ = cdims(gpu, x.shape, w.shape, flipkernel=True)
+    yc = gpu.fused_conv_bias_activation("identity", d(w), d(x), None, gd).to_numpy()
+    np.testing.assert_array_equal(yc[1:4, 1:4, 0, 0], w[::-1, ::-1, 0, 0])
+    # asymmetric padding, all ones, relu, zero bias
+    x = np.ones((28, 28, 1, 1), np.float32)
+    w = np.ones((3, 3, 1, 1), np.float32)
+    gd, _ = cdims(gpu, x.shape, w.shape, padding=(0, 1, 1, 2))
+    y = gpu.fused_conv_bias_activation("relu", d(w), d(x), d(np.zeros(1)), gd).to_numpy()[:, :, 0, 0]
+    assert y.shape == (27, 29)
+    assert (y[0, 0], y[1, 1], y[26, 0], y[0, 28], y[0, 27], y[26, 28]) == (6.0, 9.0, 4.0, 3.0, 6.0, 2.0)
+
+
+CASES = [
+    # x shape, w shape, stride, pad, dilation, groups, flip
+    ((6, 5, 4, 2), (2, 2, 4, 6), 1, 0, 1, 1, False),
+    ((6, 5, 4, 2), (2, 2, 4, 6), 2, 1, 1, 1, False),
+    ((6, 5, 4, 2), (2, 2, 2, 6), 1, 1, 1, 2, False),
+    ((7, 8, 3, 2), (3, 3, 3, 5), (2, 1), (0, 1, 2, 1), (1, 2), 1, False),
+    ((7, 8, 3, 2), (3, 2, 3, 5), 1, 1, 1, 1, True),
+    ((16, 16, 16, 4), (3, 3, 16, 32), 1, 1, 1, 1, False),
+    ((14, 14, 64, 3), (3, 3, 64, 128), 1, 1, 1, 1, False),
+    ((15, 13, 32, 2), (3, 3, 8, 64), 2, 1, 1, 4, False),
+    ((12, 12, 24, 2), (5, 5, 24, 40), 1, 2, 2, 1, True),
+    ((9, 9, 8, 5), (1, 1, 8, 16), 1, 0, 1, 1, False),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_conv_and_gradients(gpu, dtype, case):
+    xs, ws, stride, pad, dil, groups, flip = CASES[case]
+    rng = np.random.default_rng(100 + case)
+    gd, od = cdims(gpu, xs, ws, stride=stride, padding=pad, dilation=dil, groups=groups, flipkernel=flip)
+    fan_in = ws[0] * ws[1] * ws[2]
+    x, w, dy = host_inputs(dtype, rng.normal(size=xs), rng.normal(size=ws) * np.sqrt(2.0 / fan_in), rng.normal(size=od.y_shape()))
+    tag = f"{dtype} case {case}"
+    y = gpu.conv(dev(gpu, x, dtype), dev(gpu, w, dtype), gd)
+    assert_close(y.to_numpy(), O.conv(f64(x), f64(w), od), dtype, tag + " conv")
+    dx = gpu.conv_data_grad(dev(gpu, dy, dtype), dev(gpu, w, dtype), gd)
+    assert_close(dx.to_numpy(), O.conv_data_grad(f64(dy), f64(w), od), dtype, tag + " dgrad")
+    dw = gpu.conv_filter_grad(dev(gpu, x, dtype), dev(gpu, dy, dtype), gd)
+    assert_close(dw.to_numpy(), O.conv_filter_grad(f64(x), f64(dy), od), dtype, tag + " wgrad")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("act", ["identity", "sigmoid", "gelu", "relu"])
+def test_fused_conv_pullback(gpu, dtype, act):
+    rng = np.random.default_rng(abs(hash((dtype, act))) % 2 ** 31)
+    for case in (1, 2, 5, 7):
+        xs, ws, stride, pad, dil, groups, flip = CASES[case]
+        gd, od = cdims(gpu, xs, ws, stride=stride, padding=pad, dilation=dil, groups=groups, flipkernel=flip)
+        fan_in = ws[0] * ws[1] * ws[2]
+        for with_bias in (True, False):
+            x, w, b, delta = host_inputs(dtype, rng.normal(size=xs), rng.normal(size=ws) * np.sqrt(2.0 / fan_in),
+                                         rng.normal(size=ws[3]) * 0.1 if with_bias else None, rng.normal(size=od.y_shape()))
+            tag = f"{dtype} {act} case {case} bias={with_bias}"
+            y, back = gpu.pullback(gpu.fused_conv_bias_activation, act, dev(gpu, w, dtype), dev(gpu, x, dtype), dev(gpu, b, dtype), gd)
+            wy, wdw, wdx, wdb = O.fused_conv_pullback(act, f64(w), f64(x), f64(b), od, f64(delta))
+            assert_close(y.to_numpy(), wy, dtype, tag + " y")
+            gw, gx, gb = back(dev(gpu, delta, dtype))
+            if dtype == "bf16":
+                # y, the pre-activation and dz are stored in bf16 between the passes
+                pre = O.bias_add(O.conv(f64(x), f64(w), od), f64(b))
+                yq, preq = (f64(O.round_to_bf16(a.astype(np.float32))) for a in (wy, pre))
+                dzx = O.grad_activation(f64(delta), yq, act, preq)
+                dz = f64(O.round_to_bf16(dzx.astype(np.float32)))
+                wdw, wdx = O.conv_filter_grad(f64(x), dz, od), O.conv_data_grad(dz, f64(w), od)
+                wdb = O.grad_bias_add(b, dzx)
+            assert_close(gw.to_numpy(), wdw, dtype, tag + " dw")
+            assert_close(gx.to_numpy(), wdx, dtype, tag + " dx")
+            if with_bias:
+                assert_close(gb.to_numpy(), wdb, dtype, tag + " db", rel=None if dtype == "f32" else 2e-2)
+            else:
+                assert gb is None
+
+
+def test_dimension_mismatch(gpu):
+    with pytest.raises(gpu.DimensionMismatch):
+        gpu.DenseConvDims((8, 8, 4, 2), (3, 3, 3, 6))
+    d = lambda *s: gpu.DeviceArray.from_numpy(np.ones(s, np.float32))
+    gd = gpu.DenseConvDims((8, 8, 4, 2), (3, 3, 4, 6))
+    with pytest.raises(gpu.DimensionMismatch):
+        gpu.fused_conv_bias_activation("relu", d(3, 3, 4, 6), d(8, 8, 4, 3), None, gd)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_config5_full_size(gpu, dtype):
+    """BASELINE config 5 at full size: x 56x56x128x64, w 3x3x128x128 Kaiming-normal, stride 1,
+    pad 1, relu.  Forward and input gradient: fp64 oracle on two images.  Filter gradient: the
+    adjoint identity <dw, w'> == <dz, conv(x, w')> against the (checked) forward kernel plus an
+    fp64 oracle on a two-image batch.  Bias gradient: fp64 channel sums."""
+    rng = np.random.default_rng(1004)
+    xs, ws = (56, 56, 128, 64), (3, 3, 128, 128)
+    gd, od = cdims(gpu, xs, ws, padding=1)
+    x = rng.standard_normal(size=xs, dtype=np.float32)
+    w = (np.sqrt(2.0 / 1152) * rng.standard_normal(size=ws, dtype=np.float32))
+    b = (0.01 * rng.standard_normal(128)).astype(np.float32)
+    delta = rng.standard_normal(size=xs[:2] + (128, 64), dtype=np.float32)
+    x, w, b, delta = host_inputs(dtype, x, w, b, delta)
+    dx_, dw_, db_, dd_ = (dev(gpu, a, dtype) for a in (x, w, b, delta))
+    y, back = gpu.pullback(gpu.fused_conv_bias_activation, "relu", dw_, dx_, db_, gd)
+    gw, gx, gb = back(dd_)
+    yh = y.to_numpy()
+    sub = [3, 60]
+    od2 = O.ConvDims(xs[:3] + (2,), ws, padding=1)
+    wy = O.fused_conv_bias_activation("relu", f64(w), f64(x[..., sub]), f64(b), od2)
+    assert_close(yh[..., sub], wy, dtype, "config5 y")
+    dz = f64(delta) * (yh > 0)                                    # relu: derivative from the stored output
+    if dtype == "bf16":
+        dz = f64(O.round_to_bf16(dz.astype(np.float32)))
+    assert_close(gx.to_numpy()[..., sub], O.conv_data_grad(dz[..., sub], f64(w), od2), dtype, "config5 dx")
+    assert_close(gb.to_numpy(), (f64(delta) * (yh > 0)).sum(axis=(0, 1, 3)), dtype, "config5 db",
+                 rel=None if dtype == "f32" else 2e-2, scale=rms(delta) * 300)
+    # adjoint identity for the filter gradient
+    wp = host_inputs(dtype, rng.standard_normal(size=ws, dtype=np.float32))[0]
+    cwp = gpu.conv(dx_, dev(gpu, wp, dtype), gd).to_numpy().astype(np.float64)
+    lhs = float((gw.to_numpy().astype(np.float64) * f64(wp)).sum())
+    rhs = float((dz * cwp).sum())
+    assert abs(lhs - rhs) <= (2e-4 if dtype == "f32" else 2e-2) * max(abs(rhs), np.sqrt(dz.size)), (lhs, rhs)
+    # and an oracle check of the same kernel on a two-image batch
+    gd2 = gpu.DenseConvDims(xs[:3] + (2,), ws, padding=1)
+    dzq = dz[..., sub].astype(np.float32)
+    gw2 = gpu.conv_filter_grad(dev(gpu, x[..., sub], dtype), dev(gpu, dzq, dtype), gd2)
+    assert_close(gw2.to_numpy(), O.conv_filter_grad(f64(x[..., sub]), f64(dzq), od2), dtype, "config5 dw (2 images)")
