@@ -181,7 +181,148 @@ class C2BatchnormBiasAct(Workload):
                           f"normalise loop is threaded: {threads} OpenMP threads; all other passes are serial SIMD loops)"}
 
 
-WORKLOADS = {"C2": C2BatchnormBiasAct}
+class _ApiWorkload(Workload):
+    """Workloads driven through the host API mirror (pullback closures); outputs come from the
+    library's pooled allocator, so no hipMalloc happens inside the timed region."""
+
+    def setup(self, lux):
+        self.lux = lux
+        self.build(lux)
+        self.step()               # allocate pool blocks and workspaces once
+
+    def d(self, a, dtype=None):
+        return self.lux.DeviceArray.from_numpy(a, dtype or self.storage)
+
+    @property
+    def storage(self):
+        return "bf16" if self.dtype == "bf16" else "f32"
+
+
+class C1Dense(_ApiWorkload):
+    """BASELINE config 1: fused_dense_bias_activation 128 -> 256, batch 64, tanh, fp32."""
+    name, dtype, bound = "C1", "f32", "mfma"
+    description = "fused_dense_bias_activation(tanh) fwd+bwd, W 256x128, x 128x64 fp32 (latency-bound)"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1000)
+        lim = np.sqrt(6.0 / 384.0)
+        self.W = self.d(rng.uniform(-lim, lim, size=(256, 128)).astype(np.float32))
+        self.x = self.d(rng.standard_normal(size=(128, 64)).astype(np.float32))
+        self.b = self.d((0.01 * rng.standard_normal(256)).astype(np.float32))
+        self.delta = self.d(rng.standard_normal(size=(256, 64)).astype(np.float32))
+
+    def step(self):
+        y, back = self.lux.pullback(self.lux.fused_dense_bias_activation, "tanh", self.W, self.x, self.b)
+        back(self.delta)
+
+    def work_per_step(self):
+        return 3 * 2.0 * 256 * 128 * 64
+
+    def kernel_work(self):
+        return {"dense_gemm_kernel<f32>": 2.0 * 256 * 128 * 64}
+
+
+class C3Groupnorm(_ApiWorkload):
+    """BASELINE config 3: groupnorm(32 groups) + swish, x 64x64x256x16."""
+    name, bound = "C3", "hbm"
+    shape, groups = (64, 64, 256, 16), 32
+
+    def __init__(self, dtype="f32"):
+        self.dtype = dtype
+        self.name = "C3" if dtype == "f32" else "C3bf16"
+        self.description = f"groupnorm(32 groups, swish) fwd+bwd, x 64x64x256x16 {dtype}"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1002)
+        self.x = self.d(rng.standard_normal(size=self.shape, dtype=np.float32))
+        self.g = self.d(rng.uniform(0.8, 1.2, 256).astype(np.float32))
+        self.b = self.d((0.05 * rng.standard_normal(256)).astype(np.float32))
+        self.delta = self.d(rng.standard_normal(size=self.shape, dtype=np.float32))
+
+    def step(self):
+        y, back = self.lux.pullback(self.lux.groupnorm, self.x, self.g, self.b, self.groups, "swish", 1e-5)
+        back(self.delta)
+
+    @property
+    def E(self):
+        return int(np.prod(self.shape)) * (4 if self.dtype == "f32" else 2)
+
+    def work_per_step(self):
+        return 5 * self.E        # fwd: x in, y out; bwd: delta, x in, dx out
+
+    def kernel_work(self):
+        return {"gn_fwd_kernel": 2 * self.E, "gn_bwd_kernel": 3 * self.E}
+
+
+class C4TransformerMLP(_ApiWorkload):
+    """BASELINE config 4: layernorm(4096 x 8192) -> dense 4096->11008 gelu -> dense 11008->4096,
+    bf16 storage, fp32 accumulation."""
+    name, dtype, bound = "C4", "bf16", "mfma"
+    description = "layernorm + dense(4096->11008, gelu) + dense(11008->4096) fwd+bwd, 8192 tokens, bf16/fp32-acc"
+    D, F, Ntok = 4096, 11008, 8192
+
+    def build(self, lux):
+        rng = np.random.default_rng(1003)
+        D, F, N = self.D, self.F, self.Ntok
+        std = np.sqrt(2.0 / (D + F))
+        self.x = self.d(rng.standard_normal(size=(D, N), dtype=np.float32))
+        self.g = self.d(rng.uniform(0.5, 1.5, (D, 1)).astype(np.float32))
+        self.b = self.d((0.1 * rng.standard_normal((D, 1))).astype(np.float32))
+        self.W1 = self.d(std * rng.standard_normal(size=(F, D), dtype=np.float32))
+        self.b1 = self.d(np.zeros(F, np.float32))
+        self.W2 = self.d(std * rng.standard_normal(size=(D, F), dtype=np.float32))
+        self.b2 = self.d(np.zeros(D, np.float32))
+        self.delta = self.d(0.02 * rng.standard_normal(size=(D, N), dtype=np.float32))
+
+    def step(self):
+        lux = self.lux
+        h0, back_ln = lux.pullback(lux.layernorm, self.x, self.g, self.b, "identity", (1,), 1e-5)
+        h1, back_d1 = lux.pullback(lux.fused_dense_bias_activation, "gelu", self.W1, h0, self.b1)
+        h2, back_d2 = lux.pullback(lux.fused_dense_bias_activation, "identity", self.W2, h1, self.b2)
+        dW2, dh1, db2 = back_d2(self.delta)
+        dW1, dh0, db1 = back_d1(dh1)
+        back_ln(dh0)
+
+    def work_per_step(self):
+        return 6 * 2.0 * self.D * self.F * self.Ntok      # six GEMMs (the metric counts GEMM flops only)
+
+    def kernel_work(self):
+        return {"dense_gemm_kernel<bf16>": 2.0 * self.D * self.F * self.Ntok}
+
+
+class C5Conv(_ApiWorkload):
+    """BASELINE config 5: fused_conv_bias_activation 3x3, 128->128, 56x56, batch 64, pad 1, relu."""
+    bound = "mfma"
+    xs, ws = (56, 56, 128, 64), (3, 3, 128, 128)
+
+    def __init__(self, dtype="f32"):
+        self.dtype = dtype
+        self.name = "C5" if dtype == "f32" else "C5bf16"
+        self.description = f"fused_conv_bias_activation(relu) 3x3 128->128, x 56x56x128x64, pad 1, fwd+bwd {dtype}"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1004)
+        self.cd = lux.DenseConvDims(self.xs, self.ws, padding=1)
+        self.x = self.d(rng.standard_normal(size=self.xs, dtype=np.float32))
+        self.w = self.d(np.sqrt(2.0 / 1152) * rng.standard_normal(size=self.ws, dtype=np.float32))
+        self.b = self.d((0.01 * rng.standard_normal(128)).astype(np.float32))
+        self.delta = self.d(rng.standard_normal(size=self.cd.y_shape, dtype=np.float32))
+
+    def step(self):
+        y, back = self.lux.pullback(self.lux.fused_conv_bias_activation, "relu", self.w, self.x, self.b, self.cd)
+        back(self.delta)
+
+    def work_per_step(self):
+        return 3 * 2.0 * (56 * 56 * 64) * 128 * 1152
+
+    def kernel_work(self):
+        f = 2.0 * (56 * 56 * 64) * 128 * 1152
+        t = "bf16" if self.dtype == "bf16" else "f32"
+        return {f"conv_fprop_kernel<{t}>": f, f"conv_dgrad_kernel<{t}>": f, f"conv_wgrad_kernel<{t}>": f}
+
+
+WORKLOADS = {"C1": C1Dense, "C2": C2BatchnormBiasAct, "C3": lambda: C3Groupnorm("f32"), "C3bf16": lambda: C3Groupnorm("bf16"),
+             "C4": C4TransformerMLP, "C5": lambda: C5Conv("f32"), "C5bf16": lambda: C5Conv("bf16")}
 
 
 # ----------------------------------------------------------------------------- timing
@@ -215,8 +356,8 @@ def kernel_profile(lux, fn, steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline (0 disables it)")
     args = ap.parse_args()
@@ -228,6 +369,11 @@ def main():
     lux = load_package()
     lux.init(0)
     wl = WORKLOADS[args.workload]()
+    heavy = args.workload in ("C4", "C5", "C5bf16")
+    if args.steps is None:
+        args.steps = 20 if heavy else 200
+    if args.warmup is None:
+        args.warmup = 3 if heavy else 20
     wl.setup(lux)
 
     ms_gpu, ms_wall = timed(lux, wl.step, args.steps, args.warmup)

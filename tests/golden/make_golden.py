@@ -1,0 +1,81 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/luxlib_golden.npz: small input/output vectors of every operator on the
+path, on the deterministic inputs the reference's own tests use
+(`generate_fixed_array`, lib/LuxLib/test/shared_testsetup.jl:69-73), with outputs from the
+fp64 oracle, plus the reference's known-answer vectors as plain data.
+
+The reference is Julia and cannot run here, so nothing is imported from it: the oracle that
+produces these outputs is pinned independently (tests/test_oracle_*.py).  Run from the repo
+root:  python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import luxlib_oracle as O  # noqa: E402
+
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "luxlib_golden.npz")
+
+
+def fixed(shape, shift=0.0, scale=1.0):
+    return (O.generate_fixed_array(np.float64, shape) - shift) * scale
+
+
+def main():
+    g = {}
+    # --- reference known answers (test/core_layers/normalize_tests.jl:10-49, basic_tests.jl:151-194,
+    #     conv_tests.jl:54-69) stored as data
+    g["kat_bn_x"] = np.array([[1.0, 3.0, 5.0], [2.0, 4.0, 6.0]])
+    g["kat_bn_y"] = np.array([[-1.22474, 0.0, 1.22474], [-1.22474, 0.0, 1.22474]])
+    g["kat_bn_running_mean"] = np.array([0.3, 0.4])
+    g["kat_bn_running_var"] = np.array([1.3, 1.3])
+    g["kat_conv_pad_counts"] = np.array([6.0, 9.0, 4.0, 3.0, 6.0, 2.0])
+
+    # --- dense (dense_tests.jl sizes): W 4x32, x 32x3, tanh, inputs scaled like the reference (1e-3 offsets)
+    W, x, b = fixed((4, 32), 0.5), fixed((32, 3), 0.5, 2.0), fixed((4,), 0.5)
+    delta = fixed((4, 3), 0.3)
+    y, dW, dx, db = O.fused_dense_pullback("tanh", W, x, b, delta)
+    g.update(dense_W=W, dense_x=x, dense_b=b, dense_delta=delta, dense_y=y, dense_dW=dW, dense_dx=dx, dense_db=db)
+
+    # --- bias_activation (bias_act_tests.jl shape (2,2,3,4)), gelu
+    x, b, delta = fixed((2, 2, 3, 4), 0.5, 3.0), fixed((3,), 0.5), fixed((2, 2, 3, 4), 0.4)
+    y, dx, db = O.bias_activation_pullback("gelu", x, b, delta)
+    g.update(ba_x=x, ba_b=b, ba_delta=delta, ba_y=y, ba_dx=dx, ba_db=db)
+
+    # --- batchnorm (batchnorm_tests.jl shape (4,4,6,2)), training, relu
+    x = fixed((4, 4, 6, 2), 0.5, 2.0) + 0.05 * np.sin(np.arange(192)).reshape((4, 4, 6, 2), order="F")
+    gm, bt, rm, rv = fixed((6,), -0.5), fixed((6,), 0.5), fixed((6,), 0.5), fixed((6,), -0.5)
+    delta = np.cos(np.arange(192)).reshape((4, 4, 6, 2), order="F")
+    y, rm2, rv2 = O.batchnorm(x, gm, bt, rm, rv, True, "relu", 0.1, 1e-5)
+    dx, dg, dbt = O.batchnorm_pullback(x, gm, bt, "relu", 1e-5, delta)
+    g.update(bn_x=x, bn_gamma=gm, bn_beta=bt, bn_rmean=rm, bn_rvar=rv, bn_delta=delta, bn_y=y, bn_rmean_out=rm2,
+             bn_rvar_out=rv2, bn_dx=dx, bn_dgamma=dg, bn_dbeta=dbt)
+
+    # --- groupnorm (groupnorm_tests.jl shape (4,4,6,2), 3 groups), swish
+    y = O.groupnorm(x, gm, bt, 3, "swish", 1e-5)
+    dx, dg, dbt = O.groupnorm_pullback(x, gm, bt, 3, "swish", 1e-5, delta)
+    g.update(gn_y=y, gn_dx=dx, gn_dgamma=dg, gn_dbeta=dbt)
+
+    # --- layernorm (layernorm_tests.jl shape (4,4,6,2), dims 1:3, affine (4,4,6,1))
+    lg, lb = fixed((4, 4, 6, 1), -0.5), fixed((4, 4, 6, 1), 0.5)
+    y = O.layernorm(x, lg, lb, "identity", (0, 1, 2), 1e-5)
+    dx, dg, dbt = O.layernorm_pullback(x, lg, lb, "identity", (0, 1, 2), 1e-5, delta)
+    g.update(ln_gamma=lg, ln_beta=lb, ln_y=y, ln_dx=dx, ln_dgamma=dg, ln_dbeta=dbt)
+
+    # --- conv (conv_tests.jl: kernel (2,2), stride 2, pad 1, groups 2), sigmoid
+    xs, ws = (6, 5, 4, 2), (2, 2, 2, 6)
+    cx, cw, cb = fixed(xs, 0.5, 2.0), fixed(ws, 0.5), fixed((6,), 0.5)
+    cd = O.ConvDims(xs, ws, stride=2, padding=1, groups=2)
+    cdelta = np.cos(np.arange(int(np.prod(cd.y_shape())))).reshape(cd.y_shape(), order="F")
+    y, dw, dx, db = O.fused_conv_pullback("sigmoid", cw, cx, cb, cd, cdelta)
+    g.update(conv_x=cx, conv_w=cw, conv_b=cb, conv_delta=cdelta, conv_y=y, conv_dw=dw, conv_dx=dx, conv_db=db)
+
+    np.savez_compressed(OUT, **{k: np.asarray(v, dtype=np.float64) for k, v in g.items()})
+    print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(g), "arrays")
+
+
+if __name__ == "__main__":
+    main()
