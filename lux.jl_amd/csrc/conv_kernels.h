@@ -73,7 +73,7 @@ struct ConvGatherLoaderK {
     static constexpr bool KMAJOR = true;
     static constexpr int CHUNKS = ROWS * Tr::BK / Tr::VEC;
     static constexpr int PER_THREAD = CHUNKS / kGemmThreads;
-    uint4 reg[PER_THREAD];
+    u32x4_v reg[PER_THREAD];
     const GatherK<T>& g;
     int m0, K;
     __device__ __forceinline__ ConvGatherLoaderK(const GatherK<T>& gg, int row0, int k_total) : g(gg), m0(row0), K(k_total) {}
@@ -85,11 +85,11 @@ struct ConvGatherLoaderK {
             const int r = id / (Tr::BK / Tr::VEC);
             const int k = k0 + (id % (Tr::BK / Tr::VEC)) * Tr::VEC;
             const int m = m0 + r;
-            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            u32x4_v v = {0u, 0u, 0u, 0u};
             if (m < g.M && k < K) {
                 if (g.vec_ok) {          // K % VEC == 0 and chunks never straddle a tap
                     int64_t off;
-                    if (g.locate(m, k, off)) v = *reinterpret_cast<const uint4*>(g.src + off);
+                    if (g.locate(m, k, off)) v = *reinterpret_cast<const u32x4_v*>(g.src + off);
                 } else {
                     T tmp[Tr::VEC];
 #pragma unroll
@@ -97,7 +97,7 @@ struct ConvGatherLoaderK {
                         int64_t off;
                         tmp[e] = (k + e < K && g.locate(m, k + e, off)) ? g.src[off] : T(0);
                     }
-                    v = *reinterpret_cast<const uint4*>(tmp);
+                    v = *reinterpret_cast<const u32x4_v*>(tmp);
                 }
             }
             reg[i] = v;
@@ -109,7 +109,7 @@ struct ConvGatherLoaderK {
         for (int i = 0; i < PER_THREAD; ++i) {
             const int id = threadIdx.x + i * kGemmThreads;
             const int r = id / (Tr::BK / Tr::VEC), k = (id % (Tr::BK / Tr::VEC)) * Tr::VEC;
-            *reinterpret_cast<uint4*>(lds + lds_chunk_offset<T, true, ROWS>(r, k)) = reg[i];
+            *reinterpret_cast<u32x4_v*>(lds + lds_chunk_offset<T, true, ROWS>(r, k)) = reg[i];
         }
     }
 };
@@ -226,7 +226,7 @@ struct ConvGatherLoaderMN {
     static constexpr bool KMAJOR = false;
     static constexpr int CHUNKS = ROWS * Tr::BK / Tr::VEC;
     static constexpr int PER_THREAD = CHUNKS / kGemmThreads;
-    uint4 reg[PER_THREAD];
+    u32x4_v reg[PER_THREAD];
     const GatherMN<T>& g;
     int m0, kbase, Kend;       // Kend = one past the last k' of this slice
     __device__ __forceinline__ ConvGatherLoaderMN(const GatherMN<T>& gg, int row0, int kb, int ke)
@@ -238,11 +238,11 @@ struct ConvGatherLoaderMN {
             const int id = threadIdx.x + i * kGemmThreads;
             const int kp = kbase + k0 + id / (ROWS / Tr::VEC);
             const int mrow = m0 + (id % (ROWS / Tr::VEC)) * Tr::VEC;
-            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            u32x4_v v = {0u, 0u, 0u, 0u};
             if (kp < Kend && mrow < g.Mrows) {
                 if (g.vec_ok) {
                     int64_t off;
-                    if (g.locate(mrow, kp, off)) v = *reinterpret_cast<const uint4*>(g.src + off);
+                    if (g.locate(mrow, kp, off)) v = *reinterpret_cast<const u32x4_v*>(g.src + off);
                 } else {
                     T tmp[Tr::VEC];
 #pragma unroll
@@ -250,7 +250,7 @@ struct ConvGatherLoaderMN {
                         int64_t off;
                         tmp[e] = (mrow + e < g.Mrows && g.locate(mrow + e, kp, off)) ? g.src[off] : T(0);
                     }
-                    v = *reinterpret_cast<const uint4*>(tmp);
+                    v = *reinterpret_cast<const u32x4_v*>(tmp);
                 }
             }
             reg[i] = v;
@@ -262,7 +262,7 @@ struct ConvGatherLoaderMN {
         for (int i = 0; i < PER_THREAD; ++i) {
             const int id = threadIdx.x + i * kGemmThreads;
             const int k = id / (ROWS / Tr::VEC), r = (id % (ROWS / Tr::VEC)) * Tr::VEC;
-            *reinterpret_cast<uint4*>(lds + lds_chunk_offset<T, false, ROWS>(r, k)) = reg[i];
+            *reinterpret_cast<u32x4_v*>(lds + lds_chunk_offset<T, false, ROWS>(r, k)) = reg[i];
         }
     }
 };

@@ -32,6 +32,7 @@ typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
 typedef float f32x16_v __attribute__((ext_vector_type(16)));
 typedef short s16x4_v __attribute__((ext_vector_type(4)));
 typedef short s16x8_v __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_v __attribute__((ext_vector_type(4)));
 
 constexpr int kGemmThreads = 256;
 
@@ -81,17 +82,22 @@ __device__ __forceinline__ int lds_chunk_offset(int r, int k) {
 // Loader policy of the mainloop: load(k0) fetches this thread's share of the stage that starts
 // at k0 into registers, store(lds) writes it to the stage buffer.  TileLoader reads a plain
 // strided matrix; the convolution kernels provide gathering loaders with the same interface.
-template <typename T, bool KMAJOR_, int ROWS>
+template <typename T, bool KMAJOR_, int ROWS, bool FULL = false>
 struct TileLoader {
     using Tr = GemmTraits<T>;
     static constexpr bool KMAJOR = KMAJOR_;
     static constexpr int CHUNKS = ROWS * Tr::BK / Tr::VEC;
     static constexpr int PER_THREAD = CHUNKS / kGemmThreads;
     static_assert(CHUNKS % kGemmThreads == 0, "tile must split evenly over the workgroup");
-    uint4 reg[PER_THREAD];
+    u32x4_v reg[PER_THREAD];
     Operand<T> op;
     int r0, K;
-    __device__ __forceinline__ TileLoader(const Operand<T>& o, int row0, int k_total) : op(o), r0(row0), K(k_total) {}
+    uint32_t voff;   // FULL: byte offset of this thread's first chunk inside the tile (32-bit)
+    __device__ __forceinline__ TileLoader(const Operand<T>& o, int row0, int k_total) : op(o), r0(row0), K(k_total) {
+        int r, k;
+        coords(threadIdx.x, r, k);
+        voff = (uint32_t)(((int64_t)r * op.sr + (int64_t)k * op.sk) * (int64_t)sizeof(T));
+    }
 
     __device__ __forceinline__ static void coords(int id, int& r, int& k) {
         if constexpr (KMAJOR) {
@@ -110,21 +116,31 @@ struct TileLoader {
             coords(threadIdx.x + i * kGemmThreads, r, k);
             r += r0;
             k += k0;
-            uint4 v = make_uint4(0u, 0u, 0u, 0u);
-            const int rem = KMAJOR ? (K - k) : (op.rows - r);     // valid elements along the chunk
-            const bool in = KMAJOR ? (r < op.rows) : (k < K);
-            if (in && rem > 0) {
-                const T* src = op.p + (int64_t)r * op.sr + (int64_t)k * op.sk;
-                if (op.vec_ok && rem >= Tr::VEC) {
-                    v = *reinterpret_cast<const uint4*>(src);
-                } else {
-                    T tmp[Tr::VEC];
+            if constexpr (FULL) {
+                // whole tiles, aligned: no predication; uniform 64-bit base (scalar registers) plus
+                // one 32-bit per-thread offset.  Chunk i of a thread lies a uniform step further.
+                constexpr int STEP = KMAJOR ? kGemmThreads / (Tr::BK / Tr::VEC) : kGemmThreads / (ROWS / Tr::VEC);
+                const int64_t ubase = KMAJOR ? ((int64_t)(r0 + i * STEP) * op.sr + (int64_t)k0 * op.sk)
+                                             : ((int64_t)r0 * op.sr + (int64_t)(k0 + i * STEP) * op.sk);
+                const char* up = reinterpret_cast<const char*>(op.p + ubase);
+                reg[i] = *reinterpret_cast<const u32x4_v*>(up + voff);
+            } else {
+                u32x4_v v = {0u, 0u, 0u, 0u};
+                const int rem = KMAJOR ? (K - k) : (op.rows - r);     // valid elements along the chunk
+                const bool in = KMAJOR ? (r < op.rows) : (k < K);
+                if (in && rem > 0) {
+                    const T* src = op.p + (int64_t)r * op.sr + (int64_t)k * op.sk;
+                    if (op.vec_ok && rem >= Tr::VEC) {
+                        v = *reinterpret_cast<const u32x4_v*>(src);
+                    } else {
+                        T tmp[Tr::VEC];
 #pragma unroll
-                    for (int e = 0; e < Tr::VEC; ++e) tmp[e] = e < rem ? src[e] : T(0);
-                    v = *reinterpret_cast<const uint4*>(tmp);
+                        for (int e = 0; e < Tr::VEC; ++e) tmp[e] = e < rem ? src[e] : T(0);
+                        v = *reinterpret_cast<const u32x4_v*>(tmp);
+                    }
                 }
+                reg[i] = v;
             }
-            reg[i] = v;
         }
     }
 
@@ -133,7 +149,7 @@ struct TileLoader {
         for (int i = 0; i < PER_THREAD; ++i) {
             int r, k;
             coords(threadIdx.x + i * kGemmThreads, r, k);
-            *reinterpret_cast<uint4*>(lds + lds_chunk_offset<T, KMAJOR, ROWS>(r, k)) = reg[i];
+            *reinterpret_cast<u32x4_v*>(lds + lds_chunk_offset<T, KMAJOR, ROWS>(r, k)) = reg[i];
         }
     }
 };
@@ -146,7 +162,7 @@ __device__ __forceinline__ bf16x8_v load_frag_bf16(const bf16_t* lds, int rbase,
     if constexpr (KMAJOR) {
         const int r = rbase + (l & 31);
         const int chunk = 2 * kk + (l >> 5);
-        const uint4 v = *reinterpret_cast<const uint4*>(lds + r * 64 + ((chunk ^ (r & 7)) << 3));
+        const u32x4_v v = *reinterpret_cast<const u32x4_v*>(lds + r * 64 + ((chunk ^ (r & 7)) << 3));
         return __builtin_bit_cast(bf16x8_v, v);
     } else {
         constexpr int STRIDE = ROWS + GemmTraits<bf16_t>::PAD_MN;
@@ -195,12 +211,12 @@ __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, i
 // ----------------------------------------------------------------------------- mainloop
 // Accumulates the (2*WM*32) x (2*WN*32) tile at (m0, n0).  acc[wm][wn][r] of lane l belongs to
 //   m = m0 + wave_m*WM*32 + wm*32 + l%32,   n = n0 + wave_n*WN*32 + wn*32 + 8*(r/4) + 4*(l/32) + r%4.
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false>
 struct GemmMainloop {
     using Tr = GemmTraits<T>;
     static constexpr int TILE_M = 2 * WM * 32, TILE_N = 2 * WN * 32;
-    using PlainLoaderA = TileLoader<T, A_KMAJOR, TILE_M>;
-    using PlainLoaderB = TileLoader<T, B_KMAJOR, TILE_N>;
+    using PlainLoaderA = TileLoader<T, A_KMAJOR, TILE_M, FULL>;
+    using PlainLoaderB = TileLoader<T, B_KMAJOR, TILE_N, FULL>;
     static constexpr int A_ELEMS = lds_tile_elems<T, A_KMAJOR>(TILE_M);
     static constexpr int B_ELEMS = lds_tile_elems<T, B_KMAJOR>(TILE_N);
     static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
@@ -227,21 +243,7 @@ struct GemmMainloop {
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
         const int KT = (K + Tr::BK - 1) / Tr::BK;
-        la.load(0);
-        lb.load(0);
-        la.store(lds);
-        lb.store(lds + A_ELEMS);
-        __syncthreads();
-        for (int kt = 0; kt < KT; ++kt) {
-            T* cur = lds + (kt & 1) * STAGE_ELEMS;
-            T* nxt = lds + ((kt + 1) & 1) * STAGE_ELEMS;
-            const bool more = kt + 1 < KT;
-            if (more) {
-                la.load((kt + 1) * Tr::BK);
-                lb.load((kt + 1) * Tr::BK);
-            }
-            const T* As = cur;
-            const T* Bs = cur + A_ELEMS;
+        auto compute = [&](const T* As, const T* Bs) {
             if constexpr (sizeof(T) == 2) {
 #pragma unroll
                 for (int kk = 0; kk < Tr::BK / 16; ++kk) {
@@ -273,12 +275,39 @@ struct GemmMainloop {
                                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][s], fa[i][s], acc[i][j], 0, 0, 0);
                 }
             }
-            if (more) {
-                la.store(nxt);
-                lb.store(nxt + A_ELEMS);
+        };
+        // Global loads run two stages ahead of the MFMAs (two register sets), LDS is double
+        // buffered: while stage kt is consumed from one LDS buffer, stage kt+1 waits in the
+        // first register set for its LDS slot and stage kt+2 is in flight into the second.
+        LoaderA la2 = la;
+        LoaderB lb2 = lb;
+        T* buf0 = lds;
+        T* buf1 = lds + STAGE_ELEMS;
+        la.load(0);
+        lb.load(0);
+        la.store(buf0);
+        lb.store(buf0 + A_ELEMS);
+        if (KT > 1) { la.load(Tr::BK); lb.load(Tr::BK); }
+        if (KT > 2) { la2.load(2 * Tr::BK); lb2.load(2 * Tr::BK); }
+        __syncthreads();
+        int kt = 0;
+        for (; kt + 2 <= KT; kt += 2) {
+            // even stage: buf0 holds kt, set 1 holds kt+1, set 2 holds kt+2
+            compute(buf0, buf0 + A_ELEMS);
+            la.store(buf1);
+            lb.store(buf1 + A_ELEMS);
+            if (kt + 3 < KT) { la.load((kt + 3) * Tr::BK); lb.load((kt + 3) * Tr::BK); }
+            __syncthreads();
+            // odd stage: buf1 holds kt+1, set 2 holds kt+2, set 1 holds kt+3
+            compute(buf1, buf1 + A_ELEMS);
+            if (kt + 2 < KT) {
+                la2.store(buf0);
+                lb2.store(buf0 + A_ELEMS);
+                if (kt + 4 < KT) { la2.load((kt + 4) * Tr::BK); lb2.load((kt + 4) * Tr::BK); }
             }
             __syncthreads();
         }
+        if (kt < KT) compute(buf0, buf0 + A_ELEMS);   // odd number of stages: the last one sits in buf0
     }
 
     // Calls f(m, n, value) for every element of the tile owned by this lane.

@@ -26,9 +26,9 @@ __device__ __forceinline__ float apply_act(int act, float x) {
     }
 }
 
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR>
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL>
 __global__ __launch_bounds__(kGemmThreads) void dense_gemm_kernel(DenseArgs<T> a) {
-    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR>;
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
     int tm, tn;
@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kGemmThreads) void dense_gemm_kernel(DenseArgs<T> a
     ML::run(a.A, a.B, a.K, m0, n0, lds, acc);
     const int act = a.act;
     ML::for_each(acc, m0, n0, [&](int m, int n, float v) {
-        if (m < a.M && n < a.N) {
+        if (FULL || (m < a.M && n < a.N)) {
             if (a.bias) v += ld(a.bias + m);
             const int64_t off = m + (int64_t)n * a.ldc;
             if (a.pre) st(a.pre + off, v);
@@ -47,12 +47,12 @@ __global__ __launch_bounds__(kGemmThreads) void dense_gemm_kernel(DenseArgs<T> a
     });
 }
 
-template <typename T, int WM, int WN, bool AK, bool BKM>
-int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
-    using ML = GemmMainloop<T, WM, WN, AK, BKM>;
+template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL>
+int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
+    using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL>;
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
-    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM>;
+    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL>;
     static bool attr_set = false;
     if (!attr_set) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -65,14 +65,34 @@ int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
     return LUXHIP_OK;
 }
 
+// whole, aligned tiles take the kernel variant without bounds checks (big tiles only)
+template <typename T, int WM, int WN, bool AK, bool BKM>
+int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
+    using ML = GemmMainloop<T, WM, WN, AK, BKM>;
+    if constexpr (WM * WN >= 4) {
+        const bool full = a.M % ML::TILE_M == 0 && a.N % ML::TILE_N == 0 && a.K % GemmTraits<T>::BK == 0 && a.K > 0 &&
+                          a.A.vec_ok && a.B.vec_ok &&
+                          256 * std::max(a.A.sr, a.A.sk) * (int64_t)sizeof(T) < (1ll << 31) &&
+                          256 * std::max(a.B.sr, a.B.sk) * (int64_t)sizeof(T) < (1ll << 31);
+        if (full) return launch_cfg_full<T, WM, WN, AK, BKM, true>(s, a);
+    }
+    return launch_cfg_full<T, WM, WN, AK, BKM, false>(s, a);
+}
+
+int gemm_tile_override();   // gemm.hip: LUXHIP_GEMM_TILE=42|22|11 forces a tile (tuning aid), 0 = automatic
+
 template <typename T, bool AK, bool BKM>
 int launch_layout(hipStream_t s, DenseArgs<T>& a) {
-    // largest tile that still yields at least ~one workgroup per compute unit
-    const int64_t cus = std::max(1, num_cus());
-    const int64_t t256 = ceil_div(a.M, 256) * ceil_div(a.N, 256);
+    switch (gemm_tile_override()) {
+        case 42: return launch_cfg<T, 4, 2, AK, BKM>(s, a);
+        case 22: return launch_cfg<T, 2, 2, AK, BKM>(s, a);
+        case 11: return launch_cfg<T, 1, 1, AK, BKM>(s, a);
+        default: break;
+    }
+    // 128 x 128 tiles (two workgroups per compute unit) measured fastest on large problems;
+    // 64 x 64 for small ones
     const int64_t t128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
-    if (t256 >= cus) return launch_cfg<T, 4, 4, AK, BKM>(s, a);
-    if (t128 >= cus / 2 || (a.M > 64 && a.N > 64 && t128 >= 4)) return launch_cfg<T, 2, 2, AK, BKM>(s, a);
+    if (a.M > 64 && a.N > 64 && t128 >= 4) return launch_cfg<T, 2, 2, AK, BKM>(s, a);
     return launch_cfg<T, 1, 1, AK, BKM>(s, a);
 }
 

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from oracle import luxlib_oracle as O
-from tests.util import assert_close, dev, f64, host_inputs, rms
+from tests.util import stable_seed, assert_close, dev, f64, host_inputs, rms
 
 pytestmark = pytest.mark.gpu
 
@@ -24,12 +24,17 @@ def dx_scale(x, g, groups, eps, delta):
 @pytest.mark.parametrize("act", ["identity", "relu", "sigmoid_fast", "swish", "gelu"])
 @pytest.mark.parametrize("affine", [True, False])
 def test_forward_and_pullback(gpu, dtype, act, affine):
-    rng = np.random.default_rng(abs(hash((dtype, act, affine))) % 2 ** 31)
+    rng = np.random.default_rng(stable_seed(dtype, act, affine))
     for shape, groups in CASES:
         Cc = shape[-2]
-        x, g, b, delta = host_inputs(dtype, rng.normal(size=shape), rng.uniform(0.8, 1.2, Cc) if affine else None,
-                                     rng.normal(size=Cc) * 0.05 if affine else None, rng.normal(size=shape))
         eps = 1e-5 if dtype == "f32" else 1e-3
+        for _ in range(50):
+            x, g, b, delta = host_inputs(dtype, rng.normal(size=shape), rng.uniform(0.8, 1.2, Cc) if affine else None,
+                                         rng.normal(size=Cc) * 0.05 if affine else None, rng.normal(size=shape))
+            # keep the pre-activation away from relu's kink: a sign flip there is a discontinuity,
+            # not a rounding difference
+            if act != "relu" or np.abs(O.groupnorm(f64(x), f64(g), f64(b), groups, "identity", eps)).min() > 1e-3:
+                break
         tag = f"{dtype} {act} {shape} G={groups} affine={affine}"
         y, back = gpu.pullback(gpu.groupnorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), groups, act, eps)
         wy = O.groupnorm(f64(x), f64(g), f64(b), groups, act, eps)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from oracle import luxlib_oracle as O
-from tests.util import assert_close, dev, f64, host_inputs, rms
+from tests.util import stable_seed, assert_close, dev, f64, host_inputs, rms
 
 pytestmark = pytest.mark.gpu
 
@@ -25,13 +25,17 @@ def test_invariants_without_affine(gpu):
 @pytest.mark.parametrize("act", ["identity", "relu", "gelu", "tanh"])
 @pytest.mark.parametrize("affine", [True, False])
 def test_forward_and_pullback(gpu, dtype, act, affine):
-    rng = np.random.default_rng(abs(hash((dtype, act, affine))) % 2 ** 31)
+    rng = np.random.default_rng(stable_seed(dtype, act, affine))
     for shape, nd in CASES:
         pshape = shape[:nd] + (1,) * (len(shape) - nd)
-        x, g, b, delta = host_inputs(dtype, rng.normal(size=shape), rng.uniform(0.5, 1.5, pshape) if affine else None,
-                                     rng.normal(size=pshape) if affine else None, rng.normal(size=shape))
         eps = 1e-5 if dtype == "f32" else 1e-3
         dims_np, dims_jl = tuple(range(nd)), tuple(range(1, nd + 1))
+        for _ in range(50):
+            x, g, b, delta = host_inputs(dtype, rng.normal(size=shape), rng.uniform(0.5, 1.5, pshape) if affine else None,
+                                         rng.normal(size=pshape) if affine else None, rng.normal(size=shape))
+            # keep the pre-activation away from relu's kink (a sign flip is a discontinuity)
+            if act != "relu" or shape[0] > 4000 or np.abs(O.layernorm(f64(x), f64(g), f64(b), "identity", dims_np, eps)).min() > 1e-4:
+                break
         tag = f"{dtype} {act} {shape} nd={nd} affine={affine}"
         y, back = gpu.pullback(gpu.layernorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), act, dims_jl, eps)
         wy = O.layernorm(f64(x), f64(g), f64(b), act, dims_np, eps)

@@ -59,3 +59,9 @@ def f64(a):
 def rms(a):
     a = np.asarray(a, dtype=np.float64)
     return float(np.sqrt(np.mean(a * a))) if a.size else 0.0
+
+
+def stable_seed(*parts):
+    """Seed that does not depend on Python's per-process string hashing."""
+    import zlib
+    return zlib.crc32(repr(parts).encode()) & 0x7FFFFFFF
