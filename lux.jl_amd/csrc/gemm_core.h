@@ -8,18 +8,21 @@
 // consecutive m: stores to the column-major C are contiguous and a per-m bias is one value per
 // lane.
 //
-// Storage types:  bf16 -> v_mfma_f32_32x32x16_bf16 (BK = 64 per stage),
+// Storage types:  bf16 -> v_mfma_f32_32x32x16_bf16 (BK = 32 per stage),
 //                 fp32 -> v_mfma_f32_32x32x2_f32   (BK = 16 per stage).
 //
 // Each operand tile is staged global -> registers -> LDS (double buffered, one barrier per
 // stage) in the layout that matches how it lies in memory:
-//   K-major operand  (k contiguous): LDS [row][BK]; bf16 rows are 128 B with an XOR swizzle of
-//       the 16-byte chunk index so that the ds_read_b128 fragment reads of 8 consecutive rows
-//       fall into different banks; fp32 rows are padded by 4 floats.
-//   MN-major operand (m or n contiguous, k strided): LDS [k][rows + pad]; bf16 fragments are
-//       read with ds_read_b64_tr_b16 (the LDS transpose read of gfx950), which hands each lane
-//       the 4 consecutive k of its own row out of a 4(k) x 16(rows) block; fp32 fragments are
-//       plain ds_read_b32.
+//   K-major operand  (k contiguous): LDS [row][BK]; bf16 rows are 64 B (BK = 32) with an XOR
+//       swizzle of the 16-byte chunk index by (row/4)%4 so that the ds_read_b128 fragment reads
+//       of 16 consecutive rows fall into different banks; fp32 rows are padded by 4 floats.
+//   MN-major operand (m or n contiguous, k strided): LDS [k][rows]; bf16 rows are unpadded and
+//       their 64-byte granules XOR-swizzled with k&3; fragments are read with
+//       ds_read_b64_tr_b16 (the LDS transpose read of gfx950), which hands each lane the 4
+//       consecutive k of its own row out of a 4(k) x 16(rows) block (the 4 k-rows of a block
+//       then sit in 4 different bank groups); fp32 rows are padded and read with ds_read_b32.
+// Whole aligned bf16 tiles skip the registers: global_load_lds_dwordx4 writes 64 lanes x 16
+// bytes linearly into LDS, and each lane fetches the chunk that the swizzle wants there.
 // The same (lane group, slot) -> k assignment is used for both operands of an MFMA, which is
 // all the instruction needs.
 #pragma once
@@ -40,16 +43,26 @@ template <typename T>
 struct GemmTraits;
 template <>
 struct GemmTraits<bf16_t> {
-    static constexpr int BK = 64, VEC = 8, KSTEP = 16;   // KSTEP: k consumed per fragment load
-    static constexpr int PAD_MN = 16;
+    static constexpr int BK = 32, VEC = 8, KSTEP = 16;   // KSTEP: k consumed per fragment load
+    static constexpr int PAD_MN = 0;    // MN-major rows are swizzled instead of padded
     __host__ __device__ static constexpr int kmajor_stride() { return BK; }
 };
 template <>
 struct GemmTraits<float> {
     static constexpr int BK = 16, VEC = 4, KSTEP = 8;
-    static constexpr int PAD_MN = 4;
+    static constexpr int PAD_MN = 8;    // 4 k-rows apart = 128 bytes apart modulo the 256-byte bank period
     __host__ __device__ static constexpr int kmajor_stride() { return BK + 4; }
 };
+
+// The LDS of gfx950 has 64 banks of 4 bytes (256-byte period).  bf16 swizzles are chosen so that
+// the lanes served together hit 256 distinct bytes:
+//   K-major rows of 64 bytes: ds_read_b128 serves 16 lanes (16 rows) at a time; rows r and r+4
+//       share a bank offset, so the chunk index is XORed with (r/4)%4.
+//   MN-major [k][rows]: a transpose read serves two 16-lane blocks at a time, each 4 k-rows x 32
+//       bytes at row offsets g and g+32 bytes; XORing the row index with (k%4) << 5 moves the 4
+//       k-rows into 4 different 64-byte granules (tiles narrower than 128 rows have only room for
+//       32-byte granules).
+__host__ __device__ constexpr int mn_swizzle_shift(int rows) { return rows >= 128 ? 5 : 4; }
 
 // elements of one LDS stage of an operand tile with `rows` rows
 template <typename T, bool KMAJOR>
@@ -72,23 +85,24 @@ template <typename T, bool KMAJOR, int ROWS>
 __device__ __forceinline__ int lds_chunk_offset(int r, int k) {
     using Tr = GemmTraits<T>;
     if constexpr (KMAJOR) {
-        if constexpr (sizeof(T) == 2) return r * Tr::BK + (((k >> 3) ^ (r & 7)) << 3);
+        if constexpr (sizeof(T) == 2) return r * Tr::BK + (((k >> 3) ^ ((r >> 2) & 3)) << 3);
         else return r * Tr::kmajor_stride() + k;
     } else {
-        return k * (ROWS + Tr::PAD_MN) + r;
+        if constexpr (sizeof(T) == 2) return k * ROWS + (r ^ ((k & 3) << mn_swizzle_shift(ROWS)));   // r is a multiple of 8
+        else return k * (ROWS + Tr::PAD_MN) + r;
     }
 }
 
 // Loader policy of the mainloop: load(k0) fetches this thread's share of the stage that starts
 // at k0 into registers, store(lds) writes it to the stage buffer.  TileLoader reads a plain
 // strided matrix; the convolution kernels provide gathering loaders with the same interface.
-template <typename T, bool KMAJOR_, int ROWS, bool FULL = false>
+template <typename T, bool KMAJOR_, int ROWS, bool FULL = false, int THREADS = kGemmThreads>
 struct TileLoader {
     using Tr = GemmTraits<T>;
     static constexpr bool KMAJOR = KMAJOR_;
     static constexpr int CHUNKS = ROWS * Tr::BK / Tr::VEC;
-    static constexpr int PER_THREAD = CHUNKS / kGemmThreads;
-    static_assert(CHUNKS % kGemmThreads == 0, "tile must split evenly over the workgroup");
+    static constexpr int PER_THREAD = CHUNKS / THREADS;
+    static_assert(CHUNKS % THREADS == 0, "tile must split evenly over the workgroup");
     u32x4_v reg[PER_THREAD];
     Operand<T> op;
     int r0, K;
@@ -113,13 +127,13 @@ struct TileLoader {
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
             int r, k;
-            coords(threadIdx.x + i * kGemmThreads, r, k);
+            coords(threadIdx.x + i * THREADS, r, k);
             r += r0;
             k += k0;
             if constexpr (FULL) {
                 // whole tiles, aligned: no predication; uniform 64-bit base (scalar registers) plus
                 // one 32-bit per-thread offset.  Chunk i of a thread lies a uniform step further.
-                constexpr int STEP = KMAJOR ? kGemmThreads / (Tr::BK / Tr::VEC) : kGemmThreads / (ROWS / Tr::VEC);
+                constexpr int STEP = KMAJOR ? THREADS / (Tr::BK / Tr::VEC) : THREADS / (ROWS / Tr::VEC);
                 const int64_t ubase = KMAJOR ? ((int64_t)(r0 + i * STEP) * op.sr + (int64_t)k0 * op.sk)
                                              : ((int64_t)r0 * op.sr + (int64_t)(k0 + i * STEP) * op.sk);
                 const char* up = reinterpret_cast<const char*>(op.p + ubase);
@@ -148,9 +162,56 @@ struct TileLoader {
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
             int r, k;
-            coords(threadIdx.x + i * kGemmThreads, r, k);
+            coords(threadIdx.x + i * THREADS, r, k);
             *reinterpret_cast<u32x4_v*>(lds + lds_chunk_offset<T, KMAJOR, ROWS>(r, k)) = reg[i];
         }
+    }
+};
+
+// Direct global -> LDS loader for whole, aligned bf16 tiles.  One wave instruction fills 1 KiB
+// of the stage linearly (lane i -> byte 16*i after a wave-uniform base); lane i therefore
+// fetches the global chunk whose swizzled home is that slot.
+template <bool KMAJOR_, int ROWS, int THREADS = kGemmThreads>
+struct DirectLoader {
+    using T = bf16_t;
+    static constexpr bool KMAJOR = KMAJOR_;
+    static constexpr int BK = GemmTraits<bf16_t>::BK;
+    static constexpr int CPR = KMAJOR ? BK / 8 : ROWS / 8;         // 16-byte chunks per LDS row
+    static constexpr int INSTR = ROWS * BK / 8 / THREADS;          // instructions per thread and stage
+    static_assert(INSTR >= 1 && (ROWS * BK / 8) % THREADS == 0, "stage must split evenly over the workgroup");
+    static constexpr int STEP = THREADS / CPR;                // LDS rows covered per instruction of the workgroup
+    const char* base;      // uniform: first element of the tile (row r0, k = 0)
+    int64_t step_bytes;    // uniform: global distance between consecutive instructions of a thread
+    int64_t k_bytes;       // uniform: global distance of one k step
+    uint32_t voff;         // per thread
+    uint32_t lds_off;      // uniform per wave: byte offset of this wave's first 1 KiB block in the tile
+    __device__ __forceinline__ DirectLoader(const Operand<T>& op, int r0) {
+        const int q = threadIdx.x, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const int row = q / CPR, slot = q % CPR;
+        if constexpr (KMAJOR) {
+            const int chunk = slot ^ ((row >> 2) & 3);
+            voff = (uint32_t)(((int64_t)row * op.sr + chunk * 8) * 2);
+            base = reinterpret_cast<const char*>(op.p + (int64_t)r0 * op.sr);
+            step_bytes = (int64_t)STEP * op.sr * 2;
+            k_bytes = 2;
+        } else {
+            const int r = (slot * 8) ^ ((row & 3) << mn_swizzle_shift(ROWS));   // row = k within the pass
+            voff = (uint32_t)(((int64_t)row * op.sk + r) * 2);
+            base = reinterpret_cast<const char*>(op.p + r0);
+            step_bytes = (int64_t)STEP * op.sk * 2;
+            k_bytes = op.sk * 2;
+        }
+        lds_off = (uint32_t)w * 1024u;
+    }
+    // stage starting at k0 -> tile at `lds_tile` (uniform)
+    __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
+        typedef __attribute__((address_space(3))) void* lds_vp;
+        typedef const __attribute__((address_space(1))) void* glb_vp;
+        const char* g = base + (int64_t)k0 * k_bytes;
+        char* l = reinterpret_cast<char*>(lds_tile) + lds_off;
+#pragma unroll
+        for (int i = 0; i < INSTR; ++i)
+            __builtin_amdgcn_global_load_lds((glb_vp)(g + i * step_bytes + voff), (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
     }
 };
 
@@ -162,15 +223,15 @@ __device__ __forceinline__ bf16x8_v load_frag_bf16(const bf16_t* lds, int rbase,
     if constexpr (KMAJOR) {
         const int r = rbase + (l & 31);
         const int chunk = 2 * kk + (l >> 5);
-        const u32x4_v v = *reinterpret_cast<const u32x4_v*>(lds + r * 64 + ((chunk ^ (r & 7)) << 3));
+        const u32x4_v v = *reinterpret_cast<const u32x4_v*>(lds + r * 32 + ((chunk ^ ((r >> 2) & 3)) << 3));
         return __builtin_bit_cast(bf16x8_v, v);
     } else {
-        constexpr int STRIDE = ROWS + GemmTraits<bf16_t>::PAD_MN;
+        constexpr int STRIDE = ROWS;
         const int b = l >> 4, s = l & 15;
         const int r = rbase + ((b & 1) << 4) + ((s & 3) << 2);
         const int k = kk * 16 + ((b >> 1) << 3) + (s >> 2);
         typedef __attribute__((address_space(3))) s16x4_v* lds_ptr;
-        const bf16_t* p0 = lds + k * STRIDE + r;
+        const bf16_t* p0 = lds + k * STRIDE + (r ^ ((k & 3) << mn_swizzle_shift(ROWS)));   // k and k+4 share the swizzle
         const s16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
         const s16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 4 * STRIDE));
         s16x8_v v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -211,22 +272,101 @@ __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, i
 // ----------------------------------------------------------------------------- mainloop
 // Accumulates the (2*WM*32) x (2*WN*32) tile at (m0, n0).  acc[wm][wn][r] of lane l belongs to
 //   m = m0 + wave_m*WM*32 + wm*32 + l%32,   n = n0 + wave_n*WN*32 + wn*32 + 8*(r/4) + 4*(l/32) + r%4.
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false>
+// NWN = waves along n (2 -> 4 waves per workgroup, 4 -> 8 waves); always 2 waves along m.
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false, int NWN = 2>
 struct GemmMainloop {
     using Tr = GemmTraits<T>;
-    static constexpr int TILE_M = 2 * WM * 32, TILE_N = 2 * WN * 32;
-    using PlainLoaderA = TileLoader<T, A_KMAJOR, TILE_M, FULL>;
-    using PlainLoaderB = TileLoader<T, B_KMAJOR, TILE_N, FULL>;
+    static constexpr int THREADS = 2 * NWN * 64;
+    static constexpr int TILE_M = 2 * WM * 32, TILE_N = NWN * WN * 32;
+    using PlainLoaderA = TileLoader<T, A_KMAJOR, TILE_M, FULL, THREADS>;
+    using PlainLoaderB = TileLoader<T, B_KMAJOR, TILE_N, FULL, THREADS>;
     static constexpr int A_ELEMS = lds_tile_elems<T, A_KMAJOR>(TILE_M);
     static constexpr int B_ELEMS = lds_tile_elems<T, B_KMAJOR>(TILE_N);
     static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
-    static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * sizeof(T);
+    static constexpr bool DIRECT = FULL && sizeof(T) == 2;     // global -> LDS without registers
+    static constexpr int NST = DIRECT ? 4 : 2;                  // LDS stages
+    static constexpr size_t LDS_BYTES = NST * (size_t)STAGE_ELEMS * sizeof(T);
 
     __device__ __forceinline__ static void run(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0, T* lds,
                                                f32x16_v (&acc)[WM][WN]) {
-        PlainLoaderA la(A, m0, K);
-        PlainLoaderB lb(B, n0, K);
-        run(la, lb, K, lds, acc);
+        if constexpr (FULL && sizeof(T) == 2) {
+            run_direct(A, B, K, m0, n0, lds, acc);
+        } else {
+            PlainLoaderA la(A, m0, K);
+            PlainLoaderB lb(B, n0, K);
+            run(la, lb, K, lds, acc);
+        }
+    }
+
+    __device__ __forceinline__ static void zero(f32x16_v (&acc)[WM][WN]) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    }
+
+    __device__ __forceinline__ static void compute_bf16(const bf16_t* As, const bf16_t* Bs, int wave_m, int wave_n,
+                                                        f32x16_v (&acc)[WM][WN]) {
+#pragma unroll
+        for (int kk = 0; kk < Tr::BK / 16; ++kk) {
+            bf16x8_v fa[WM], fb[WN];
+#pragma unroll
+            for (int i = 0; i < WM; ++i) fa[i] = load_frag_bf16<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kk);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) fb[j] = load_frag_bf16<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kk);
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // Whole aligned bf16 tiles: stages go from global memory straight into LDS (no staging
+    // registers, no ds_write).  NST LDS stages: while stage kt is consumed, stages kt+1 ..
+    // kt+NST-2 are in flight or landed and stage kt+NST-1 is issued into the buffer that stage
+    // kt-1 has just left.  One barrier per stage.
+    __device__ __forceinline__ static void run_direct(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0,
+                                                      T* lds, f32x16_v (&acc)[WM][WN]) {
+        const int w = threadIdx.x >> 6;
+        const int wave_m = (w & 1) * (WM * 32), wave_n = (w >> 1) * (WN * 32);
+        zero(acc);
+        using LA = DirectLoader<A_KMAJOR, TILE_M, THREADS>;
+        using LB = DirectLoader<B_KMAJOR, TILE_N, THREADS>;
+        LA la(A, m0);
+        LB lb(B, n0);
+        constexpr int IPS = LA::INSTR + LB::INSTR;               // load instructions per thread and stage
+        constexpr int PENDING = (NST - 2) * IPS;                 // loads of later stages that may stay in flight
+        static_assert(PENDING < 64, "vmcnt range");
+        // s_waitcnt vmcnt(PENDING) lgkmcnt(0): expcnt left at its maximum; lgkmcnt(0) retires this wave's
+        // LDS reads of the previous stage before the barrier lets other waves refill that buffer
+        constexpr int WAIT_IMM = (PENDING & 0xF) | (0x7 << 4) | ((PENDING >> 4) << 14);
+        const int KT = K / Tr::BK;
+#pragma unroll
+        for (int st = 0; st < NST - 1; ++st)
+            if (st < KT) {
+                la.issue(st * Tr::BK, lds + st * STAGE_ELEMS);
+                lb.issue(st * Tr::BK, lds + st * STAGE_ELEMS + A_ELEMS);
+            }
+        int cur = 0, fill = NST - 1;                             // buffer of stage kt, buffer to refill
+        for (int kt = 0; kt < KT; ++kt) {
+            if (kt + NST - 2 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+            else __builtin_amdgcn_s_waitcnt(0);                  // tail: fewer stages are in flight
+            // bare barrier: __syncthreads() would add a fence that drains every load in flight.
+            // This wave's share of stage kt has landed (wait above) and its LDS reads of stage
+            // kt-1 were consumed by MFMAs already, so nothing else has to be waited for.
+            __builtin_amdgcn_s_barrier();
+            if (kt + NST - 1 < KT) {
+                la.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS);
+                lb.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS + A_ELEMS);
+            }
+            const T* cb = lds + cur * STAGE_ELEMS;
+            compute_bf16(reinterpret_cast<const bf16_t*>(cb), reinterpret_cast<const bf16_t*>(cb + A_ELEMS), wave_m, wave_n, acc);
+            cur = cur + 1 == NST ? 0 : cur + 1;
+            fill = fill + 1 == NST ? 0 : fill + 1;
+        }
     }
 
     // k range [0, K) in stages of BK; the loaders decide what a stage contains

@@ -26,9 +26,9 @@ __device__ __forceinline__ float apply_act(int act, float x) {
     }
 }
 
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL>
-__global__ __launch_bounds__(kGemmThreads) void dense_gemm_kernel(DenseArgs<T> a) {
-    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL>;
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN>
+__global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
     int tm, tn;
@@ -47,12 +47,12 @@ __global__ __launch_bounds__(kGemmThreads) void dense_gemm_kernel(DenseArgs<T> a
     });
 }
 
-template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL>
+template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL, int NWN = 2>
 int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
-    using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL>;
+    using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL, NWN>;
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
-    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL>;
+    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL, NWN>;
     static bool attr_set = false;
     if (!attr_set) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -60,37 +60,46 @@ int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
         attr_set = true;
     }
     ProfScope ps(sizeof(T) == 2 ? "dense_gemm_kernel<bf16>" : "dense_gemm_kernel<f32>", s);
-    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(kGemmThreads), ML::LDS_BYTES, s>>>(a);
+    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }
 
 // whole, aligned tiles take the kernel variant without bounds checks (big tiles only)
-template <typename T, int WM, int WN, bool AK, bool BKM>
-int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
-    using ML = GemmMainloop<T, WM, WN, AK, BKM>;
-    if constexpr (WM * WN >= 4) {
-        const bool full = a.M % ML::TILE_M == 0 && a.N % ML::TILE_N == 0 && a.K % GemmTraits<T>::BK == 0 && a.K > 0 &&
-                          a.A.vec_ok && a.B.vec_ok &&
-                          256 * std::max(a.A.sr, a.A.sk) * (int64_t)sizeof(T) < (1ll << 31) &&
-                          256 * std::max(a.B.sr, a.B.sk) * (int64_t)sizeof(T) < (1ll << 31);
-        if (full) return launch_cfg_full<T, WM, WN, AK, BKM, true>(s, a);
-    }
-    return launch_cfg_full<T, WM, WN, AK, BKM, false>(s, a);
+template <typename T, int TILE_M, int TILE_N>
+bool whole_tiles(const DenseArgs<T>& a) {
+    return a.M % TILE_M == 0 && a.N % TILE_N == 0 && a.K % GemmTraits<T>::BK == 0 && a.K > 0 && a.A.vec_ok && a.B.vec_ok &&
+           256 * std::max(a.A.sr, a.A.sk) * (int64_t)sizeof(T) < (1ll << 31) &&
+           256 * std::max(a.B.sr, a.B.sk) * (int64_t)sizeof(T) < (1ll << 31);
 }
 
-int gemm_tile_override();   // gemm.hip: LUXHIP_GEMM_TILE=42|22|11 forces a tile (tuning aid), 0 = automatic
+template <typename T, int WM, int WN, bool AK, bool BKM, int NWN = 2>
+int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
+    using ML = GemmMainloop<T, WM, WN, AK, BKM, false, NWN>;
+    if constexpr (WM * WN >= 4) {
+        if (whole_tiles<T, ML::TILE_M, ML::TILE_N>(a)) return launch_cfg_full<T, WM, WN, AK, BKM, true, NWN>(s, a);
+    }
+    return launch_cfg_full<T, WM, WN, AK, BKM, false, NWN>(s, a);
+}
+
+int gemm_tile_override();   // gemm.hip: LUXHIP_GEMM_TILE=82|42|22|11 forces a tile (tuning aid), 0 = automatic
 
 template <typename T, bool AK, bool BKM>
 int launch_layout(hipStream_t s, DenseArgs<T>& a) {
     switch (gemm_tile_override()) {
+        case 82: return launch_cfg<T, 4, 2, AK, BKM, 4>(s, a);   // 8 waves, 256 x 256
         case 42: return launch_cfg<T, 4, 2, AK, BKM>(s, a);
         case 22: return launch_cfg<T, 2, 2, AK, BKM>(s, a);
         case 11: return launch_cfg<T, 1, 1, AK, BKM>(s, a);
         default: break;
     }
-    // 128 x 128 tiles (two workgroups per compute unit) measured fastest on large problems;
-    // 64 x 64 for small ones
+    // bf16 problems of whole 256 x 256 tiles that fill the chip: eight waves, operands streamed
+    // straight into LDS.  Otherwise 128 x 128 tiles (two workgroups per compute unit) measured
+    // fastest on large problems; 64 x 64 for small ones.
+    if constexpr (sizeof(T) == 2) {
+        if (whole_tiles<T, 256, 256>(a) && (int64_t)(a.M / 256) * (a.N / 256) >= 128)
+            return launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, a);
+    }
     const int64_t t128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
     if (a.M > 64 && a.N > 64 && t128 >= 4) return launch_cfg<T, 2, 2, AK, BKM>(s, a);
     return launch_cfg<T, 1, 1, AK, BKM>(s, a);
