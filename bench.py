@@ -137,7 +137,8 @@ class C2BatchnormBiasAct(Workload):
 
     def kernel_work(self):
         E = self.E
-        return {"bn_stats_kernel": 1 * E, "bn_apply_kernel": 2 * E, "bias_act_fwd_kernel": 2 * E,
+        return {"bn_fwd_resident_kernel": 2 * E, "bn_bwd_resident_kernel": 3 * E,
+                "bn_stats_kernel": 1 * E, "bn_apply_kernel": 2 * E, "bias_act_fwd_kernel": 2 * E,
                 "bias_act_bwd_channel_kernel": 3 * E, "bn_bwd_reduce_kernel": 2 * E, "bn_bwd_apply_kernel": 3 * E}
 
     def cpu_baseline(self, budget_s: float):
@@ -360,6 +361,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline (0 disables it)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library tuning switch (luxhip_set_option), e.g. bn_resident=0; may be repeated")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path is single-GPU; no collective is part of it); "
@@ -368,6 +371,9 @@ def main():
 
     lux = load_package()
     lux.init(0)
+    for opt in args.option:
+        name, _, val = opt.partition("=")
+        lux.set_option(name, int(val))
     wl = WORKLOADS[args.workload]()
     heavy = args.workload in ("C4", "C5", "C5bf16")
     if args.steps is None:
@@ -407,7 +413,7 @@ def main():
         "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype,
         "data": "synthetic", "config": {"workload": f"{wl.name}: {wl.description}"},
-        "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
+        "options": args.option, "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
         "ms_per_step_host_clock": round(ms_wall, 5), "roofline": roofline, "kernels": kernels,
     }
     if hasattr(wl, "step_fused"):

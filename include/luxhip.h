@@ -81,6 +81,12 @@ int luxhip_event_destroy(luxhip_event_t e);
  * luxhip_profile_report synchronises, writes a JSON array of {kernel, count, total_ms, min_ms,
  * max_ms} into buf and clears the log. */
 int luxhip_profile_enable(int on);
+/* Tuning switches (no counterpart in LuxLib; tests use them to reach every code path):
+ *   "bn_resident"   1 (default) / 0: single-pass batchnorm kernels that keep the tensor in registers
+ *   "bn_spin_limit" polls after which a resident batchnorm workgroup stops waiting for its peer
+ *                   workgroups and recomputes their share itself (default 2^22; 0 = never wait)
+ *   "gemm_tile"     0 automatic (default), 82 | 42 | 22 | 11 force a GEMM tile shape */
+int luxhip_set_option(const char* name, int64_t value);
 int luxhip_profile_report(char* buf, size_t len);
 
 /* Pooled device allocator (size-bucketed free lists; luxhip_free returns the block to the

@@ -37,6 +37,11 @@ def init(device: int = 0, own_stream: bool = True):
     _initialised = True
 
 
+def set_option(name: str, value: int):
+    """Tuning switch of the library (luxhip_set_option): "bn_resident", "bn_spin_limit", "gemm_tile"."""
+    _lib.call("luxhip_set_option", name.encode(), int(value))
+
+
 def synchronize():
     _lib.call("luxhip_stream_synchronize", current_stream())
 

@@ -52,6 +52,7 @@ SIGNATURES = {
     "luxhip_event_destroy": [_vp],
     "luxhip_profile_enable": [_i],
     "luxhip_profile_report": [C.c_char_p, _sz],
+    "luxhip_set_option": [C.c_char_p, _i64],
     "luxhip_malloc": [C.POINTER(_vp), _sz],
     "luxhip_free": [_vp],
     "luxhip_trim": [],

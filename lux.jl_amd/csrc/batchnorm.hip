@@ -2,20 +2,27 @@
 // pullback, as HBM-bound streaming kernels over the (I, C, N) view.
 //
 // Channel c owns the rows (n*C + c)*I .. +I for every n.  Reduction kernels use a (S, C)
-// grid: workgroup (s, c) streams a contiguous slice of channel c's I*N elements and writes one
-// partial; a one-wave-per-channel finalize kernel combines the S partials in a fixed order
-// (deterministic, no floating-point atomics, no device-wide fences inside the streaming
-// kernels: an agent-scope fence per workgroup writes back the L2 and costs far more than the
-// extra launch) and writes the per-channel results.
+// grid: workgroup (s, c) works on a contiguous slice of channel c's I*N elements and publishes
+// one partial result; partials are always combined in slice order, so results do not depend on
+// scheduling.  No floating-point atomics and no cache-wide fences (see common.h, cross-workgroup
+// hand-off).
 //
-//   forward, training : bn_stats_kernel (read x) -> partials
-//                       bn_stats_finalize_kernel -> mean, invstd, scale, shift, running stats
+// Resident path (tensor fits the register file: C*S <= compute units, slice <= 8 vectors per
+// thread of a 1024-thread workgroup), one kernel and one trip through HBM per tensor:
+//   forward : bn_fwd_resident_kernel  load x -> slice statistics -> publish, wait for the other
+//             slices of the channel -> mean/invstd (+ running stats, saved stats) -> write y
+//   pullback: bn_bwd_resident_kernel  load delta, x -> slice sums -> publish, wait -> dgamma, dbeta
+//             -> write dx
+//   All workgroups of the grid are resident at once (one per compute unit), so the wait ends as
+//   soon as the slowest peer has published.  The wait is bounded all the same: a workgroup that
+//   gives up recomputes the peers' partials itself from global memory.
+// Streaming path (any size):
+//   forward, training : bn_stats_kernel (read x) -> partials; the workgroup of a channel that
+//                       arrives last combines them -> mean, invstd, scale, shift, running stats
 //                       bn_apply_kernel  (read x, write y)
-//   forward, inference: bn_infer_prep_kernel (C threads) -> scale, shift
-//                       bn_apply_kernel
-//   pullback          : bn_bwd_reduce_kernel (read delta, x) -> partials
-//                       bn_bwd_finalize_kernel -> dgamma, dbeta, per-channel coefficients
-//                       bn_bwd_apply_kernel  (read delta, x, write dx)
+//   forward, inference: bn_infer_prep_kernel (C threads) -> scale, shift;  bn_apply_kernel
+//   pullback          : bn_bwd_reduce_kernel (read delta, x) -> partials; last arriver -> dgamma,
+//                       dbeta, per-channel coefficients;  bn_bwd_apply_kernel (read delta, x, write dx)
 #include <algorithm>
 
 #include "common.h"
@@ -60,18 +67,62 @@ __device__ __forceinline__ void chan_merge(float& n, float& mean, float& m2, flo
 }
 
 // ------------------------------------------------------------------------------- statistics
+struct BnFwdParams {
+    const void *gamma, *beta, *rmean, *rvar;   // storage type T
+    void *rmean_out, *rvar_out;                // NULL: running statistics are not updated
+    float *save_mean, *save_invstd;            // may be NULL
+    float count, momentum, eps;
+};
+
+// Wave-wide: combines S partial (count, mean, M2) triples read through `get(i, k)` in a fixed
+// tree order; lane 0 holds the result.
+template <typename Get>
+__device__ __forceinline__ void merge_stat_partials(uint32_t S, Get get, float& n, float& mean, float& m2) {
+    const uint32_t lane = threadIdx.x & 63;
+    n = 0.0f; mean = 0.0f; m2 = 0.0f;
+    for (uint32_t i = lane; i < S; i += kWave) chan_merge(n, mean, m2, get(i, 0), get(i, 1), get(i, 2));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float nb = __shfl_xor(n, off, kWave), mb = __shfl_xor(mean, off, kWave), qb = __shfl_xor(m2, off, kWave);
+        chan_merge(n, mean, m2, nb, mb, qb);
+    }
+}
+
+// One thread: every per-channel result of the forward pass from the channel's (mean, M2).
+template <typename T>
+__device__ __forceinline__ void bn_fwd_channel_results(const BnFwdParams& p, uint32_t c, float mean, float m2,
+                                                       float* scale, float* shift, float& sc, float& sh) {
+    const T* gamma = static_cast<const T*>(p.gamma);
+    const T* beta = static_cast<const T*>(p.beta);
+    const float var = m2 / p.count;
+    const float invstd = 1.0f / sqrtf(var + p.eps);
+    sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
+    sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+    if (scale) { scale[c] = sc; shift[c] = sh; }
+    if (p.save_mean) p.save_mean[c] = mean;
+    if (p.save_invstd) p.save_invstd[c] = invstd;
+    if (p.rmean_out) {
+        const float m1 = p.momentum, m3 = 1.0f - p.momentum;
+        const float m2c = p.momentum * p.count / (p.count - 1.0f);
+        st(static_cast<T*>(p.rmean_out) + c, m3 * ld(static_cast<const T*>(p.rmean) + c) + m1 * mean);
+        st(static_cast<T*>(p.rvar_out) + c, m3 * ld(static_cast<const T*>(p.rvar) + c) + m2c * var);
+    }
+}
+
 // Partial (count, mean, M2) of slice s of channel c -> partial[(c*S + s)*3 ..].  A workgroup
-// keeps its slice (up to kStatVecs vectors per thread) in registers and makes two passes over
-// the registers: workgroup mean, then the sum of squared deviations from it (exact two-pass
-// statistics per slice; slices are combined with Chan's formula by the finalize kernel).
+// keeps its slice (up to kStatVecs vectors per thread per trip) in registers and makes two
+// passes over the registers: workgroup mean, then the sum of squared deviations from it (exact
+// two-pass statistics per trip; trips and slices are combined with Chan's formula).
 constexpr int kStatVecs = 4;
 template <typename T, int VEC>
-__global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(const T* __restrict__ x, float* partial, ChanGeom g) {
+__global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(const T* __restrict__ x, float* partial, uint32_t* counters,
+                                                              uint32_t cstride, float* scale, float* shift,
+                                                              BnFwdParams prm, ChanGeom g) {
     __shared__ float sm[kBnThreads / 64];
+    __shared__ uint32_t last_flag;
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     const uint32_t q0 = s * g.chunk, q1 = min(q0 + g.chunk, g.nq);
-    const float cnt = (float)((q1 - q0) * VEC);
-    float n = 0.0f, mean = 0.0f, m2 = 0.0f;   // running (count, mean, M2) over the passes of the outer loop
+    float n = 0.0f, mean = 0.0f, m2 = 0.0f;   // running (count, mean, M2) over the trips of the outer loop
     for (uint32_t base = q0; base < q1; base += kBnThreads * kStatVecs) {
         float v[kStatVecs][VEC];
         bool ok[kStatVecs];
@@ -101,45 +152,19 @@ __global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(const T* __restric
         const float m2b = block_sum(dev, sm);
         chan_merge(n, mean, m2, nb, mb, m2b);
     }
-    (void)cnt;
+    float* mine = partial + ((size_t)c * S + s) * 3;
     if (threadIdx.x == 0) {
-        float* p = partial + ((size_t)c * S + s) * 3;
-        p[0] = n; p[1] = mean; p[2] = m2;
+        publish(mine, n);
+        publish(mine + 1, mean);
+        publish(mine + 2, m2);
+        publish_done();
     }
-}
-
-// One wave per channel merges the S partials (fixed tree order) and writes every per-channel
-// result of the forward pass.  S <= kBnThreads.
-template <typename T>
-__global__ __launch_bounds__(kWave) void bn_stats_finalize_kernel(
-    const float* __restrict__ partial, uint32_t S, const T* __restrict__ gamma, const T* __restrict__ beta,
-    const T* __restrict__ rmean, const T* __restrict__ rvar, T* rmean_out, T* rvar_out, float* save_mean,
-    float* save_invstd, float* scale, float* shift, float count, float momentum, float eps) {
-    const uint32_t c = blockIdx.x;
-    const float* p = partial + (size_t)c * S * 3;
-    float n = 0.0f, mean = 0.0f, m2 = 0.0f;
-    for (uint32_t i = threadIdx.x; i < S; i += kWave) chan_merge(n, mean, m2, p[3 * i], p[3 * i + 1], p[3 * i + 2]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float nb = __shfl_xor(n, off, kWave), mb = __shfl_xor(mean, off, kWave), qb = __shfl_xor(m2, off, kWave);
-        chan_merge(n, mean, m2, nb, mb, qb);
-    }
-    if (threadIdx.x == 0) {
-        const float var = m2 / count;
-        const float invstd = 1.0f / sqrtf(var + eps);
-        const float gm = gamma ? ld(gamma + c) : 1.0f;
-        const float bt = beta ? ld(beta + c) : 0.0f;
-        const float sc = gm * invstd;
-        scale[c] = sc;
-        shift[c] = fmaf(-mean, sc, bt);
-        if (save_mean) save_mean[c] = mean;
-        if (save_invstd) save_invstd[c] = invstd;
-        if (rmean_out) {
-            const float m1 = momentum, m3 = 1.0f - momentum;
-            const float m2c = momentum * count / (count - 1.0f);
-            st(rmean_out + c, m3 * ld(rmean + c) + m1 * mean);
-            st(rvar_out + c, m3 * ld(rvar + c) + m2c * var);
-        }
+    if (!arrive_last(counters + (size_t)c * cstride, S, &last_flag)) return;
+    if (threadIdx.x < kWave) {
+        const float* p = partial + (size_t)c * S * 3;
+        merge_stat_partials(S, [&](uint32_t i, int k) { return fetch(p + 3 * i + k); }, n, mean, m2);
+        float sc, sh;
+        if (threadIdx.x == 0) bn_fwd_channel_results<T>(prm, c, mean, m2, scale, shift, sc, sh);
     }
 }
 
@@ -189,12 +214,30 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const T* __restric
 }
 
 // ------------------------------------------------------------------------------- pullback
-// Partials of s1 = sum dy and s2 = sum dy * (x - mean) * invstd, dy = delta * act'(recomputed).
+// One thread: dgamma, dbeta and the coefficients of dx = A*dy + B*(x - mean) + D from the
+// channel sums s1 = sum dy, s2 = sum dy * xhat.
+template <typename T>
+__device__ __forceinline__ void bn_bwd_channel_results(uint32_t c, float s1, float s2, const T* gamma, float invstd,
+                                                       T* dgamma, T* dbeta, float inv_count, int stats_from_batch,
+                                                       float& A, float& B, float& D) {
+    const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
+    if (dgamma) st(dgamma + c, s2);
+    if (dbeta) st(dbeta + c, s1);
+    A = sc;
+    B = stats_from_batch ? -sc * invstd * s2 * inv_count : 0.0f;
+    D = stats_from_batch ? -sc * s1 * inv_count : 0.0f;
+}
+
+// Partials of s1 = sum dy and s2 = sum dy * (x - mean) * invstd, dy = delta * act'(recomputed);
+// the workgroup of a channel that arrives last adds them in slice order and writes dgamma, dbeta
+// and coef[c], coef[C + c], coef[2C + c] = A, B, D.
 template <typename T, int ACT, int VEC>
 __global__ __launch_bounds__(kBnThreads) void bn_bwd_reduce_kernel(
     const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
-    const float* __restrict__ save_mean, const float* __restrict__ save_invstd, float* partial, ChanGeom g) {
+    const float* __restrict__ save_mean, const float* __restrict__ save_invstd, float* partial, uint32_t* counters,
+    uint32_t cstride, T* dgamma, T* dbeta, float* coef, float inv_count, int stats_from_batch, ChanGeom g) {
     __shared__ float sm[kBnThreads / 64];
+    __shared__ uint32_t last_flag;
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     const uint32_t q0 = s * g.chunk, q1 = min(q0 + g.chunk, g.nq);
     const float mean = save_mean[c], invstd = save_invstd[c];
@@ -232,32 +275,24 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_reduce_kernel(
     s1 = block_sum(s1, sm);
     s2 = block_sum(s2, sm);
     if (threadIdx.x == 0) {
-        partial[((size_t)c * S + s) * 2] = s1;
-        partial[((size_t)c * S + s) * 2 + 1] = s2;
+        publish(partial + ((size_t)c * S + s) * 2, s1);
+        publish(partial + ((size_t)c * S + s) * 2 + 1, s2);
+        publish_done();
     }
-}
-
-// One wave per channel: dgamma, dbeta and the coefficients of dx = A*dy + B*(x - mean) + D.
-template <typename T>
-__global__ __launch_bounds__(kWave) void bn_bwd_finalize_kernel(const float* __restrict__ partial, uint32_t S,
-                                                                const T* __restrict__ gamma,
-                                                                const float* __restrict__ save_invstd, T* dgamma,
-                                                                T* dbeta, float* coef, uint32_t C, float inv_count,
-                                                                int stats_from_batch) {
-    const uint32_t c = blockIdx.x;
-    const float* p = partial + (size_t)c * S * 2;
-    float t1 = 0.0f, t2 = 0.0f;
-    for (uint32_t i = threadIdx.x; i < S; i += kWave) { t1 += p[2 * i]; t2 += p[2 * i + 1]; }
-    t1 = wave_sum(t1);
-    t2 = wave_sum(t2);
-    if (threadIdx.x == 0) {
-        const float invstd = save_invstd[c];
-        const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
-        if (dgamma) st(dgamma + c, t2);
-        if (dbeta) st(dbeta + c, t1);
-        coef[c] = sc;
-        coef[C + c] = stats_from_batch ? -sc * invstd * t2 * inv_count : 0.0f;
-        coef[2 * C + c] = stats_from_batch ? -sc * t1 * inv_count : 0.0f;
+    if (!arrive_last(counters + (size_t)c * cstride, S, &last_flag)) return;
+    if (threadIdx.x < kWave) {
+        const float* p = partial + (size_t)c * S * 2;
+        float t1 = 0.0f, t2 = 0.0f;
+        for (uint32_t i = threadIdx.x; i < S; i += kWave) { t1 += fetch(p + 2 * i); t2 += fetch(p + 2 * i + 1); }
+        t1 = wave_sum(t1);
+        t2 = wave_sum(t2);
+        if (threadIdx.x == 0) {
+            float A, B, D;
+            bn_bwd_channel_results<T>(c, t1, t2, gamma, invstd, dgamma, dbeta, inv_count, stats_from_batch, A, B, D);
+            coef[c] = A;
+            coef[g.C + c] = B;
+            coef[2 * g.C + c] = D;
+        }
     }
 }
 
@@ -304,6 +339,263 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const T* __res
     }
 }
 
+// ------------------------------------------------------------------------------- resident path
+constexpr int kResThreads = 1024;   // one workgroup per compute unit
+constexpr int kResVecs = 8;         // 16-byte vectors per thread held in registers
+constexpr int kResMaxSlices = 256;
+
+// Slice `slice` of channel c -> registers.  Vector u of a thread is vector q0 + u*1024 + tid of
+// the slice; loads past the end of the slice are redirected to its last vector (every load is
+// unconditional, so all of them are in flight together) and ignored by the users of v.
+template <typename T>
+__device__ __forceinline__ void res_load(const T* __restrict__ p, const ChanGeom& g, uint32_t c, uint32_t slice,
+                                         raw16_t (&v)[kResVecs]) {
+    constexpr int VEC = Vec<T>::N;
+    const uint32_t q0 = slice * g.chunk, q1 = min(q0 + g.chunk, g.nq);
+#pragma unroll
+    for (int u = 0; u < kResVecs; ++u) {
+        const uint32_t q = min(q0 + u * kResThreads + threadIdx.x, q1 - 1);
+        v[u] = *reinterpret_cast<const raw16_t*>(p + g.offset(q, c, VEC));
+    }
+}
+
+// Exact two-pass (count, mean, M2) of the slice held in v; every thread receives the result.
+template <typename T>
+__device__ __forceinline__ void res_slice_stats(const ChanGeom& g, uint32_t slice, const raw16_t (&v)[kResVecs],
+                                                float* sm, float& n, float& mean, float& m2) {
+    constexpr int VEC = Vec<T>::N;
+    const uint32_t q0 = slice * g.chunk, q1 = min(q0 + g.chunk, g.nq);
+    float sum = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kResVecs; ++u)
+        if (q0 + u * kResThreads + threadIdx.x < q1) {
+            float f[VEC];
+            Vec<T>::unpack(v[u], f);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum += f[k];
+        }
+    n = (float)((q1 - q0) * VEC);
+    mean = block_sum(sum, sm) / n;
+    float dev = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kResVecs; ++u)
+        if (q0 + u * kResThreads + threadIdx.x < q1) {
+            float f[VEC];
+            Vec<T>::unpack(v[u], f);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) dev = fmaf(f[k] - mean, f[k] - mean, dev);
+        }
+    m2 = block_sum(dev, sm);
+}
+
+// Wave 0 polls the S flags of channel c until they show `epoch`; false for the whole workgroup
+// if any poll loop ran out of tries.  Contains a workgroup barrier.
+__device__ __forceinline__ bool res_wait_peers(const uint32_t* flags, uint32_t S, uint32_t epoch, uint32_t spin_limit,
+                                               uint32_t* lds_ok) {
+    if (threadIdx.x < kWave) {
+        bool ok = true;
+        for (uint32_t i = threadIdx.x; i < S; i += kWave) {
+            uint32_t tries = 0;
+            while (fetch(flags + i) != epoch) {
+                if (tries++ >= spin_limit) { ok = false; break; }
+                __builtin_amdgcn_s_sleep(4);
+            }
+        }
+        const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+        if (threadIdx.x == 0) *lds_ok = all_ok ? 1u : 0u;
+    }
+    __syncthreads();
+    return *lds_ok != 0u;
+}
+
+template <typename T, int ACT>
+__global__ __launch_bounds__(kResThreads) void bn_fwd_resident_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                      float* partial, uint32_t* flags, uint32_t epoch,
+                                                                      uint32_t spin_limit, BnFwdParams prm, ChanGeom g) {
+    constexpr int VEC = Vec<T>::N;
+    __shared__ float sm[kResThreads / 64];
+    __shared__ float parts[kResMaxSlices * 3];
+    __shared__ float bc[2];
+    __shared__ uint32_t lds_ok;
+    const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
+    raw16_t v[kResVecs];
+    res_load<T>(x, g, c, s, v);
+    float n, mean, m2;
+    res_slice_stats<T>(g, s, v, sm, n, mean, m2);
+    float* chan_part = partial + (size_t)c * S * 3;
+    uint32_t* chan_flags = flags + (size_t)c * S;
+    if (threadIdx.x == 0) {
+        publish(chan_part + 3 * s, n);
+        publish(chan_part + 3 * s + 1, mean);
+        publish(chan_part + 3 * s + 2, m2);
+        publish_done();
+        publish(chan_flags + s, epoch);
+    }
+    if (res_wait_peers(chan_flags, S, epoch, spin_limit, &lds_ok)) {
+        for (uint32_t i = threadIdx.x; i < 3 * S; i += kResThreads) parts[i] = fetch(chan_part + i);
+    } else {
+        // a peer did not show up in time: its share is recomputed here, the own slice last so
+        // that v holds it again afterwards
+        for (uint32_t i = 0; i <= S; ++i) {
+            const uint32_t slice = i < S ? i : s;
+            __syncthreads();
+            res_load<T>(x, g, c, slice, v);
+            res_slice_stats<T>(g, slice, v, sm, n, mean, m2);
+            if (threadIdx.x == 0 && i < S) { parts[3 * i] = n; parts[3 * i + 1] = mean; parts[3 * i + 2] = m2; }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < kWave) {
+        merge_stat_partials(S, [&](uint32_t i, int k) { return parts[3 * i + k]; }, n, mean, m2);
+        if (threadIdx.x == 0) {
+            float sc, sh;
+            BnFwdParams q = prm;
+            if (s != 0) { q.save_mean = nullptr; q.save_invstd = nullptr; q.rmean_out = nullptr; }  // slice 0 writes
+            bn_fwd_channel_results<T>(q, c, mean, m2, nullptr, nullptr, sc, sh);
+            bc[0] = sc;
+            bc[1] = sh;
+        }
+    }
+    __syncthreads();
+    const float sc = bc[0], sh = bc[1];
+    const uint32_t q0 = s * g.chunk, q1 = min(q0 + g.chunk, g.nq);
+#pragma unroll
+    for (int u = 0; u < kResVecs; ++u) {
+        const uint32_t q = q0 + u * kResThreads + threadIdx.x;
+        if (q < q1) {
+            float f[VEC];
+            Vec<T>::unpack(v[u], f);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) f[k] = Act<ACT>::f(fmaf(f[k], sc, sh));
+            *reinterpret_cast<raw16_t*>(y + g.offset(q, c, VEC)) = Vec<T>::pack(f);
+        }
+    }
+}
+
+// dy of the slice in place of delta (d), slice sums s1 = sum dy, s2 = sum dy * xhat.
+template <typename T, int ACT>
+__device__ __forceinline__ void res_bwd_slice_sums(const ChanGeom& g, uint32_t slice, raw16_t (&d)[kResVecs],
+                                                   const raw16_t (&v)[kResVecs], float mean, float invstd, float sc,
+                                                   float sh, float* sm, float& s1, float& s2) {
+    constexpr int VEC = Vec<T>::N;
+    const uint32_t q0 = slice * g.chunk, q1 = min(q0 + g.chunk, g.nq);
+    s1 = 0.0f;
+    s2 = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kResVecs; ++u)
+        if (q0 + u * kResThreads + threadIdx.x < q1) {
+            float fd[VEC], fx[VEC];
+            Vec<T>::unpack(d[u], fd);
+            Vec<T>::unpack(v[u], fx);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float dy = fd[k];
+                if constexpr (ACT != LUXHIP_ACT_IDENTITY) {
+                    const float pre = fmaf(fx[k], sc, sh);
+                    dy *= Act<ACT>::d(Act<ACT>::f(pre), pre);
+                }
+                s1 += dy;
+                s2 = fmaf(dy, (fx[k] - mean) * invstd, s2);
+            }
+        }
+    s1 = block_sum(s1, sm);
+    s2 = block_sum(s2, sm);
+}
+
+template <typename T, int ACT>
+__global__ __launch_bounds__(kResThreads) void bn_bwd_resident_kernel(
+    const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
+    const float* __restrict__ save_mean, const float* __restrict__ save_invstd, T* __restrict__ dx, T* dgamma, T* dbeta,
+    float* partial, uint32_t* flags, uint32_t epoch, uint32_t spin_limit, float inv_count, int stats_from_batch,
+    ChanGeom g) {
+    constexpr int VEC = Vec<T>::N;
+    __shared__ float sm[kResThreads / 64];
+    __shared__ float parts[kResMaxSlices * 2];
+    __shared__ float bc[3];
+    __shared__ uint32_t lds_ok;
+    const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
+    const float mean = save_mean[c], invstd = save_invstd[c];
+    const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
+    const float sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+    raw16_t d[kResVecs], v[kResVecs];
+    res_load<T>(delta, g, c, s, d);
+    res_load<T>(x, g, c, s, v);
+    float s1, s2;
+    res_bwd_slice_sums<T, ACT>(g, s, d, v, mean, invstd, sc, sh, sm, s1, s2);
+    float* chan_part = partial + (size_t)c * S * 2;
+    uint32_t* chan_flags = flags + (size_t)c * S;
+    if (threadIdx.x == 0) {
+        publish(chan_part + 2 * s, s1);
+        publish(chan_part + 2 * s + 1, s2);
+        publish_done();
+        publish(chan_flags + s, epoch);
+    }
+    if (res_wait_peers(chan_flags, S, epoch, spin_limit, &lds_ok)) {
+        for (uint32_t i = threadIdx.x; i < 2 * S; i += kResThreads) parts[i] = fetch(chan_part + i);
+    } else {
+        for (uint32_t i = 0; i <= S; ++i) {   // recompute the peers' sums; own slice last (d, v restored)
+            const uint32_t slice = i < S ? i : s;
+            __syncthreads();
+            res_load<T>(delta, g, c, slice, d);
+            res_load<T>(x, g, c, slice, v);
+            res_bwd_slice_sums<T, ACT>(g, slice, d, v, mean, invstd, sc, sh, sm, s1, s2);
+            if (threadIdx.x == 0 && i < S) { parts[2 * i] = s1; parts[2 * i + 1] = s2; }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < kWave) {
+        float t1 = 0.0f, t2 = 0.0f;
+        for (uint32_t i = threadIdx.x; i < S; i += kWave) { t1 += parts[2 * i]; t2 += parts[2 * i + 1]; }
+        t1 = wave_sum(t1);
+        t2 = wave_sum(t2);
+        if (threadIdx.x == 0) {
+            float A, B, D;
+            bn_bwd_channel_results<T>(c, t1, t2, gamma, invstd, s == 0 ? dgamma : nullptr, s == 0 ? dbeta : nullptr,
+                                      inv_count, stats_from_batch, A, B, D);
+            bc[0] = A; bc[1] = B; bc[2] = D;
+        }
+    }
+    __syncthreads();
+    const float A = bc[0], B = bc[1], D = bc[2];
+    const uint32_t q0 = s * g.chunk, q1 = min(q0 + g.chunk, g.nq);
+#pragma unroll
+    for (int u = 0; u < kResVecs; ++u) {
+        const uint32_t q = q0 + u * kResThreads + threadIdx.x;
+        if (q < q1) {
+            float fd[VEC], fx[VEC], o[VEC];
+            Vec<T>::unpack(d[u], fd);
+            Vec<T>::unpack(v[u], fx);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float dy = fd[k];
+                if constexpr (ACT != LUXHIP_ACT_IDENTITY) {
+                    const float pre = fmaf(fx[k], sc, sh);
+                    dy *= Act<ACT>::d(Act<ACT>::f(pre), pre);
+                }
+                o[k] = fmaf(A, dy, fmaf(B, fx[k] - mean, D));
+            }
+            *reinterpret_cast<raw16_t*>(dx + g.offset(q, c, VEC)) = Vec<T>::pack(o);
+        }
+    }
+}
+
+// Slices per channel for the resident path, 0 if the tensor does not qualify.
+static int64_t resident_slices(int64_t I, int64_t C, int64_t N, int vec, bool aligned) {
+    if (!option_bn_resident() || !aligned || I % vec != 0) return 0;
+    const int64_t cus = num_cus();
+    if (C > cus) return 0;
+    const int64_t nq = I * N / vec;
+    const int64_t per_wg = (int64_t)kResThreads * kResVecs;
+    const int64_t s_need = ceil_div(nq, per_wg);
+    const int64_t s_max = std::min<int64_t>(cus / C, kResMaxSlices);
+    if (s_need > s_max) return 0;
+    // as many slices as fit (more compute units busy) while a slice keeps at least one vector per thread
+    int64_t S = std::min<int64_t>(s_max, std::max<int64_t>(s_need, nq / kResThreads));
+    if (S < 1) S = 1;
+    if ((size_t)(C * S) > kWorkspaceFlags) return 0;
+    return S;
+}
+
 // ------------------------------------------------------------------------------- host side
 static ChanGeom make_geom(int64_t I, int64_t C, int64_t N, int vec, int64_t* S_out) {
     ChanGeom g;
@@ -343,6 +635,39 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     const bool vec = aligned16(x) && aligned16(y) && I % V == 0;
     const int vv = vec ? V : 1;
     const bool batch_stats = training || rmean == nullptr;
+    const bool upd = training && rmean != nullptr;
+    BnFwdParams prm;
+    prm.gamma = gamma; prm.beta = beta; prm.rmean = rmean; prm.rvar = rvar;
+    prm.rmean_out = upd ? rmean_out : nullptr;
+    prm.rvar_out = upd ? rvar_out : nullptr;
+    prm.save_mean = save_mean; prm.save_invstd = save_invstd;
+    prm.count = (float)(I * N); prm.momentum = momentum; prm.eps = eps;
+
+    const int64_t SR = batch_stats ? resident_slices(I, C, N, V, vec) : 0;
+    if (SR > 0) {
+        ChanGeom g;
+        g.nq = (uint32_t)(I * N / V);
+        g.vec_per_row = (uint32_t)(I / V);
+        g.C = (uint32_t)C;
+        g.rowdiv = FastDiv(g.vec_per_row);
+        g.chunk = (uint32_t)ceil_div(g.nq, SR);
+        const int64_t S = ceil_div(g.nq, g.chunk);
+        Workspace ws;
+        int rc = get_workspace(s, (size_t)C * 3 * S * sizeof(float), &ws);
+        if (rc != LUXHIP_OK) return rc;
+        float* partial = reinterpret_cast<float*>(ws.data);
+        const uint32_t spin = (uint32_t)option_bn_spin_limit();
+        dim3 grid((unsigned)S, (unsigned)C);
+#define LAUNCH_RES(A) bn_fwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(x, y, partial, ws.flags, ws.epoch, spin, prm, g)
+        {
+            ProfScope ps("bn_fwd_resident_kernel", s);
+            LUX_DISPATCH_ACT(act, LAUNCH_RES);
+        }
+#undef LAUNCH_RES
+        LUX_CHECK_LAUNCH();
+        return LUXHIP_OK;
+    }
+
     int64_t S = 1;
     ChanGeom g = make_geom(I, C, N, vv, &S);
     Workspace ws;
@@ -352,19 +677,10 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     float* shift = scale + C;
     float* partial = shift + C;
     if (batch_stats) {
-        const bool upd = training && rmean != nullptr;
         dim3 grid((unsigned)S, (unsigned)C);
-        {
-            ProfScope ps("bn_stats_kernel", s);
-            if (vec) bn_stats_kernel<T, V><<<grid, kBnThreads, 0, s>>>(x, partial, g);
-            else bn_stats_kernel<T, 1><<<grid, kBnThreads, 0, s>>>(x, partial, g);
-        }
-        LUX_CHECK_LAUNCH();
-        ProfScope ps("bn_stats_finalize_kernel", s);
-        bn_stats_finalize_kernel<T><<<(unsigned)C, kWave, 0, s>>>(partial, (uint32_t)S, gamma, beta, rmean, rvar,
-                                                                 upd ? rmean_out : nullptr, upd ? rvar_out : nullptr,
-                                                                 save_mean, save_invstd, scale, shift, (float)(I * N),
-                                                                 momentum, eps);
+        ProfScope ps("bn_stats_kernel", s);
+        if (vec) bn_stats_kernel<T, V><<<grid, kBnThreads, 0, s>>>(x, partial, ws.counters, counter_stride(C), scale, shift, prm, g);
+        else bn_stats_kernel<T, 1><<<grid, kBnThreads, 0, s>>>(x, partial, ws.counters, counter_stride(C), scale, shift, prm, g);
     } else {
         ProfScope ps("bn_infer_prep_kernel", s);
         bn_infer_prep_kernel<T><<<(unsigned)ceil_div(C, 256), 256, 0, s>>>(gamma, beta, rmean, rvar, save_mean,
@@ -394,6 +710,35 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     constexpr int V = Vec<T>::N;
     const bool vec = aligned16(x) && aligned16(delta) && aligned16(dx) && I % V == 0;
     const int vv = vec ? V : 1;
+    const float inv_count = 1.0f / (float)(I * N);
+
+    const int64_t SR = resident_slices(I, C, N, V, vec);
+    if (SR > 0) {
+        ChanGeom g;
+        g.nq = (uint32_t)(I * N / V);
+        g.vec_per_row = (uint32_t)(I / V);
+        g.C = (uint32_t)C;
+        g.rowdiv = FastDiv(g.vec_per_row);
+        g.chunk = (uint32_t)ceil_div(g.nq, SR);
+        const int64_t S = ceil_div(g.nq, g.chunk);
+        Workspace ws;
+        int rc = get_workspace(s, (size_t)C * 2 * S * sizeof(float), &ws);
+        if (rc != LUXHIP_OK) return rc;
+        float* partial = reinterpret_cast<float*>(ws.data);
+        const uint32_t spin = (uint32_t)option_bn_spin_limit();
+        dim3 grid((unsigned)S, (unsigned)C);
+#define LAUNCH_RES(A)                                                                                               \
+    bn_bwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, \
+                                                              partial, ws.flags, ws.epoch, spin, inv_count, stats_from_batch, g)
+        {
+            ProfScope ps("bn_bwd_resident_kernel", s);
+            LUX_DISPATCH_ACT(act, LAUNCH_RES);
+        }
+#undef LAUNCH_RES
+        LUX_CHECK_LAUNCH();
+        return LUXHIP_OK;
+    }
+
     int64_t S = 1;
     ChanGeom g = make_geom(I, C, N, vv, &S);
     Workspace ws;
@@ -401,14 +746,13 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     if (rc != LUXHIP_OK) return rc;
     float* coef = reinterpret_cast<float*>(ws.data);
     float* partial = coef + 3 * C;
-    const float inv_count = 1.0f / (float)(I * N);
     dim3 grid((unsigned)S, (unsigned)C);
     const uint32_t tv = (uint32_t)(I * C * N / vv);
     const FastDiv rowdiv((uint32_t)(I / vv)), cdiv((uint32_t)C);
 #define LAUNCH_REDUCE(A)                                                                                            \
     do {                                                                                                            \
-        if (vec) bn_bwd_reduce_kernel<T, A, V><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, partial, g); \
-        else bn_bwd_reduce_kernel<T, A, 1><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, partial, g);     \
+        if (vec) bn_bwd_reduce_kernel<T, A, V><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, partial, ws.counters, counter_stride(C), dgamma, dbeta, coef, inv_count, stats_from_batch, g); \
+        else bn_bwd_reduce_kernel<T, A, 1><<<grid, kBnThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, partial, ws.counters, counter_stride(C), dgamma, dbeta, coef, inv_count, stats_from_batch, g);     \
     } while (0)
 #define LAUNCH_BWD_APPLY(A)                                                                                         \
     do {                                                                                                            \
@@ -418,12 +762,6 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     {
         ProfScope ps("bn_bwd_reduce_kernel", s);
         LUX_DISPATCH_ACT(act, LAUNCH_REDUCE);
-    }
-    LUX_CHECK_LAUNCH();
-    {
-        ProfScope ps("bn_bwd_finalize_kernel", s);
-        bn_bwd_finalize_kernel<T><<<(unsigned)C, kWave, 0, s>>>(partial, (uint32_t)S, gamma, save_invstd, dgamma, dbeta, coef,
-                                                               (uint32_t)C, inv_count, stats_from_batch);
     }
     LUX_CHECK_LAUNCH();
     {

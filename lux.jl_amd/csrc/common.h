@@ -12,12 +12,32 @@ namespace luxhip {
 int set_error(int status, const char* fmt, ...);
 bool initialized();
 int num_cus();
+// Tuning switches set through luxhip_set_option (defaults in runtime.hip).
+int64_t option_bn_resident();     // 1: single-pass batchnorm kernels for tensors that fit the register file
+int64_t option_bn_spin_limit();   // polls before a resident workgroup stops waiting for its peers
+int64_t option_gemm_tile();       // 0 automatic, else 82 | 42 | 22 | 11
 
 // Per-stream scratch owned by the library (partial results of the reduction kernels,
 // per-channel coefficients).  get_workspace grows it on demand; kernels on one stream are
 // ordered, so consecutive operators may share it.
+// `counters`: kWorkspaceCounters arrival counters, all zero whenever no kernel of the stream is
+// running (the workgroup that arrives last puts its counter back to zero).
+// `flags`: kWorkspaceFlags words that resident kernels set to `epoch`, a value no earlier call on
+// the stream has used (so the flags never need clearing).
+constexpr size_t kWorkspaceCounters = 65536;
+constexpr size_t kWorkspaceFlags = 4096;
+// Counters of different channels are spread over different cache lines where the channel count
+// allows it: arrivals of all channels in one line would queue up behind each other.
+inline uint32_t counter_stride(int64_t channels) {
+    uint32_t st = 64;
+    while (st > 1 && (int64_t)st * channels > (int64_t)kWorkspaceCounters) st >>= 1;
+    return st;
+}
 struct Workspace {
     char* data;  // >= the requested number of bytes, 256-byte aligned
+    uint32_t* counters;
+    uint32_t* flags;
+    uint32_t epoch;
 };
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out);
 
@@ -97,11 +117,23 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
     return (bf16_t)(u >> 16);
 }
 
+typedef uint32_t raw16_t __attribute__((ext_vector_type(4)));   // 16 bytes as they lie in memory
+
 template <typename T>
 struct Vec;  // 16-byte vector access
 template <>
 struct Vec<float> {
     static constexpr int N = 4;
+    __device__ __forceinline__ static void unpack(raw16_t r, float (&v)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(r[i]);
+    }
+    __device__ __forceinline__ static raw16_t pack(const float (&v)[4]) {
+        raw16_t r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = __float_as_uint(v[i]);
+        return r;
+    }
     __device__ __forceinline__ static void load(const float* p, float (&v)[4]) {
         float4 t = *reinterpret_cast<const float4*>(p);
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
@@ -113,6 +145,19 @@ struct Vec<float> {
 template <>
 struct Vec<bf16_t> {
     static constexpr int N = 8;
+    __device__ __forceinline__ static void unpack(raw16_t r, float (&v)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(r[i] << 16);
+            v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+        }
+    }
+    __device__ __forceinline__ static raw16_t pack(const float (&v)[8]) {
+        raw16_t r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+        return r;
+    }
     __device__ __forceinline__ static void load(const bf16_t* p, float (&v)[8]) {
         uint4 t = *reinterpret_cast<const uint4*>(p);
         uint32_t w[4] = {t.x, t.y, t.z, t.w};
@@ -258,6 +303,45 @@ __device__ __forceinline__ float block_sum(float v, float* smem) {
     for (int i = 0; i < nw; ++i) t += smem[i];
     __syncthreads();
     return t;
+}
+
+// ----------------------------------------------------------------------------- cross-workgroup hand-off
+// Partial results travel between workgroups through agent-scope atomic stores and loads, which
+// go past the per-XCD L2 caches, so no cache-wide release fence (an L2 write-back of everything
+// the kernel has stored so far) is needed.  Protocol: every thread that published waits for its
+// stores (publish_done), the workgroup synchronises and one thread bumps the arrival counter
+// (arrive_last); the workgroup that arrives last reads everybody's values with fetch().
+__device__ __forceinline__ void publish(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t fetch(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void publish(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float fetch(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Call after the last publish of a thread and before the workgroup barrier that precedes arrive().
+__device__ __forceinline__ void publish_done() {
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_waitcnt(0);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+// True in every thread of the workgroup that arrives last out of `expected`; that workgroup also
+// puts the counter back to zero for the next kernel.  `flag` is one word of LDS.  Contains
+// workgroup barriers: all threads must call it.
+__device__ __forceinline__ bool arrive_last(uint32_t* counter, uint32_t expected, uint32_t* flag) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev + 1 == expected;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    return *flag != 0u;
 }
 
 }  // namespace luxhip

@@ -134,14 +134,18 @@ __global__ __launch_bounds__(kThreads) void act_bwd_kernel(const T* __restrict__
 }
 
 // "channel" layout: grid (S, C).  Workgroup (s, c) handles vectors [s*chunk, (s+1)*chunk) of
-// the nq = I*N/VEC vectors of channel c and writes its partial sum.
+// the nq = I*N/VEC vectors of channel c and publishes its partial sum; the workgroup of a
+// channel that arrives last adds the S partials in index order (same result on every run).
 template <typename T, int ACT, int VEC>
 __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T* __restrict__ delta,
                                                                         const T* __restrict__ out,
-                                                                        const T* __restrict__ pre, T* dx,
-                                                                        float* partial, uint32_t nq, uint32_t chunk, FastDiv rowdiv,
+                                                                        const T* __restrict__ pre, T* dx, T* dbias,
+                                                                        float* partial, uint32_t* counters,
+                                                                        uint32_t cstride, uint32_t nq,
+                                                                        uint32_t chunk, FastDiv rowdiv,
                                                                         uint32_t vec_per_row, uint32_t C) {
     __shared__ float smem[kThreads / 64];
+    __shared__ uint32_t last_flag;
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     const uint32_t q0 = s * chunk;
     const uint32_t q1 = min(q0 + chunk, nq);
@@ -156,17 +160,17 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T*
         for (int k = 0; k < VEC; ++k) acc += r[k];
     }
     acc = block_sum(acc, smem);
-    if (threadIdx.x == 0) partial[(size_t)c * S + s] = acc;
-}
-
-// dbias[c] = sum_s partial[c][s]; one wave per channel, fixed order.
-template <typename T>
-__global__ __launch_bounds__(64) void channel_finalize_kernel(const float* __restrict__ partial, T* dbias, uint32_t S) {
-    const uint32_t c = blockIdx.x;
-    float t = 0.0f;
-    for (uint32_t i = threadIdx.x; i < S; i += 64) t += partial[(size_t)c * S + i];
-    t = wave_sum(t);
-    if (threadIdx.x == 0) st(dbias + c, t);
+    if (threadIdx.x == 0) {
+        publish(partial + (size_t)c * S + s, acc);
+        publish_done();
+    }
+    if (!arrive_last(counters + (size_t)c * cstride, S, &last_flag)) return;
+    if (threadIdx.x < 64) {
+        float t = 0.0f;
+        for (uint32_t i = threadIdx.x; i < S; i += 64) t += fetch(partial + (size_t)c * S + i);
+        t = wave_sum(t);
+        if (threadIdx.x == 0) st(dbias + c, t);
+    }
 }
 
 // "plane" layout: P = I*C contiguous elements per n.  grid (ceil(P/(T*VEC)), S); a thread
@@ -309,23 +313,21 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
         int rc = get_workspace(s, (size_t)C * S * sizeof(float), &ws);
         if (rc != LUXHIP_OK) return rc;
         float* partial = reinterpret_cast<float*>(ws.data);
+        uint32_t* counters = ws.counters;
         const FastDiv rowdiv((uint32_t)(I / vv));
         dim3 grid((unsigned)S, (unsigned)C);
 #define LAUNCH_CH(A)                                                                                               \
     do {                                                                                                           \
         if (vec)                                                                                                   \
-            bias_act_bwd_channel_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+            bias_act_bwd_channel_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, counters, counter_stride(C), nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
         else                                                                                                       \
-            bias_act_bwd_channel_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, partial, nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+            bias_act_bwd_channel_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, counters, counter_stride(C), nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
     } while (0)
         {
             ProfScope ps("bias_act_bwd_channel_kernel", s);
             LUX_DISPATCH_ACT(act, LAUNCH_CH);
         }
 #undef LAUNCH_CH
-        LUX_CHECK_LAUNCH();
-        ProfScope ps2("channel_finalize_kernel", s);
-        channel_finalize_kernel<T><<<(unsigned)C, 64, 0, s>>>(partial, dbias, (uint32_t)S);
         LUX_CHECK_LAUNCH();
         return LUXHIP_OK;
     }

@@ -12,13 +12,7 @@ namespace luxhip {
 int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* delta,
                           const void* out, const void* pre, void* dx, void* dbias);   // elementwise.hip
 
-int gemm_tile_override() {
-    static const int v = [] {
-        const char* e = getenv("LUXHIP_GEMM_TILE");
-        return e ? atoi(e) : 0;
-    }();
-    return v;
-}
+int gemm_tile_override() { return (int)option_gemm_tile(); }
 
 template <typename T>
 static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const T* A, int64_t lda,

@@ -1,9 +1,11 @@
 // libluxhip runtime: context, error reporting, streams, events, pooled device memory and
 // the per-stream workspace used by the reduction kernels.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <map>
 #include <string>
 #include <mutex>
@@ -29,6 +31,8 @@ struct Pool {
 struct WsEntry {
     void* base = nullptr;
     size_t data_bytes = 0;
+    uint32_t* counters = nullptr;   // kWorkspaceCounters words, zero between kernels, then kWorkspaceFlags words
+    uint32_t epoch = 0;
 };
 std::map<hipStream_t, WsEntry> g_ws;
 
@@ -73,6 +77,21 @@ int set_error(int status, const char* fmt, ...) {
 bool initialized() { return g_init; }
 int num_cus() { return g_cus; }
 
+namespace {
+std::atomic<int64_t> g_opt_bn_resident{1}, g_opt_bn_spin_limit{int64_t(1) << 22}, g_opt_gemm_tile{-1};
+}
+int64_t option_bn_resident() { return g_opt_bn_resident.load(); }
+int64_t option_bn_spin_limit() { return g_opt_bn_spin_limit.load(); }
+int64_t option_gemm_tile() {
+    int64_t v = g_opt_gemm_tile.load();
+    if (v < 0) {   // not set through the API: the environment variable LUXHIP_GEMM_TILE, read once
+        const char* e = getenv("LUXHIP_GEMM_TILE");
+        v = e ? atoll(e) : 0;
+        g_opt_gemm_tile.store(v);
+    }
+    return v;
+}
+
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     std::lock_guard<std::mutex> lk(g_mu);
     WsEntry& e = g_ws[s];
@@ -89,7 +108,19 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
         e.base = p;
         e.data_bytes = want;
     }
+    if (e.counters == nullptr) {
+        void* c = nullptr;
+        constexpr size_t words = kWorkspaceCounters + kWorkspaceFlags;
+        LUX_CHECK_HIP(hipMalloc(&c, words * sizeof(uint32_t)));
+        hipError_t rc = hipMemsetAsync(c, 0, words * sizeof(uint32_t), s);
+        if (rc != hipSuccess) { (void)hipFree(c); LUX_CHECK_HIP(rc); }
+        e.counters = reinterpret_cast<uint32_t*>(c);
+    }
     out->data = reinterpret_cast<char*>(e.base);
+    out->counters = e.counters;
+    out->flags = e.counters + kWorkspaceCounters;
+    if (++e.epoch == 0) e.epoch = 1;   // 0 is what freshly cleared flags hold
+    out->epoch = e.epoch;
     return LUXHIP_OK;
 }
 
@@ -133,8 +164,10 @@ int luxhip_shutdown(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     if (!g_init) return LUXHIP_OK;
     (void)hipDeviceSynchronize();
-    for (auto& kv : g_ws)
+    for (auto& kv : g_ws) {
         if (kv.second.base) (void)hipFree(kv.second.base);
+        if (kv.second.counters) (void)hipFree(kv.second.counters);
+    }
     g_ws.clear();
     for (auto& kv : g_pool.free_blocks) (void)hipFree(kv.second);
     g_pool.free_blocks.clear();
@@ -146,6 +179,23 @@ int luxhip_shutdown(void) {
 }
 
 const char* luxhip_last_error(void) { return g_err; }
+
+int luxhip_set_option(const char* name, int64_t value) {
+    LUX_INVALID_IF(name == nullptr, "set_option: name must not be NULL");
+    if (strcmp(name, "bn_resident") == 0) {
+        g_opt_bn_resident.store(value != 0);
+    } else if (strcmp(name, "bn_spin_limit") == 0) {
+        LUX_INVALID_IF(value < 0 || value > (int64_t(1) << 30), "set_option: bn_spin_limit out of range");
+        g_opt_bn_spin_limit.store(value);
+    } else if (strcmp(name, "gemm_tile") == 0) {
+        LUX_INVALID_IF(value != 0 && value != 82 && value != 42 && value != 22 && value != 11,
+                       "set_option: gemm_tile must be 0, 82, 42, 22 or 11");
+        g_opt_gemm_tile.store(value);
+    } else {
+        return set_error(LUXHIP_INVALID, "set_option: unknown option '%s'", name);
+    }
+    return LUXHIP_OK;
+}
 
 int luxhip_device_info(char* name, size_t name_len, int* compute_units, int64_t* total_mem) {
     LUX_REQUIRE_INIT();
@@ -179,6 +229,7 @@ int luxhip_stream_destroy(luxhip_stream_t s) {
         auto it = g_ws.find((hipStream_t)s);
         if (it != g_ws.end()) {
             if (it->second.base) (void)hipFree(it->second.base);
+            if (it->second.counters) (void)hipFree(it->second.counters);
             g_ws.erase(it);
         }
     }

@@ -33,14 +33,27 @@ def test_reference_known_answer(gpu):
     assert st2["running_mean"] is st["running_mean"]
 
 
-SHAPES = [(4, 4, 6, 2), (8, 2), (3, 5, 4), (16, 16, 8, 4), (64, 3, 5), (32, 32, 16, 8)]
+SHAPES = [(4, 4, 6, 2), (8, 2), (3, 5, 4), (16, 16, 8, 4), (64, 3, 5), (32, 32, 16, 8), (40, 40, 3, 7)]
+
+
+@pytest.fixture(params=["resident", "streaming", "no_wait"])
+def bn_path(gpu, request):
+    """The three ways the library can run a training-mode batchnorm: single-pass kernels that keep
+    the tensor in registers (default where it fits), the two-kernel streaming path, and the
+    single-pass kernels with the wait for peer workgroups cut to zero polls, which makes every
+    workgroup recompute its peers' partial results itself (the bounded-wait exit)."""
+    gpu.set_option("bn_resident", 0 if request.param == "streaming" else 1)
+    gpu.set_option("bn_spin_limit", 0 if request.param == "no_wait" else 1 << 22)
+    yield request.param
+    gpu.set_option("bn_resident", 1)
+    gpu.set_option("bn_spin_limit", 1 << 22)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("act", ["identity", "relu", "sigmoid_fast", "swish", "gelu", "tanh"])
 @pytest.mark.parametrize("affine", [True, False])
 @pytest.mark.parametrize("track", [True, False])
-def test_training_forward_and_pullback(gpu, dtype, act, affine, track):
+def test_training_forward_and_pullback(gpu, bn_path, dtype, act, affine, track):
     rng = np.random.default_rng(stable_seed(dtype, act, affine, track))
     for shape in SHAPES:
         Cc = shape[-2]
@@ -62,7 +75,7 @@ def test_training_forward_and_pullback(gpu, dtype, act, affine, track):
         (y, st), back = gpu.pullback(gpu.batchnorm, *args, True, act, 0.1, eps)
         wy, wrm, wrv = O.batchnorm(f64(x), f64(g), f64(b), f64(rm), f64(rv), True, act, 0.1, eps)
         wy32 = O.batchnorm(x, g, b, rm, rv, True, act, 0.1, eps)[0]
-        tag = f"{dtype} {act} {shape} affine={affine} track={track}"
+        tag = f"{bn_path} {dtype} {act} {shape} affine={affine} track={track}"
         assert_close(y.to_numpy(), wy, dtype, tag + " y", want32=wy32)
         if track:
             assert_close(st["running_mean"].to_numpy(), wrm, dtype, tag + " running_mean")
@@ -123,7 +136,7 @@ def test_large_mean_small_variance_is_stable(gpu):
     assert abs(y.to_numpy().std() - 1) < 1e-2
 
 
-def test_config2_full_size(gpu):
+def test_config2_full_size(gpu, bn_path):
     """BASELINE config 2 at full size: x 32x32x64x128 ~ N(0.5, 2), train mode.  Checked against
     the fp64 oracle on a channel subset plus size-independent invariants (zero mean / unit
     variance per channel before the affine map; sum(dx) == 0 and sum(dx * xhat) == 0 per
