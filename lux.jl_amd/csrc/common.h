@@ -38,7 +38,9 @@ struct Workspace {
     uint32_t* counters;
     uint32_t* flags;
     uint32_t epoch;
+    const void* zeros;   // kWorkspaceZeroBytes bytes that are never written
 };
+constexpr size_t kWorkspaceZeroBytes = 256;
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out);
 
 // Optional per-kernel timing with HIP events on the launch stream (luxhip_profile_enable).

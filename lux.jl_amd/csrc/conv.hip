@@ -137,27 +137,57 @@ static void fill_gather(GatherK<T>& q, const ConvGeom& g, bool dgrad) {
 }
 
 // fprop (dgrad == false): out = y; dgrad: out = dx.  src is the channel-contiguous activation,
-// wm the packed filter (all groups).
+// wm the packed filter (all groups), zeros a few zero bytes in device memory.
 template <typename T>
 static int run_conv_gemm(hipStream_t s, const ConvGeom& g, bool dgrad, const T* src, const T* wm, const T* bias, T* out,
-                         T* pre, int act) {
+                         T* pre, int act, const void* zeros) {
     const int Tt = g.kW * g.kH;
+    const int Cg = dgrad ? g.Cout_g : g.Cin_g;
+    const int64_t src_elems = dgrad ? (int64_t)g.OW * g.OH * g.Cout * g.N : (int64_t)g.W * g.H * g.Cin * g.N;
+    // whole-tap stages: a K stage never straddles a filter tap; the transposed-convolution index
+    // map of dgrad is only that simple for unit stride
+    const bool tap_path = Cg % GemmTraits<T>::BK == 0 && (!dgrad || (g.sw == 1 && g.sh == 1)) && aligned16(src) &&
+                          aligned16(wm) && src_elems < (int64_t(1) << 30);
     for (int grp = 0; grp < g.groups; ++grp) {
-        ConvGemmArgs<T> a;
-        fill_gather(a.gather, g, dgrad);
-        a.gather.src = src;
-        a.gather.c_off = grp * a.gather.Cg;
-        a.gather.vec_ok = a.gather.vec_ok && aligned16(src);
-        a.K = Tt * a.gather.Cg;
-        a.Ncols = dgrad ? g.Cin_g : g.Cout_g;
-        a.Wm.p = wm + (size_t)grp * a.Ncols * a.K;
-        a.Wm.sr = a.K; a.Wm.sk = 1; a.Wm.rows = a.Ncols;
-        a.Wm.vec_ok = aligned16(a.Wm.p) && ((size_t)a.K * sizeof(T)) % 16 == 0;
-        a.out = out; a.pre = pre; a.bias = bias;
-        a.Ctot_out = dgrad ? g.Cin : g.Cout;
-        a.col_off = grp * a.Ncols;
-        a.act = act;
-        int rc = launch_conv_gemm_any<T>(s, a);
+        const int Ncols = dgrad ? g.Cin_g : g.Cout_g;
+        const int K = Tt * Cg;
+        Operand<T> Wm;
+        Wm.p = wm + (size_t)grp * Ncols * K;
+        Wm.sr = K; Wm.sk = 1; Wm.rows = Ncols;
+        Wm.vec_ok = aligned16(Wm.p) && ((size_t)K * sizeof(T)) % 16 == 0;
+        int rc;
+        if (tap_path) {
+            ConvTapArgs<T> a;
+            TapGeom<T>& q = a.tap;
+            q.kW = g.kW; q.sw = g.sw; q.sh = g.sh; q.pw = g.pw; q.ph = g.ph; q.dw = g.dw; q.dh = g.dh;
+            q.dgrad = dgrad;
+            q.Cg = Cg;
+            if (!dgrad) { q.Ctot = g.Cin; q.P = g.OW; q.PQ = g.OW * g.OH; q.SP = g.W; q.SQ = g.H; }
+            else { q.Ctot = g.Cout; q.P = g.W; q.PQ = g.W * g.H; q.SP = g.OW; q.SQ = g.OH; }
+            q.M = q.PQ * g.N;
+            q.divP = FastDiv((uint32_t)q.P); q.divPQ = FastDiv((uint32_t)q.PQ); q.divCg = FastDiv((uint32_t)q.Cg);
+            q.divkW = FastDiv((uint32_t)g.kW);
+            q.src = src + (size_t)grp * Cg;
+            q.zero = zeros;
+            a.Wm = Wm; a.K = K; a.Ncols = Ncols;
+            a.out = out; a.pre = pre; a.bias = bias;
+            a.Ctot_out = dgrad ? g.Cin : g.Cout;
+            a.col_off = grp * Ncols;
+            a.act = act;
+            rc = launch_conv_tap_any<T>(s, a);
+        } else {
+            ConvGemmArgs<T> a;
+            fill_gather(a.gather, g, dgrad);
+            a.gather.src = src;
+            a.gather.c_off = grp * a.gather.Cg;
+            a.gather.vec_ok = a.gather.vec_ok && aligned16(src);
+            a.K = K; a.Ncols = Ncols; a.Wm = Wm;
+            a.out = out; a.pre = pre; a.bias = bias;
+            a.Ctot_out = dgrad ? g.Cin : g.Cout;
+            a.col_off = grp * a.Ncols;
+            a.act = act;
+            rc = launch_conv_gemm_any<T>(s, a);
+        }
         if (rc != LUXHIP_OK) return rc;
     }
     return LUXHIP_OK;
@@ -229,7 +259,7 @@ static int conv_fwd_t(hipStream_t s, int act, const ConvGeom& g, const T* x, con
     T* wF = reinterpret_cast<T*>(ws.data + xb);
     if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
     if ((rc = pack_filter<T>(s, w, wF, g, 0)) != LUXHIP_OK) return rc;
-    return run_conv_gemm<T>(s, g, false, xT, wF, bias, y, pre, act);
+    return run_conv_gemm<T>(s, g, false, xT, wF, bias, y, pre, act, ws.zeros);
 }
 
 template <typename T>
@@ -243,7 +273,7 @@ static int conv_bwd_data_t(hipStream_t s, const ConvGeom& g, const T* dy, const 
     T* wD = reinterpret_cast<T*>(ws.data + yb);
     if ((rc = transpose_to_cwhn<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
     if ((rc = pack_filter<T>(s, w, wD, g, 1)) != LUXHIP_OK) return rc;
-    return run_conv_gemm<T>(s, g, true, dyT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY);
+    return run_conv_gemm<T>(s, g, true, dyT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY, ws.zeros);
 }
 
 template <typename T>
@@ -289,7 +319,7 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
     if ((rc = transpose_to_cwhn<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
     if (dx != nullptr) {
         if ((rc = pack_filter<T>(s, w, wD, g, 1)) != LUXHIP_OK) return rc;
-        if ((rc = run_conv_gemm<T>(s, g, true, dzT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY)) != LUXHIP_OK) return rc;
+        if ((rc = run_conv_gemm<T>(s, g, true, dzT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY, ws.zeros)) != LUXHIP_OK) return rc;
     }
     if (dw != nullptr) {
         if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;

@@ -8,4 +8,9 @@ int launch_conv_gemm_any<float>(hipStream_t s, ConvGemmArgs<float>& a) {
     if (a.Ncols > 64 && a.gather.M > 64) return launch_conv_gemm<float, 2, 2>(s, a);
     return launch_conv_gemm<float, 1, 1>(s, a);
 }
+// whole-tap stages through registers: 128 x 128 tiles (two workgroups per compute unit)
+template <>
+int launch_conv_tap_any<float>(hipStream_t s, ConvTapArgs<float>& a) {
+    return launch_conv_tap<float, 2, 2, 2, 0>(s, a);
+}
 }  // namespace luxhip

@@ -127,18 +127,44 @@ struct ConvGemmArgs {
     int tiles_m, tiles_n;
 };
 
-__device__ __forceinline__ float conv_apply_act(int act, float x) {
-    switch (act) {
-        case LUXHIP_ACT_RELU: return Act<LUXHIP_ACT_RELU>::f(x);
-        case LUXHIP_ACT_TANH: return Act<LUXHIP_ACT_TANH>::f(x);
-        case LUXHIP_ACT_SIGMOID: return Act<LUXHIP_ACT_SIGMOID>::f(x);
-        case LUXHIP_ACT_SWISH: return Act<LUXHIP_ACT_SWISH>::f(x);
-        case LUXHIP_ACT_GELU: return Act<LUXHIP_ACT_GELU>::f(x);
-        case LUXHIP_ACT_SOFTPLUS: return Act<LUXHIP_ACT_SOFTPLUS>::f(x);
-        case LUXHIP_ACT_LOGSIGMOID: return Act<LUXHIP_ACT_LOGSIGMOID>::f(x);
-        case LUXHIP_ACT_LISHT: return Act<LUXHIP_ACT_LISHT>::f(x);
-        default: return x;
+// Epilogue of fprop / dgrad: element (m = (p, q, n), col) -> out[(m - n*PQ) + PQ*(col_off + col +
+// Ctot_out*n)], with bias per output channel and the activation.  The image index of a row is
+// decoded once per row, the channel terms once per column.
+template <class ML, typename T, int WM, int WN>
+__device__ __forceinline__ void conv_epilogue(const f32x16_v (&acc)[WM][WN], int m0, int n0, int M, int PQ, FastDiv divPQ,
+                                              int Ncols, int col_off, int Ctot_out, const T* bias, T* out, T* pre, int act) {
+    const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
+    int64_t rowoff[WM];
+    bool mok[WM];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const int m = mb + i * 32;
+        mok[i] = m < M;
+        const int n = (int)divPQ.div((uint32_t)(mok[i] ? m : 0));
+        rowoff[i] = (int64_t)(m - n * PQ) + (int64_t)PQ * Ctot_out * n;
     }
+    static_for<WN * 16>([&](auto JR) {
+        {
+            constexpr int j = decltype(JR)::value / 16, r = decltype(JR)::value % 16;
+            const int col = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
+            if (col < Ncols) {
+                const float b = bias ? ld(bias + col_off + col) : 0.0f;
+                const int64_t coloff = (int64_t)PQ * (col_off + col);
+                float v[WM];
+#pragma unroll
+                for (int i = 0; i < WM; ++i) v[i] = acc[i][j][r] + b;
+                if (pre) {
+#pragma unroll
+                    for (int i = 0; i < WM; ++i)
+                        if (mok[i]) st(pre + coloff + rowoff[i], v[i]);
+                }
+                act_vec(act, v);
+#pragma unroll
+                for (int i = 0; i < WM; ++i)
+                    if (mok[i]) st(out + coloff + rowoff[i], v[i]);
+            }
+        }
+    });
 }
 
 // fprop and dgrad share this kernel (the gather loader's `dgrad` flag picks the index map).
@@ -155,18 +181,7 @@ __global__ __launch_bounds__(kGemmThreads) void conv_gemm_kernel(ConvGemmArgs<T>
     typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
     f32x16_v acc[WM][WN];
     ML::run(la, lb, a.K, lds, acc);
-    const int PQ = g.PQ, M = g.M;
-    const FastDiv divPQ = g.divPQ;
-    ML::for_each(acc, m0, n0, [&](int m, int col, float v) {
-        if (m < M && col < a.Ncols) {
-            const int n = (int)divPQ.div((uint32_t)m);
-            const int ch = a.col_off + col;
-            if (a.bias) v += ld(a.bias + ch);
-            const int64_t off = (int64_t)(m - n * PQ) + (int64_t)PQ * (ch + (int64_t)a.Ctot_out * n);
-            if (a.pre) st(a.pre + off, v);
-            st(a.out + off, conv_apply_act(a.act, v));
-        }
-    });
+    conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
 }
 
 template <typename T, int WM, int WN>
@@ -187,6 +202,193 @@ int launch_conv_gemm(hipStream_t s, ConvGemmArgs<T>& a) {
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }
+
+// ----------------------------------------------------------------------------- whole-tap stages
+// When the channels per group are a multiple of BK, a K stage lies inside one filter tap: the
+// tap (ka, kb) and first channel of a stage are uniform scalars, and the (p, q, n) decode of a
+// thread's rows does not depend on the stage, so it is done once.  Element offset of row m at
+// the stage that starts at k0:  pos0(m) + tap_delta(k0)  with
+//   pos0      = ((n*SQ + qs)*SP + ps)*Ctot     (ps, qs: source position for tap offset 0)
+//   tap_delta = (dq*SP + dp)*Ctot + c0         (dp, dq: the tap's shift of that position)
+// valid when 0 <= ps+dp < SP and 0 <= qs+dq < SQ.  fprop: ps = p*sw, dp = ka*dw - pw.  dgrad
+// (unit stride only): ps = p, dp = pw - ka*dw.
+template <typename T>
+struct TapGeom {
+    const T* src;              // channel-contiguous source, first channel of the group
+    const void* zero;          // 16 zero bytes in device memory (padding and rows past M)
+    int Ctot, Cg;
+    int P, PQ, M;
+    int SP, SQ;
+    int kW, sw, sh, pw, ph, dw, dh;
+    int dgrad;
+    FastDiv divP, divPQ, divCg, divkW;
+};
+
+template <int N>
+struct TapRows {
+    int pos0[N], ps[N], qs[N];
+    template <typename T>
+    __device__ __forceinline__ void init(const TapGeom<T>& g, int m_first, int m_step) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int m = m_first + i * m_step;
+            if (m < g.M) {
+                const int n = (int)g.divPQ.div((uint32_t)m);
+                const int rem = m - n * g.PQ;
+                const int q = (int)g.divP.div((uint32_t)rem);
+                const int p = rem - q * g.P;
+                ps[i] = g.dgrad ? p : p * g.sw;
+                qs[i] = g.dgrad ? q : q * g.sh;
+                // ps, qs may exceed the source extent (strided windows); the 64-bit product keeps pos0 exact
+                pos0[i] = (int)((((int64_t)n * g.SQ + qs[i]) * g.SP + ps[i]) * g.Ctot);
+            } else {
+                ps[i] = -(1 << 24);   // never valid
+                qs[i] = 0;
+                pos0[i] = 0;
+            }
+        }
+    }
+};
+
+struct TapStage {
+    int dp, dq, delta;
+    template <typename T>
+    __device__ __forceinline__ TapStage(const TapGeom<T>& g, int k0) {
+        const int t = (int)g.divCg.div((uint32_t)k0);
+        const int c0 = k0 - t * g.Cg;
+        const int kb = (int)g.divkW.div((uint32_t)t);
+        const int ka = t - kb * g.kW;
+        dp = g.dgrad ? g.pw - ka * g.dw : ka * g.dw - g.pw;
+        dq = g.dgrad ? g.ph - kb * g.dh : kb * g.dh - g.ph;
+        delta = (dq * g.SP + dp) * g.Ctot + c0;
+    }
+};
+
+// bf16, straight into LDS (same slot assignment as DirectLoader<true, ROWS, THREADS>)
+template <int ROWS, int THREADS>
+struct ConvDirectLoaderK {
+    using T = bf16_t;
+    static constexpr bool KMAJOR = true;
+    static constexpr int BK = GemmTraits<bf16_t>::BK, CPR = BK / 8;
+    static constexpr int INSTR = ROWS * CPR / THREADS, STEP = THREADS / CPR;
+    static_assert(INSTR >= 1 && (ROWS * CPR) % THREADS == 0 && STEP % 16 == 0, "stage must split evenly over the workgroup");
+    const TapGeom<T>& g;
+    TapRows<INSTR> rows;
+    int chunk_el;          // element offset of this thread's 16-byte chunk inside a row's stage
+    uint32_t lds_off;
+    __device__ __forceinline__ ConvDirectLoaderK(const TapGeom<T>& gg, int m0) : g(gg) {
+        const int q = threadIdx.x, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const int row = q / CPR, slot = q % CPR;
+        chunk_el = (slot ^ ((row >> 2) & 3)) * 8;     // STEP is a multiple of 16: same swizzle for every i
+        lds_off = (uint32_t)w * 1024u;
+        rows.init(g, m0 + row, STEP);
+    }
+    __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
+        typedef __attribute__((address_space(3))) void* lds_vp;
+        typedef const __attribute__((address_space(1))) void* glb_vp;
+        const TapStage st(g, k0);
+        char* l = reinterpret_cast<char*>(lds_tile) + lds_off;
+#pragma unroll
+        for (int i = 0; i < INSTR; ++i) {
+            const bool valid = (unsigned)(rows.ps[i] + st.dp) < (unsigned)g.SP && (unsigned)(rows.qs[i] + st.dq) < (unsigned)g.SQ;
+            const T* src = g.src + ((int64_t)rows.pos0[i] + st.delta + chunk_el);
+            const void* p = valid ? static_cast<const void*>(src) : g.zero;
+            __builtin_amdgcn_global_load_lds((glb_vp)p, (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
+        }
+    }
+};
+
+// any storage type, through registers (interface of TileLoader)
+template <typename T, int ROWS, int THREADS>
+struct ConvTapLoaderK {
+    using Tr = GemmTraits<T>;
+    static constexpr bool KMAJOR = true;
+    static constexpr int CPR = Tr::BK / Tr::VEC;
+    static constexpr int PER_THREAD = ROWS * CPR / THREADS, STEP = THREADS / CPR;
+    static_assert(PER_THREAD >= 1 && (ROWS * CPR) % THREADS == 0, "tile must split evenly over the workgroup");
+    u32x4_v reg[PER_THREAD];
+    const TapGeom<T>& g;
+    TapRows<PER_THREAD> rows;
+    int chunk_el;
+    __device__ __forceinline__ ConvTapLoaderK(const TapGeom<T>& gg, int m0) : g(gg) {
+        chunk_el = (threadIdx.x % CPR) * Tr::VEC;
+        rows.init(g, m0 + threadIdx.x / CPR, STEP);
+    }
+    __device__ __forceinline__ void load(int k0) {
+        const TapStage st(g, k0);
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            const bool valid = (unsigned)(rows.ps[i] + st.dp) < (unsigned)g.SP && (unsigned)(rows.qs[i] + st.dq) < (unsigned)g.SQ;
+            const T* src = g.src + ((int64_t)rows.pos0[i] + st.delta + chunk_el);
+            const u32x4_v* p = reinterpret_cast<const u32x4_v*>(valid ? static_cast<const void*>(src) : g.zero);
+            reg[i] = *p;
+        }
+    }
+    __device__ __forceinline__ void store(T* lds) const {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            const int r = threadIdx.x / CPR + i * STEP;
+            *reinterpret_cast<u32x4_v*>(lds + lds_chunk_offset<T, true, ROWS>(r, chunk_el)) = reg[i];
+        }
+    }
+};
+
+template <typename T>
+struct ConvTapArgs {
+    TapGeom<T> tap;
+    Operand<T> Wm;                     // filter matrix, K-major, rows = output columns of this group
+    int K, Ncols;
+    T* out;
+    T* pre;
+    const T* bias;
+    int Ctot_out, col_off, act;
+    int tiles_m, tiles_n;
+};
+
+template <typename T, int WM, int WN, int NWN, int NST>
+__global__ __launch_bounds__(2 * NWN * 64) void conv_tap_kernel(ConvTapArgs<T> a) {
+    constexpr bool DIRECT = sizeof(T) == 2;
+    using ML = GemmMainloop<T, WM, WN, true, true, DIRECT, NWN, NST>;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    int tm, tn;
+    tile_coords(a.tiles_m, a.tiles_n, tm, tn);
+    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+    const TapGeom<T>& g = a.tap;
+    f32x16_v acc[WM][WN];
+    if constexpr (DIRECT) {
+        ConvDirectLoaderK<ML::TILE_M, ML::THREADS> la(g, m0);
+        DirectLoader<true, ML::TILE_N, ML::THREADS, true> lb(a.Wm, n0, g.zero);
+        ML::run_pipeline(la, lb, a.K, lds, acc);
+    } else {
+        ConvTapLoaderK<T, ML::TILE_M, ML::THREADS> la(g, m0);
+        typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
+        ML::run(la, lb, a.K, lds, acc);
+    }
+    conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
+}
+
+template <typename T, int WM, int WN, int NWN, int NST>
+int launch_conv_tap(hipStream_t s, ConvTapArgs<T>& a) {
+    using ML = GemmMainloop<T, WM, WN, true, true, sizeof(T) == 2, NWN, NST>;
+    a.tiles_m = (int)ceil_div(a.tap.M, ML::TILE_M);
+    a.tiles_n = (int)ceil_div(a.Ncols, ML::TILE_N);
+    auto kernel = conv_tap_kernel<T, WM, WN, NWN, NST>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)ML::LDS_BYTES));
+        attr_set = true;
+    }
+    ProfScope ps(a.tap.dgrad ? (sizeof(T) == 2 ? "conv_dgrad_kernel<bf16>" : "conv_dgrad_kernel<f32>")
+                             : (sizeof(T) == 2 ? "conv_fprop_kernel<bf16>" : "conv_fprop_kernel<f32>"), s);
+    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T>
+int launch_conv_tap_any(hipStream_t s, ConvTapArgs<T>& a);   // picks the tile; conv_inst_*.hip
 
 template <typename T>
 int launch_conv_gemm_any(hipStream_t s, ConvGemmArgs<T>& a);   // picks the tile; conv_inst_*.hip

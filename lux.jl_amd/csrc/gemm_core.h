@@ -27,15 +27,52 @@
 // all the instruction needs.
 #pragma once
 
+#include <type_traits>
+#include <utility>
+
 #include "common.h"
 
 namespace luxhip {
+
+// f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N-1>): a loop that is
+// expanded by the front end, for bodies the loop unroller gives up on (accumulator registers can
+// only be indexed by compile-time constants).
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
 
 typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
 typedef float f32x16_v __attribute__((ext_vector_type(16)));
 typedef short s16x4_v __attribute__((ext_vector_type(4)));
 typedef short s16x8_v __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_v __attribute__((ext_vector_type(4)));
+
+// Activation over a few values at a time: the epilogues branch on the runtime activation id once
+// per column of the accumulator tile, and only those few values are live in VGPRs meanwhile.
+template <int ACT, int N>
+__device__ __forceinline__ void act_vec_as(float (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = Act<ACT>::f(v[i]);
+}
+template <int N>
+__device__ __forceinline__ void act_vec(int act, float (&v)[N]) {
+    switch (act) {
+        case LUXHIP_ACT_RELU: act_vec_as<LUXHIP_ACT_RELU>(v); break;
+        case LUXHIP_ACT_TANH: act_vec_as<LUXHIP_ACT_TANH>(v); break;
+        case LUXHIP_ACT_SIGMOID: act_vec_as<LUXHIP_ACT_SIGMOID>(v); break;
+        case LUXHIP_ACT_SWISH: act_vec_as<LUXHIP_ACT_SWISH>(v); break;
+        case LUXHIP_ACT_GELU: act_vec_as<LUXHIP_ACT_GELU>(v); break;
+        case LUXHIP_ACT_SOFTPLUS: act_vec_as<LUXHIP_ACT_SOFTPLUS>(v); break;
+        case LUXHIP_ACT_LOGSIGMOID: act_vec_as<LUXHIP_ACT_LOGSIGMOID>(v); break;
+        case LUXHIP_ACT_LISHT: act_vec_as<LUXHIP_ACT_LISHT>(v); break;
+        default: break;
+    }
+}
 
 constexpr int kGemmThreads = 256;
 
@@ -168,10 +205,11 @@ struct TileLoader {
     }
 };
 
-// Direct global -> LDS loader for whole, aligned bf16 tiles.  One wave instruction fills 1 KiB
-// of the stage linearly (lane i -> byte 16*i after a wave-uniform base); lane i therefore
-// fetches the global chunk whose swizzled home is that slot.
-template <bool KMAJOR_, int ROWS, int THREADS = kGemmThreads>
+// Direct global -> LDS loader for aligned bf16 tiles.  One wave instruction fills 1 KiB of the
+// stage linearly (lane i -> byte 16*i after a wave-uniform base); lane i therefore fetches the
+// global chunk whose swizzled home is that slot.  BOUNDED: rows at or past op.rows read from
+// `zero` (16 zero bytes somewhere in device memory) instead, so partial tiles need no branch.
+template <bool KMAJOR_, int ROWS, int THREADS = kGemmThreads, bool BOUNDED = false>
 struct DirectLoader {
     using T = bf16_t;
     static constexpr bool KMAJOR = KMAJOR_;
@@ -180,12 +218,15 @@ struct DirectLoader {
     static constexpr int INSTR = ROWS * BK / 8 / THREADS;          // instructions per thread and stage
     static_assert(INSTR >= 1 && (ROWS * BK / 8) % THREADS == 0, "stage must split evenly over the workgroup");
     static constexpr int STEP = THREADS / CPR;                // LDS rows covered per instruction of the workgroup
+    static_assert(!BOUNDED || KMAJOR, "row bounds are implemented for K-major operands");
     const char* base;      // uniform: first element of the tile (row r0, k = 0)
+    const char* zero;      // BOUNDED only
     int64_t step_bytes;    // uniform: global distance between consecutive instructions of a thread
     int64_t k_bytes;       // uniform: global distance of one k step
     uint32_t voff;         // per thread
     uint32_t lds_off;      // uniform per wave: byte offset of this wave's first 1 KiB block in the tile
-    __device__ __forceinline__ DirectLoader(const Operand<T>& op, int r0) {
+    int rows_left;         // BOUNDED: valid rows from this thread's first row on (may be <= 0)
+    __device__ __forceinline__ DirectLoader(const Operand<T>& op, int r0, const void* zero_page = nullptr) {
         const int q = threadIdx.x, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
         const int row = q / CPR, slot = q % CPR;
         if constexpr (KMAJOR) {
@@ -202,6 +243,8 @@ struct DirectLoader {
             k_bytes = op.sk * 2;
         }
         lds_off = (uint32_t)w * 1024u;
+        zero = reinterpret_cast<const char*>(zero_page);
+        rows_left = op.rows - r0 - row;
     }
     // stage starting at k0 -> tile at `lds_tile` (uniform)
     __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
@@ -210,8 +253,11 @@ struct DirectLoader {
         const char* g = base + (int64_t)k0 * k_bytes;
         char* l = reinterpret_cast<char*>(lds_tile) + lds_off;
 #pragma unroll
-        for (int i = 0; i < INSTR; ++i)
-            __builtin_amdgcn_global_load_lds((glb_vp)(g + i * step_bytes + voff), (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
+        for (int i = 0; i < INSTR; ++i) {
+            const char* src = g + i * step_bytes + voff;
+            if constexpr (BOUNDED) src = i * STEP < rows_left ? src : zero;
+            __builtin_amdgcn_global_load_lds((glb_vp)src, (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
+        }
     }
 };
 
@@ -273,7 +319,7 @@ __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, i
 // Accumulates the (2*WM*32) x (2*WN*32) tile at (m0, n0).  acc[wm][wn][r] of lane l belongs to
 //   m = m0 + wave_m*WM*32 + wm*32 + l%32,   n = n0 + wave_n*WN*32 + wn*32 + 8*(r/4) + 4*(l/32) + r%4.
 // NWN = waves along n (2 -> 4 waves per workgroup, 4 -> 8 waves); always 2 waves along m.
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false, int NWN = 2>
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false, int NWN = 2, int NSTAGES = 0>
 struct GemmMainloop {
     using Tr = GemmTraits<T>;
     static constexpr int THREADS = 2 * NWN * 64;
@@ -284,7 +330,7 @@ struct GemmMainloop {
     static constexpr int B_ELEMS = lds_tile_elems<T, B_KMAJOR>(TILE_N);
     static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
     static constexpr bool DIRECT = FULL && sizeof(T) == 2;     // global -> LDS without registers
-    static constexpr int NST = DIRECT ? 4 : 2;                  // LDS stages
+    static constexpr int NST = NSTAGES > 0 ? NSTAGES : (DIRECT ? 4 : 2);   // LDS stages
     static constexpr size_t LDS_BYTES = NST * (size_t)STAGE_ELEMS * sizeof(T);
 
     __device__ __forceinline__ static void run(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0, T* lds,
@@ -325,18 +371,24 @@ struct GemmMainloop {
     }
 
     // Whole aligned bf16 tiles: stages go from global memory straight into LDS (no staging
-    // registers, no ds_write).  NST LDS stages: while stage kt is consumed, stages kt+1 ..
-    // kt+NST-2 are in flight or landed and stage kt+NST-1 is issued into the buffer that stage
-    // kt-1 has just left.  One barrier per stage.
+    // registers, no ds_write).
     __device__ __forceinline__ static void run_direct(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0,
                                                       T* lds, f32x16_v (&acc)[WM][WN]) {
+        DirectLoader<A_KMAJOR, TILE_M, THREADS> la(A, m0);
+        DirectLoader<B_KMAJOR, TILE_N, THREADS> lb(B, n0);
+        run_pipeline(la, lb, K, lds, acc);
+    }
+
+    // Direct-to-LDS pipeline over loaders with an issue(k0, lds_tile) method and INSTR loads per
+    // thread and stage.  NST LDS stages: while stage kt is consumed, stages kt+1 .. kt+NST-2 are
+    // in flight or landed and stage kt+NST-1 is issued into the buffer that stage kt-1 has just
+    // left.  One barrier per stage.  K must be a multiple of BK.
+    template <class LA, class LB>
+    __device__ __forceinline__ static void run_pipeline(const LA& la, const LB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
+        static_assert(sizeof(T) == 2, "direct-to-LDS staging is implemented for bf16");
         const int w = threadIdx.x >> 6;
         const int wave_m = (w & 1) * (WM * 32), wave_n = (w >> 1) * (WN * 32);
         zero(acc);
-        using LA = DirectLoader<A_KMAJOR, TILE_M, THREADS>;
-        using LB = DirectLoader<B_KMAJOR, TILE_N, THREADS>;
-        LA la(A, m0);
-        LB lb(B, n0);
         constexpr int IPS = LA::INSTR + LB::INSTR;               // load instructions per thread and stage
         constexpr int PENDING = (NST - 2) * IPS;                 // loads of later stages that may stay in flight
         static_assert(PENDING < 64, "vmcnt range");
@@ -355,8 +407,8 @@ struct GemmMainloop {
             if (kt + NST - 2 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
             else __builtin_amdgcn_s_waitcnt(0);                  // tail: fewer stages are in flight
             // bare barrier: __syncthreads() would add a fence that drains every load in flight.
-            // This wave's share of stage kt has landed (wait above) and its LDS reads of stage
-            // kt-1 were consumed by MFMAs already, so nothing else has to be waited for.
+            // This wave's share of stage kt has landed and its LDS reads of stage kt-1 have
+            // returned (wait above), so nothing else has to be waited for.
             __builtin_amdgcn_s_barrier();
             if (kt + NST - 1 < KT) {
                 la.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS);
@@ -448,6 +500,15 @@ struct GemmMainloop {
             __syncthreads();
         }
         if (kt < KT) compute(buf0, buf0 + A_ELEMS);   // odd number of stages: the last one sits in buf0
+    }
+
+    // First m and n of this lane inside the tile at (m0, n0); element acc[i][j][r] belongs to
+    // m = lane_m + 32*i,  n = lane_n + 32*j + 8*(r/4) + r%4.
+    __device__ __forceinline__ static int lane_m(int m0) {
+        return m0 + ((threadIdx.x >> 6) & 1) * (WM * 32) + (threadIdx.x & 31);
+    }
+    __device__ __forceinline__ static int lane_n(int n0) {
+        return n0 + (threadIdx.x >> 7) * (WN * 32) + (((threadIdx.x & 63) >> 5) << 2);
     }
 
     // Calls f(m, n, value) for every element of the tile owned by this lane.

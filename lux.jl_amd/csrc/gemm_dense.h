@@ -12,20 +12,6 @@
 
 namespace luxhip {
 
-__device__ __forceinline__ float apply_act(int act, float x) {
-    switch (act) {
-        case LUXHIP_ACT_RELU: return Act<LUXHIP_ACT_RELU>::f(x);
-        case LUXHIP_ACT_TANH: return Act<LUXHIP_ACT_TANH>::f(x);
-        case LUXHIP_ACT_SIGMOID: return Act<LUXHIP_ACT_SIGMOID>::f(x);
-        case LUXHIP_ACT_SWISH: return Act<LUXHIP_ACT_SWISH>::f(x);
-        case LUXHIP_ACT_GELU: return Act<LUXHIP_ACT_GELU>::f(x);
-        case LUXHIP_ACT_SOFTPLUS: return Act<LUXHIP_ACT_SOFTPLUS>::f(x);
-        case LUXHIP_ACT_LOGSIGMOID: return Act<LUXHIP_ACT_LOGSIGMOID>::f(x);
-        case LUXHIP_ACT_LISHT: return Act<LUXHIP_ACT_LISHT>::f(x);
-        default: return x;
-    }
-}
-
 template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN>
 __global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
     using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN>;
@@ -36,13 +22,32 @@ __global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a
     const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
     f32x16_v acc[WM][WN];
     ML::run(a.A, a.B, a.K, m0, n0, lds, acc);
+    // epilogue: bias is per m (one value per lane and i), the column base per (j, r)
+    const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
+    float bv[WM];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) bv[i] = (a.bias && (FULL || mb + i * 32 < a.M)) ? ld(a.bias + mb + i * 32) : 0.0f;
     const int act = a.act;
-    ML::for_each(acc, m0, n0, [&](int m, int n, float v) {
-        if (FULL || (m < a.M && n < a.N)) {
-            if (a.bias) v += ld(a.bias + m);
-            const int64_t off = m + (int64_t)n * a.ldc;
-            if (a.pre) st(a.pre + off, v);
-            st(a.C + off, apply_act(act, v));
+    static_for<WN * 16>([&](auto JR) {
+        {
+            constexpr int j = decltype(JR)::value / 16, r = decltype(JR)::value % 16;
+            const int n = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
+            if (FULL || n < a.N) {
+                float v[WM];
+#pragma unroll
+                for (int i = 0; i < WM; ++i) v[i] = acc[i][j][r] + bv[i];
+                if (a.pre) {
+                    T* pcol = a.pre + (int64_t)n * a.ldc;
+#pragma unroll
+                    for (int i = 0; i < WM; ++i)
+                        if (FULL || mb + i * 32 < a.M) st(pcol + mb + i * 32, v[i]);
+                }
+                act_vec(act, v);
+                T* ccol = a.C + (int64_t)n * a.ldc;
+#pragma unroll
+                for (int i = 0; i < WM; ++i)
+                    if (FULL || mb + i * 32 < a.M) st(ccol + mb + i * 32, v[i]);
+            }
         }
     });
 }

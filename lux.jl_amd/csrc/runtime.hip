@@ -110,7 +110,7 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     }
     if (e.counters == nullptr) {
         void* c = nullptr;
-        constexpr size_t words = kWorkspaceCounters + kWorkspaceFlags;
+        constexpr size_t words = kWorkspaceCounters + kWorkspaceFlags + kWorkspaceZeroBytes / 4;
         LUX_CHECK_HIP(hipMalloc(&c, words * sizeof(uint32_t)));
         hipError_t rc = hipMemsetAsync(c, 0, words * sizeof(uint32_t), s);
         if (rc != hipSuccess) { (void)hipFree(c); LUX_CHECK_HIP(rc); }
@@ -119,6 +119,7 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     out->data = reinterpret_cast<char*>(e.base);
     out->counters = e.counters;
     out->flags = e.counters + kWorkspaceCounters;
+    out->zeros = e.counters + kWorkspaceCounters + kWorkspaceFlags;
     if (++e.epoch == 0) e.epoch = 1;   // 0 is what freshly cleared flags hold
     out->epoch = e.epoch;
     return LUXHIP_OK;

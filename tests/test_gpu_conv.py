@@ -48,6 +48,11 @@ CASES = [
     ((15, 13, 32, 2), (3, 3, 8, 64), 2, 1, 1, 4, False),
     ((12, 12, 24, 2), (5, 5, 24, 40), 1, 2, 2, 1, True),
     ((9, 9, 8, 5), (1, 1, 8, 16), 1, 0, 1, 1, False),
+    # channel counts per group that are multiples of the K stage (whole-tap kernels), with
+    # strides, dilation, asymmetric padding, groups, partial column tiles and > 128 columns
+    ((13, 11, 64, 3), (3, 2, 32, 64), (2, 1), (1, 0, 2, 1), (1, 2), 2, True),
+    ((10, 12, 64, 2), (3, 3, 32, 96), 1, (2, 1, 0, 2), 2, 2, False),
+    ((8, 8, 32, 5), (3, 3, 32, 320), 1, 1, 1, 1, False),
 ]
 
 
@@ -72,7 +77,7 @@ def test_conv_and_gradients(gpu, dtype, case):
 @pytest.mark.parametrize("act", ["identity", "sigmoid", "gelu", "relu"])
 def test_fused_conv_pullback(gpu, dtype, act):
     rng = np.random.default_rng(stable_seed(dtype, act))
-    for case in (1, 2, 5, 7):
+    for case in (1, 2, 5, 7, 10, 11):
         xs, ws, stride, pad, dil, groups, flip = CASES[case]
         gd, od = cdims(gpu, xs, ws, stride=stride, padding=pad, dilation=dil, groups=groups, flipkernel=flip)
         fan_in = ws[0] * ws[1] * ws[2]
