@@ -16,6 +16,7 @@ int num_cus();
 int64_t option_bn_resident();     // 1: single-pass batchnorm kernels for tensors that fit the register file
 int64_t option_bn_spin_limit();   // polls before a resident workgroup stops waiting for its peers
 int64_t option_gemm_tile();       // 0 automatic, else 82 | 42 | 22 | 11
+int64_t option_conv_tile();       // 0 automatic, else a tile code of the bf16 whole-tap convolution kernels
 
 // Per-stream scratch owned by the library (partial results of the reduction kernels,
 // per-channel coefficients).  get_workspace grows it on demand; kernels on one stream are
@@ -111,12 +112,13 @@ struct FastDiv {
 typedef uint16_t bf16_t;  // raw bfloat16 bits
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    // round to nearest even; NaN stays NaN
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+// round to nearest even, NaN stays NaN: v_cvt_pk_bf16_f32 of gfx950
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {   // lo in bits 15:0
+    const f32x2_hw v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_hw));
 }
 
 typedef uint32_t raw16_t __attribute__((ext_vector_type(4)));   // 16 bytes as they lie in memory
@@ -157,7 +159,7 @@ struct Vec<bf16_t> {
     __device__ __forceinline__ static raw16_t pack(const float (&v)[8]) {
         raw16_t r;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) r[i] = f32x2_to_bf16x2(v[2 * i], v[2 * i + 1]);
         return r;
     }
     __device__ __forceinline__ static void load(const bf16_t* p, float (&v)[8]) {
@@ -173,7 +175,7 @@ struct Vec<bf16_t> {
         uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            w[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+            w[i] = f32x2_to_bf16x2(v[2 * i], v[2 * i + 1]);
         *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 };

@@ -129,17 +129,18 @@ struct ConvGemmArgs {
 
 // Epilogue of fprop / dgrad: element (m = (p, q, n), col) -> out[(m - n*PQ) + PQ*(col_off + col +
 // Ctot_out*n)], with bias per output channel and the activation.  The image index of a row is
-// decoded once per row, the channel terms once per column.
-template <class ML, typename T, int WM, int WN>
-__device__ __forceinline__ void conv_epilogue(const f32x16_v (&acc)[WM][WN], int m0, int n0, int M, int PQ, FastDiv divPQ,
-                                              int Ncols, int col_off, int Ctot_out, const T* bias, T* out, T* pre, int act) {
+// decoded once per row, the channel terms once per column.  CHECK (tiles that stick out of the
+// matrix), HAS_ACT and HAS_PRE are resolved once per tile.
+template <class ML, typename T, int WM, int WN, bool CHECK, bool HAS_ACT, bool HAS_PRE>
+__device__ __forceinline__ void conv_epilogue_as(const f32x16_v (&acc)[WM][WN], int m0, int n0, int M, int PQ, FastDiv divPQ,
+                                                 int Ncols, int col_off, int Ctot_out, const T* bias, T* out, T* pre, int act) {
     const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
     int64_t rowoff[WM];
     bool mok[WM];
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
         const int m = mb + i * 32;
-        mok[i] = m < M;
+        mok[i] = !CHECK || m < M;
         const int n = (int)divPQ.div((uint32_t)(mok[i] ? m : 0));
         rowoff[i] = (int64_t)(m - n * PQ) + (int64_t)PQ * Ctot_out * n;
     }
@@ -147,41 +148,64 @@ __device__ __forceinline__ void conv_epilogue(const f32x16_v (&acc)[WM][WN], int
         {
             constexpr int j = decltype(JR)::value / 16, r = decltype(JR)::value % 16;
             const int col = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
-            if (col < Ncols) {
+            if (!CHECK || col < Ncols) {
                 const float b = bias ? ld(bias + col_off + col) : 0.0f;
                 const int64_t coloff = (int64_t)PQ * (col_off + col);
                 float v[WM];
 #pragma unroll
                 for (int i = 0; i < WM; ++i) v[i] = acc[i][j][r] + b;
-                if (pre) {
+                if constexpr (HAS_PRE) {
 #pragma unroll
                     for (int i = 0; i < WM; ++i)
-                        if (mok[i]) st(pre + coloff + rowoff[i], v[i]);
+                        if (!CHECK || mok[i]) st(pre + coloff + rowoff[i], v[i]);
                 }
-                act_vec(act, v);
+                if constexpr (HAS_ACT) act_vec(act, v);
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
-                    if (mok[i]) st(out + coloff + rowoff[i], v[i]);
+                    if (!CHECK || mok[i]) st(out + coloff + rowoff[i], v[i]);
             }
         }
     });
 }
+template <class ML, typename T, int WM, int WN>
+__device__ __forceinline__ void conv_epilogue(const f32x16_v (&acc)[WM][WN], int m0, int n0, int M, int PQ, FastDiv divPQ,
+                                              int Ncols, int col_off, int Ctot_out, const T* bias, T* out, T* pre, int act) {
+    const bool check = m0 + ML::TILE_M > M || n0 + ML::TILE_N > Ncols;
+    const bool has_act = act != LUXHIP_ACT_IDENTITY, has_pre = pre != nullptr;
+#define LUX_CONV_EPI(C, A, P) conv_epilogue_as<ML, T, WM, WN, C, A, P>(acc, m0, n0, M, PQ, divPQ, Ncols, col_off, Ctot_out, bias, out, pre, act)
+    if (check) {                                 // rare: general variants
+        if (has_pre) LUX_CONV_EPI(true, true, true);
+        else LUX_CONV_EPI(true, true, false);
+    } else if (!has_act && !has_pre) {
+        LUX_CONV_EPI(false, false, false);
+    } else if (!has_pre) {
+        LUX_CONV_EPI(false, true, false);
+    } else {
+        LUX_CONV_EPI(false, true, true);
+    }
+#undef LUX_CONV_EPI
+}
 
 // fprop and dgrad share this kernel (the gather loader's `dgrad` flag picks the index map).
+// Persistent: workgroup b handles tiles b, b + gridDim.x, ...
 template <typename T, int WM, int WN>
 __global__ __launch_bounds__(kGemmThreads) void conv_gemm_kernel(ConvGemmArgs<T> a) {
     using ML = GemmMainloop<T, WM, WN, true, true>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
-    int tm, tn;
-    tile_coords(a.tiles_m, a.tiles_n, tm, tn);
-    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
     const GatherK<T>& g = a.gather;
-    ConvGatherLoaderK<T, ML::TILE_M> la(g, m0, a.K);
-    typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
-    f32x16_v acc[WM][WN];
-    ML::run(la, lb, a.K, lds, acc);
-    conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
+    const int total = a.tiles_m * a.tiles_n;
+    for (int t = blockIdx.x; t < total; t += gridDim.x) {
+        int tm, tn;
+        tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
+        const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+        ConvGatherLoaderK<T, ML::TILE_M> la(g, m0, a.K);
+        typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
+        f32x16_v acc[WM][WN];
+        ML::run(la, lb, a.K, lds, acc);
+        conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
+        __syncthreads();   // every wave is done with the LDS stages before the next tile refills them
+    }
 }
 
 template <typename T, int WM, int WN>
@@ -190,15 +214,16 @@ int launch_conv_gemm(hipStream_t s, ConvGemmArgs<T>& a) {
     a.tiles_m = (int)ceil_div(a.gather.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.Ncols, ML::TILE_N);
     auto kernel = conv_gemm_kernel<T, WM, WN>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static int resident = 0;   // workgroups that fit the device at once
+    if (resident == 0) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)ML::LDS_BYTES));
-        attr_set = true;
+        resident = persistent_grid(kernel, kGemmThreads, ML::LDS_BYTES, int64_t(1) << 40);
     }
+    const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
     ProfScope ps(a.gather.dgrad ? (sizeof(T) == 2 ? "conv_dgrad_kernel<bf16>" : "conv_dgrad_kernel<f32>")
                                 : (sizeof(T) == 2 ? "conv_fprop_kernel<bf16>" : "conv_fprop_kernel<f32>"), s);
-    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(kGemmThreads), ML::LDS_BYTES, s>>>(a);
+    kernel<<<dim3((unsigned)grid), dim3(kGemmThreads), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }
@@ -281,8 +306,9 @@ struct ConvDirectLoaderK {
         const int row = q / CPR, slot = q % CPR;
         chunk_el = (slot ^ ((row >> 2) & 3)) * 8;     // STEP is a multiple of 16: same swizzle for every i
         lds_off = (uint32_t)w * 1024u;
-        rows.init(g, m0 + row, STEP);
+        move_to(m0);
     }
+    __device__ __forceinline__ void move_to(int m0) { rows.init(g, m0 + (int)threadIdx.x / CPR, STEP); }
     __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
         typedef __attribute__((address_space(3))) void* lds_vp;
         typedef const __attribute__((address_space(1))) void* glb_vp;
@@ -314,6 +340,7 @@ struct ConvTapLoaderK {
         chunk_el = (threadIdx.x % CPR) * Tr::VEC;
         rows.init(g, m0 + threadIdx.x / CPR, STEP);
     }
+    __device__ __forceinline__ ConvTapLoaderK(const ConvTapLoaderK&) = default;
     __device__ __forceinline__ void load(int k0) {
         const TapStage st(g, k0);
 #pragma unroll
@@ -345,44 +372,71 @@ struct ConvTapArgs {
     int tiles_m, tiles_n;
 };
 
-template <typename T, int WM, int WN, int NWN, int NST>
-__global__ __launch_bounds__(2 * NWN * 64) void conv_tap_kernel(ConvTapArgs<T> a) {
+// Persistent: workgroup b handles tiles b, b + gridDim.x, ...  On the direct-to-LDS path the
+// first stages of the next tile are issued before the epilogue of the current one.
+template <typename T, int WM, int WN, int NWN, int NST, int NWM>
+__global__ __launch_bounds__(NWM * NWN * 64) void conv_tap_kernel(ConvTapArgs<T> a) {
     constexpr bool DIRECT = sizeof(T) == 2;
-    using ML = GemmMainloop<T, WM, WN, true, true, DIRECT, NWN, NST>;
+    using ML = GemmMainloop<T, WM, WN, true, true, DIRECT, NWN, NST, NWM>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
-    int tm, tn;
-    tile_coords(a.tiles_m, a.tiles_n, tm, tn);
-    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
     const TapGeom<T>& g = a.tap;
+    const int total = a.tiles_m * a.tiles_n;
     f32x16_v acc[WM][WN];
+    int tm, tn;
     if constexpr (DIRECT) {
+        int t = blockIdx.x;
+        tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
+        int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
         ConvDirectLoaderK<ML::TILE_M, ML::THREADS> la(g, m0);
         DirectLoader<true, ML::TILE_N, ML::THREADS, true> lb(a.Wm, n0, g.zero);
-        ML::run_pipeline(la, lb, a.K, lds, acc);
+        ML::pipeline_fill(la, lb, a.K, lds);
+        for (;;) {
+            ML::pipeline_loop(la, lb, a.K, lds, acc);
+            const int tnext = t + gridDim.x;
+            int m0n = 0, n0n = 0;
+            if (tnext < total) {
+                tile_coords(tnext, a.tiles_m, a.tiles_n, tm, tn);
+                m0n = tm * ML::TILE_M;
+                n0n = tn * ML::TILE_N;
+                la.move_to(m0n);
+                lb.move_to(a.Wm, n0n);
+                ML::pipeline_drain();
+                ML::pipeline_fill(la, lb, a.K, lds);
+            }
+            conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
+            if (tnext >= total) break;
+            t = tnext; m0 = m0n; n0 = n0n;
+        }
     } else {
-        ConvTapLoaderK<T, ML::TILE_M, ML::THREADS> la(g, m0);
-        typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
-        ML::run(la, lb, a.K, lds, acc);
+        for (int t = blockIdx.x; t < total; t += gridDim.x) {
+            tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
+            const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+            ConvTapLoaderK<T, ML::TILE_M, ML::THREADS> la(g, m0);
+            typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
+            ML::run(la, lb, a.K, lds, acc);
+            conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
+            __syncthreads();   // every wave is done with the LDS stages before the next tile refills them
+        }
     }
-    conv_epilogue<ML, T, WM, WN>(acc, m0, n0, g.M, g.PQ, g.divPQ, a.Ncols, a.col_off, a.Ctot_out, a.bias, a.out, a.pre, a.act);
 }
 
-template <typename T, int WM, int WN, int NWN, int NST>
+template <typename T, int WM, int WN, int NWN, int NST, int NWM = 2>
 int launch_conv_tap(hipStream_t s, ConvTapArgs<T>& a) {
-    using ML = GemmMainloop<T, WM, WN, true, true, sizeof(T) == 2, NWN, NST>;
+    using ML = GemmMainloop<T, WM, WN, true, true, sizeof(T) == 2, NWN, NST, NWM>;
     a.tiles_m = (int)ceil_div(a.tap.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.Ncols, ML::TILE_N);
-    auto kernel = conv_tap_kernel<T, WM, WN, NWN, NST>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    auto kernel = conv_tap_kernel<T, WM, WN, NWN, NST, NWM>;
+    static int resident = 0;   // workgroups that fit the device at once
+    if (resident == 0) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)ML::LDS_BYTES));
-        attr_set = true;
+        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
     }
+    const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
     ProfScope ps(a.tap.dgrad ? (sizeof(T) == 2 ? "conv_dgrad_kernel<bf16>" : "conv_dgrad_kernel<f32>")
                              : (sizeof(T) == 2 ? "conv_fprop_kernel<bf16>" : "conv_fprop_kernel<f32>"), s);
-    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
+    kernel<<<dim3((unsigned)grid), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

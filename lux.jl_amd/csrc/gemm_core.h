@@ -27,6 +27,7 @@
 // all the instruction needs.
 #pragma once
 
+#include <algorithm>
 #include <type_traits>
 #include <utility>
 
@@ -232,19 +233,22 @@ struct DirectLoader {
         if constexpr (KMAJOR) {
             const int chunk = slot ^ ((row >> 2) & 3);
             voff = (uint32_t)(((int64_t)row * op.sr + chunk * 8) * 2);
-            base = reinterpret_cast<const char*>(op.p + (int64_t)r0 * op.sr);
             step_bytes = (int64_t)STEP * op.sr * 2;
             k_bytes = 2;
         } else {
             const int r = (slot * 8) ^ ((row & 3) << mn_swizzle_shift(ROWS));   // row = k within the pass
             voff = (uint32_t)(((int64_t)row * op.sk + r) * 2);
-            base = reinterpret_cast<const char*>(op.p + r0);
             step_bytes = (int64_t)STEP * op.sk * 2;
             k_bytes = op.sk * 2;
         }
         lds_off = (uint32_t)w * 1024u;
         zero = reinterpret_cast<const char*>(zero_page);
-        rows_left = op.rows - r0 - row;
+        move_to(op, r0);
+    }
+    // tile that starts at row r0 of the same operand
+    __device__ __forceinline__ void move_to(const Operand<T>& op, int r0) {
+        base = reinterpret_cast<const char*>(op.p + (KMAJOR ? (int64_t)r0 * op.sr : (int64_t)r0));
+        rows_left = op.rows - r0 - (int)threadIdx.x / CPR;
     }
     // stage starting at k0 -> tile at `lds_tile` (uniform)
     __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
@@ -301,12 +305,16 @@ __device__ __forceinline__ void load_frag_f32(const float* lds, int rbase, int k
 }
 
 // ----------------------------------------------------------------------------- tile -> C coordinates
-// XCD-aware ordering: consecutive workgroup ids land on different XCDs (8 of them, each with
-// its own L2), so ids are first regrouped per XCD and then walked in groups of 8 tiles along m.
-__device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int nb = gridDim.x, bid = blockIdx.x;
+// Tile `id` of `nb` = tiles_m * tiles_n tiles -> (tm, tn).  Workgroups walk the tiles in
+// strides of the grid size (a multiple of 8 whenever there are more tiles than workgroups), so
+// the tiles with id % 8 == x are all processed on XCD x (consecutive workgroup ids land on
+// different XCDs, 8 of them, each with its own L2).  Ids are therefore first regrouped per XCD
+// and then walked in groups of 8 tiles along m, which keeps the operand rows and columns that
+// one L2 sees close together.
+__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int nb = tiles_m * tiles_n;
     const int per = nb >> 3;
-    const int lid = bid < (per << 3) ? (bid & 7) * per + (bid >> 3) : bid;
+    const int lid = id < (per << 3) ? (id & 7) * per + (id >> 3) : id;
     constexpr int GROUP = 8;
     const int in_group = GROUP * tiles_n;
     const int first_m = (lid / in_group) * GROUP;
@@ -315,15 +323,26 @@ __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, i
     tn = (lid % in_group) / gsize;
 }
 
+// Workgroups of a persistent tile kernel: as many as stay resident at once, at most one per tile.
+template <typename Kernel>
+inline int persistent_grid(Kernel kernel, int threads, size_t lds_bytes, int64_t tiles) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds_bytes) != hipSuccess || per_cu < 1)
+        per_cu = 1;
+    const int64_t cus = num_cus() > 0 ? num_cus() : 256;
+    return (int)std::min<int64_t>(tiles, cus * per_cu);
+}
+
 // ----------------------------------------------------------------------------- mainloop
 // Accumulates the (2*WM*32) x (2*WN*32) tile at (m0, n0).  acc[wm][wn][r] of lane l belongs to
 //   m = m0 + wave_m*WM*32 + wm*32 + l%32,   n = n0 + wave_n*WN*32 + wn*32 + 8*(r/4) + 4*(l/32) + r%4.
-// NWN = waves along n (2 -> 4 waves per workgroup, 4 -> 8 waves); always 2 waves along m.
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false, int NWN = 2, int NSTAGES = 0>
+// NWM x NWN waves per workgroup (along m, along n); wave w sits at (w % NWM, w / NWM).
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false, int NWN = 2, int NSTAGES = 0,
+          int NWM = 2>
 struct GemmMainloop {
     using Tr = GemmTraits<T>;
-    static constexpr int THREADS = 2 * NWN * 64;
-    static constexpr int TILE_M = 2 * WM * 32, TILE_N = NWN * WN * 32;
+    static constexpr int THREADS = NWM * NWN * 64;
+    static constexpr int TILE_M = NWM * WM * 32, TILE_N = NWN * WN * 32;
     using PlainLoaderA = TileLoader<T, A_KMAJOR, TILE_M, FULL, THREADS>;
     using PlainLoaderB = TileLoader<T, B_KMAJOR, TILE_N, FULL, THREADS>;
     static constexpr int A_ELEMS = lds_tile_elems<T, A_KMAJOR>(TILE_M);
@@ -383,11 +402,30 @@ struct GemmMainloop {
     // thread and stage.  NST LDS stages: while stage kt is consumed, stages kt+1 .. kt+NST-2 are
     // in flight or landed and stage kt+NST-1 is issued into the buffer that stage kt-1 has just
     // left.  One barrier per stage.  K must be a multiple of BK.
+    //   pipeline_fill : issues the first NST-1 stages of a tile.  All waves must have finished
+    //                   reading the LDS stages of the previous tile (pipeline_drain).
+    //   pipeline_loop : consumes all stages of the tile; acc is overwritten.
+    // Other vector-memory operations of the wave that are still outstanding (the previous tile's
+    // epilogue stores) only make the vmcnt waits more conservative: loads return in order.
     template <class LA, class LB>
-    __device__ __forceinline__ static void run_pipeline(const LA& la, const LB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
+    __device__ __forceinline__ static void pipeline_fill(const LA& la, const LB& lb, int K, T* lds) {
         static_assert(sizeof(T) == 2, "direct-to-LDS staging is implemented for bf16");
+        const int KT = K / Tr::BK;
+#pragma unroll
+        for (int st = 0; st < NST - 1; ++st)
+            if (st < KT) {
+                la.issue(st * Tr::BK, lds + st * STAGE_ELEMS);
+                lb.issue(st * Tr::BK, lds + st * STAGE_ELEMS + A_ELEMS);
+            }
+    }
+    __device__ __forceinline__ static void pipeline_drain() {
+        __builtin_amdgcn_s_waitcnt(0xF | (0x7 << 4) | (0x3 << 14));   // lgkmcnt(0): own LDS reads returned
+        __builtin_amdgcn_s_barrier();
+    }
+    template <class LA, class LB>
+    __device__ __forceinline__ static void pipeline_loop(const LA& la, const LB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
         const int w = threadIdx.x >> 6;
-        const int wave_m = (w & 1) * (WM * 32), wave_n = (w >> 1) * (WN * 32);
+        const int wave_m = (w % NWM) * (WM * 32), wave_n = (w / NWM) * (WN * 32);
         zero(acc);
         constexpr int IPS = LA::INSTR + LB::INSTR;               // load instructions per thread and stage
         constexpr int PENDING = (NST - 2) * IPS;                 // loads of later stages that may stay in flight
@@ -396,12 +434,6 @@ struct GemmMainloop {
         // LDS reads of the previous stage before the barrier lets other waves refill that buffer
         constexpr int WAIT_IMM = (PENDING & 0xF) | (0x7 << 4) | ((PENDING >> 4) << 14);
         const int KT = K / Tr::BK;
-#pragma unroll
-        for (int st = 0; st < NST - 1; ++st)
-            if (st < KT) {
-                la.issue(st * Tr::BK, lds + st * STAGE_ELEMS);
-                lb.issue(st * Tr::BK, lds + st * STAGE_ELEMS + A_ELEMS);
-            }
         int cur = 0, fill = NST - 1;                             // buffer of stage kt, buffer to refill
         for (int kt = 0; kt < KT; ++kt) {
             if (kt + NST - 2 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
@@ -420,13 +452,18 @@ struct GemmMainloop {
             fill = fill + 1 == NST ? 0 : fill + 1;
         }
     }
+    template <class LA, class LB>
+    __device__ __forceinline__ static void run_pipeline(const LA& la, const LB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
+        pipeline_fill(la, lb, K, lds);
+        pipeline_loop(la, lb, K, lds, acc);
+    }
 
     // k range [0, K) in stages of BK; the loaders decide what a stage contains
     template <class LoaderA, class LoaderB>
     __device__ __forceinline__ static void run(LoaderA& la, LoaderB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
         static_assert(LoaderA::KMAJOR == A_KMAJOR && LoaderB::KMAJOR == B_KMAJOR, "loader layout mismatch");
         const int w = threadIdx.x >> 6;
-        const int wave_m = (w & 1) * (WM * 32), wave_n = (w >> 1) * (WN * 32);
+        const int wave_m = (w % NWM) * (WM * 32), wave_n = (w / NWM) * (WN * 32);
 #pragma unroll
         for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -505,18 +542,18 @@ struct GemmMainloop {
     // First m and n of this lane inside the tile at (m0, n0); element acc[i][j][r] belongs to
     // m = lane_m + 32*i,  n = lane_n + 32*j + 8*(r/4) + r%4.
     __device__ __forceinline__ static int lane_m(int m0) {
-        return m0 + ((threadIdx.x >> 6) & 1) * (WM * 32) + (threadIdx.x & 31);
+        return m0 + ((threadIdx.x >> 6) % NWM) * (WM * 32) + (threadIdx.x & 31);
     }
     __device__ __forceinline__ static int lane_n(int n0) {
-        return n0 + (threadIdx.x >> 7) * (WN * 32) + (((threadIdx.x & 63) >> 5) << 2);
+        return n0 + ((threadIdx.x >> 6) / NWM) * (WN * 32) + (((threadIdx.x & 63) >> 5) << 2);
     }
 
     // Calls f(m, n, value) for every element of the tile owned by this lane.
     template <typename F>
     __device__ __forceinline__ static void for_each(const f32x16_v (&acc)[WM][WN], int m0, int n0, F&& f) {
         const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
-        const int mb = m0 + (w & 1) * (WM * 32) + (l & 31);
-        const int nb = n0 + (w >> 1) * (WN * 32) + ((l >> 5) << 2);
+        const int mb = m0 + (w % NWM) * (WM * 32) + (l & 31);
+        const int nb = n0 + (w / NWM) * (WN * 32) + ((l >> 5) << 2);
 #pragma unroll
         for (int i = 0; i < WM; ++i)
 #pragma unroll

@@ -12,44 +12,90 @@
 
 namespace luxhip {
 
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN>
-__global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
-    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN>;
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    T* lds = reinterpret_cast<T*>(lds_raw);
-    int tm, tn;
-    tile_coords(a.tiles_m, a.tiles_n, tm, tn);
-    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
-    f32x16_v acc[WM][WN];
-    ML::run(a.A, a.B, a.K, m0, n0, lds, acc);
-    // epilogue: bias is per m (one value per lane and i), the column base per (j, r)
+// Epilogue of one tile: C = act(acc + bias), optional pre-activation copy.  CHECK: bounds tests;
+// HAS_ACT / HAS_PRE are resolved once per tile, so the per-element code has no branches.
+template <class ML, typename T, int WM, int WN, bool CHECK, bool HAS_ACT, bool HAS_PRE>
+__device__ __forceinline__ void dense_epilogue_as(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int m0, int n0) {
     const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
     float bv[WM];
 #pragma unroll
-    for (int i = 0; i < WM; ++i) bv[i] = (a.bias && (FULL || mb + i * 32 < a.M)) ? ld(a.bias + mb + i * 32) : 0.0f;
+    for (int i = 0; i < WM; ++i) bv[i] = (a.bias && (!CHECK || mb + i * 32 < a.M)) ? ld(a.bias + mb + i * 32) : 0.0f;
     const int act = a.act;
     static_for<WN * 16>([&](auto JR) {
         {
             constexpr int j = decltype(JR)::value / 16, r = decltype(JR)::value % 16;
             const int n = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
-            if (FULL || n < a.N) {
+            if (!CHECK || n < a.N) {
                 float v[WM];
 #pragma unroll
                 for (int i = 0; i < WM; ++i) v[i] = acc[i][j][r] + bv[i];
-                if (a.pre) {
-                    T* pcol = a.pre + (int64_t)n * a.ldc;
+                if constexpr (HAS_PRE) {
+                    T* pcol = a.pre + (int64_t)n * a.ldc + mb;
 #pragma unroll
                     for (int i = 0; i < WM; ++i)
-                        if (FULL || mb + i * 32 < a.M) st(pcol + mb + i * 32, v[i]);
+                        if (!CHECK || mb + i * 32 < a.M) st(pcol + i * 32, v[i]);
                 }
-                act_vec(act, v);
-                T* ccol = a.C + (int64_t)n * a.ldc;
+                if constexpr (HAS_ACT) act_vec(act, v);
+                T* ccol = a.C + (int64_t)n * a.ldc + mb;
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
-                    if (FULL || mb + i * 32 < a.M) st(ccol + mb + i * 32, v[i]);
+                    if (!CHECK || mb + i * 32 < a.M) st(ccol + i * 32, v[i]);
             }
         }
     });
+}
+template <class ML, typename T, int WM, int WN, bool FULL>
+__device__ __forceinline__ void dense_epilogue(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int m0, int n0) {
+    const bool has_act = a.act != LUXHIP_ACT_IDENTITY, has_pre = a.pre != nullptr;
+    if (!has_act && !has_pre) dense_epilogue_as<ML, T, WM, WN, !FULL, false, false>(acc, a, m0, n0);
+    else if (!has_pre) dense_epilogue_as<ML, T, WM, WN, !FULL, true, false>(acc, a, m0, n0);
+    else dense_epilogue_as<ML, T, WM, WN, !FULL, true, true>(acc, a, m0, n0);
+}
+
+// Persistent: workgroup b handles tiles b, b + gridDim.x, ...  On the direct-to-LDS path the
+// first stages of the next tile are issued before the epilogue of the current one, so the
+// stores overlap with the loads.
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN>
+__global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN>;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    const int total = a.tiles_m * a.tiles_n;
+    f32x16_v acc[WM][WN];
+    int tm, tn;
+    if constexpr (ML::DIRECT) {
+        int t = blockIdx.x;
+        tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
+        int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+        DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(a.A, m0);
+        DirectLoader<B_KMAJOR, ML::TILE_N, ML::THREADS> lb(a.B, n0);
+        ML::pipeline_fill(la, lb, a.K, lds);
+        for (;;) {
+            ML::pipeline_loop(la, lb, a.K, lds, acc);
+            const int tnext = t + gridDim.x;
+            int m0n = 0, n0n = 0;
+            if (tnext < total) {
+                tile_coords(tnext, a.tiles_m, a.tiles_n, tm, tn);
+                m0n = tm * ML::TILE_M;
+                n0n = tn * ML::TILE_N;
+                la.move_to(a.A, m0n);
+                lb.move_to(a.B, n0n);
+                ML::pipeline_drain();
+                ML::pipeline_fill(la, lb, a.K, lds);
+            }
+            dense_epilogue<ML, T, WM, WN, FULL>(acc, a, m0, n0);
+            if (tnext >= total) break;
+            t = tnext; m0 = m0n; n0 = n0n;
+        }
+    } else {
+        for (int t = blockIdx.x; t < total; t += gridDim.x) {
+            tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
+            const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+            ML::run(a.A, a.B, a.K, m0, n0, lds, acc);
+            dense_epilogue<ML, T, WM, WN, FULL>(acc, a, m0, n0);
+            __syncthreads();   // every wave is done with the LDS stages before the next tile refills them
+        }
+    }
 }
 
 template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL, int NWN = 2>
@@ -58,14 +104,15 @@ int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
     auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL, NWN>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static int resident = 0;   // workgroups that fit the device at once
+    if (resident == 0) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)ML::LDS_BYTES));
-        attr_set = true;
+        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
     }
+    const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
     ProfScope ps(sizeof(T) == 2 ? "dense_gemm_kernel<bf16>" : "dense_gemm_kernel<f32>", s);
-    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
+    kernel<<<dim3((unsigned)grid), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

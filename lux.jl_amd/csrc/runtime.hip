@@ -78,10 +78,11 @@ bool initialized() { return g_init; }
 int num_cus() { return g_cus; }
 
 namespace {
-std::atomic<int64_t> g_opt_bn_resident{1}, g_opt_bn_spin_limit{int64_t(1) << 22}, g_opt_gemm_tile{-1};
+std::atomic<int64_t> g_opt_bn_resident{1}, g_opt_bn_spin_limit{int64_t(1) << 22}, g_opt_gemm_tile{-1}, g_opt_conv_tile{0};
 }
 int64_t option_bn_resident() { return g_opt_bn_resident.load(); }
 int64_t option_bn_spin_limit() { return g_opt_bn_spin_limit.load(); }
+int64_t option_conv_tile() { return g_opt_conv_tile.load(); }
 int64_t option_gemm_tile() {
     int64_t v = g_opt_gemm_tile.load();
     if (v < 0) {   // not set through the API: the environment variable LUXHIP_GEMM_TILE, read once
@@ -192,6 +193,10 @@ int luxhip_set_option(const char* name, int64_t value) {
         LUX_INVALID_IF(value != 0 && value != 82 && value != 42 && value != 22 && value != 11,
                        "set_option: gemm_tile must be 0, 82, 42, 22 or 11");
         g_opt_gemm_tile.store(value);
+    } else if (strcmp(name, "conv_tile") == 0) {
+        LUX_INVALID_IF(value != 0 && value != 82 && value != 83 && value != 84 && value != 42,
+                       "set_option: conv_tile must be 0, 82, 83, 84 or 42");
+        g_opt_conv_tile.store(value);
     } else {
         return set_error(LUXHIP_INVALID, "set_option: unknown option '%s'", name);
     }
