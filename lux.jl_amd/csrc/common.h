@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/luxhip.h"
 
 namespace luxhip {
@@ -198,7 +200,11 @@ __device__ __forceinline__ void st<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf1
 // and the pre-activation `x`.
 template <int ACT>
 struct Act;
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+// 1 / (1 + e^-x) with the hardware exponential and reciprocal (about 2 ulp each); the argument
+// is clamped so that e^-x stays finite
+__device__ __forceinline__ float sigmoidf_(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-fmaxf(x, -80.0f)));
+}
 template <>
 struct Act<LUXHIP_ACT_IDENTITY> {
     static constexpr bool needs_pre = false;
@@ -289,10 +295,24 @@ inline bool act_needs_pre(int act) {
 // ----------------------------------------------------------------------------- reductions
 constexpr int kWave = 64;
 
+// Sum over the 64 lanes of a wave, every lane receives the total.  Data-parallel-primitive
+// moves inside the VALU (no trip through the LDS crossbar): butterfly inside each row of 16
+// lanes, then the row totals are passed along (row_bcast15, row_bcast31) so that lane 63 holds
+// the wave total, which a scalar read broadcasts.  Fixed order: same result on every run.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    auto dpp_add = [](float x, auto ctrl, auto row_mask, auto bound) {
+        const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value, decltype(row_mask)::value,
+                                                  0xF, decltype(bound)::value);
+        return x + __int_as_float(t);
+    };
+    using std::integral_constant;
+    v = dpp_add(v, integral_constant<int, 0xB1>{}, integral_constant<int, 0xF>{}, integral_constant<bool, true>{});    // quad_perm [1,0,3,2]
+    v = dpp_add(v, integral_constant<int, 0x4E>{}, integral_constant<int, 0xF>{}, integral_constant<bool, true>{});    // quad_perm [2,3,0,1]
+    v = dpp_add(v, integral_constant<int, 0x141>{}, integral_constant<int, 0xF>{}, integral_constant<bool, true>{});   // row_half_mirror
+    v = dpp_add(v, integral_constant<int, 0x140>{}, integral_constant<int, 0xF>{}, integral_constant<bool, true>{});   // row_mirror
+    v = dpp_add(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{}, integral_constant<bool, false>{});  // row_bcast15 -> rows 1, 3
+    v = dpp_add(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{}, integral_constant<bool, false>{});  // row_bcast31 -> rows 2, 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // Sum over the workgroup; every thread receives the total.  `smem` needs blockDim.x/64

@@ -33,6 +33,49 @@ __global__ __launch_bounds__(256) void whcn_to_cwhn_kernel(const T* __restrict__
     }
 }
 
+// Same transform with 16-byte global accesses on both sides (P and C multiples of the vector
+// length, aligned pointers): a 64(p) x 64(c) tile goes through LDS as tile[c][p]; the row pitch
+// (66 two-byte or 65 four-byte elements) spreads the strided reads of the second phase over
+// the banks.
+template <typename T>
+__global__ __launch_bounds__(256) void whcn_to_cwhn_vec_kernel(const T* __restrict__ in, T* __restrict__ out, int P, int C) {
+    constexpr int V = 16 / sizeof(T), TP = 64, TC = 64;
+    constexpr int PITCH = TP + 4 / sizeof(T);   // 66 (bf16) / 65 (fp32) elements: rows stay 4-byte aligned
+    __shared__ __align__(16) T tile[TC * PITCH];
+    const int n = blockIdx.z;
+    const int p0 = blockIdx.x * TP, c0 = blockIdx.y * TC;
+    const T* src = in + (size_t)n * C * P;
+    T* dst = out + (size_t)n * C * P;
+    // phase 1: vectors along p
+    constexpr int VP = TP / V;                       // vectors per tile row
+#pragma unroll
+    for (int it = 0; it < TC * VP / 256; ++it) {
+        const int idx = threadIdx.x + it * 256;
+        const int c = idx / VP, pv = idx % VP;
+        if (c0 + c < C && p0 + pv * V < P) {
+            const raw16_t v = *reinterpret_cast<const raw16_t*>(src + (size_t)(c0 + c) * P + p0 + pv * V);
+            uint32_t* row = reinterpret_cast<uint32_t*>(tile + c * PITCH + pv * V);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) row[k] = v[k];
+        }
+    }
+    __syncthreads();
+    // phase 2: vectors along c
+    constexpr int VC = TC / V;
+#pragma unroll
+    for (int it = 0; it < TP * VC / 256; ++it) {
+        const int idx = threadIdx.x + it * 256;
+        const int pp = idx / VC, cv = idx % VC;
+        if (p0 + pp < P && c0 + cv * V < C) {
+            raw16_t r;
+            T* e = reinterpret_cast<T*>(&r);
+#pragma unroll
+            for (int k = 0; k < V; ++k) e[k] = tile[(cv * V + k) * PITCH + pp];
+            *reinterpret_cast<raw16_t*>(dst + (size_t)(p0 + pp) * C + c0 + cv * V) = r;
+        }
+    }
+}
+
 // wF[(co*T + t)*Cin_g + ci] (fprop, K = T*Cin_g) or wD[((g*Cin_g + ci)*T + t)*Cout_g + col]
 // (dgrad, K = T*Cout_g) from w[a + kW*(b + kH*(ci + Cin_g*co))]; tap t = ka + kW*kb with
 // a = flip ? ka : kW-1-ka (same for b).
@@ -104,9 +147,13 @@ static inline size_t align256(size_t b) { return (b + 255) & ~size_t(255); }
 template <typename T>
 static int transpose_to_cwhn(hipStream_t s, const T* in, T* out, int P, int C, int N) {
     ProfScope ps("whcn_to_cwhn_kernel", s);
-    dim3 grid((unsigned)ceil_div(P, 32), (unsigned)ceil_div(C, 32), (unsigned)N);
+    constexpr int V = 16 / (int)sizeof(T);
+    const bool vec = P % V == 0 && C % V == 0 && aligned16(in) && aligned16(out);
+    const int tile = vec ? 64 : 32;
+    dim3 grid((unsigned)ceil_div(P, tile), (unsigned)ceil_div(C, tile), (unsigned)N);
     LUX_UNSUPPORTED_IF(grid.y > 65535 || grid.z > 65535, "conv: too many channels or images for the layout transform");
-    whcn_to_cwhn_kernel<T><<<grid, 256, 0, s>>>(in, out, P, C);
+    if (vec) whcn_to_cwhn_vec_kernel<T><<<grid, 256, 0, s>>>(in, out, P, C);
+    else whcn_to_cwhn_kernel<T><<<grid, 256, 0, s>>>(in, out, P, C);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

@@ -128,7 +128,7 @@ __device__ __forceinline__ void wave_channel_accumulate(float* accg, float* accb
     unsigned long long todo = __ballot(active);
     while (todo) {
         const int first = __ffsll((long long)todo) - 1;
-        const uint32_t j0 = __shfl(j, first, kWave);
+        const uint32_t j0 = (uint32_t)__builtin_amdgcn_readlane((int)j, first);   // first is uniform
         const bool sel = active && j == j0;
         const float ta = wave_sum(sel ? a : 0.0f);
         const float tb = wave_sum(sel ? b : 0.0f);
@@ -206,6 +206,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                         const float xh = (v[u][e] - mean) * invstd;
                         s1 += gv[e];
                         s2 = fmaf(gv[e], xh, s2);
+                        d[u][e] = gv[e];            // dy * gamma replaces delta: the second pass needs only this
                     }
                 }
                 if constexpr (AFFINE) {
@@ -254,7 +255,15 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = u * T_ + threadIdx.x;
-            if (q < g.nvec) emit(q, d[u], v[u]);
+            if (q < g.nvec) {                       // d[u] holds dy * gamma
+                float o[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float xh = (v[u][e] - mean) * invstd;
+                    o[e] = invstd * (d[u][e] - s1 - xh * s2);
+                }
+                gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
+            }
         }
     } else {
         for (uint32_t q = threadIdx.x; q < g.nvec; q += T_) {

@@ -36,12 +36,17 @@ struct WsEntry {
 };
 std::map<hipStream_t, WsEntry> g_ws;
 
+// One event is recorded after every profiled launch; a launch that directly follows another
+// profiled launch on the same stream takes that event as its start, so a launch costs one event
+// record and its time runs from the end of its predecessor to its own end.
 struct ProfEntry {
     const char* name;
-    hipEvent_t a, b;
+    hipStream_t stream;
+    int a, b;   // indices into g_prof_events, b < 0 while the scope is open
 };
 bool g_prof = false;
 std::vector<ProfEntry> g_prof_entries;
+std::vector<hipEvent_t> g_prof_events;
 
 size_t round_size(size_t b) {
     if (b == 0) b = 1;
@@ -50,20 +55,30 @@ size_t round_size(size_t b) {
 }
 }  // namespace
 
+static int prof_record(hipStream_t s) {   // g_mu held
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return -1;
+    if (hipEventRecord(e, s) != hipSuccess) { (void)hipEventDestroy(e); return -1; }
+    g_prof_events.push_back(e);
+    return (int)g_prof_events.size() - 1;
+}
 ProfScope::ProfScope(const char* n, hipStream_t s) : name(n), stream(s), active(g_prof) {
     if (!active) return;
-    ProfEntry e{n, nullptr, nullptr};
-    if (hipEventCreate(&e.a) != hipSuccess || hipEventCreate(&e.b) != hipSuccess) { active = false; return; }
-    (void)hipEventRecord(e.a, s);
     std::lock_guard<std::mutex> lk(g_mu);
-    g_prof_entries.push_back(e);
+    int a = -1;
+    if (!g_prof_entries.empty() && g_prof_entries.back().stream == s && g_prof_entries.back().b >= 0)
+        a = g_prof_entries.back().b;
+    else
+        a = prof_record(s);
+    if (a < 0) { active = false; return; }
+    g_prof_entries.push_back(ProfEntry{n, s, a, -1});
 }
 ProfScope::~ProfScope() {
     if (!active) return;
     std::lock_guard<std::mutex> lk(g_mu);
-    // the matching entry is the last one with this name and stream still open
+    // the matching entry is the last one with this name still open
     for (auto it = g_prof_entries.rbegin(); it != g_prof_entries.rend(); ++it)
-        if (it->name == name) { (void)hipEventRecord(it->b, stream); break; }
+        if (it->name == name && it->b < 0) { it->b = prof_record(stream); break; }
 }
 
 int set_error(int status, const char* fmt, ...) {
@@ -285,15 +300,15 @@ int luxhip_profile_report(char* buf, size_t len) {
     std::map<std::string, Agg> agg;
     for (auto& e : g_prof_entries) {
         float ms = 0.0f;
-        if (hipEventElapsedTime(&ms, e.a, e.b) == hipSuccess) {
+        if (e.a >= 0 && e.b >= 0 && hipEventElapsedTime(&ms, g_prof_events[e.a], g_prof_events[e.b]) == hipSuccess) {
             Agg& a = agg[e.name];
             a.count++; a.total += ms;
             if (ms < a.mn) a.mn = ms;
             if (ms > a.mx) a.mx = ms;
         }
-        (void)hipEventDestroy(e.a);
-        (void)hipEventDestroy(e.b);
     }
+    for (hipEvent_t ev : g_prof_events) (void)hipEventDestroy(ev);
+    g_prof_events.clear();
     g_prof_entries.clear();
     size_t off = 0;
     off += snprintf(buf + off, len - off, "[");
