@@ -372,21 +372,27 @@ struct GemmMainloop {
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
     }
 
+    // All fragment reads of the stage are issued up front (LDS returns in order, so the MFMAs of
+    // the first k-step start while the reads of the second are still in flight).
     __device__ __forceinline__ static void compute_bf16(const bf16_t* As, const bf16_t* Bs, int wave_m, int wave_n,
                                                         f32x16_v (&acc)[WM][WN]) {
+        constexpr int KK = Tr::BK / 16;
+        bf16x8_v fa[KK][WM], fb[KK][WN];
 #pragma unroll
-        for (int kk = 0; kk < Tr::BK / 16; ++kk) {
-            bf16x8_v fa[WM], fb[WN];
+        for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
-            for (int i = 0; i < WM; ++i) fa[i] = load_frag_bf16<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kk);
+            for (int j = 0; j < WN; ++j) fb[kk][j] = load_frag_bf16<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kk);
 #pragma unroll
-            for (int j = 0; j < WN; ++j) fb[j] = load_frag_bf16<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kk);
+            for (int i = 0; i < WM; ++i) fa[kk][i] = load_frag_bf16<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kk);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // keep the reads ahead of the MFMAs (the scheduler would sink them to save registers)
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
             for (int i = 0; i < WM; ++i)
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
-        }
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
     }
 
     // Whole aligned bf16 tiles: stages go from global memory straight into LDS (no staging

@@ -55,9 +55,9 @@ __device__ __forceinline__ void dense_epilogue(const f32x16_v (&acc)[WM][WN], co
 // Persistent: workgroup b handles tiles b, b + gridDim.x, ...  On the direct-to-LDS path the
 // first stages of the next tile are issued before the epilogue of the current one, so the
 // stores overlap with the loads.
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN>
-__global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
-    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN>;
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
+__global__ __launch_bounds__(NWM * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
     const int total = a.tiles_m * a.tiles_n;
@@ -98,12 +98,12 @@ __global__ __launch_bounds__(2 * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a
     }
 }
 
-template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL, int NWN = 2>
+template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL, int NWN = 2, int NWM = 2>
 int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
-    using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL, NWN>;
+    using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL, NWN, 0, NWM>;
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
-    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL, NWN>;
+    auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL, NWN, NWM>;
     static int resident = 0;   // workgroups that fit the device at once
     if (resident == 0) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
