@@ -213,6 +213,27 @@ __global__ __launch_bounds__(64) void plane_finalize_kernel(const float* __restr
     if (threadIdx.x == 0) st(dbias + c, acc);
 }
 
+// I == 1 (dense layout): dbias[c] = sum_s partial[s][c] with threads along c.  Workgroup of 64
+// channels x 16 slice groups: group g adds slices g, g+16, ...; the group sums are added in order.
+template <typename T>
+__global__ __launch_bounds__(1024) void plane_finalize_dense_kernel(const float* __restrict__ partial, T* dbias, uint32_t C,
+                                                                    uint32_t S) {
+    __shared__ float sg[16][64];
+    const uint32_t cx = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const uint32_t c = blockIdx.x * 64 + cx;
+    float t = 0.0f;
+    if (c < C)
+        for (uint32_t s = grp; s < S; s += 16) t += partial[(size_t)s * C + c];
+    sg[grp][cx] = t;
+    __syncthreads();
+    if (grp == 0 && c < C) {
+        t = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 16; ++g) t += sg[g][cx];
+        st(dbias + c, t);
+    }
+}
+
 static inline unsigned grid_for(uint32_t total_vec) {
     return (unsigned)ceil_div(total_vec, kThreads * kUnroll);
 }
@@ -360,7 +381,8 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
 #undef LAUNCH_PL
     LUX_CHECK_LAUNCH();
     ProfScope ps2("plane_finalize_kernel", s);
-    plane_finalize_kernel<T><<<(unsigned)C, 64, 0, s>>>(partial, dbias, (uint32_t)P, (uint32_t)I, (uint32_t)S);
+    if (I == 1) plane_finalize_dense_kernel<T><<<(unsigned)ceil_div(C, 64), 1024, 0, s>>>(partial, dbias, (uint32_t)C, (uint32_t)S);
+    else plane_finalize_kernel<T><<<(unsigned)C, 64, 0, s>>>(partial, dbias, (uint32_t)P, (uint32_t)I, (uint32_t)S);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

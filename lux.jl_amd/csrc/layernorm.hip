@@ -27,6 +27,21 @@ __device__ __forceinline__ void ln_store(T* p, size_t off, const float (&v)[VEC]
     else Vec<T>::store(p + off, v);
 }
 
+// A vector kept in registers between the passes: the 16 bytes as they lie in memory (bf16 stays
+// packed, which halves the register footprint), or one float for the scalar kernels.
+template <typename T, int VEC>
+struct Kept {
+    using type = raw16_t;
+    __device__ __forceinline__ static type load(const T* p, size_t off) { return *reinterpret_cast<const raw16_t*>(p + off); }
+    __device__ __forceinline__ static void get(const type& k, float (&v)[VEC]) { Vec<T>::unpack(k, v); }
+};
+template <typename T>
+struct Kept<T, 1> {
+    using type = float;
+    __device__ __forceinline__ static type load(const T* p, size_t off) { return ld(p + off); }
+    __device__ __forceinline__ static void get(const type& k, float (&v)[1]) { v[0] = k; }
+};
+
 // Sum over the threads that share a column: the wave (WAVE) or the workgroup.
 template <bool WAVE>
 __device__ __forceinline__ float col_sum(float v, float* sm) {
@@ -36,7 +51,7 @@ __device__ __forceinline__ float col_sum(float v, float* sm) {
 
 // ------------------------------------------------------------------------------- forward
 template <typename T, int ACT, int VEC, bool WAVE, bool CACHED>
-__global__ void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, T* y,
+__global__ __launch_bounds__(WAVE ? 256 : 1024) void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, T* y,
                               float* save_mean, float* save_invstd, uint32_t nvec, uint32_t R, float inv_L, float eps) {
     __shared__ float sm[16];
     const uint32_t tpc = WAVE ? 64u : blockDim.x;                       // threads per column
@@ -44,20 +59,20 @@ __global__ void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
     const uint32_t r = WAVE ? blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6) : blockIdx.x;
     if (r >= R) return;                                                 // whole waves / workgroups only
     const size_t base = (size_t)r * nvec * VEC;
-    float v[CACHED ? kLnCache : 1][VEC];
+    using K = Kept<T, VEC>;
+    typename K::type kv[CACHED ? kLnCache : 1];   // cached: the column; loads past its end re-read the last vector
+    float v[1][VEC];
     float sum = 0.0f;
     if constexpr (CACHED) {
 #pragma unroll
-        for (int u = 0; u < kLnCache; ++u) {
-            const uint32_t q = u * tpc + t;
-            if (q < nvec) ln_load<T, VEC>(x, base + (size_t)q * VEC, v[u]);
-        }
+        for (int u = 0; u < kLnCache; ++u) kv[u] = K::load(x, base + (size_t)min(u * tpc + t, nvec - 1) * VEC);
 #pragma unroll
         for (int u = 0; u < kLnCache; ++u) {
             const uint32_t q = u * tpc + t;
             if (q < nvec) {
+                K::get(kv[u], v[0]);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) sum += v[u][e];
+                for (int e = 0; e < VEC; ++e) sum += v[0][e];
             }
         }
     } else {
@@ -74,8 +89,9 @@ __global__ void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
         for (int u = 0; u < kLnCache; ++u) {
             const uint32_t q = u * tpc + t;
             if (q < nvec) {
+                K::get(kv[u], v[0]);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) dev = fmaf(v[u][e] - mean, v[u][e] - mean, dev);
+                for (int e = 0; e < VEC; ++e) dev = fmaf(v[0][e] - mean, v[0][e] - mean, dev);
             }
         }
     } else {
@@ -109,7 +125,10 @@ __global__ void ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
 #pragma unroll
         for (int u = 0; u < kLnCache; ++u) {
             const uint32_t q = u * tpc + t;
-            if (q < nvec) emit(q, v[u]);
+            if (q < nvec) {
+                K::get(kv[u], v[0]);
+                emit(q, v[0]);
+            }
         }
     } else {
         for (uint32_t q = t; q < nvec; q += tpc) {
@@ -145,7 +164,7 @@ __device__ __forceinline__ void ln_dy(const T* gamma, const T* beta, uint32_t q,
 }
 
 template <typename T, int ACT, int VEC, bool WAVE, bool CACHED>
-__global__ void ln_bwd_dx_kernel(const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma,
+__global__ __launch_bounds__(WAVE ? 256 : 1024) void ln_bwd_dx_kernel(const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma,
                                  const T* __restrict__ beta, const float* __restrict__ save_mean,
                                  const float* __restrict__ save_invstd, T* dx, uint32_t nvec, uint32_t R, float inv_L) {
     __shared__ float sm[16];
@@ -155,7 +174,9 @@ __global__ void ln_bwd_dx_kernel(const T* __restrict__ delta, const T* __restric
     if (r >= R) return;
     const size_t base = (size_t)r * nvec * VEC;
     const float mean = save_mean[r], invstd = save_invstd[r];
-    float d[CACHED ? kLnCache : 1][VEC], v[CACHED ? kLnCache : 1][VEC];
+    using K = Kept<T, VEC>;
+    typename K::type kd[CACHED ? kLnCache : 1], kv[CACHED ? kLnCache : 1];
+    float d[1][VEC], v[1][VEC];
     float s1 = 0.0f, s2 = 0.0f;
     auto accumulate = [&](uint32_t q, const float (&dv)[VEC], const float (&xv)[VEC]) {
         float dy[VEC], gm[VEC];
@@ -170,16 +191,18 @@ __global__ void ln_bwd_dx_kernel(const T* __restrict__ delta, const T* __restric
     if constexpr (CACHED) {
 #pragma unroll
         for (int u = 0; u < kLnCache; ++u) {
-            const uint32_t q = u * tpc + t;
-            if (q < nvec) {
-                ln_load<T, VEC>(delta, base + (size_t)q * VEC, d[u]);
-                ln_load<T, VEC>(x, base + (size_t)q * VEC, v[u]);
-            }
+            const size_t off = base + (size_t)min(u * tpc + t, nvec - 1) * VEC;   // past the end: re-read the last vector
+            kd[u] = K::load(delta, off);
+            kv[u] = K::load(x, off);
         }
 #pragma unroll
         for (int u = 0; u < kLnCache; ++u) {
             const uint32_t q = u * tpc + t;
-            if (q < nvec) accumulate(q, d[u], v[u]);
+            if (q < nvec) {
+                K::get(kd[u], d[0]);
+                K::get(kv[u], v[0]);
+                accumulate(q, d[0], v[0]);
+            }
         }
     } else {
         for (uint32_t q = t; q < nvec; q += tpc) {
@@ -204,7 +227,11 @@ __global__ void ln_bwd_dx_kernel(const T* __restrict__ delta, const T* __restric
 #pragma unroll
         for (int u = 0; u < kLnCache; ++u) {
             const uint32_t q = u * tpc + t;
-            if (q < nvec) emit(q, d[u], v[u]);
+            if (q < nvec) {
+                K::get(kd[u], d[0]);
+                K::get(kv[u], v[0]);
+                emit(q, d[0], v[0]);
+            }
         }
     } else {
         for (uint32_t q = t; q < nvec; q += tpc) {
@@ -261,18 +288,30 @@ __global__ __launch_bounds__(64) void ln_param_grad_kernel(const T* __restrict__
     for (int e = 0; e < VEC; ++e) { pg[o + e] = ag[e]; pb[o + e] = ab[e]; }
 }
 
+// dgamma[l] = sum_s pg[s][l], dbeta likewise.  Workgroup of 64 positions x 16 slice groups:
+// group g adds slices g, g+16, ... and the 16 group sums are added in group order.
 template <typename T>
-__global__ void ln_param_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, T* dgamma, T* dbeta,
-                                         uint32_t L, uint32_t S) {
-    const uint32_t l = blockIdx.x * blockDim.x + threadIdx.x;
-    if (l >= L) return;
+__global__ __launch_bounds__(1024) void ln_param_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb,
+                                                                 T* dgamma, T* dbeta, uint32_t L, uint32_t S) {
+    __shared__ float sg[16][64], sb[16][64];
+    const uint32_t lx = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const uint32_t l = blockIdx.x * 64 + lx;
     float tg = 0.0f, tb = 0.0f;
-    for (uint32_t s = 0; s < S; ++s) {
-        tg += pg[(size_t)s * L + l];
-        tb += pb[(size_t)s * L + l];
+    if (l < L)
+        for (uint32_t s = grp; s < S; s += 16) {
+            tg += pg[(size_t)s * L + l];
+            tb += pb[(size_t)s * L + l];
+        }
+    sg[grp][lx] = tg;
+    sb[grp][lx] = tb;
+    __syncthreads();
+    if (grp == 0 && l < L) {
+        tg = 0.0f; tb = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 16; ++g) { tg += sg[g][lx]; tb += sb[g][lx]; }
+        if (dgamma) st(dgamma + l, tg);
+        if (dbeta) st(dbeta + l, tb);
     }
-    if (dgamma) st(dgamma + l, tg);
-    if (dbeta) st(dbeta + l, tb);
 }
 
 // ------------------------------------------------------------------------------- host side
@@ -378,7 +417,7 @@ static int ln_bwd_impl(hipStream_t s, int act, int64_t L, int64_t R, const T* de
         }
         LUX_CHECK_LAUNCH();
         ProfScope ps2("ln_param_finalize_kernel", s);
-        ln_param_finalize_kernel<T><<<(unsigned)ceil_div(L, 256), 256, 0, s>>>(pg, pb, dgamma, dbeta, (uint32_t)L, (uint32_t)S);
+        ln_param_finalize_kernel<T><<<(unsigned)ceil_div(L, 64), 1024, 0, s>>>(pg, pb, dgamma, dbeta, (uint32_t)L, (uint32_t)S);
         LUX_CHECK_LAUNCH();
     }
     return LUXHIP_OK;
