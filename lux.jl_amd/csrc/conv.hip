@@ -248,7 +248,9 @@ static int wgrad_plan(const ConvGeom& g, int* slices, int* kslice, bool* small) 
     const int tile = *small ? 64 : 128;
     const int64_t tiles = ceil_div(Mrows, tile) * ceil_div(g.Cout_g, tile);
     const int64_t Ktotal = (int64_t)g.OW * g.OH * g.N;
-    int64_t want = std::max<int64_t>(1, ceil_div(2 * (int64_t)std::max(1, num_cus()), tiles * g.groups));
+    // as many slices as keep every workgroup resident at once (two per compute unit): one more
+    // would add a whole round for a single straggler
+    int64_t want = std::max<int64_t>(1, 2 * (int64_t)std::max(1, num_cus()) / (tiles * g.groups));
     int64_t ks = ceil_div(ceil_div(Ktotal, want), BK) * BK;
     ks = std::max<int64_t>(ks, 4 * BK);
     *kslice = (int)ks;
@@ -265,29 +267,64 @@ static size_t wgrad_partial_bytes(const ConvGeom& g) {
     return align256((size_t)slices * g.kW * g.kH * g.Cin_g * g.Cout_g * sizeof(float));
 }
 
+// bf16 fast path of the filter gradient: conditions under which conv_wgrad_direct_kernel applies
 template <typename T>
-static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dyT, float* partial, T* dw) {
+static bool wgrad_direct_ok(const ConvGeom& g, const void* xT, const void* dy) {
+    if (sizeof(T) != 2) return false;
+    const int64_t PQ = (int64_t)g.OW * g.OH;
+    return PQ % GemmTraits<T>::BK == 0 && g.Cin_g % 8 == 0 && g.Cin % 8 == 0 && aligned16(xT) && aligned16(dy) &&
+           (int64_t)g.W * g.H * g.Cin * g.N < (int64_t(1) << 30) && PQ * g.Cout * g.N < (int64_t(1) << 30);
+}
+
+// dy: WHCN cotangent (used by the direct bf16 kernel); dyT: its channel-contiguous copy (used by
+// the general kernel; may be NULL when wgrad_direct_ok).
+template <typename T>
+static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy, const T* dyT, float* partial, T* dw,
+                     const void* zeros) {
     constexpr int V = GemmTraits<T>::VEC;
     int slices, kslice;
     bool small;
     int rc = wgrad_plan<T>(g, &slices, &kslice, &small);
     if (rc != LUXHIP_OK) return rc;
+    const bool direct = wgrad_direct_ok<T>(g, xT, dy);
     for (int grp = 0; grp < g.groups; ++grp) {
-        ConvWgradArgs<T> a;
-        GatherMN<T>& q = a.gather;
-        q.src = xT; q.Ctot = g.Cin; q.c_off = grp * g.Cin_g; q.Cg = g.Cin_g; q.Mrows = g.kW * g.kH * g.Cin_g;
-        q.OW = g.OW; q.OWOH = g.OW * g.OH; q.SP = g.W; q.SQ = g.H; q.kW = g.kW; q.sw = g.sw; q.sh = g.sh; q.pw = g.pw;
-        q.ph = g.ph; q.dw = g.dw; q.dh = g.dh;
-        q.vec_ok = (g.Cin_g % V == 0) && (g.Cin % V == 0) && aligned16(xT);
-        q.divOW = FastDiv((uint32_t)q.OW); q.divOWOH = FastDiv((uint32_t)q.OWOH); q.divCg = FastDiv((uint32_t)q.Cg);
-        q.divkW = FastDiv((uint32_t)g.kW);
-        a.dyT = dyT; a.Cout = g.Cout; a.co_off = grp * g.Cout_g; a.Cout_g = g.Cout_g;
-        a.Ktotal = g.OW * g.OH * g.N; a.kslice = kslice; a.partial = partial;
-        a.dy_vec_ok = (g.Cout % V == 0) && (g.Cout_g % V == 0) && aligned16(dyT);
-        rc = launch_conv_wgrad_any<T>(s, a, slices, small);
+        const int Mrows = g.kW * g.kH * g.Cin_g;
+        if (direct) {
+            if constexpr (sizeof(T) == 2) {
+                ConvWgradDirectArgs a;
+                WgradGeomA& q = a.A;
+                q.src = reinterpret_cast<const bf16_t*>(xT) + (size_t)grp * g.Cin_g;
+                q.zero = zeros;
+                q.Ctot = g.Cin; q.Cg = g.Cin_g; q.Mrows = Mrows;
+                q.OW = g.OW; q.OWOH = g.OW * g.OH; q.SP = g.W; q.SQ = g.H;
+                q.kW = g.kW; q.sw = g.sw; q.sh = g.sh; q.pw = g.pw; q.ph = g.ph; q.dw = g.dw; q.dh = g.dh;
+                q.divOW = FastDiv((uint32_t)q.OW); q.divOWOH = FastDiv((uint32_t)q.OWOH);
+                q.divCg = FastDiv((uint32_t)q.Cg); q.divkW = FastDiv((uint32_t)g.kW);
+                WgradGeomB& b = a.B;
+                b.dy = reinterpret_cast<const bf16_t*>(dy);
+                b.zero = zeros;
+                b.PQ = g.OW * g.OH; b.Cout = g.Cout; b.co_off = grp * g.Cout_g; b.Ncols = g.Cout_g;
+                b.divPQ = FastDiv((uint32_t)b.PQ);
+                a.Ktotal = g.OW * g.OH * g.N; a.kslice = kslice; a.partial = partial;
+                rc = launch_conv_wgrad_direct(s, a, slices);
+            }
+        } else {
+            ConvWgradArgs<T> a;
+            GatherMN<T>& q = a.gather;
+            q.src = xT; q.Ctot = g.Cin; q.c_off = grp * g.Cin_g; q.Cg = g.Cin_g; q.Mrows = Mrows;
+            q.OW = g.OW; q.OWOH = g.OW * g.OH; q.SP = g.W; q.SQ = g.H; q.kW = g.kW; q.sw = g.sw; q.sh = g.sh; q.pw = g.pw;
+            q.ph = g.ph; q.dw = g.dw; q.dh = g.dh;
+            q.vec_ok = (g.Cin_g % V == 0) && (g.Cin % V == 0) && aligned16(xT);
+            q.divOW = FastDiv((uint32_t)q.OW); q.divOWOH = FastDiv((uint32_t)q.OWOH); q.divCg = FastDiv((uint32_t)q.Cg);
+            q.divkW = FastDiv((uint32_t)g.kW);
+            a.dyT = dyT; a.Cout = g.Cout; a.co_off = grp * g.Cout_g; a.Cout_g = g.Cout_g;
+            a.Ktotal = g.OW * g.OH * g.N; a.kslice = kslice; a.partial = partial;
+            a.dy_vec_ok = (g.Cout % V == 0) && (g.Cout_g % V == 0) && aligned16(dyT);
+            rc = launch_conv_wgrad_any<T>(s, a, slices, small);
+        }
         if (rc != LUXHIP_OK) return rc;
         ProfScope ps("wgrad_reduce_kernel", s);
-        const int total = q.Mrows * g.Cout_g;
+        const int total = Mrows * g.Cout_g;
         wgrad_reduce_kernel<T><<<(unsigned)ceil_div(total, 256), 256, 0, s>>>(partial, dw, g, grp, slices);
         LUX_CHECK_LAUNCH();
     }
@@ -335,8 +372,10 @@ static int conv_bwd_filter_t(hipStream_t s, const ConvGeom& g, const T* x, const
     T* dyT = reinterpret_cast<T*>(ws.data + xb);
     float* partial = reinterpret_cast<float*>(ws.data + xb + yb);
     if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
-    if ((rc = transpose_to_cwhn<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
-    return run_wgrad<T>(s, g, xT, dyT, partial, dw);
+    if (!wgrad_direct_ok<T>(g, xT, dy)) {   // the direct kernel reads dy as it is
+        if ((rc = transpose_to_cwhn<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
+    }
+    return run_wgrad<T>(s, g, xT, dy, dyT, partial, dw, ws.zeros);
 }
 
 template <typename T>
@@ -370,7 +409,7 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
     }
     if (dw != nullptr) {
         if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
-        if ((rc = run_wgrad<T>(s, g, xT, dzT, partial, dw)) != LUXHIP_OK) return rc;
+        if ((rc = run_wgrad<T>(s, g, xT, dzp, dzT, partial, dw, ws.zeros)) != LUXHIP_OK) return rc;
     }
     return LUXHIP_OK;
 }

@@ -576,6 +576,139 @@ int launch_conv_wgrad(hipStream_t s, ConvWgradArgs<T>& a, int slices) {
     return LUXHIP_OK;
 }
 
+// ----------------------------------------------------------------------------- wgrad, bf16 straight into LDS
+// A(m' = (tap, ci), k' = (ow, oh, n)) gathered from the channel-contiguous xT into the MN-major
+// LDS layout: a thread's 16-byte chunk always covers the same 8 channels of the same tap, so
+// tap and channel are decoded once; the output position of each load is decoded per stage.
+// B(k', co) comes from dy in its original WHCN layout, where the positions of one image and
+// channel are contiguous: K-major, no transposed copy of dy, 16-byte LDS reads.  Needs
+// OW*OH % BK == 0 (a stage never straddles two images) and slices of whole stages.
+struct WgradGeomA {
+    const bf16_t* src;         // xT + first channel of the group
+    const void* zero;
+    int Ctot, Cg, Mrows;
+    int OW, OWOH, SP, SQ;
+    int kW, sw, sh, pw, ph, dw, dh;
+    FastDiv divOW, divOWOH, divCg, divkW;
+};
+
+template <int ROWS, int THREADS>
+struct WgradDirectLoaderA {
+    using T = bf16_t;
+    static constexpr bool KMAJOR = false;
+    static constexpr int BK = GemmTraits<bf16_t>::BK, CPR = ROWS / 8;
+    static constexpr int INSTR = ROWS * BK / 8 / THREADS, STEP = THREADS / CPR;   // STEP: k rows per instruction
+    static_assert(INSTR >= 1 && (ROWS * BK / 8) % THREADS == 0 && STEP % 4 == 0, "stage must split evenly over the workgroup");
+    const WgradGeomA& g;
+    int kbeg, krow;            // first k' of the slice, this thread's k row inside an instruction's block
+    int dpx, dqy, coff;        // tap shift of the source position, channel offset
+    bool valid_m;
+    uint32_t lds_off;
+    __device__ __forceinline__ WgradDirectLoaderA(const WgradGeomA& gg, int m0, int kb_) : g(gg), kbeg(kb_) {
+        const int q = threadIdx.x, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        krow = q / CPR;
+        const int slot = q % CPR;
+        const int r = (slot * 8) ^ ((krow & 3) << mn_swizzle_shift(ROWS));   // (krow + i*STEP) & 3 == krow & 3
+        const int m = m0 + r;
+        valid_m = m < g.Mrows;
+        const int t = (int)g.divCg.div((uint32_t)(valid_m ? m : 0));
+        coff = (valid_m ? m : 0) - t * g.Cg;
+        const int kb = (int)g.divkW.div((uint32_t)t), ka = t - kb * g.kW;
+        dpx = ka * g.dw - g.pw;
+        dqy = kb * g.dh - g.ph;
+        lds_off = (uint32_t)w * 1024u;
+    }
+    __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
+        typedef __attribute__((address_space(3))) void* lds_vp;
+        typedef const __attribute__((address_space(1))) void* glb_vp;
+        char* l = reinterpret_cast<char*>(lds_tile) + lds_off;
+#pragma unroll
+        for (int i = 0; i < INSTR; ++i) {
+            const int kp = kbeg + k0 + krow + i * STEP;
+            const int n = (int)g.divOWOH.div((uint32_t)kp);
+            const int rem = kp - n * g.OWOH;
+            const int oh = (int)g.divOW.div((uint32_t)rem);
+            const int ow = rem - oh * g.OW;
+            const int sp = ow * g.sw + dpx, sq = oh * g.sh + dqy;
+            const bool valid = valid_m && (unsigned)sp < (unsigned)g.SP && (unsigned)sq < (unsigned)g.SQ;
+            const T* src = g.src + ((((int64_t)n * g.SQ + sq) * g.SP + sp) * g.Ctot + coff);
+            const void* p = valid ? static_cast<const void*>(src) : g.zero;
+            __builtin_amdgcn_global_load_lds((glb_vp)p, (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
+        }
+    }
+};
+
+struct WgradGeomB {
+    const bf16_t* dy;          // WHCN
+    const void* zero;
+    int PQ, Cout, co_off, Ncols;
+    FastDiv divPQ;
+};
+
+template <int ROWS, int THREADS>
+struct WgradDirectLoaderB {
+    using T = bf16_t;
+    static constexpr bool KMAJOR = true;
+    static constexpr int BK = GemmTraits<bf16_t>::BK, CPR = BK / 8;
+    static constexpr int INSTR = ROWS * CPR / THREADS, STEP = THREADS / CPR;
+    static_assert(INSTR >= 1 && (ROWS * CPR) % THREADS == 0 && STEP % 16 == 0, "stage must split evenly over the workgroup");
+    const WgradGeomB& g;
+    int kbeg, col0, rows_left;
+    int voff;                  // elements: row * PQ + chunk * 8
+    uint32_t lds_off;
+    __device__ __forceinline__ WgradDirectLoaderB(const WgradGeomB& gg, int n0, int kb_) : g(gg), kbeg(kb_), col0(n0) {
+        const int q = threadIdx.x, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const int row = q / CPR, slot = q % CPR;
+        voff = row * g.PQ + ((slot ^ ((row >> 2) & 3)) << 3);
+        rows_left = g.Ncols - n0 - row;
+        lds_off = (uint32_t)w * 1024u;
+    }
+    __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
+        typedef __attribute__((address_space(3))) void* lds_vp;
+        typedef const __attribute__((address_space(1))) void* glb_vp;
+        const int kp = kbeg + k0;                                  // uniform
+        const int n = (int)g.divPQ.div((uint32_t)kp);
+        const T* base = g.dy + (kp - n * g.PQ) + (int64_t)g.PQ * (g.co_off + col0 + (int64_t)g.Cout * n);
+        char* l = reinterpret_cast<char*>(lds_tile) + lds_off;
+#pragma unroll
+        for (int i = 0; i < INSTR; ++i) {
+            const T* src = base + voff + (int64_t)i * STEP * g.PQ;
+            const void* p = i * STEP < rows_left ? static_cast<const void*>(src) : g.zero;
+            __builtin_amdgcn_global_load_lds((glb_vp)p, (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
+        }
+    }
+};
+
+struct ConvWgradDirectArgs {
+    WgradGeomA A;
+    WgradGeomB B;
+    int Ktotal, kslice;
+    float* partial;            // [slice][Mrows][Ncols]
+    int tiles_m, tiles_n;
+};
+
+template <int WM, int WN, int NWN, int NST, int NWM>
+__global__ __launch_bounds__(NWM * NWN * 64) void conv_wgrad_direct_kernel(ConvWgradDirectArgs a) {
+    using ML = GemmMainloop<bf16_t, WM, WN, false, true, true, NWN, NST, NWM>;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
+    const int tile = blockIdx.x, slice = blockIdx.y;
+    const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
+    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+    const int kbeg = slice * a.kslice, kend = min(kbeg + a.kslice, a.Ktotal);
+    WgradDirectLoaderA<ML::TILE_M, ML::THREADS> la(a.A, m0, kbeg);
+    WgradDirectLoaderB<ML::TILE_N, ML::THREADS> lb(a.B, n0, kbeg);
+    f32x16_v acc[WM][WN];
+    ML::run_pipeline(la, lb, kend - kbeg, lds, acc);
+    const int Mrows = a.A.Mrows, Ncols = a.B.Ncols;
+    float* out = a.partial + (size_t)slice * Mrows * Ncols;
+    ML::for_each(acc, m0, n0, [&](int m, int col, float v) {
+        if (m < Mrows && col < Ncols) out[(size_t)m + (size_t)col * Mrows] = v;
+    });
+}
+
+int launch_conv_wgrad_direct(hipStream_t s, ConvWgradDirectArgs& a, int slices);   // conv_inst_wgrad_bf16.hip
+
 template <typename T>
 int launch_conv_wgrad_any(hipStream_t s, ConvWgradArgs<T>& a, int slices, bool small);   // conv_inst_*.hip
 

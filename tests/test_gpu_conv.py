@@ -53,6 +53,9 @@ CASES = [
     ((13, 11, 64, 3), (3, 2, 32, 64), (2, 1), (1, 0, 2, 1), (1, 2), 2, True),
     ((10, 12, 64, 2), (3, 3, 32, 96), 1, (2, 1, 0, 2), 2, 2, False),
     ((8, 8, 32, 5), (3, 3, 32, 320), 1, 1, 1, 1, False),
+    # output planes of a multiple of 32 positions (bf16 filter gradient straight from the WHCN cotangent)
+    ((16, 8, 32, 3), (3, 3, 16, 48), 1, 1, 1, 2, False),
+    ((16, 8, 16, 2), (3, 3, 16, 24), (2, 1), (1, 1, 1, 1), 1, 1, True),
 ]
 
 
@@ -77,7 +80,7 @@ def test_conv_and_gradients(gpu, dtype, case):
 @pytest.mark.parametrize("act", ["identity", "sigmoid", "gelu", "relu"])
 def test_fused_conv_pullback(gpu, dtype, act):
     rng = np.random.default_rng(stable_seed(dtype, act))
-    for case in (1, 2, 5, 7, 10, 11):
+    for case in (1, 2, 5, 7, 10, 11, 13):
         xs, ws, stride, pad, dil, groups, flip = CASES[case]
         gd, od = cdims(gpu, xs, ws, stride=stride, padding=pad, dilation=dil, groups=groups, flipkernel=flip)
         fan_in = ws[0] * ws[1] * ws[2]
