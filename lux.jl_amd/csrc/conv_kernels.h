@@ -130,8 +130,8 @@ struct ConvGemmArgs {
 // Epilogue of fprop / dgrad: element (m = (p, q, n), col) -> out[(m - n*PQ) + PQ*(col_off + col +
 // Ctot_out*n)], with bias per output channel and the activation.  The image index of a row is
 // decoded once per row, the channel terms once per column.  CHECK (tiles that stick out of the
-// matrix), HAS_ACT and HAS_PRE are resolved once per tile.
-template <class ML, typename T, int WM, int WN, bool CHECK, bool HAS_ACT, bool HAS_PRE>
+// matrix), the activation mode and HAS_PRE are resolved once per tile.
+template <class ML, typename T, int WM, int WN, bool CHECK, int ACT_MODE, bool HAS_PRE>
 __device__ __forceinline__ void conv_epilogue_as(const f32x16_v (&acc)[WM][WN], int m0, int n0, int M, int PQ, FastDiv divPQ,
                                                  int Ncols, int col_off, int Ctot_out, const T* bias, T* out, T* pre, int act) {
     const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
@@ -159,7 +159,8 @@ __device__ __forceinline__ void conv_epilogue_as(const f32x16_v (&acc)[WM][WN], 
                     for (int i = 0; i < WM; ++i)
                         if (!CHECK || mok[i]) st(pre + coloff + rowoff[i], v[i]);
                 }
-                if constexpr (HAS_ACT) act_vec(act, v);
+                if constexpr (ACT_MODE == 1) act_vec_as<LUXHIP_ACT_RELU>(v);
+                else if constexpr (ACT_MODE == 2) act_vec(act, v);
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
                     if (!CHECK || mok[i]) st(out + coloff + rowoff[i], v[i]);
@@ -171,17 +172,20 @@ template <class ML, typename T, int WM, int WN>
 __device__ __forceinline__ void conv_epilogue(const f32x16_v (&acc)[WM][WN], int m0, int n0, int M, int PQ, FastDiv divPQ,
                                               int Ncols, int col_off, int Ctot_out, const T* bias, T* out, T* pre, int act) {
     const bool check = m0 + ML::TILE_M > M || n0 + ML::TILE_N > Ncols;
-    const bool has_act = act != LUXHIP_ACT_IDENTITY, has_pre = pre != nullptr;
+    const bool has_pre = pre != nullptr;
+    // activation: 0 none, 1 relu (inline), 2 any (dispatched per column of the accumulator tile)
 #define LUX_CONV_EPI(C, A, P) conv_epilogue_as<ML, T, WM, WN, C, A, P>(acc, m0, n0, M, PQ, divPQ, Ncols, col_off, Ctot_out, bias, out, pre, act)
     if (check) {                                 // rare: general variants
-        if (has_pre) LUX_CONV_EPI(true, true, true);
-        else LUX_CONV_EPI(true, true, false);
-    } else if (!has_act && !has_pre) {
-        LUX_CONV_EPI(false, false, false);
-    } else if (!has_pre) {
-        LUX_CONV_EPI(false, true, false);
+        if (has_pre) LUX_CONV_EPI(true, 2, true);
+        else LUX_CONV_EPI(true, 2, false);
+    } else if (has_pre) {
+        LUX_CONV_EPI(false, 2, true);
+    } else if (act == LUXHIP_ACT_IDENTITY) {
+        LUX_CONV_EPI(false, 0, false);
+    } else if (act == LUXHIP_ACT_RELU) {
+        LUX_CONV_EPI(false, 1, false);
     } else {
-        LUX_CONV_EPI(false, true, true);
+        LUX_CONV_EPI(false, 2, false);
     }
 #undef LUX_CONV_EPI
 }

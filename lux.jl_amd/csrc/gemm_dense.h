@@ -13,8 +13,8 @@
 namespace luxhip {
 
 // Epilogue of one tile: C = act(acc + bias), optional pre-activation copy.  CHECK: bounds tests;
-// HAS_ACT / HAS_PRE are resolved once per tile, so the per-element code has no branches.
-template <class ML, typename T, int WM, int WN, bool CHECK, bool HAS_ACT, bool HAS_PRE>
+// the activation mode and HAS_PRE are resolved once per tile, so the common cases have no branch per element.
+template <class ML, typename T, int WM, int WN, bool CHECK, int ACT_MODE, bool HAS_PRE>
 __device__ __forceinline__ void dense_epilogue_as(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int m0, int n0) {
     const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
     float bv[WM];
@@ -35,7 +35,8 @@ __device__ __forceinline__ void dense_epilogue_as(const f32x16_v (&acc)[WM][WN],
                     for (int i = 0; i < WM; ++i)
                         if (!CHECK || mb + i * 32 < a.M) st(pcol + i * 32, v[i]);
                 }
-                if constexpr (HAS_ACT) act_vec(act, v);
+                if constexpr (ACT_MODE == 1) act_vec_as<LUXHIP_ACT_RELU>(v);
+                else if constexpr (ACT_MODE == 2) act_vec(act, v);
                 T* ccol = a.C + (int64_t)n * a.ldc + mb;
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
@@ -46,10 +47,11 @@ __device__ __forceinline__ void dense_epilogue_as(const f32x16_v (&acc)[WM][WN],
 }
 template <class ML, typename T, int WM, int WN, bool FULL>
 __device__ __forceinline__ void dense_epilogue(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int m0, int n0) {
-    const bool has_act = a.act != LUXHIP_ACT_IDENTITY, has_pre = a.pre != nullptr;
-    if (!has_act && !has_pre) dense_epilogue_as<ML, T, WM, WN, !FULL, false, false>(acc, a, m0, n0);
-    else if (!has_pre) dense_epilogue_as<ML, T, WM, WN, !FULL, true, false>(acc, a, m0, n0);
-    else dense_epilogue_as<ML, T, WM, WN, !FULL, true, true>(acc, a, m0, n0);
+    // activation: 0 none, 1 relu (inline), 2 any (dispatched per column of the accumulator tile)
+    if (a.pre != nullptr) dense_epilogue_as<ML, T, WM, WN, !FULL, 2, true>(acc, a, m0, n0);
+    else if (a.act == LUXHIP_ACT_IDENTITY) dense_epilogue_as<ML, T, WM, WN, !FULL, 0, false>(acc, a, m0, n0);
+    else if (a.act == LUXHIP_ACT_RELU) dense_epilogue_as<ML, T, WM, WN, !FULL, 1, false>(acc, a, m0, n0);
+    else dense_epilogue_as<ML, T, WM, WN, !FULL, 2, false>(acc, a, m0, n0);
 }
 
 // Persistent: workgroup b handles tiles b, b + gridDim.x, ...  On the direct-to-LDS path the
