@@ -150,21 +150,41 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T*
     const uint32_t q0 = s * chunk;
     const uint32_t q1 = min(q0 + chunk, nq);
     float acc = 0.0f;
-    for (uint32_t q = q0 + threadIdx.x; q < q1; q += kThreads) {
-        const uint32_t n = rowdiv.div(q);
-        const size_t off = ((size_t)q + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
-        float r[VEC];
-        dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
-        if (dx) store_vec<T, VEC>(dx, off, r);
+    // One vector per thread (the usual split): the partial sum is handed over before dx is
+    // stored, so the hand-off does not wait for the stores.
+    const bool single = chunk <= kThreads;
+    float r0[VEC];
+    size_t off0 = 0;
+    bool have0 = false;
+    if (single) {
+        const uint32_t q = q0 + threadIdx.x;
+        if (q < q1) {
+            const uint32_t n = rowdiv.div(q);
+            off0 = ((size_t)q + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
+            dx_vec<T, ACT, VEC>(delta, out, pre, off0, r0);
+            have0 = true;
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc += r[k];
+            for (int k = 0; k < VEC; ++k) acc += r0[k];
+        }
+    } else {
+        for (uint32_t q = q0 + threadIdx.x; q < q1; q += kThreads) {
+            const uint32_t n = rowdiv.div(q);
+            const size_t off = ((size_t)q + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
+            float r[VEC];
+            dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
+            if (dx) store_vec<T, VEC>(dx, off, r);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc += r[k];
+        }
     }
     acc = block_sum(acc, smem);
     if (threadIdx.x == 0) {
         publish(partial + (size_t)c * S + s, acc);
         publish_done();
     }
-    if (!arrive_last(counters + (size_t)c * cstride, S, &last_flag)) return;
+    const bool last = arrive_last(counters + (size_t)c * cstride, S, &last_flag);
+    if (single && have0 && dx) store_vec<T, VEC>(dx, off0, r0);
+    if (!last) return;
     if (threadIdx.x < 64) {
         float t = 0.0f;
         for (uint32_t i = threadIdx.x; i < S; i += 64) t += fetch(partial + (size_t)c * S + i);
