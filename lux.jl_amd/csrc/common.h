@@ -184,6 +184,7 @@ struct Vec<bf16_t> {
 
 template <typename T>
 __device__ __forceinline__ float ld(const T* p);
+
 template <>
 __device__ __forceinline__ float ld<float>(const float* p) { return *p; }
 template <>
@@ -194,6 +195,26 @@ template <>
 __device__ __forceinline__ void st<float>(float* p, float v) { *p = v; }
 template <>
 __device__ __forceinline__ void st<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// A vector kept in registers between the passes: the 16 bytes as they lie in memory (bf16 stays
+// packed, which halves the register footprint), or one float for the scalar kernels.
+template <typename T, int VEC>
+struct Kept {
+    using type = raw16_t;
+    __device__ __forceinline__ static type load(const T* p, size_t off) { return *reinterpret_cast<const raw16_t*>(p + off); }
+    __device__ __forceinline__ static void get(const type& k, float (&v)[VEC]) { Vec<T>::unpack(k, v); }
+};
+template <typename T>
+struct Kept<T, 1> {
+    using type = float;
+    __device__ __forceinline__ static type load(const T* p, size_t off) { return ld(p + off); }
+    __device__ __forceinline__ static void get(const type& k, float (&v)[1]) { v[0] = k; }
+};
+template <typename T, int VEC>
+__device__ __forceinline__ typename Kept<T, VEC>::type keep(const float (&v)[VEC]) {   // the reverse of get()
+    if constexpr (VEC == 1) return v[0];
+    else return Vec<T>::pack(v);
+}
 
 // ----------------------------------------------------------------------------- activations
 // value f(x) and the derivative LuxLib multiplies the cotangent by, given the output `o`

@@ -7,8 +7,9 @@
 //     the registers (slices of up to kGnCache vectors per thread x 1024 threads);
 //   * streaming kernels handle larger slices with a second read of the slice.
 // Per-channel gradients (dgamma, dbeta) are accumulated per wave in LDS in program order,
-// combined across waves in a fixed order, written as [N][C] partials and reduced over N by a
-// finalize kernel: deterministic, no floating-point atomics.
+// combined across waves in a fixed order, published as [N][C] partials and added over N, in
+// sample order, by the workgroup of each group that arrives last: deterministic, no
+// floating-point atomics, no extra launch.
 #include <algorithm>
 
 #include "common.h"
@@ -44,22 +45,22 @@ __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
     const uint32_t k = slice % g.G;
     const size_t base = (size_t)slice * g.nvec * VEC;
     const uint32_t T_ = blockDim.x;
-    float v[CACHED ? kGnCache : 1][VEC];
+    using K = Kept<T, VEC>;
+    typename K::type kv[CACHED ? kGnCache : 1];   // cached: the slice as it lies in memory; loads past its end re-read the last vector
+    float v[1][VEC];
 
     // pass 1: mean
     float sum = 0.0f;
     if constexpr (CACHED) {
 #pragma unroll
-        for (int u = 0; u < kGnCache; ++u) {
-            const uint32_t q = u * T_ + threadIdx.x;
-            if (q < g.nvec) gn_load<T, VEC>(x, base + (size_t)q * VEC, v[u]);
-        }
+        for (int u = 0; u < kGnCache; ++u) kv[u] = K::load(x, base + (size_t)min(u * T_ + threadIdx.x, g.nvec - 1) * VEC);
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = u * T_ + threadIdx.x;
             if (q < g.nvec) {
+                K::get(kv[u], v[0]);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) sum += v[u][e];
+                for (int e = 0; e < VEC; ++e) sum += v[0][e];
             }
         }
     } else {
@@ -77,8 +78,9 @@ __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = u * T_ + threadIdx.x;
             if (q < g.nvec) {
+                K::get(kv[u], v[0]);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) dev = fmaf(v[u][e] - mean, v[u][e] - mean, dev);
+                for (int e = 0; e < VEC; ++e) dev = fmaf(v[0][e] - mean, v[0][e] - mean, dev);
             }
         }
     } else {
@@ -108,7 +110,10 @@ __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = u * T_ + threadIdx.x;
-            if (q < g.nvec) emit(q, v[u]);
+            if (q < g.nvec) {
+                K::get(kv[u], v[0]);
+                emit(q, v[0]);
+            }
         }
     } else {
         for (uint32_t q = threadIdx.x; q < g.nvec; q += T_) {
@@ -143,7 +148,8 @@ __device__ __forceinline__ void wave_channel_accumulate(float* accg, float* accb
 template <typename T, int ACT, int VEC, bool CACHED, bool AFFINE>
 __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma,
                               const T* __restrict__ beta, const float* __restrict__ save_mean,
-                              const float* __restrict__ save_invstd, T* dx, float* pdg, float* pdb, GnGeom g) {
+                              const float* __restrict__ save_invstd, T* dx, float* pdg, float* pdb, T* dgamma,
+                              T* dbeta, uint32_t* counters, uint32_t cstride, uint32_t N, GnGeom g) {
     extern __shared__ float lds[];                  // [16] reduction scratch, then [nw][Cg] x 2
     float* sm = lds;
     const uint32_t T_ = blockDim.x, nw = T_ >> 6, w = threadIdx.x >> 6;
@@ -156,7 +162,13 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         for (uint32_t i = threadIdx.x; i < 2 * nw * g.Cg; i += T_) lds[16 + i] = 0.0f;
         __syncthreads();
     }
-    float d[CACHED ? kGnCache : 1][VEC], v[CACHED ? kGnCache : 1][VEC];
+    using K = Kept<T, VEC>;
+    typename K::type kd[CACHED ? kGnCache : 1], kv[CACHED ? kGnCache : 1];
+    float d[1][VEC], v[1][VEC];
+    // fp32 storage: after the first pass kd holds dy * gamma, so the second pass needs no
+    // activation derivative; bf16 storage keeps delta (packing dy * gamma would round it) and
+    // recomputes
+    constexpr bool KEEP_G = sizeof(T) == 4;
     float s1 = 0.0f, s2 = 0.0f;
 
     // dy and g = dy * gamma for one vector; also returns the channel's parameters
@@ -185,11 +197,9 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     if constexpr (CACHED) {
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
-            const uint32_t q = u * T_ + threadIdx.x;
-            if (q < g.nvec) {
-                gn_load<T, VEC>(delta, base + (size_t)q * VEC, d[u]);
-                gn_load<T, VEC>(x, base + (size_t)q * VEC, v[u]);
-            }
+            const size_t off = base + (size_t)min(u * T_ + threadIdx.x, g.nvec - 1) * VEC;   // past the end: last vector again
+            kd[u] = K::load(delta, off);
+            kv[u] = K::load(x, off);
         }
     }
     if constexpr (CACHED) {
@@ -200,14 +210,16 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                 const bool active = q < g.nvec;
                 float gv[VEC], a = 0.0f, b = 0.0f;
                 if (active) {
-                    grad_terms(q, d[u], v[u], gv, a, b);
+                    K::get(kd[u], d[0]);
+                    K::get(kv[u], v[0]);
+                    grad_terms(q, d[0], v[0], gv, a, b);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        const float xh = (v[u][e] - mean) * invstd;
+                        const float xh = (v[0][e] - mean) * invstd;
                         s1 += gv[e];
                         s2 = fmaf(gv[e], xh, s2);
-                        d[u][e] = gv[e];            // dy * gamma replaces delta: the second pass needs only this
                     }
+                    if constexpr (KEEP_G) kd[u] = keep<T, VEC>(gv);
                 }
                 if constexpr (AFFINE) {
                     // the first lane of the wave decides whether the wave has work this round
@@ -241,6 +253,35 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     s1 = block_sum(s1, sm) * g.inv_m;
     s2 = block_sum(s2, sm) * g.inv_m;
 
+    // Parameter gradients first (they only need the first pass), so that their hand-off does not
+    // wait for the dx stores below.
+    if constexpr (AFFINE) {
+        for (uint32_t j = threadIdx.x; j < g.Cg; j += T_) {
+            float tg = 0.0f, tb = 0.0f;
+            for (uint32_t ww = 0; ww < nw; ++ww) {
+                tg += lds[16 + (size_t)ww * g.Cg + j];
+                tb += lds[16 + (size_t)(nw + ww) * g.Cg + j];
+            }
+            publish(pdg + (size_t)n * g.C + k * g.Cg + j, tg);
+            publish(pdb + (size_t)n * g.C + k * g.Cg + j, tb);
+        }
+        publish_done();
+        // the workgroup of group k that arrives last (one per sample) adds the N per-sample
+        // partials of the group's channels in sample order
+        uint32_t* last_flag = reinterpret_cast<uint32_t*>(lds + 15);   // a word of the reduction scratch that is free now
+        if (arrive_last(counters + (size_t)k * cstride, N, last_flag)) {
+            for (uint32_t j = threadIdx.x; j < g.Cg; j += T_) {
+                float tg = 0.0f, tb = 0.0f;
+                for (uint32_t nn = 0; nn < N; ++nn) {
+                    tg += fetch(pdg + (size_t)nn * g.C + k * g.Cg + j);
+                    tb += fetch(pdb + (size_t)nn * g.C + k * g.Cg + j);
+                }
+                if (dgamma) st(dgamma + k * g.Cg + j, tg);
+                if (dbeta) st(dbeta + k * g.Cg + j, tb);
+            }
+        }
+    }
+
     auto emit = [&](uint32_t q, const float (&dv)[VEC], const float (&xv)[VEC]) {
         float gv[VEC], a, b, o[VEC];
         grad_terms(q, dv, xv, gv, a, b);
@@ -255,14 +296,20 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = u * T_ + threadIdx.x;
-            if (q < g.nvec) {                       // d[u] holds dy * gamma
-                float o[VEC];
+            if (q < g.nvec) {
+                K::get(kd[u], d[0]);
+                K::get(kv[u], v[0]);
+                if constexpr (KEEP_G) {             // kd[u] holds dy * gamma
+                    float o[VEC];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const float xh = (v[u][e] - mean) * invstd;
-                    o[e] = invstd * (d[u][e] - s1 - xh * s2);
+                    for (int e = 0; e < VEC; ++e) {
+                        const float xh = (v[0][e] - mean) * invstd;
+                        o[e] = invstd * (d[0][e] - s1 - xh * s2);
+                    }
+                    gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
+                } else {
+                    emit(q, d[0], v[0]);
                 }
-                gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
             }
         }
     } else {
@@ -272,33 +319,6 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
             emit(q, d[0], v[0]);
         }
     }
-    if constexpr (AFFINE) {
-        __syncthreads();
-        for (uint32_t j = threadIdx.x; j < g.Cg; j += T_) {
-            float tg = 0.0f, tb = 0.0f;
-            for (uint32_t ww = 0; ww < nw; ++ww) {
-                tg += lds[16 + (size_t)ww * g.Cg + j];
-                tb += lds[16 + (size_t)(nw + ww) * g.Cg + j];
-            }
-            pdg[(size_t)n * g.C + k * g.Cg + j] = tg;
-            pdb[(size_t)n * g.C + k * g.Cg + j] = tb;
-        }
-    }
-}
-
-// dgamma[c] = sum_n pdg[n][c], dbeta[c] = sum_n pdb[n][c]
-template <typename T>
-__global__ void gn_param_finalize_kernel(const float* __restrict__ pdg, const float* __restrict__ pdb, T* dgamma,
-                                         T* dbeta, uint32_t C, uint32_t N) {
-    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    float tg = 0.0f, tb = 0.0f;
-    for (uint32_t n = 0; n < N; ++n) {
-        tg += pdg[(size_t)n * C + c];
-        tb += pdb[(size_t)n * C + c];
-    }
-    if (dgamma) st(dgamma + c, tg);
-    if (dbeta) st(dbeta + c, tb);
 }
 
 // ------------------------------------------------------------------------------- host side
@@ -377,19 +397,23 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
         LUX_UNSUPPORTED_IF(lds_bytes > 60 * 1024, "groupnorm_bwd: %u channels per group exceed the LDS accumulators", L.g.Cg);
     }
     float *pdg = nullptr, *pdb = nullptr;
+    uint32_t* counters = nullptr;
+    const uint32_t cstride = counter_stride(G);
     if (affine) {
+        LUX_UNSUPPORTED_IF((size_t)G > kWorkspaceCounters, "groupnorm_bwd: more than %zu groups", kWorkspaceCounters);
         Workspace ws;
         int rc = get_workspace(s, (size_t)2 * N * C * sizeof(float), &ws);
         if (rc != LUXHIP_OK) return rc;
         pdg = reinterpret_cast<float*>(ws.data);
         pdb = pdg + (size_t)N * C;
+        counters = ws.counters;
     }
     {
         ProfScope ps("gn_bwd_kernel", s);
 #define GN_BWD_A(A, VV, CA)                                                                                           \
     do {                                                                                                              \
-        if (affine) gn_bwd_kernel<T, A, VV, CA, true><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, L.g); \
-        else gn_bwd_kernel<T, A, VV, CA, false><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, L.g);       \
+        if (affine) gn_bwd_kernel<T, A, VV, CA, true><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g); \
+        else gn_bwd_kernel<T, A, VV, CA, false><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g);       \
     } while (0)
 #define GN_BWD(A)                                                                                                     \
     do {                                                                                                              \
@@ -403,11 +427,6 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
 #undef GN_BWD_A
     }
     LUX_CHECK_LAUNCH();
-    if (affine) {
-        ProfScope ps("gn_param_finalize_kernel", s);
-        gn_param_finalize_kernel<T><<<(unsigned)ceil_div(C, 128), 128, 0, s>>>(pdg, pdb, dgamma, dbeta, (uint32_t)C, (uint32_t)N);
-        LUX_CHECK_LAUNCH();
-    }
     return LUXHIP_OK;
 }
 

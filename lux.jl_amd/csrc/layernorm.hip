@@ -27,21 +27,6 @@ __device__ __forceinline__ void ln_store(T* p, size_t off, const float (&v)[VEC]
     else Vec<T>::store(p + off, v);
 }
 
-// A vector kept in registers between the passes: the 16 bytes as they lie in memory (bf16 stays
-// packed, which halves the register footprint), or one float for the scalar kernels.
-template <typename T, int VEC>
-struct Kept {
-    using type = raw16_t;
-    __device__ __forceinline__ static type load(const T* p, size_t off) { return *reinterpret_cast<const raw16_t*>(p + off); }
-    __device__ __forceinline__ static void get(const type& k, float (&v)[VEC]) { Vec<T>::unpack(k, v); }
-};
-template <typename T>
-struct Kept<T, 1> {
-    using type = float;
-    __device__ __forceinline__ static type load(const T* p, size_t off) { return ld(p + off); }
-    __device__ __forceinline__ static void get(const type& k, float (&v)[1]) { v[0] = k; }
-};
-
 // Sum over the threads that share a column: the wave (WAVE) or the workgroup.
 template <bool WAVE>
 __device__ __forceinline__ float col_sum(float v, float* sm) {
