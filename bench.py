@@ -64,7 +64,7 @@ class Workload:
 
 
 class C2BatchnormBiasAct(Workload):
-    """BASELINE config 2: batchnorm (training, running stats updated) then bias_activation(relu),
+    """benchmark configuration 2: batchnorm (training, running stats updated) then bias_activation(relu),
     forward and pullback, fp32, x 32x32x64x128."""
     name = "C2"
     dtype = "f32"
@@ -213,7 +213,7 @@ class _ApiWorkload(Workload):
 
 
 class C1Dense(_ApiWorkload):
-    """BASELINE config 1: fused_dense_bias_activation 128 -> 256, batch 64, tanh, fp32."""
+    """benchmark configuration 1: fused_dense_bias_activation 128 -> 256, batch 64, tanh, fp32."""
     name, dtype, bound = "C1", "f32", "mfma"
     description = "fused_dense_bias_activation(tanh) fwd+bwd, W 256x128, x 128x64 fp32 (latency-bound)"
 
@@ -237,7 +237,7 @@ class C1Dense(_ApiWorkload):
 
 
 class C3Groupnorm(_ApiWorkload):
-    """BASELINE config 3: groupnorm(32 groups) + swish, x 64x64x256x16."""
+    """benchmark configuration 3: groupnorm(32 groups) + swish, x 64x64x256x16."""
     name, bound = "C3", "hbm"
     shape, groups = (64, 64, 256, 16), 32
 
@@ -269,7 +269,7 @@ class C3Groupnorm(_ApiWorkload):
 
 
 class C4TransformerMLP(_ApiWorkload):
-    """BASELINE config 4: layernorm(4096 x 8192) -> dense 4096->11008 gelu -> dense 11008->4096,
+    """benchmark configuration 4: layernorm(4096 x 8192) -> dense 4096->11008 gelu -> dense 11008->4096,
     bf16 storage, fp32 accumulation."""
     name, dtype, bound = "C4", "bf16", "mfma"
     description = "layernorm + dense(4096->11008, gelu) + dense(11008->4096) fwd+bwd, 8192 tokens, bf16/fp32-acc"
@@ -305,7 +305,7 @@ class C4TransformerMLP(_ApiWorkload):
 
 
 class C5Conv(_ApiWorkload):
-    """BASELINE config 5: fused_conv_bias_activation 3x3, 128->128, 56x56, batch 64, pad 1, relu."""
+    """benchmark configuration 5: fused_conv_bias_activation 3x3, 128->128, 56x56, batch 64, pad 1, relu."""
     bound = "mfma"
     xs, ws = (56, 56, 128, 64), (3, 3, 128, 128)
 

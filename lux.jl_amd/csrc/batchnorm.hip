@@ -9,8 +9,9 @@
 //
 // Resident path (tensor fits the register file: C*S <= compute units, slice <= 8 vectors per
 // thread of a 1024-thread workgroup), one kernel and one trip through HBM per tensor:
-//   forward : bn_fwd_resident_kernel  load x -> slice statistics -> publish, wait for the other
-//             slices of the channel -> mean/invstd (+ running stats, saved stats) -> write y
+//   forward : bn_fwd_resident_kernel  load x -> slice statistics -> publish as (value, epoch)
+//             words, collect the words of the channel's other slices -> mean/invstd (+ running
+//             stats, saved stats) -> write y
 //   pullback: bn_bwd_resident_kernel  load delta, x -> slice sums -> publish, wait -> dgamma, dbeta
 //             -> write dx
 //   All workgroups of the grid are resident at once (one per compute unit), so the wait ends as
@@ -388,52 +389,44 @@ __device__ __forceinline__ void res_slice_stats(const ChanGeom& g, uint32_t slic
     m2 = block_sum(dev, sm);
 }
 
-// Wave 0 polls the S flags of channel c until they show `epoch`; false for the whole workgroup
-// if any poll loop ran out of tries.  Contains a workgroup barrier.
-__device__ __forceinline__ bool res_wait_peers(const uint32_t* flags, uint32_t S, uint32_t epoch, uint32_t spin_limit,
-                                               uint32_t* lds_ok) {
-    if (threadIdx.x < kWave) {
-        bool ok = true;
-        for (uint32_t i = threadIdx.x; i < S; i += kWave) {
-            uint32_t tries = 0;
-            while (fetch(flags + i) != epoch) {
-                if (tries++ >= spin_limit) { ok = false; break; }
-                __builtin_amdgcn_s_sleep(4);
-            }
+// The nw = K*S exchange words of a channel (K per slice) -> parts[0..nw) in LDS.  Thread i polls
+// word i until it carries `epoch`; false for the whole workgroup if any poll ran out of tries.
+// Contains workgroup barriers.
+__device__ __forceinline__ bool res_collect(const uint64_t* words, uint32_t nw, uint32_t epoch, uint32_t spin_limit,
+                                            float* parts) {
+    int failed = 0;
+    if (threadIdx.x < nw) {
+        uint32_t tries = 0;
+        for (;;) {
+            const uint64_t wv = fetch_tagged(words + threadIdx.x);
+            if ((uint32_t)(wv >> 32) == epoch) { parts[threadIdx.x] = __uint_as_float((uint32_t)wv); break; }
+            if (tries++ >= spin_limit) { failed = 1; break; }
+            __builtin_amdgcn_s_sleep(2);
         }
-        const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
-        if (threadIdx.x == 0) *lds_ok = all_ok ? 1u : 0u;
     }
-    __syncthreads();
-    return *lds_ok != 0u;
+    return __syncthreads_or(failed) == 0;
 }
 
 template <typename T, int ACT>
 __global__ __launch_bounds__(kResThreads) void bn_fwd_resident_kernel(const T* __restrict__ x, T* __restrict__ y,
-                                                                      float* partial, uint32_t* flags, uint32_t epoch,
+                                                                      uint64_t* words, uint32_t epoch,
                                                                       uint32_t spin_limit, BnFwdParams prm, ChanGeom g) {
     constexpr int VEC = Vec<T>::N;
     __shared__ float sm[kResThreads / 64];
     __shared__ float parts[kResMaxSlices * 3];
     __shared__ float bc[2];
-    __shared__ uint32_t lds_ok;
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     raw16_t v[kResVecs];
     res_load<T>(x, g, c, s, v);
     float n, mean, m2;
     res_slice_stats<T>(g, s, v, sm, n, mean, m2);
-    float* chan_part = partial + (size_t)c * S * 3;
-    uint32_t* chan_flags = flags + (size_t)c * S;
+    uint64_t* chan_words = words + (size_t)c * S * 3;
     if (threadIdx.x == 0) {
-        publish(chan_part + 3 * s, n);
-        publish(chan_part + 3 * s + 1, mean);
-        publish(chan_part + 3 * s + 2, m2);
-        publish_done();
-        publish(chan_flags + s, epoch);
+        publish_tagged(chan_words + 3 * s, n, epoch);
+        publish_tagged(chan_words + 3 * s + 1, mean, epoch);
+        publish_tagged(chan_words + 3 * s + 2, m2, epoch);
     }
-    if (res_wait_peers(chan_flags, S, epoch, spin_limit, &lds_ok)) {
-        for (uint32_t i = threadIdx.x; i < 3 * S; i += kResThreads) parts[i] = fetch(chan_part + i);
-    } else {
+    if (!res_collect(chan_words, 3 * S, epoch, spin_limit, parts)) {
         // a peer did not show up in time: its share is recomputed here, the own slice last so
         // that v holds it again afterwards
         for (uint32_t i = 0; i <= S; ++i) {
@@ -506,13 +499,11 @@ template <typename T, int ACT>
 __global__ __launch_bounds__(kResThreads) void bn_bwd_resident_kernel(
     const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const float* __restrict__ save_mean, const float* __restrict__ save_invstd, T* __restrict__ dx, T* dgamma, T* dbeta,
-    float* partial, uint32_t* flags, uint32_t epoch, uint32_t spin_limit, float inv_count, int stats_from_batch,
-    ChanGeom g) {
+    uint64_t* words, uint32_t epoch, uint32_t spin_limit, float inv_count, int stats_from_batch, ChanGeom g) {
     constexpr int VEC = Vec<T>::N;
     __shared__ float sm[kResThreads / 64];
     __shared__ float parts[kResMaxSlices * 2];
     __shared__ float bc[3];
-    __shared__ uint32_t lds_ok;
     const uint32_t c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
     const float mean = save_mean[c], invstd = save_invstd[c];
     const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
@@ -522,17 +513,12 @@ __global__ __launch_bounds__(kResThreads) void bn_bwd_resident_kernel(
     res_load<T>(x, g, c, s, v);
     float s1, s2;
     res_bwd_slice_sums<T, ACT>(g, s, d, v, mean, invstd, sc, sh, sm, s1, s2);
-    float* chan_part = partial + (size_t)c * S * 2;
-    uint32_t* chan_flags = flags + (size_t)c * S;
+    uint64_t* chan_words = words + (size_t)c * S * 2;
     if (threadIdx.x == 0) {
-        publish(chan_part + 2 * s, s1);
-        publish(chan_part + 2 * s + 1, s2);
-        publish_done();
-        publish(chan_flags + s, epoch);
+        publish_tagged(chan_words + 2 * s, s1, epoch);
+        publish_tagged(chan_words + 2 * s + 1, s2, epoch);
     }
-    if (res_wait_peers(chan_flags, S, epoch, spin_limit, &lds_ok)) {
-        for (uint32_t i = threadIdx.x; i < 2 * S; i += kResThreads) parts[i] = fetch(chan_part + i);
-    } else {
+    if (!res_collect(chan_words, 2 * S, epoch, spin_limit, parts)) {
         for (uint32_t i = 0; i <= S; ++i) {   // recompute the peers' sums; own slice last (d, v restored)
             const uint32_t slice = i < S ? i : s;
             __syncthreads();
@@ -592,7 +578,7 @@ static int64_t resident_slices(int64_t I, int64_t C, int64_t N, int vec, bool al
     // as many slices as fit (more compute units busy) while a slice keeps at least one vector per thread
     int64_t S = std::min<int64_t>(s_max, std::max<int64_t>(s_need, nq / kResThreads));
     if (S < 1) S = 1;
-    if ((size_t)(C * S) > kWorkspaceFlags) return 0;
+    if ((size_t)(C * S) * 6 > kWorkspaceFlags) return 0;   // three 8-byte exchange words per slice
     return S;
 }
 
@@ -653,12 +639,12 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         g.chunk = (uint32_t)ceil_div(g.nq, SR);
         const int64_t S = ceil_div(g.nq, g.chunk);
         Workspace ws;
-        int rc = get_workspace(s, (size_t)C * 3 * S * sizeof(float), &ws);
+        int rc = get_workspace(s, 0, &ws);
         if (rc != LUXHIP_OK) return rc;
-        float* partial = reinterpret_cast<float*>(ws.data);
+        uint64_t* words = reinterpret_cast<uint64_t*>(ws.flags);
         const uint32_t spin = (uint32_t)option_bn_spin_limit();
         dim3 grid((unsigned)S, (unsigned)C);
-#define LAUNCH_RES(A) bn_fwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(x, y, partial, ws.flags, ws.epoch, spin, prm, g)
+#define LAUNCH_RES(A) bn_fwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(x, y, words, ws.epoch, spin, prm, g)
         {
             ProfScope ps("bn_fwd_resident_kernel", s);
             LUX_DISPATCH_ACT(act, LAUNCH_RES);
@@ -722,14 +708,14 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         g.chunk = (uint32_t)ceil_div(g.nq, SR);
         const int64_t S = ceil_div(g.nq, g.chunk);
         Workspace ws;
-        int rc = get_workspace(s, (size_t)C * 2 * S * sizeof(float), &ws);
+        int rc = get_workspace(s, 0, &ws);
         if (rc != LUXHIP_OK) return rc;
-        float* partial = reinterpret_cast<float*>(ws.data);
+        uint64_t* words = reinterpret_cast<uint64_t*>(ws.flags);
         const uint32_t spin = (uint32_t)option_bn_spin_limit();
         dim3 grid((unsigned)S, (unsigned)C);
 #define LAUNCH_RES(A)                                                                                               \
     bn_bwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, \
-                                                              partial, ws.flags, ws.epoch, spin, inv_count, stats_from_batch, g)
+                                                              words, ws.epoch, spin, inv_count, stats_from_batch, g)
         {
             ProfScope ps("bn_bwd_resident_kernel", s);
             LUX_DISPATCH_ACT(act, LAUNCH_RES);

@@ -25,8 +25,9 @@ int64_t option_conv_tile();       // 0 automatic, else a tile code of the bf16 w
 // ordered, so consecutive operators may share it.
 // `counters`: kWorkspaceCounters arrival counters, all zero whenever no kernel of the stream is
 // running (the workgroup that arrives last puts its counter back to zero).
-// `flags`: kWorkspaceFlags words that resident kernels set to `epoch`, a value no earlier call on
-// the stream has used (so the flags never need clearing).
+// `flags`: kWorkspaceFlags words reserved for the resident kernels' (value, epoch) exchange words;
+// `epoch` is a value no earlier call on the stream has used, so the words never need clearing and
+// no other kernel writes this memory.
 constexpr size_t kWorkspaceCounters = 65536;
 constexpr size_t kWorkspaceFlags = 4096;
 // Counters of different channels are spread over different cache lines where the channel count
@@ -360,6 +361,15 @@ __device__ __forceinline__ void publish(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint32_t fetch(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// A float together with the epoch of the call that wrote it, as one 8-byte word: the reader sees
+// either an older epoch or the complete pair, so the value needs no separate flag and the writer
+// no wait between the two.
+__device__ __forceinline__ void publish_tagged(uint64_t* p, float v, uint32_t epoch) {
+    __hip_atomic_store(p, ((uint64_t)epoch << 32) | __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t fetch_tagged(const uint64_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void publish(float* p, float v) {

@@ -222,7 +222,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                     if constexpr (KEEP_G) kd[u] = keep<T, VEC>(gv);
                 }
                 if constexpr (AFFINE) {
-                    // the first lane of the wave decides whether the wave has work this round
+                    // the first lane of the wave decides whether the wave has work in this pass
                     if (u * T_ + (w << 6) < g.nvec)
                         wave_channel_accumulate(accg, accb, active ? g.chdiv.div(q) : 0u, a, b, active);
                 }

@@ -137,7 +137,7 @@ def test_large_mean_small_variance_is_stable(gpu):
 
 
 def test_config2_full_size(gpu, bn_path):
-    """BASELINE config 2 at full size: x 32x32x64x128 ~ N(0.5, 2), train mode.  Checked against
+    """benchmark configuration 2 at full size: x 32x32x64x128 ~ N(0.5, 2), train mode.  Checked against
     the fp64 oracle on a channel subset plus size-independent invariants (zero mean / unit
     variance per channel before the affine map; sum(dx) == 0 and sum(dx * xhat) == 0 per
     channel, the two conservation laws of the batchnorm pullback)."""

@@ -70,7 +70,7 @@ def test_argument_errors(gpu):
 
 
 def test_full_size_properties(gpu):
-    """BASELINE config 2's bias_activation(relu) at full size (1024, 64, 128): checked through
+    """benchmark configuration 2's bias_activation(relu) at full size (1024, 64, 128): checked through
     size-independent properties (idempotence of relu, linearity of the pullback, the bias
     gradient equals the channel sums of dx)."""
     rng = np.random.default_rng(11)

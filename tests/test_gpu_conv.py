@@ -120,7 +120,7 @@ def test_dimension_mismatch(gpu):
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_config5_full_size(gpu, dtype):
-    """BASELINE config 5 at full size: x 56x56x128x64, w 3x3x128x128 Kaiming-normal, stride 1,
+    """benchmark configuration 5 at full size: x 56x56x128x64, w 3x3x128x128 Kaiming-normal, stride 1,
     pad 1, relu.  Forward and input gradient: fp64 oracle on two images.  Filter gradient: the
     adjoint identity <dw, w'> == <dz, conv(x, w')> against the (checked) forward kernel plus an
     fp64 oracle on a two-image batch.  Bias gradient: fp64 channel sums."""

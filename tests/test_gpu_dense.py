@@ -111,7 +111,7 @@ def test_views_with_leading_dimension(gpu):
 
 
 def test_config1(gpu):
-    """BASELINE config 1: W 256x128 Glorot-uniform, x 128x64, bias 256, tanh, fp32."""
+    """benchmark configuration 1: W 256x128 Glorot-uniform, x 128x64, bias 256, tanh, fp32."""
     rng = np.random.default_rng(1000)
     lim = np.sqrt(6.0 / 384.0)
     W = rng.uniform(-lim, lim, size=(256, 128)).astype(np.float32)
@@ -130,7 +130,7 @@ def test_config1(gpu):
 
 
 def test_config4_dense_full_size(gpu):
-    """BASELINE config 4's first dense layer at full size (4096 -> 11008, 8192 tokens, gelu,
+    """benchmark configuration 4's first dense layer at full size (4096 -> 11008, 8192 tokens, gelu,
     bf16 storage / fp32 accumulation): output rows, weight-gradient rows and input-gradient
     columns are spot-checked against the fp64 oracle; linearity of the pullback in the
     cotangent is checked on the whole tensors."""

@@ -63,7 +63,7 @@ def test_argument_errors(gpu):
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_config3_full_size(gpu, dtype):
-    """BASELINE config 3 at full size: x 64x64x256x16, 32 groups, swish.  Oracle comparison on
+    """benchmark configuration 3 at full size: x 64x64x256x16, 32 groups, swish.  Oracle comparison on
     two samples; whole-tensor invariants: per-(group, sample) slices of dx sum to zero and are
     orthogonal to xhat (the two conservation laws of the normalisation pullback)."""
     rng = np.random.default_rng(1002)

@@ -71,7 +71,7 @@ def test_default_dims_and_errors(gpu):
 
 
 def test_config4_layernorm_full_size(gpu):
-    """BASELINE config 4's layernorm: 4096 features x 8192 tokens, bf16, affine.  Oracle on a
+    """benchmark configuration 4's layernorm: 4096 features x 8192 tokens, bf16, affine.  Oracle on a
     token subset; invariants on all tokens (normalised rows have zero mean / unit variance;
     dx rows sum to zero and are orthogonal to xhat)."""
     rng = np.random.default_rng(1003)
