@@ -133,6 +133,8 @@ __global__ __launch_bounds__(kThreads) void act_bwd_kernel(const T* __restrict__
     }
 }
 
+constexpr int kChanVecs = 4;   // vectors per thread of the channel-layout pullback
+
 // "channel" layout: grid (S, C).  Workgroup (s, c) handles vectors [s*chunk, (s+1)*chunk) of
 // the nq = I*N/VEC vectors of channel c and publishes its partial sum; the workgroup of a
 // channel that arrives last adds the S partials in index order (same result on every run).
@@ -150,22 +152,30 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T*
     const uint32_t q0 = s * chunk;
     const uint32_t q1 = min(q0 + chunk, nq);
     float acc = 0.0f;
-    // One vector per thread (the usual split): the partial sum is handed over before dx is
-    // stored, so the hand-off does not wait for the stores.
-    const bool single = chunk <= kThreads;
-    float r0[VEC];
-    size_t off0 = 0;
-    bool have0 = false;
+    // Up to kChanVecs vectors per thread (the usual split): all loads in flight together, and the
+    // partial sum is handed over before dx is stored, so the hand-off does not wait for the stores.
+    const bool single = chunk <= kThreads * kChanVecs;
+    float r0[kChanVecs][VEC];
+    size_t off0[kChanVecs];
+    bool have0[kChanVecs];
     if (single) {
-        const uint32_t q = q0 + threadIdx.x;
-        if (q < q1) {
-            const uint32_t n = rowdiv.div(q);
-            off0 = ((size_t)q + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
-            dx_vec<T, ACT, VEC>(delta, out, pre, off0, r0);
-            have0 = true;
+        // all loads of the thread are issued before the first use
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) acc += r0[k];
+        for (int u = 0; u < kChanVecs; ++u) {
+            const uint32_t q = q0 + u * kThreads + threadIdx.x;
+            have0[u] = q < q1;
+            const uint32_t qq = have0[u] ? q : q1 - 1;            // past the end: last vector again (ignored)
+            const uint32_t n = rowdiv.div(qq);
+            off0[u] = ((size_t)qq + (size_t)vec_per_row * ((size_t)n * (C - 1) + c)) * VEC;
         }
+#pragma unroll
+        for (int u = 0; u < kChanVecs; ++u) dx_vec<T, ACT, VEC>(delta, out, pre, off0[u], r0[u]);
+#pragma unroll
+        for (int u = 0; u < kChanVecs; ++u)
+            if (have0[u]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc += r0[u][k];
+            }
     } else {
         for (uint32_t q = q0 + threadIdx.x; q < q1; q += kThreads) {
             const uint32_t n = rowdiv.div(q);
@@ -183,7 +193,11 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_channel_kernel(const T*
         publish_done();
     }
     const bool last = arrive_last(counters + (size_t)c * cstride, S, &last_flag);
-    if (single && have0 && dx) store_vec<T, VEC>(dx, off0, r0);
+    if (single && dx) {
+#pragma unroll
+        for (int u = 0; u < kChanVecs; ++u)
+            if (have0[u]) store_vec<T, VEC>(dx, off0[u], r0[u]);
+    }
     if (!last) return;
     if (threadIdx.x < 64) {
         float t = 0.0f;
@@ -344,7 +358,7 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
         const bool vec = ptr_ok && I % V == 0;
         const int vv = vec ? V : 1;
         const uint32_t nq = (uint32_t)(I * N / vv);
-        int64_t S = ceil_div(nq, kThreads);
+        int64_t S = ceil_div(nq, kThreads * kChanVecs);
         const int64_t smax = std::min<int64_t>(kThreads, std::max<int64_t>(1, 16384 / C));
         if (S > smax) S = smax;
         if (S < 1) S = 1;
