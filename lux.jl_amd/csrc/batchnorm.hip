@@ -31,7 +31,7 @@
 namespace luxhip {
 
 constexpr int kBnThreads = 256;
-constexpr int kBnUnroll = 1;  // one 16-byte vector per thread and a huge grid streams fastest on MI355X
+constexpr int kBnUnroll = 4;  // 16-byte vectors per thread; all of a thread's loads are issued before the first use
 
 struct ChanGeom {
     uint32_t nq;           // vectors per channel = I*N / VEC
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const T* __restric
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
             idx[u] = base + u * kBnThreads + threadIdx.x;
-            if (idx[u] < total_vec) load_vec<T, VEC>(x, (size_t)idx[u] * VEC, v[u]);
+            load_vec<T, VEC>(x, (size_t)min(idx[u], total_vec - 1) * VEC, v[u]);   // past the end: ignored below
         }
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
@@ -311,10 +311,9 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const T* __res
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
             idx[u] = base + u * kBnThreads + threadIdx.x;
-            if (idx[u] < total_vec) {
-                load_vec<T, VEC>(delta, (size_t)idx[u] * VEC, d[u]);
-                load_vec<T, VEC>(x, (size_t)idx[u] * VEC, v[u]);
-            }
+            const size_t off = (size_t)min(idx[u], total_vec - 1) * VEC;   // past the end: ignored below
+            load_vec<T, VEC>(delta, off, d[u]);
+            load_vec<T, VEC>(x, off, v[u]);
         }
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {

@@ -15,7 +15,7 @@
 namespace luxhip {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 1;  // one 16-byte vector per thread and a huge grid streams fastest on MI355X
+constexpr int kUnroll = 4;  // 16-byte vectors per thread; all of a thread's loads are issued before the first use
 
 // ------------------------------------------------------------------------------- forward
 template <typename T, int ACT, int VEC, bool HAS_BIAS, bool WRITE_PRE>
@@ -29,10 +29,9 @@ __global__ __launch_bounds__(kThreads) void bias_act_fwd_kernel(const T* __restr
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             idx[u] = base + u * kThreads + threadIdx.x;
-            if (idx[u] < total_vec) {
-                if constexpr (VEC == 1) v[u][0] = ld(x + idx[u]);
-                else Vec<T>::load(x + (size_t)idx[u] * VEC, v[u]);
-            }
+            const uint32_t li = min(idx[u], total_vec - 1);      // past the end: last vector again (ignored below)
+            if constexpr (VEC == 1) v[u][0] = ld(x + li);
+            else Vec<T>::load(x + (size_t)li * VEC, v[u]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -121,14 +120,16 @@ template <typename T, int ACT, int VEC>
 __global__ __launch_bounds__(kThreads) void act_bwd_kernel(const T* __restrict__ delta, const T* __restrict__ out,
                                                            const T* __restrict__ pre, T* dx, uint32_t total_vec) {
     for (uint32_t base = blockIdx.x * (kThreads * kUnroll); base < total_vec; base += gridDim.x * (kThreads * kUnroll)) {
+        float r[kUnroll][VEC];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            uint32_t idx = base + u * kThreads + threadIdx.x;
-            if (idx < total_vec) {
-                float r[VEC];
-                dx_vec<T, ACT, VEC>(delta, out, pre, (size_t)idx * VEC, r);
-                store_vec<T, VEC>(dx, (size_t)idx * VEC, r);
-            }
+            const uint32_t li = min(base + u * kThreads + threadIdx.x, total_vec - 1);   // past the end: ignored below
+            dx_vec<T, ACT, VEC>(delta, out, pre, (size_t)li * VEC, r[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t idx = base + u * kThreads + threadIdx.x;
+            if (idx < total_vec) store_vec<T, VEC>(dx, (size_t)idx * VEC, r[u]);
         }
     }
 }
