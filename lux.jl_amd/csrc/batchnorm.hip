@@ -7,14 +7,16 @@
 // scheduling.  No floating-point atomics and no cache-wide fences (see common.h, cross-workgroup
 // hand-off).
 //
-// Resident path (tensor fits the register file: C*S <= compute units, slice <= 8 vectors per
-// thread of a 1024-thread workgroup), one kernel and one trip through HBM per tensor:
+// Resident path (tensor fits the register file: C*S <= workgroups the device holds at once,
+// slice <= 8 vectors per thread of a 512-thread workgroup, two workgroups per compute unit),
+// one kernel and one trip through HBM per tensor:
 //   forward : bn_fwd_resident_kernel  load x -> slice statistics -> publish as (value, epoch)
 //             words, collect the words of the channel's other slices -> mean/invstd (+ running
 //             stats, saved stats) -> write y
 //   pullback: bn_bwd_resident_kernel  load delta, x -> slice sums -> publish, wait -> dgamma, dbeta
 //             -> write dx
-//   All workgroups of the grid are resident at once (one per compute unit), so the wait ends as
+//   All workgroups of the grid are resident at once (the host asks the occupancy calculator how
+//   many a compute unit holds), so the wait ends as
 //   soon as the slowest peer has published.  The wait is bounded all the same: a workgroup that
 //   gives up recomputes the peers' partials itself from global memory.
 // Streaming path (any size):
@@ -25,6 +27,8 @@
 //   pullback          : bn_bwd_reduce_kernel (read delta, x) -> partials; last arriver -> dgamma,
 //                       dbeta, per-channel coefficients;  bn_bwd_apply_kernel (read delta, x, write dx)
 #include <algorithm>
+#include <mutex>
+#include <unordered_map>
 
 #include "common.h"
 
@@ -340,9 +344,10 @@ __global__ __launch_bounds__(kBnThreads) void bn_bwd_apply_kernel(const T* __res
 }
 
 // ------------------------------------------------------------------------------- resident path
-constexpr int kResThreads = 1024;   // one workgroup per compute unit
+constexpr int kResThreads = 512;    // two workgroups per compute unit
 constexpr int kResVecs = 8;         // 16-byte vectors per thread held in registers
-constexpr int kResMaxSlices = 256;
+constexpr int kResMaxSlices = kResThreads / 3;   // one thread per exchange word, three words per slice
+constexpr int kResPerCu = 1024 / kResThreads;   // resident workgroups per compute unit the kernels are compiled for
 
 // Slice `slice` of channel c -> registers.  Vector u of a thread is vector q0 + u*1024 + tid of
 // the slice; loads past the end of the slice are redirected to its last vector (every load is
@@ -407,7 +412,7 @@ __device__ __forceinline__ bool res_collect(const uint64_t* words, uint32_t nw, 
 }
 
 template <typename T, int ACT>
-__global__ __launch_bounds__(kResThreads) void bn_fwd_resident_kernel(const T* __restrict__ x, T* __restrict__ y,
+__global__ __launch_bounds__(kResThreads, kResPerCu) void bn_fwd_resident_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                       uint64_t* words, uint32_t epoch,
                                                                       uint32_t spin_limit, BnFwdParams prm, ChanGeom g) {
     constexpr int VEC = Vec<T>::N;
@@ -495,7 +500,7 @@ __device__ __forceinline__ void res_bwd_slice_sums(const ChanGeom& g, uint32_t s
 }
 
 template <typename T, int ACT>
-__global__ __launch_bounds__(kResThreads) void bn_bwd_resident_kernel(
+__global__ __launch_bounds__(kResThreads, kResPerCu) void bn_bwd_resident_kernel(
     const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const float* __restrict__ save_mean, const float* __restrict__ save_invstd, T* __restrict__ dx, T* dgamma, T* dbeta,
     uint64_t* words, uint32_t epoch, uint32_t spin_limit, float inv_count, int stats_from_batch, ChanGeom g) {
@@ -564,20 +569,35 @@ __global__ __launch_bounds__(kResThreads) void bn_bwd_resident_kernel(
     }
 }
 
+// Workgroups of a resident kernel that one compute unit holds at once (register use decides; the
+// exchange between the workgroups of a channel needs all of them on the device together).
+static int resident_per_cu(const void* kernel) {
+    static std::mutex mu;
+    static std::unordered_map<const void*, int> cache;
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = cache.find(kernel);
+    if (it != cache.end()) return it->second;
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, kResThreads, 0) != hipSuccess) n = 0;
+    cache[kernel] = n;
+    return n;
+}
+
 // Slices per channel for the resident path, 0 if the tensor does not qualify.
-static int64_t resident_slices(int64_t I, int64_t C, int64_t N, int vec, bool aligned) {
-    if (!option_bn_resident() || !aligned || I % vec != 0) return 0;
-    const int64_t cus = num_cus();
-    if (C > cus) return 0;
+static int64_t resident_slices(int64_t I, int64_t C, int64_t N, int vec, bool aligned, int per_cu) {
+    if (!option_bn_resident() || !aligned || I % vec != 0 || per_cu < 1) return 0;
+    const int64_t slots = (int64_t)per_cu * num_cus();
+    if (C > slots) return 0;
     const int64_t nq = I * N / vec;
     const int64_t per_wg = (int64_t)kResThreads * kResVecs;
     const int64_t s_need = ceil_div(nq, per_wg);
-    const int64_t s_max = std::min<int64_t>(cus / C, kResMaxSlices);
+    // slices: bounded by the resident workgroups, by one polling thread per exchange word and by
+    // the exchange area (three 8-byte words per slice)
+    const int64_t s_max = std::min<int64_t>({slots / C, (int64_t)kResMaxSlices, (int64_t)(kWorkspaceFlags / 6) / C});
     if (s_need > s_max) return 0;
     // as many slices as fit (more compute units busy) while a slice keeps at least one vector per thread
     int64_t S = std::min<int64_t>(s_max, std::max<int64_t>(s_need, nq / kResThreads));
     if (S < 1) S = 1;
-    if ((size_t)(C * S) * 6 > kWorkspaceFlags) return 0;   // three 8-byte exchange words per slice
     return S;
 }
 
@@ -628,7 +648,11 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     prm.save_mean = save_mean; prm.save_invstd = save_invstd;
     prm.count = (float)(I * N); prm.momentum = momentum; prm.eps = eps;
 
-    const int64_t SR = batch_stats ? resident_slices(I, C, N, V, vec) : 0;
+    const void* res_kernel = nullptr;
+#define PICK_RES(A) res_kernel = reinterpret_cast<const void*>(&bn_fwd_resident_kernel<T, A>)
+    LUX_DISPATCH_ACT(act, PICK_RES);
+#undef PICK_RES
+    const int64_t SR = batch_stats ? resident_slices(I, C, N, V, vec, resident_per_cu(res_kernel)) : 0;
     if (SR > 0) {
         ChanGeom g;
         g.nq = (uint32_t)(I * N / V);
@@ -697,7 +721,11 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
     const int vv = vec ? V : 1;
     const float inv_count = 1.0f / (float)(I * N);
 
-    const int64_t SR = resident_slices(I, C, N, V, vec);
+    const void* res_kernel = nullptr;
+#define PICK_RES(A) res_kernel = reinterpret_cast<const void*>(&bn_bwd_resident_kernel<T, A>)
+    LUX_DISPATCH_ACT(act, PICK_RES);
+#undef PICK_RES
+    const int64_t SR = resident_slices(I, C, N, V, vec, resident_per_cu(res_kernel));
     if (SR > 0) {
         ChanGeom g;
         g.nq = (uint32_t)(I * N / V);

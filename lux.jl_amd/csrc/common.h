@@ -29,7 +29,7 @@ int64_t option_conv_tile();       // 0 automatic, else a tile code of the bf16 w
 // `epoch` is a value no earlier call on the stream has used, so the words never need clearing and
 // no other kernel writes this memory.
 constexpr size_t kWorkspaceCounters = 65536;
-constexpr size_t kWorkspaceFlags = 4096;
+constexpr size_t kWorkspaceFlags = 16384;
 // Counters of different channels are spread over different cache lines where the channel count
 // allows it: arrivals of all channels in one line would queue up behind each other.
 inline uint32_t counter_stride(int64_t channels) {
