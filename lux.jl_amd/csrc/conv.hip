@@ -103,19 +103,45 @@ __global__ void pack_filter_kernel(const T* __restrict__ w, T* __restrict__ out,
     out[idx] = w[a + g.kW * (b + g.kH * (ci + g.Cin_g * co))];
 }
 
-// dw[a, b, ci, g*Cout_g + col] = sum over slices of partial[slice][m' = t*Cin_g + ci][col]
+// dw[a, b, ci, g*Cout_g + col] = sum over slices of partial[slice][m' = t*Cin_g + ci][col].
+// A thread owns 4 consecutive m' (one 16-byte load per slice, eight slices in flight); slices are
+// added in order.
 template <typename T>
-__global__ void wgrad_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw, ConvGeom g, int grp, int slices) {
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw, ConvGeom g,
+                                                           int grp, int slices) {
     const int Mrows = g.kW * g.kH * g.Cin_g;
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= Mrows * g.Cout_g) return;
-    const int m = idx % Mrows, col = idx / Mrows;
-    float acc = 0.0f;
-    for (int sl = 0; sl < slices; ++sl) acc += partial[(size_t)sl * Mrows * g.Cout_g + idx];
-    const int t = m / g.Cin_g, ci = m - t * g.Cin_g;
-    const int ka = t % g.kW, kb = t / g.kW;
-    const int a = g.flip ? ka : g.kW - 1 - ka, b = g.flip ? kb : g.kH - 1 - kb;
-    st(dw + a + g.kW * (b + g.kH * (ci + g.Cin_g * (grp * g.Cout_g + col))), acc);
+    const int total = Mrows * g.Cout_g;
+    const int idx = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (idx >= total) return;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool vec = (total & 3) == 0;                 // then idx + 3 < total and every slice row is 16-byte aligned
+    if (vec) {
+        int sl = 0;
+        for (; sl + 8 <= slices; sl += 8) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(partial + (size_t)(sl + u) * total + idx);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { acc[0] += v[u].x; acc[1] += v[u].y; acc[2] += v[u].z; acc[3] += v[u].w; }
+        }
+        for (; sl < slices; ++sl) {
+            const float4 v = *reinterpret_cast<const float4*>(partial + (size_t)sl * total + idx);
+            acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+        }
+    } else {
+        for (int sl = 0; sl < slices; ++sl)
+            for (int e = 0; e < 4; ++e)
+                if (idx + e < total) acc[e] += partial[(size_t)sl * total + idx + e];
+    }
+    for (int e = 0; e < 4; ++e) {
+        const int id = idx + e;
+        if (id >= total) break;
+        const int m = id % Mrows, col = id / Mrows;
+        const int t = m / g.Cin_g, ci = m - t * g.Cin_g;
+        const int ka = t % g.kW, kb = t / g.kW;
+        const int a = g.flip ? ka : g.kW - 1 - ka, b = g.flip ? kb : g.kH - 1 - kb;
+        st(dw + a + g.kW * (b + g.kH * (ci + g.Cin_g * (grp * g.Cout_g + col))), acc[e]);
+    }
 }
 
 // ----------------------------------------------------------------------------- host helpers
@@ -325,7 +351,7 @@ static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy,
         if (rc != LUXHIP_OK) return rc;
         ProfScope ps("wgrad_reduce_kernel", s);
         const int total = Mrows * g.Cout_g;
-        wgrad_reduce_kernel<T><<<(unsigned)ceil_div(total, 256), 256, 0, s>>>(partial, dw, g, grp, slices);
+        wgrad_reduce_kernel<T><<<(unsigned)ceil_div(total, 1024), 256, 0, s>>>(partial, dw, g, grp, slices);
         LUX_CHECK_LAUNCH();
     }
     return LUXHIP_OK;
