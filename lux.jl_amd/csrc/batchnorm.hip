@@ -60,17 +60,6 @@ __device__ __forceinline__ void store_vecn(T* p, size_t off, const float (&v)[VE
     else Vec<T>::store(p + off, v);
 }
 
-// Chan et al. pairwise combination of (count, mean, M2).
-__device__ __forceinline__ void chan_merge(float& n, float& mean, float& m2, float nb, float meanb, float m2b) {
-    const float nn = n + nb;
-    if (nn == 0.0f) return;
-    const float delta = meanb - mean;
-    const float f = nb / nn;
-    mean += delta * f;
-    m2 += m2b + delta * delta * n * f;
-    n = nn;
-}
-
 // ------------------------------------------------------------------------------- statistics
 struct BnFwdParams {
     const void *gamma, *beta, *rmean, *rvar;   // storage type T
@@ -393,24 +382,6 @@ __device__ __forceinline__ void res_slice_stats(const ChanGeom& g, uint32_t slic
     m2 = block_sum(dev, sm);
 }
 
-// The nw = K*S exchange words of a channel (K per slice) -> parts[0..nw) in LDS.  Thread i polls
-// word i until it carries `epoch`; false for the whole workgroup if any poll ran out of tries.
-// Contains workgroup barriers.
-__device__ __forceinline__ bool res_collect(const uint64_t* words, uint32_t nw, uint32_t epoch, uint32_t spin_limit,
-                                            float* parts) {
-    int failed = 0;
-    if (threadIdx.x < nw) {
-        uint32_t tries = 0;
-        for (;;) {
-            const uint64_t wv = fetch_tagged(words + threadIdx.x);
-            if ((uint32_t)(wv >> 32) == epoch) { parts[threadIdx.x] = __uint_as_float((uint32_t)wv); break; }
-            if (tries++ >= spin_limit) { failed = 1; break; }
-            __builtin_amdgcn_s_sleep(2);
-        }
-    }
-    return __syncthreads_or(failed) == 0;
-}
-
 template <typename T, int ACT>
 __global__ __launch_bounds__(kResThreads, kResPerCu) void bn_fwd_resident_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                       uint64_t* words, uint32_t epoch,
@@ -430,7 +401,7 @@ __global__ __launch_bounds__(kResThreads, kResPerCu) void bn_fwd_resident_kernel
         publish_tagged(chan_words + 3 * s + 1, mean, epoch);
         publish_tagged(chan_words + 3 * s + 2, m2, epoch);
     }
-    if (!res_collect(chan_words, 3 * S, epoch, spin_limit, parts)) {
+    if (!collect_tagged(chan_words, 3 * S, epoch, spin_limit, parts)) {
         // a peer did not show up in time: its share is recomputed here, the own slice last so
         // that v holds it again afterwards
         for (uint32_t i = 0; i <= S; ++i) {
@@ -522,7 +493,7 @@ __global__ __launch_bounds__(kResThreads, kResPerCu) void bn_bwd_resident_kernel
         publish_tagged(chan_words + 2 * s, s1, epoch);
         publish_tagged(chan_words + 2 * s + 1, s2, epoch);
     }
-    if (!res_collect(chan_words, 2 * S, epoch, spin_limit, parts)) {
+    if (!collect_tagged(chan_words, 2 * S, epoch, spin_limit, parts)) {
         for (uint32_t i = 0; i <= S; ++i) {   // recompute the peers' sums; own slice last (d, v restored)
             const uint32_t slice = i < S ? i : s;
             __syncthreads();

@@ -351,6 +351,17 @@ __device__ __forceinline__ float block_sum(float v, float* smem) {
     return t;
 }
 
+// Chan et al. pairwise combination of (count, mean, M2).
+__device__ __forceinline__ void chan_merge(float& n, float& mean, float& m2, float nb, float meanb, float m2b) {
+    const float nn = n + nb;
+    if (nn == 0.0f) return;
+    const float delta = meanb - mean;
+    const float f = nb / nn;
+    mean += delta * f;
+    m2 += m2b + delta * delta * n * f;
+    n = nn;
+}
+
 // ----------------------------------------------------------------------------- cross-workgroup hand-off
 // Partial results travel between workgroups through agent-scope atomic stores and loads, which
 // go past the per-XCD L2 caches, so no cache-wide release fence (an L2 write-back of everything
@@ -371,6 +382,23 @@ __device__ __forceinline__ void publish_tagged(uint64_t* p, float v, uint32_t ep
 }
 __device__ __forceinline__ uint64_t fetch_tagged(const uint64_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// words[0..nw) -> parts[0..nw) in LDS: thread i polls word i until it carries `epoch`.  False for
+// the whole workgroup if any poll ran out of tries (then parts is incomplete).  Needs nw <=
+// blockDim.x; contains workgroup barriers.
+__device__ __forceinline__ bool collect_tagged(const uint64_t* words, uint32_t nw, uint32_t epoch, uint32_t spin_limit,
+                                               float* parts) {
+    int failed = 0;
+    if (threadIdx.x < nw) {
+        uint32_t tries = 0;
+        for (;;) {
+            const uint64_t wv = fetch_tagged(words + threadIdx.x);
+            if ((uint32_t)(wv >> 32) == epoch) { parts[threadIdx.x] = __uint_as_float((uint32_t)wv); break; }
+            if (tries++ >= spin_limit) { failed = 1; break; }
+            __builtin_amdgcn_s_sleep(2);
+        }
+    }
+    return __syncthreads_or(failed) == 0;
 }
 __device__ __forceinline__ void publish(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

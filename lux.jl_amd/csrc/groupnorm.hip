@@ -5,7 +5,10 @@
 //   * cached kernels keep the slice (forward: x; pullback: delta and x) in registers, so HBM
 //     sees every tensor once: statistics, normalisation and the input gradient all come from
 //     the registers (slices of up to kGnCache vectors per thread x 1024 threads);
-//   * streaming kernels handle larger slices with a second read of the slice.
+//   * a slice too long for a 512-thread workgroup is split between two of them (each owns whole
+//     channels); the halves exchange their partial statistics as (value, epoch) words, with a
+//     bounded wait after which a workgroup recomputes its peer's share from global memory;
+//   * streaming kernels handle still larger slices with a second read of the slice.
 // Per-channel gradients (dgamma, dbeta) are accumulated per wave in LDS in program order,
 // combined across waves in a fixed order, published as [N][C] partials and added over N, in
 // sample order, by the workgroup of each group that arrives last: deterministic, no
@@ -21,6 +24,7 @@ constexpr int kGnCache = 8;  // vectors per thread kept in registers
 struct GnGeom {
     uint32_t I, Cg, G, C;
     uint32_t nvec;         // vectors per slice = I*Cg / VEC
+    uint32_t parts, pvec;  // workgroups per slice (cached kernels; 1 otherwise) and vectors per part = nvec / parts
     FastDiv chdiv;         // vector index -> channel within group: / (I / VEC)   (VEC == 1: / I)
     float inv_m;           // 1 / (I*Cg)
 };
@@ -37,6 +41,12 @@ __device__ __forceinline__ void gn_store(T* p, size_t off, const float (&v)[VEC]
 }
 
 // ------------------------------------------------------------------------------- forward
+// Exchange area of the split kernels: `epoch`-tagged words, K per part, parts of a slice adjacent.
+struct GnExchange {
+    uint64_t* words;
+    uint32_t epoch, spin_limit;
+};
+
 template <typename T, int ACT, int VEC, bool CACHED>
 __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, T* y,
                               float* save_mean, float* save_invstd, GnGeom g, float eps) {
@@ -149,13 +159,17 @@ template <typename T, int ACT, int VEC, bool CACHED, bool AFFINE>
 __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma,
                               const T* __restrict__ beta, const float* __restrict__ save_mean,
                               const float* __restrict__ save_invstd, T* dx, float* pdg, float* pdb, T* dgamma,
-                              T* dbeta, uint32_t* counters, uint32_t cstride, uint32_t N, GnGeom g) {
+                              T* dbeta, uint32_t* counters, uint32_t cstride, uint32_t N, GnGeom g, GnExchange ex) {
     extern __shared__ float lds[];                  // [16] reduction scratch, then [nw][Cg] x 2
     float* sm = lds;
     const uint32_t T_ = blockDim.x, nw = T_ >> 6, w = threadIdx.x >> 6;
     float* accg = lds + 16 + (size_t)w * g.Cg;
     float* accb = lds + 16 + (size_t)(nw + w) * g.Cg;
-    const uint32_t slice = blockIdx.x, k = slice % g.G, n = slice / g.G;
+    __shared__ float pst[2 * 4 + 2];                // exchanged part sums (parts <= 4), then the slice totals
+    const uint32_t parts = CACHED ? g.parts : 1u;
+    const uint32_t slice = blockIdx.x / parts, part = blockIdx.x - slice * parts;
+    const uint32_t k = slice % g.G, n = slice / g.G;
+    const uint32_t qbeg = part * g.pvec, qend = CACHED ? qbeg + g.pvec : g.nvec;   // this workgroup's vectors of the slice
     const size_t base = (size_t)slice * g.nvec * VEC;
     const float mean = save_mean[slice], invstd = save_invstd[slice];
     if constexpr (AFFINE) {
@@ -193,11 +207,11 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         }
     };
 
-    const uint32_t iters = (g.nvec + T_ - 1) / T_;
+    const uint32_t iters = (qend - qbeg + T_ - 1) / T_;
     if constexpr (CACHED) {
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
-            const size_t off = base + (size_t)min(u * T_ + threadIdx.x, g.nvec - 1) * VEC;   // past the end: last vector again
+            const size_t off = base + (size_t)min(qbeg + u * T_ + threadIdx.x, qend - 1) * VEC;   // past the end: last vector again
             kd[u] = K::load(delta, off);
             kv[u] = K::load(x, off);
         }
@@ -206,8 +220,8 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
             if ((uint32_t)u < iters) {              // uniform
-                const uint32_t q = u * T_ + threadIdx.x;
-                const bool active = q < g.nvec;
+                const uint32_t q = qbeg + u * T_ + threadIdx.x;
+                const bool active = q < qend;
                 float gv[VEC], a = 0.0f, b = 0.0f;
                 if (active) {
                     K::get(kd[u], d[0]);
@@ -223,7 +237,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                 }
                 if constexpr (AFFINE) {
                     // the first lane of the wave decides whether the wave has work in this pass
-                    if (u * T_ + (w << 6) < g.nvec)
+                    if (qbeg + u * T_ + (w << 6) < qend)
                         wave_channel_accumulate(accg, accb, active ? g.chdiv.div(q) : 0u, a, b, active);
                 }
             }
@@ -250,13 +264,54 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
             }
         }
     }
-    s1 = block_sum(s1, sm) * g.inv_m;
-    s2 = block_sum(s2, sm) * g.inv_m;
+    s1 = block_sum(s1, sm);
+    s2 = block_sum(s2, sm);
+    if (parts > 1) {
+        // part sums -> the other workgroups of the slice; added in part order
+        uint64_t* words = ex.words + (size_t)slice * parts * 2;
+        if (threadIdx.x == 0) {
+            publish_tagged(words + 2 * part, s1, ex.epoch);
+            publish_tagged(words + 2 * part + 1, s2, ex.epoch);
+        }
+        if (!collect_tagged(words, 2 * parts, ex.epoch, ex.spin_limit, pst)) {
+            // a peer did not show up in time: its sums are recomputed here from global memory
+            for (uint32_t i = 0; i < parts; ++i) {
+                float t1 = 0.0f, t2 = 0.0f;
+                for (uint32_t q = i * g.pvec + threadIdx.x; q < (i + 1) * g.pvec; q += T_) {
+                    float gv[VEC], a, b;
+                    gn_load<T, VEC>(delta, base + (size_t)q * VEC, d[0]);
+                    gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+                    grad_terms(q, d[0], v[0], gv, a, b);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        t1 += gv[e];
+                        t2 = fmaf(gv[e], (v[0][e] - mean) * invstd, t2);
+                    }
+                }
+                t1 = block_sum(t1, sm);
+                t2 = block_sum(t2, sm);
+                if (threadIdx.x == 0) { pst[2 * i] = t1; pst[2 * i + 1] = t2; }
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            float t1 = 0.0f, t2 = 0.0f;
+            for (uint32_t i = 0; i < parts; ++i) { t1 += pst[2 * i]; t2 += pst[2 * i + 1]; }
+            pst[8] = t1;
+            pst[9] = t2;
+        }
+        __syncthreads();
+        s1 = pst[8];
+        s2 = pst[9];
+    }
+    s1 *= g.inv_m;
+    s2 *= g.inv_m;
 
     // Parameter gradients first (they only need the first pass), so that their hand-off does not
     // wait for the dx stores below.
     if constexpr (AFFINE) {
-        for (uint32_t j = threadIdx.x; j < g.Cg; j += T_) {
+        const uint32_t jbeg = part * (g.Cg / parts), jend = jbeg + g.Cg / parts;   // a part owns whole channels
+        for (uint32_t j = jbeg + threadIdx.x; j < jend; j += T_) {
             float tg = 0.0f, tb = 0.0f;
             for (uint32_t ww = 0; ww < nw; ++ww) {
                 tg += lds[16 + (size_t)ww * g.Cg + j];
@@ -266,10 +321,10 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
             publish(pdb + (size_t)n * g.C + k * g.Cg + j, tb);
         }
         publish_done();
-        // the workgroup of group k that arrives last (one per sample) adds the N per-sample
+        // the workgroup of group k that arrives last (parts per sample) adds the N per-sample
         // partials of the group's channels in sample order
         uint32_t* last_flag = reinterpret_cast<uint32_t*>(lds + 15);   // a word of the reduction scratch that is free now
-        if (arrive_last(counters + (size_t)k * cstride, N, last_flag)) {
+        if (arrive_last(counters + (size_t)k * cstride, N * parts, last_flag)) {
             for (uint32_t j = threadIdx.x; j < g.Cg; j += T_) {
                 float tg = 0.0f, tb = 0.0f;
                 for (uint32_t nn = 0; nn < N; ++nn) {
@@ -295,8 +350,8 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     if constexpr (CACHED) {
 #pragma unroll
         for (int u = 0; u < kGnCache; ++u) {
-            const uint32_t q = u * T_ + threadIdx.x;
-            if (q < g.nvec) {
+            const uint32_t q = qbeg + u * T_ + threadIdx.x;
+            if (q < qend) {
                 K::get(kd[u], d[0]);
                 K::get(kv[u], v[0]);
                 if constexpr (KEEP_G) {             // kd[u] holds dy * gamma
@@ -342,7 +397,7 @@ struct GnLaunch {
 };
 
 template <typename T>
-static GnLaunch gn_plan(int64_t I, int64_t C, int64_t G, int64_t N, bool ptr_ok) {
+static GnLaunch gn_plan(int64_t I, int64_t C, int64_t G, int64_t N, bool ptr_ok, bool allow_split) {
     constexpr int V = Vec<T>::N;
     GnLaunch L;
     const int64_t Cg = C / G, m = I * Cg;
@@ -352,19 +407,41 @@ static GnLaunch gn_plan(int64_t I, int64_t C, int64_t G, int64_t N, bool ptr_ok)
     L.g.nvec = (uint32_t)(m / vv);
     L.g.chdiv = FastDiv((uint32_t)(I / vv));
     L.g.inv_m = 1.0f / (float)m;
+    // A slice that would need a 1024-thread workgroup can be split between two 512-thread
+    // workgroups (each owns whole channels): two of them fit a compute unit even with the
+    // pullback's register footprint, and one loads while the other computes or stores.  The halves
+    // exchange their partial sums through tagged words.  Measured: 5 % faster for the pullback,
+    // slower for the forward pass (which fits twice per compute unit anyway), so only the
+    // pullback asks for it.
+    L.g.parts = 1;
+    if (allow_split && L.vec && (int64_t)L.g.nvec > 512 * kGnCache && (int64_t)L.g.nvec <= 2 * 512 * kGnCache && Cg % 2 == 0 &&
+        (L.g.nvec / 2) % (uint32_t)(I / vv) == 0 && (size_t)(G * N) * 2 * 3 * 2 <= kWorkspaceFlags)
+        L.g.parts = 2;
+    L.g.pvec = L.g.nvec / L.g.parts;
     int64_t t = 64;
-    while (t < 1024 && t * kGnCache < L.g.nvec) t <<= 1;
+    while (t < 1024 && t * kGnCache < L.g.pvec) t <<= 1;
     L.threads = (unsigned)t;
-    L.cached = (int64_t)L.g.nvec <= t * kGnCache;
-    L.blocks = (unsigned)(G * N);
+    L.cached = (int64_t)L.g.pvec <= t * kGnCache;
+    if (!L.cached) { L.g.parts = 1; L.g.pvec = L.g.nvec; }
+    L.blocks = (unsigned)(G * N * L.g.parts);
     return L;
+}
+
+static int gn_exchange(hipStream_t s, GnExchange* ex) {
+    Workspace ws;
+    int rc = get_workspace(s, 0, &ws);
+    if (rc != LUXHIP_OK) return rc;
+    ex->words = reinterpret_cast<uint64_t*>(ws.flags);
+    ex->epoch = ws.epoch;
+    ex->spin_limit = (uint32_t)option_bn_spin_limit();
+    return LUXHIP_OK;
 }
 
 template <typename T>
 static int gn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, int64_t N, const T* x, const T* gamma,
                        const T* beta, float eps, T* y, float* save_mean, float* save_invstd) {
     constexpr int V = Vec<T>::N;
-    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(y));
+    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(y), false);
     ProfScope ps("gn_fwd_kernel", s);
 #define GN_FWD(A)                                                                                                     \
     do {                                                                                                              \
@@ -384,14 +461,19 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
                        const T* gamma, const T* beta, const float* save_mean, const float* save_invstd, T* dx,
                        T* dgamma, T* dbeta) {
     constexpr int V = Vec<T>::N;
-    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(delta) && aligned16(dx));
+    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(delta) && aligned16(dx), true);
     const bool affine = gamma != nullptr && (dgamma != nullptr || dbeta != nullptr);
     // LDS: 16 floats of reduction scratch + 2 * nw * Cg accumulators
     size_t lds_bytes = 64;
     if (affine) {
         while (L.threads > 64 && (16 + 2 * (size_t)(L.threads / 64) * L.g.Cg) * 4 > 60 * 1024) {
             L.threads >>= 1;
-            L.cached = (int64_t)L.g.nvec <= (int64_t)L.threads * kGnCache;
+            L.cached = (int64_t)L.g.pvec <= (int64_t)L.threads * kGnCache;
+        }
+        if (!L.cached && L.g.parts > 1) {           // the streaming kernel works on whole slices
+            L.g.parts = 1;
+            L.g.pvec = L.g.nvec;
+            L.blocks = (unsigned)(G * N);
         }
         lds_bytes = (16 + 2 * (size_t)(L.threads / 64) * L.g.Cg) * 4;
         LUX_UNSUPPORTED_IF(lds_bytes > 60 * 1024, "groupnorm_bwd: %u channels per group exceed the LDS accumulators", L.g.Cg);
@@ -399,6 +481,11 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
     float *pdg = nullptr, *pdb = nullptr;
     uint32_t* counters = nullptr;
     const uint32_t cstride = counter_stride(G);
+    GnExchange ex;
+    {
+        int rc = gn_exchange(s, &ex);
+        if (rc != LUXHIP_OK) return rc;
+    }
     if (affine) {
         LUX_UNSUPPORTED_IF((size_t)G > kWorkspaceCounters, "groupnorm_bwd: more than %zu groups", kWorkspaceCounters);
         Workspace ws;
@@ -412,8 +499,8 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
         ProfScope ps("gn_bwd_kernel", s);
 #define GN_BWD_A(A, VV, CA)                                                                                           \
     do {                                                                                                              \
-        if (affine) gn_bwd_kernel<T, A, VV, CA, true><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g); \
-        else gn_bwd_kernel<T, A, VV, CA, false><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g);       \
+        if (affine) gn_bwd_kernel<T, A, VV, CA, true><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g, ex); \
+        else gn_bwd_kernel<T, A, VV, CA, false><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g, ex);       \
     } while (0)
 #define GN_BWD(A)                                                                                                     \
     do {                                                                                                              \

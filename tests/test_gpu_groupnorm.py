@@ -9,7 +9,18 @@ from tests.util import stable_seed, assert_close, dev, f64, host_inputs, rms
 pytestmark = pytest.mark.gpu
 
 CASES = [((6, 2), 2), ((4, 4, 6, 2), 3), ((2, 2, 6, 2), 2), ((5, 12, 3), 4), ((16, 16, 8, 3), 2), ((64, 6, 2), 3),
-         ((32, 32, 12, 2), 1), ((8, 8, 16, 2), 16), ((96, 96, 4, 2), 1)]
+         ((32, 32, 12, 2), 1), ((8, 8, 16, 2), 16), ((96, 96, 4, 2), 1),
+         # slices that two workgroups share (fp32: 19200 elements per slice, bf16: 65536)
+         ((40, 40, 24, 2), 2), ((64, 64, 32, 2), 2)]
+
+
+@pytest.fixture(params=["wait", "no_wait"])
+def gn_path(gpu, request):
+    """Slices shared by two workgroups exchange partial statistics with a bounded wait; "no_wait"
+    cuts the wait to zero polls, so every workgroup recomputes its peer's share itself."""
+    gpu.set_option("bn_spin_limit", 0 if request.param == "no_wait" else 1 << 22)
+    yield request.param
+    gpu.set_option("bn_spin_limit", 1 << 22)
 
 
 def dx_scale(x, g, groups, eps, delta):
@@ -23,7 +34,7 @@ def dx_scale(x, g, groups, eps, delta):
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("act", ["identity", "relu", "sigmoid_fast", "swish", "gelu"])
 @pytest.mark.parametrize("affine", [True, False])
-def test_forward_and_pullback(gpu, dtype, act, affine):
+def test_forward_and_pullback(gpu, gn_path, dtype, act, affine):
     rng = np.random.default_rng(stable_seed(dtype, act, affine))
     for shape, groups in CASES:
         Cc = shape[-2]
@@ -35,7 +46,7 @@ def test_forward_and_pullback(gpu, dtype, act, affine):
             # not a rounding difference
             if act != "relu" or np.abs(O.groupnorm(f64(x), f64(g), f64(b), groups, "identity", eps)).min() > 1e-3:
                 break
-        tag = f"{dtype} {act} {shape} G={groups} affine={affine}"
+        tag = f"{gn_path} {dtype} {act} {shape} G={groups} affine={affine}"
         y, back = gpu.pullback(gpu.groupnorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), groups, act, eps)
         wy = O.groupnorm(f64(x), f64(g), f64(b), groups, act, eps)
         assert_close(y.to_numpy(), wy, dtype, tag + " y", want32=O.groupnorm(x, g, b, groups, act, np.float32(eps)))
@@ -62,7 +73,7 @@ def test_argument_errors(gpu):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_config3_full_size(gpu, dtype):
+def test_config3_full_size(gpu, gn_path, dtype):
     """benchmark configuration 3 at full size: x 64x64x256x16, 32 groups, swish.  Oracle comparison on
     two samples; whole-tensor invariants: per-(group, sample) slices of dx sum to zero and are
     orthogonal to xhat (the two conservation laws of the normalisation pullback)."""
