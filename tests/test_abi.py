@@ -53,6 +53,20 @@ def test_ops_fail_loudly_without_init(lux):
         lux.init(0)
 
 
+def test_tuning_switches_validate_their_arguments(lux):
+    """luxhip_set_option needs no device: unknown names and out-of-range values are rejected with a
+    message, known switches are accepted and can be put back to their defaults."""
+    with pytest.raises(lux.LuxHipError, match="unknown option"):
+        lux.set_option("no_such_switch", 1)
+    with pytest.raises(lux.LuxHipError, match="gemm_tile"):
+        lux.set_option("gemm_tile", 7)
+    with pytest.raises(lux.LuxHipError, match="bn_spin_limit"):
+        lux.set_option("bn_spin_limit", -1)
+    for name, value in (("bn_resident", 0), ("bn_resident", 1), ("bn_spin_limit", 0), ("bn_spin_limit", 1 << 22),
+                        ("gemm_tile", 82), ("gemm_tile", 0), ("conv_tile", 84), ("conv_tile", 0)):
+        lux.set_option(name, value)
+
+
 def test_host_side_argument_checks_need_no_device(lux):
     """Shape errors are raised on the host before anything is launched
     (impl/matmul.jl:21-34, api/groupnorm.jl:40-64, api/bias_activation.jl:38-45)."""
