@@ -30,10 +30,10 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
 # size (profiles/c2_hbm_traffic_pmc.md holds the commands and the raw counter values).
 MEASURED_TRAFFIC = {
-    ("C2", "bn_fwd_resident_kernel"): 67333668,
-    ("C2", "bias_act_fwd_kernel"): 67130943,
-    ("C2", "bias_act_bwd_channel_kernel"): 101456825,
-    ("C2", "bn_bwd_resident_kernel"): 100839051,
+    ("C2", "bn_fwd_resident_kernel"): 67764601,
+    ("C2", "bias_act_fwd_kernel"): 67138039,
+    ("C2", "bias_act_bwd_channel_kernel"): 100918103,
+    ("C2", "bn_bwd_resident_kernel"): 100979652,
 }
 METRIC = "fwd+bwd TFLOP/s & HBM GB/s (% MI355X roofline) per LuxLib fused op, 1 GPU"
 

@@ -259,17 +259,20 @@ struct Act<LUXHIP_ACT_SWISH> {
 };
 template <>
 struct Act<LUXHIP_ACT_GELU> {
+    // 0.5 x (1 + tanh u) with u = sqrt(2/pi) (x + 0.044715 x^3) is x * sigmoid(2u) exactly
+    // (1 + tanh u = 2 sigmoid(2u)): no cancellation for negative x, and one exponential plus one
+    // reciprocal instead of a tanh.
     static constexpr bool needs_pre = true;
     __device__ __forceinline__ static float f(float x) {
-        float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-        return 0.5f * x * (1.0f + tanhf(u));
+        const float u2 = 1.5957691216057308f * (x + 0.044715f * x * x * x);
+        return x * sigmoidf_(u2);
     }
     __device__ __forceinline__ static float d(float, float x) {
-        float x2 = x * x;
-        float u = 0.7978845608028654f * (x + 0.044715f * x2 * x);
-        float t = tanhf(u);
-        float du = 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x2);
-        return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * du;
+        const float x2 = x * x;
+        const float u2 = 1.5957691216057308f * (x + 0.044715f * x2 * x);
+        const float s = sigmoidf_(u2);
+        const float du2 = 1.5957691216057308f * (1.0f + 3.0f * 0.044715f * x2);
+        return s + x * s * (1.0f - s) * du2;
     }
 };
 template <>
