@@ -151,8 +151,44 @@ int launch_layout(hipStream_t s, DenseArgs<T>& a) {
     // straight into LDS.  Otherwise 128 x 128 tiles (two workgroups per compute unit) measured
     // fastest on large problems; 64 x 64 for small ones.
     if constexpr (sizeof(T) == 2) {
-        if (whole_tiles<T, 256, 256>(a) && (int64_t)(a.M / 256) * (a.N / 256) >= 128)
+        if (whole_tiles<T, 256, 256>(a) && (int64_t)(a.M / 256) * (a.N / 256) >= 128) {
+            // The 256 x 256 tiles are walked in rounds of one per compute unit.  When the last
+            // round would be mostly empty, the matrix is cut along m or n: the part that makes
+            // whole rounds keeps the big tiles, the rest (at most 10 % of the tiles) goes to
+            // 128 x 128 tiles, which fill the compute units two at a time.
+            const int64_t tm = a.M / 256, tn = a.N / 256, cus = num_cus() > 0 ? num_cus() : 256;
+            const int64_t rem = (tm * tn) % cus;
+            if (rem != 0 && rem * 10 < cus * 7) {
+                for (int along_m = 1; along_m >= 0; --along_m) {
+                    const int64_t t_cut = along_m ? tm : tn, t_other = along_m ? tn : tm;
+                    int64_t keep = t_cut - 1;
+                    while (keep > 0 && (keep * t_other) % cus != 0) --keep;
+                    if (keep <= 0 || (t_cut - keep) * 10 > t_cut) continue;   // measured: a 7 % rest pays off, a 26 % rest does not
+                    DenseArgs<T> big = a, rest = a;
+                    const int64_t cut = keep * 256;
+                    if (along_m) {
+                        big.M = (int)cut;
+                        rest.M = a.M - (int)cut;
+                        rest.A.p = a.A.p + cut * a.A.sr;
+                        rest.C = a.C + cut;
+                        if (a.pre) rest.pre = a.pre + cut;
+                        if (a.bias) rest.bias = a.bias + cut;
+                    } else {
+                        big.N = (int)cut;
+                        rest.N = a.N - (int)cut;
+                        rest.B.p = a.B.p + cut * a.B.sr;
+                        rest.C = a.C + cut * a.ldc;
+                        if (a.pre) rest.pre = a.pre + cut * a.ldc;
+                    }
+                    big.A.rows = big.M; big.B.rows = big.N;
+                    rest.A.rows = rest.M; rest.B.rows = rest.N;
+                    int rc = launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, big);
+                    if (rc != LUXHIP_OK) return rc;
+                    return launch_cfg<T, 2, 2, AK, BKM>(s, rest);
+                }
+            }
             return launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, a);
+        }
     }
     const int64_t t128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
     if (a.M > 64 && a.N > 64 && t128 >= 4) return launch_cfg<T, 2, 2, AK, BKM>(s, a);

@@ -164,3 +164,23 @@ def test_config4_dense_full_size(gpu):
     gW2, gx2, _ = back(dev(gpu, 2 * delta, "bf16"))
     np.testing.assert_array_equal(gW2.to_numpy()[rows], 2 * gW.to_numpy()[rows])
     np.testing.assert_array_equal(gx2.to_numpy()[:, cols], 2 * gx.to_numpy()[:, cols])
+
+
+@pytest.mark.parametrize("ragged", ["m", "n"])
+def test_ragged_tile_rounds_bf16(gpu, ragged):
+    """43 x 32 tiles of 256 x 256 do not fill whole rounds of one tile per compute unit: the
+    library cuts such a problem into a part of whole rounds and a rest on smaller tiles.  Rows and
+    columns on both sides of the cut and at the far end are compared with the fp64 oracle."""
+    rng = np.random.default_rng(77)
+    M, N = (11008, 8192) if ragged == "m" else (8192, 11008)
+    K = 64
+    A, B, bias = host_inputs("bf16", rng.normal(size=(M, K)), rng.normal(size=(K, N)), rng.normal(size=M))
+    got = gpu.matmul(dev(gpu, A, "bf16"), dev(gpu, B, "bf16"), dev(gpu, bias, "bf16")).to_numpy()
+    want = lambda r, c: f64(A[r]) @ f64(B[:, c]) + f64(bias[r])[:, None]
+    full = slice(None)
+    cut = 10240   # 40 of the 43 tiles along the ragged dimension keep the big tiles
+    edge = np.r_[0:4, cut - 130:cut + 130, (M if ragged == "m" else N) - 4:(M if ragged == "m" else N)]
+    if ragged == "m":
+        assert_close(got[edge], want(edge, full), "bf16", "ragged m rows")
+    else:
+        assert_close(got[:, edge], want(full, edge), "bf16", "ragged n cols")
