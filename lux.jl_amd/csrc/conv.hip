@@ -247,6 +247,7 @@ static int run_conv_gemm(hipStream_t s, const ConvGeom& g, bool dgrad, const T* 
             a.Ctot_out = dgrad ? g.Cin : g.Cout;
             a.col_off = grp * Ncols;
             a.act = act;
+            a.m_begin = 0;
             rc = launch_conv_tap_any<T>(s, a);
         } else {
             ConvGemmArgs<T> a;

@@ -374,6 +374,7 @@ struct ConvTapArgs {
     const T* bias;
     int Ctot_out, col_off, act;
     int tiles_m, tiles_n;
+    int m_begin;                       // first row of this launch (rows m_begin .. tap.M are tiled)
 };
 
 // Persistent: workgroup b handles tiles b, b + gridDim.x, ...  On the direct-to-LDS path the
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void conv_tap_kernel(ConvTapArgs<T>
     if constexpr (DIRECT) {
         int t = blockIdx.x;
         tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
-        int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+        int m0 = a.m_begin + tm * ML::TILE_M, n0 = tn * ML::TILE_N;
         ConvDirectLoaderK<ML::TILE_M, ML::THREADS> la(g, m0);
         DirectLoader<true, ML::TILE_N, ML::THREADS, true> lb(a.Wm, n0, g.zero);
         ML::pipeline_fill(la, lb, a.K, lds);
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void conv_tap_kernel(ConvTapArgs<T>
             int m0n = 0, n0n = 0;
             if (tnext < total) {
                 tile_coords(tnext, a.tiles_m, a.tiles_n, tm, tn);
-                m0n = tm * ML::TILE_M;
+                m0n = a.m_begin + tm * ML::TILE_M;
                 n0n = tn * ML::TILE_N;
                 la.move_to(m0n);
                 lb.move_to(a.Wm, n0n);
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void conv_tap_kernel(ConvTapArgs<T>
     } else {
         for (int t = blockIdx.x; t < total; t += gridDim.x) {
             tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
-            const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+            const int m0 = a.m_begin + tm * ML::TILE_M, n0 = tn * ML::TILE_N;
             ConvTapLoaderK<T, ML::TILE_M, ML::THREADS> la(g, m0);
             typename ML::PlainLoaderB lb(a.Wm, n0, a.K);
             ML::run(la, lb, a.K, lds, acc);
@@ -425,18 +426,30 @@ __global__ __launch_bounds__(NWM * NWN * 64) void conv_tap_kernel(ConvTapArgs<T>
     }
 }
 
+// Workgroups of conv_tap_kernel<...> that the device holds at once (0 on error); also raises the
+// kernel's dynamic LDS limit on first use.
+template <typename T, int WM, int WN, int NWN, int NST, int NWM = 2>
+int conv_tap_resident() {
+    using ML = GemmMainloop<T, WM, WN, true, true, sizeof(T) == 2, NWN, NST, NWM>;
+    static int resident = 0;
+    if (resident == 0) {
+        auto kernel = conv_tap_kernel<T, WM, WN, NWN, NST, NWM>;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)ML::LDS_BYTES) != hipSuccess)
+            return 0;
+        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
+    }
+    return resident;
+}
+
 template <typename T, int WM, int WN, int NWN, int NST, int NWM = 2>
 int launch_conv_tap(hipStream_t s, ConvTapArgs<T>& a) {
     using ML = GemmMainloop<T, WM, WN, true, true, sizeof(T) == 2, NWN, NST, NWM>;
-    a.tiles_m = (int)ceil_div(a.tap.M, ML::TILE_M);
+    a.tiles_m = (int)ceil_div(a.tap.M - a.m_begin, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.Ncols, ML::TILE_N);
     auto kernel = conv_tap_kernel<T, WM, WN, NWN, NST, NWM>;
-    static int resident = 0;   // workgroups that fit the device at once
-    if (resident == 0) {
-        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)ML::LDS_BYTES));
-        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
-    }
+    const int resident = conv_tap_resident<T, WM, WN, NWN, NST, NWM>();
+    LUX_UNSUPPORTED_IF(resident <= 0, "conv: the kernel does not fit the device");
     const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
     ProfScope ps(a.tap.dgrad ? (sizeof(T) == 2 ? "conv_dgrad_kernel<bf16>" : "conv_dgrad_kernel<f32>")
                              : (sizeof(T) == 2 ? "conv_fprop_kernel<bf16>" : "conv_fprop_kernel<f32>"), s);

@@ -136,7 +136,7 @@ def test_config5_full_size(gpu, dtype):
     y, back = gpu.pullback(gpu.fused_conv_bias_activation, "relu", dw_, dx_, db_, gd)
     gw, gx, gb = back(dd_)
     yh = y.to_numpy()
-    sub = [3, 60]
+    sub = [3, 63]          # the last image lies in the rows that the fp32 kernels give to a second launch
     od2 = O.ConvDims(xs[:3] + (2,), ws, padding=1)
     wy = O.fused_conv_bias_activation("relu", f64(w), f64(x[..., sub]), f64(b), od2)
     assert_close(yh[..., sub], wy, dtype, "config5 y")
