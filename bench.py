@@ -409,10 +409,19 @@ def main():
     prof = kernel_profile(lux, wl.step, min(args.steps, 100))
     kw = wl.kernel_work()
     kernels = []
+    # "<name>+tail" is a second launch that finishes the rows of <name>: one kernel's work, so its
+    # time is added to <name>'s
+    tails = {k["kernel"][:-5]: k for k in prof if k["kernel"].endswith("+tail")}
+    prof = [dict(k) for k in prof if not k["kernel"].endswith("+tail")]
     for k in prof:
+        if k["kernel"] in tails:
+            k["total_ms"] += tails[k["kernel"]]["total_ms"]
+            k["tail_launches"] = tails[k["kernel"]]["count"]
         avg_ms = k["total_ms"] / max(k["count"], 1)
         w = kw.get(k["kernel"])
         ent = {"kernel": k["kernel"], "avg_us": round(avg_ms * 1e3, 3), "launches": k["count"]}
+        if "tail_launches" in k:
+            ent["tail_launches"] = k["tail_launches"]
         if w:
             ach = w / (avg_ms * 1e-3) / (1e9 if wl.bound == "hbm" else 1e12)
             ent.update({"algorithmic": w, "achieved": round(ach, 1), "frac": round(ach / peak, 4)})

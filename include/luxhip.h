@@ -168,6 +168,18 @@ int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64
                          const float* save_mean, const float* save_invstd, void* dx, void* dgamma,
                          void* dbeta);
 
+/* instancenorm = the groupnorm kernels with G = C (statistics per channel and sample,
+ * src/impl/normalization.jl:191-208) plus, in training with running statistics, this update
+ * (update_normalization_statistics, src/impl/normalization.jl:91-110, reduce dims 1..N-2):
+ *   rmean_out[c] = (1-m) rmean[c] + m mean_n(mu[c,n]),
+ *   rvar_out[c]  = (1-m) rvar[c]  + m I/(I-1) mean_n(var[c,n]),   var = 1/invstd^2 - eps.
+ * save_mean, save_invstd: (C, N) fp32 as written by luxhip_groupnorm_fwd with G = C and the same
+ * eps; rmean, rvar, rmean_out, rvar_out: length C in the storage dtype. */
+int luxhip_instancenorm_running_stats(luxhip_stream_t s, int dtype, int64_t I, int64_t C, int64_t N,
+                                      const float* save_mean, const float* save_invstd, double eps,
+                                      double momentum, const void* rmean, const void* rvar, void* rmean_out,
+                                      void* rvar_out);
+
 /* ---------------------------------------------------------------- layernorm ----------
  * x, y, delta, dx: (L, R): statistics over the L leading (contiguous) elements of each of
  * the R columns.  gamma, beta, dgamma, dbeta: length L (elementwise affine over the

@@ -19,7 +19,8 @@ from ._lib import LuxHipError, Unsupported
 from .array import DeviceArray, StatArray, current_stream, set_stream
 from .luxlib import (ArgumentError, DenseConvDims, DimensionMismatch, DEFAULT_DIMS, batchnorm, bias_activation,
                      bias_activation_inplace, conv, conv_data_grad, conv_filter_grad, default_epsilon,
-                     fused_conv_bias_activation, fused_dense_bias_activation, groupnorm, layernorm, matmul, pullback,
+                     fast_activation, fast_activation_inplace, fused_conv_bias_activation, fused_dense_bias_activation,
+                     groupnorm, instancenorm, layernorm, matmul, pullback, rrule_fast_activation, rrule_instancenorm,
                      rrule_batchnorm, rrule_bias_activation, rrule_fused_conv_bias_activation,
                      rrule_fused_dense_bias_activation, rrule_groupnorm, rrule_layernorm)
 

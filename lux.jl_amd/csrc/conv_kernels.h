@@ -451,8 +451,11 @@ int launch_conv_tap(hipStream_t s, ConvTapArgs<T>& a) {
     const int resident = conv_tap_resident<T, WM, WN, NWN, NST, NWM>();
     LUX_UNSUPPORTED_IF(resident <= 0, "conv: the kernel does not fit the device");
     const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
-    ProfScope ps(a.tap.dgrad ? (sizeof(T) == 2 ? "conv_dgrad_kernel<bf16>" : "conv_dgrad_kernel<f32>")
-                             : (sizeof(T) == 2 ? "conv_fprop_kernel<bf16>" : "conv_fprop_kernel<f32>"), s);
+    // a launch that finishes the rows of another one is reported as "<name>+tail"
+    static const char* const names[2][2][2] = {
+        {{"conv_fprop_kernel<f32>", "conv_fprop_kernel<f32>+tail"}, {"conv_dgrad_kernel<f32>", "conv_dgrad_kernel<f32>+tail"}},
+        {{"conv_fprop_kernel<bf16>", "conv_fprop_kernel<bf16>+tail"}, {"conv_dgrad_kernel<bf16>", "conv_dgrad_kernel<bf16>+tail"}}};
+    ProfScope ps(names[sizeof(T) == 2][a.tap.dgrad ? 1 : 0][a.m_begin > 0], s);
     kernel<<<dim3((unsigned)grid), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;

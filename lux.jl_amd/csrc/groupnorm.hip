@@ -517,7 +517,38 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
     return LUXHIP_OK;
 }
 
+// instancenorm's running statistics: the statistics of the (channel, sample) slices averaged over
+// the batch, the variance with the n / (n - 1) correction of a slice of n = I values.
+template <typename T>
+__global__ void in_running_stats_kernel(const float* __restrict__ mean, const float* __restrict__ invstd, int C, int N,
+                                        float eps, float momentum, float corrected, const T* __restrict__ rmean,
+                                        const T* __restrict__ rvar, T* __restrict__ rmean_out, T* __restrict__ rvar_out) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float sm = 0.f, sv = 0.f;
+    for (int n = 0; n < N; ++n) {
+        const float is = invstd[c + (size_t)C * n];
+        sm += mean[c + (size_t)C * n];
+        sv += 1.f / (is * is) - eps;
+    }
+    st<T>(rmean_out + c, (1.f - momentum) * ld<T>(rmean + c) + momentum * (sm / (float)N));
+    st<T>(rvar_out + c, (1.f - momentum) * ld<T>(rvar + c) + corrected * (sv / (float)N));
+}
+
+template <typename T>
+static int in_running_stats_impl(hipStream_t s, int64_t I, int64_t C, int64_t N, const float* mean, const float* invstd,
+                                 float eps, float momentum, const T* rmean, const T* rvar, T* rmean_out, T* rvar_out) {
+    const float m = (float)I;
+    const float corrected = momentum * m / (m - 1.f);            // update_normalization_statistics
+    ProfScope ps("in_running_stats_kernel", s);
+    in_running_stats_kernel<T><<<dim3((unsigned)ceil_div(C, 256)), dim3(256), 0, s>>>(mean, invstd, (int)C, (int)N, eps, momentum,
+                                                                                      corrected, rmean, rvar, rmean_out, rvar_out);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
 }  // namespace luxhip
+
 
 using namespace luxhip;
 
@@ -554,6 +585,25 @@ int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64
                                   (const float*)beta, save_mean, save_invstd, (float*)dx, (float*)dgamma, (float*)dbeta);
     return gn_bwd_impl<bf16_t>((hipStream_t)s, act, I, C, G, N, (const bf16_t*)delta, (const bf16_t*)x, (const bf16_t*)gamma,
                                (const bf16_t*)beta, save_mean, save_invstd, (bf16_t*)dx, (bf16_t*)dgamma, (bf16_t*)dbeta);
+}
+
+int luxhip_instancenorm_running_stats(luxhip_stream_t s, int dtype, int64_t I, int64_t C, int64_t N, const float* save_mean,
+                                      const float* save_invstd, double eps, double momentum, const void* rmean,
+                                      const void* rvar, void* rmean_out, void* rvar_out) {
+    LUX_REQUIRE_INIT();
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_INVALID_IF(I < 0 || C < 0 || N < 0, "invalid dimension");
+    if (C == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(I * N == 0, "instancenorm_running_stats: statistics of empty slices");
+    LUX_UNSUPPORTED_IF(C * N >= 2147483648LL, "instancenorm_running_stats: too many slices");
+    LUX_INVALID_IF(save_mean == nullptr || save_invstd == nullptr || rmean == nullptr || rvar == nullptr ||
+                       rmean_out == nullptr || rvar_out == nullptr,
+                   "instancenorm_running_stats: no argument may be NULL");
+    if (dtype == LUXHIP_F32)
+        return in_running_stats_impl<float>((hipStream_t)s, I, C, N, save_mean, save_invstd, (float)eps, (float)momentum,
+                                            (const float*)rmean, (const float*)rvar, (float*)rmean_out, (float*)rvar_out);
+    return in_running_stats_impl<bf16_t>((hipStream_t)s, I, C, N, save_mean, save_invstd, (float)eps, (float)momentum,
+                                         (const bf16_t*)rmean, (const bf16_t*)rvar, (bf16_t*)rmean_out, (bf16_t*)rvar_out);
 }
 
 }  // extern "C"

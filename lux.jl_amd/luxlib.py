@@ -120,6 +120,37 @@ def rrule_bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray])
     return y, back
 
 
+# ------------------------------------------------------------------------------- fast_activation
+def fast_activation(act: str, x: DeviceArray) -> DeviceArray:
+    """`fast_activation(σ, x)` (api/activation.jl:55-57): σ.(x) into a new array."""
+    aid = _act_id(act)
+    y = DeviceArray(x.shape, x.dtype)
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, aid, 1, 1, x.size, x.ptr, None, y.ptr, None)
+    return y
+
+
+def fast_activation_inplace(act: str, x: DeviceArray) -> DeviceArray:
+    """`fast_activation!!(σ, x)` (api/activation.jl:27-29): overwrites and returns x."""
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, _act_id(act), 1, 1, x.size, x.ptr, None, x.ptr, None)
+    return x
+
+
+def rrule_fast_activation(act: str, x: DeviceArray):
+    """CRC.rrule(activation!!) (impl/activation.jl:20-49): (y, Δ -> (∂x,)); ∂x = Δ·dσ(y, x)
+    (∇activation, impl/activation.jl:135-154).  x itself is the saved pre-activation."""
+    aid = _act_id(act)
+    y = DeviceArray(x.shape, x.dtype)
+    _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, aid, 1, 1, x.size, x.ptr, None, y.ptr, None)
+
+    def back(delta: DeviceArray):
+        dx = DeviceArray(x.shape, x.dtype)
+        _lib.call("luxhip_bias_activation_bwd", current_stream(), x.code, aid, 1, 1, x.size, delta.ptr, y.ptr,
+                  x.ptr if aid in _NEEDS_PRE else None, dx.ptr, None)
+        return (dx,)
+
+    return y, back
+
+
 # ------------------------------------------------------------------------------- dense
 def _check_dense(weight, x, b):
     if weight.ndim != 2 or x.ndim != 2:
@@ -280,6 +311,67 @@ def rrule_groupnorm(x, scale, bias, groups, act="identity", epsilon=None):
         return dx, dg, db
 
     return y, back
+
+
+# ------------------------------------------------------------------------------- instancenorm
+def _instancenorm_fwd(x, scale, bias, rmean, rvar, training, act, momentum, epsilon, save):
+    if x.ndim <= 2:
+        raise AssertionError(f"`ndims(x) = {x.ndim}` must be at least > 2.")      # api/instancenorm.jl:75-78
+    dt = _same_dtype(x, scale, bias, rmean, rvar)
+    I, Cc, N = _icn(x)
+    for v in (scale, bias, rmean, rvar):
+        if v is not None and (v.ndim != 1 or v.shape[0] != Cc):
+            raise ArgumentError("Invalid Dimensions!")      # get_norm_reshape_dims, impl/normalization.jl:178-185
+    if (scale is None) != (bias is None) or (rmean is None) != (rvar is None):
+        raise ArgumentError("scale/bias and running_mean/running_var must be given in pairs")
+    if epsilon is None:
+        epsilon = default_epsilon(dt)
+    if not training and rmean is not None:
+        # the running statistics stand in for every sample's statistics: the inference batchnorm
+        # kernels compute exactly that (impl/normalization.jl:122-127)
+        y, stats, saved = _batchnorm_fwd(x, scale, bias, rmean, rvar, False, act, 0.0, epsilon, save)
+        return y, stats, ("running",) + tuple(saved)
+    upd = training and rmean is not None
+    y, (sm, si) = _groupnorm_fwd(x, scale, bias, Cc, act, epsilon, save or upd)
+    stats = {"running_mean": rmean, "running_var": rvar}
+    if upd:
+        rm_out, rv_out = DeviceArray((Cc,), dt), DeviceArray((Cc,), dt)
+        _lib.call("luxhip_instancenorm_running_stats", current_stream(), x.code, I, Cc, N, sm.ptr, si.ptr, float(epsilon),
+                  float(momentum), rmean.ptr, rvar.ptr, rm_out.ptr, rv_out.ptr)
+        stats = {"running_mean": rm_out, "running_var": rv_out}
+    return y, stats, ("sample", sm, si, float(epsilon))
+
+
+def instancenorm(x: DeviceArray, scale, bias, running_mean, running_var, training, act: str = "identity",
+                 momentum: float = 0.1, epsilon: Optional[float] = None):
+    """`instancenorm(x, scale, bias, running_mean, running_var, training, σ, momentum, epsilon)`
+    (api/instancenorm.jl:45-73): statistics per channel and sample over the leading dims; returns
+    `(y, {"running_mean": .., "running_var": ..})`.  The legacy form without running statistics
+    (:33-43) is `instancenorm(x, scale, bias, None, None, training, σ)`."""
+    y, stats, _ = _instancenorm_fwd(x, scale, bias, running_mean, running_var, bool(training), act, momentum, epsilon, False)
+    return y, stats
+
+
+def rrule_instancenorm(x, scale, bias, running_mean, running_var, training, act="identity", momentum=0.1, epsilon=None):
+    """((y, stats), Δ -> (∂x, ∂γ, ∂β)): the pullback of the generic `normalization`
+    (impl/normalization.jl:143-165) with reduce dims 1..N-2; running statistics are constants."""
+    y, stats, saved = _instancenorm_fwd(x, scale, bias, running_mean, running_var, bool(training), act, momentum, epsilon, True)
+    I, Cc, N = _icn(x)
+    aid = _act_id(act)
+
+    def back(delta: DeviceArray):
+        dx = DeviceArray(x.shape, x.dtype)
+        dg = None if scale is None else DeviceArray((Cc,), x.dtype)
+        db = None if bias is None else DeviceArray((Cc,), x.dtype)
+        if saved[0] == "running":
+            _lib.call("luxhip_batchnorm_bwd", current_stream(), x.code, aid, I, Cc, N, delta.ptr, x.ptr, _p(scale), _p(bias),
+                      saved[1].ptr, saved[2].ptr, 0, dx.ptr, _p(dg), _p(db))
+        else:
+            _lib.call("luxhip_groupnorm_bwd", current_stream(), x.code, aid, I, Cc, Cc, N, delta.ptr, x.ptr, _p(scale),
+                      _p(bias), saved[1].ptr, saved[2].ptr, dx.ptr, _p(dg), _p(db))
+        return dx, dg, db
+
+    return (y, stats), back
 
 
 # ------------------------------------------------------------------------------- layernorm
@@ -468,6 +560,8 @@ _RRULES = {
     fused_dense_bias_activation: rrule_fused_dense_bias_activation,
     batchnorm: rrule_batchnorm,
     groupnorm: rrule_groupnorm,
+    instancenorm: rrule_instancenorm,
+    fast_activation: rrule_fast_activation,
     layernorm: rrule_layernorm,
     fused_conv_bias_activation: rrule_fused_conv_bias_activation,
 }

@@ -22,6 +22,8 @@ tests/test_oracle_*.py):
                                         torch F.batch_norm autograd, finite differences
   * groupnorm (+bwd) .................. torch F.group_norm autograd, finite differences
   * layernorm (+bwd) .................. mean~0/std~1 invariant, torch F.layer_norm autograd
+  * instancenorm (+running stats, bwd)  torch F.instance_norm (values, running statistics,
+                                        autograd), groupnorm with G = C, finite differences
   * conv / dgrad / wgrad .............. reference known answers (impulse response,
                                         asymmetric-pad counts), brute-force 7-loop direct
                                         convolution, torch conv2d with flipped kernel
@@ -428,6 +430,71 @@ def groupnorm_pullback(x, gamma, beta, groups: int, act: str, eps, delta):
     dvar = -(dxt * xmu).sum(axis=axes, keepdims=True) * T(0.5) * idenom * idenom
     dxv = dxt + mean_var_pullback(xv, mu, axes, dmu, dvar)
     dx = np.swapaxes(dxv, -3, -2).reshape(x.shape)
+    return dx, (None if gamma is None else dgamma), (None if beta is None else dbeta)
+
+
+# --------------------------------------------------------------------------------------
+# instancenorm  (api/instancenorm.jl:33-80, impl/normalization.jl:143-208: the generic
+# `normalization` with reduce dims 1..N-2)
+# --------------------------------------------------------------------------------------
+def instancenorm(x, gamma, beta, rmean, rvar, training: bool, act: str = "identity", momentum=0.1, eps=None):
+    """Returns (y, running_mean', running_var').  Statistics per (channel, sample) over the
+    leading dims (biased variance); with running statistics in training mode the per-sample
+    statistics are averaged over the batch first (impl/normalization.jl:104-107) and the
+    variance is corrected by m/(m-1), m = number of reduced elements (:108-109).  Inference
+    with running statistics uses them for every sample (:122-127)."""
+    x = np.asarray(x)
+    assert x.ndim > 2, "`ndims(x)` must be at least > 2."       # api/instancenorm.jl:75-78
+    T = x.dtype.type
+    if eps is None:
+        eps = default_epsilon(x.dtype)
+    C = x.shape[-2]
+    axes = tuple(range(x.ndim - 2))
+    cs = _chan_shape(x, C)
+    rmean_new, rvar_new = rmean, rvar
+    if training or rmean is None:
+        mu, var = mean_var(x, axes, corrected=False)
+        if training and rmean is not None:
+            m = T(np.prod([x.shape[a] for a in axes]))
+            mom = T(momentum)
+            rmean_new = (T(1) - mom) * np.asarray(rmean) + mom * mu.mean(axis=-1).reshape(C)
+            rvar_new = (T(1) - mom) * np.asarray(rvar) + (mom * m / (m - T(1))) * var.mean(axis=-1).reshape(C)
+    else:
+        mu, var = np.asarray(rmean).reshape(cs), np.asarray(rvar).reshape(cs)
+    y = _affine_normalize(act, x, mu, var, gamma, beta, T(eps), cs)
+    return y, rmean_new, rvar_new
+
+
+def instancenorm_pullback(x, gamma, beta, act: str, eps, delta, *, training=True, rmean=None, rvar=None):
+    """(∂x, ∂γ, ∂β) of instancenorm: AD of the generic `normalization` (affine_normalize,
+    impl/normalization.jl:3-17, and the mean_var rrule, impl/common_ops.jl:45-61, with
+    n = the number of reduced elements); running statistics are constants."""
+    x = np.asarray(x)
+    T = x.dtype.type
+    C = x.shape[-2]
+    axes = tuple(range(x.ndim - 2))
+    par_axes = axes + (x.ndim - 1,)
+    cs = _chan_shape(x, C)
+    from_x = training or rmean is None
+    if from_x:
+        mu, var = mean_var(x, axes)
+    else:
+        mu, var = np.asarray(rmean).reshape(cs), np.asarray(rvar).reshape(cs)
+    eps = T(eps)
+    idenom = T(1) / np.sqrt(var + eps)
+    g = np.ones(cs, x.dtype) if gamma is None else np.asarray(gamma).reshape(cs)
+    b = np.zeros(cs, x.dtype) if beta is None else np.asarray(beta).reshape(cs)
+    gp = g * idenom
+    pre = x * gp + (b - mu * gp)
+    dy = grad_activation(delta, act_value(act, pre), act, pre)
+    xmu = x - mu
+    dbeta = dy.sum(axis=par_axes)
+    dgamma = (dy * xmu * idenom).sum(axis=par_axes)
+    dx = dy * gp
+    if from_x:
+        dmu = -dx.sum(axis=axes, keepdims=True)
+        dvar = -(dx * xmu).sum(axis=axes, keepdims=True) * T(0.5) * idenom * idenom
+        dx = dx + mean_var_pullback(x, mu, axes, dmu, dvar)
     return dx, (None if gamma is None else dgamma), (None if beta is None else dbeta)
 
 

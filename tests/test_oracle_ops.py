@@ -215,6 +215,71 @@ def test_groupnorm_equals_instance_stats_when_groups_eq_channels():
     np.testing.assert_allclose(y.std(axis=0), 1, rtol=1e-12)
 
 
+# ----------------------------------------------------------------------------- instancenorm
+@pytest.mark.parametrize("shape", [(4, 4, 6, 2), (7, 3, 4), (3, 2, 2, 5, 3)])
+@pytest.mark.parametrize("act", ["identity", "relu", "swish"])
+@pytest.mark.parametrize("affine", [True, False])
+def test_instancenorm_vs_torch(shape, act, affine):
+    # shapes of lib/LuxLib/test/normalization/instancenorm_tests.jl; torch.nn.functional.instance_norm
+    # is the library routine (values, running statistics averaged over the batch, autograd)
+    from tests.test_oracle_activations import TORCH
+    x = RNG.normal(size=shape) * 1.5 + 0.3
+    C = shape[-2]
+    g = RNG.uniform(0.5, 1.5, C) if affine else None
+    b = RNG.normal(size=C) if affine else None
+    rm, rv = RNG.normal(size=C), RNG.uniform(0.5, 2, C)
+    delta = RNG.normal(size=shape)
+    eps = 1e-5
+    perm = (len(shape) - 1, len(shape) - 2) + tuple(range(len(shape) - 2))
+    inv = np.argsort(perm)
+    tx = torch.tensor(np.transpose(x, perm).copy(), requires_grad=True)
+    tg = torch.tensor(g, requires_grad=True) if affine else None
+    tb = torch.tensor(b, requires_grad=True) if affine else None
+    trm, trv = torch.tensor(rm), torch.tensor(rv)
+    ty = TORCH[act](F.instance_norm(tx, trm, trv, tg, tb, True, 0.1, eps))
+    ty.backward(torch.tensor(np.transpose(delta, perm).copy()))
+    y, rm_n, rv_n = O.instancenorm(x, g, b, rm, rv, True, act, 0.1, eps)
+    dx, dg, db = O.instancenorm_pullback(x, g, b, act, eps, delta)
+    np.testing.assert_allclose(y, np.transpose(ty.detach().numpy(), inv), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(rm_n, trm.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(rv_n, trv.numpy(), rtol=1e-12)
+    np.testing.assert_allclose(dx, np.transpose(tx.grad.numpy(), inv), rtol=1e-8, atol=1e-10)
+    if affine:
+        np.testing.assert_allclose(dg, tg.grad.numpy(), rtol=1e-9, atol=1e-11)
+        np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-9, atol=1e-11)
+    # the same statistics as groupnorm with one channel per group
+    np.testing.assert_allclose(y, O.groupnorm(x, g, b, C, act, eps), rtol=1e-12, atol=1e-13)
+    gdx, gdg, gdb = O.groupnorm_pullback(x, g, b, C, act, eps, delta)
+    np.testing.assert_allclose(dx, gdx, rtol=1e-10, atol=1e-12)
+    # without running statistics nothing is updated; in inference they replace the sample statistics
+    y0, r0, v0 = O.instancenorm(x, g, b, None, None, True, act, 0.1, eps)
+    assert r0 is None and v0 is None
+    np.testing.assert_array_equal(y0, y)
+    yi, ri, vi = O.instancenorm(x, g, b, rm, rv, False, act, 0.1, eps)
+    assert ri is rm and vi is rv
+    tyi = TORCH[act](F.instance_norm(tx.detach(), torch.tensor(rm), torch.tensor(rv), None if not affine else tg.detach(),
+                                     None if not affine else tb.detach(), False, 0.1, eps))
+    np.testing.assert_allclose(yi, np.transpose(tyi.numpy(), inv), rtol=1e-10, atol=1e-11)
+
+
+def test_instancenorm_inference_pullback_finite_differences():
+    x = RNG.normal(size=(3, 4, 2))
+    g, b = RNG.uniform(0.5, 1.5, 4), RNG.normal(size=4)
+    rm, rv = RNG.normal(size=4), RNG.uniform(0.5, 2, 4)
+    delta = RNG.normal(size=x.shape)
+    for training, stats in ((False, (rm, rv)), (False, (None, None)), (True, (rm, rv))):
+        loss = lambda xx: float((O.instancenorm(xx, g, b, stats[0], stats[1], training, "swish", 0.1, 1e-5)[0] * delta).sum())
+        dx, dg, db = O.instancenorm_pullback(x, g, b, "swish", 1e-5, delta, training=training, rmean=stats[0], rvar=stats[1])
+        np.testing.assert_allclose(dx, fd_grad(loss, x), rtol=1e-5, atol=1e-7)
+        lg = lambda gg: float((O.instancenorm(x, gg, b, stats[0], stats[1], training, "swish", 0.1, 1e-5)[0] * delta).sum())
+        np.testing.assert_allclose(dg, fd_grad(lg, g), rtol=1e-5, atol=1e-7)
+
+
+def test_instancenorm_needs_three_dims():
+    with pytest.raises(AssertionError):
+        O.instancenorm(np.ones((4, 3)), None, None, None, None, True)
+
+
 # ----------------------------------------------------------------------------- layernorm
 def test_layernorm_invariants():
     # lib/LuxLib/test/normalization/layernorm_tests.jl:54-57: mean ~ 0, std ~ 1 without affine
