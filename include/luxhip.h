@@ -180,6 +180,39 @@ int luxhip_instancenorm_running_stats(luxhip_stream_t s, int dtype, int64_t I, i
                                       double momentum, const void* rmean, const void* rvar, void* rmean_out,
                                       void* rvar_out);
 
+/* ---------------------------------------------------------------- dropout ----------
+ * The reference draws its noise with `rand!(rng, y)` from the array package's generator
+ * (src/impl/dropout.jl:171-190); here a counter-based Philox4x32-10 stream stands in for it:
+ * element e takes lane e % 4 of the block with counter offset + e / 4 under the 64-bit key `seed`.
+ * A caller advances `offset` by ceil(n / 4) per call (the analogue of the replicated rng that the
+ * reference returns).  Uniform values in [0, 1): (u >> 8) 2^-24 (fp32), (u >> 24) 2^-8 (bf16). */
+
+/* rand!(rng, out) (src/impl/dropout.jl:173-176, 186-187). */
+int luxhip_rand_uniform(luxhip_stream_t s, int dtype, int64_t n, uint64_t seed, uint64_t offset, void* out);
+
+/* dropout with a full-size mask in one pass (src/impl/dropout.jl:3-6): mask = (noise > T(p)) T(invp)
+ * (generate_dropout_mask!, :200-218), y = x .* mask (dropout_dot_mul, :220); the noise is never
+ * stored.  x == y == NULL: only the mask (generate_dropout_mask, :179-190, for masks that are
+ * broadcast over x).  mask == NULL: only y. */
+int luxhip_dropout_fwd(luxhip_stream_t s, int dtype, int64_t n, uint64_t seed, uint64_t offset, double p,
+                       double invp, const void* x, void* y, void* mask);
+
+/* Impl.generate_dropout_mask!(y, opmode, p, invp) (src/impl/dropout.jl:200-218) on stored noise,
+ * in place: y = (y > T(p)) T(invp). */
+int luxhip_dropout_mask(luxhip_stream_t s, int dtype, int64_t n, double p, double invp, void* noise_to_mask);
+
+/* dropout_dot_mul(x, mask) = x .* mask (src/impl/dropout.jl:220) and its pullback dx = delta .* mask
+ * (:222-228).  mask_shape[d] is x_shape[d] or 1 (dropout_shape, :74-78); both column-major. */
+int luxhip_dropout_mul(luxhip_stream_t s, int dtype, int ndim, const int64_t* x_shape, const int64_t* mask_shape,
+                       const void* x, const void* mask, void* y);
+
+/* alpha_dropout(opmode, noise, p, x, alpha, A, B) (src/impl/dropout.jl:84-89):
+ * y = muladd(ifelse(noise > p, x, T(alpha)), T(A), T(B)); pullback (:137-150): dx = delta (noise > p) A. */
+int luxhip_alpha_dropout_fwd(luxhip_stream_t s, int dtype, int64_t n, const void* noise, double p, const void* x,
+                             double alpha, double A, double B, void* y);
+int luxhip_alpha_dropout_bwd(luxhip_stream_t s, int dtype, int64_t n, const void* noise, double p,
+                             const void* delta, double A, void* dx);
+
 /* ---------------------------------------------------------------- layernorm ----------
  * x, y, delta, dx: (L, R): statistics over the L leading (contiguous) elements of each of
  * the R columns.  gamma, beta, dgamma, dbeta: length L (elementwise affine over the

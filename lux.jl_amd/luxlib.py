@@ -13,6 +13,7 @@ Julia's column-major layout and logical shapes (W, H, C, N) / (features, batch).
 from __future__ import annotations
 
 import ctypes as C
+import math
 from dataclasses import dataclass, field
 from typing import Optional, Sequence, Tuple
 
@@ -149,6 +150,121 @@ def rrule_fast_activation(act: str, x: DeviceArray):
         return (dx,)
 
     return y, back
+
+
+# ------------------------------------------------------------------------------- dropout
+@dataclass(frozen=True)
+class PhiloxRNG:
+    """The generator state handed to dropout in place of Julia's `rng`: a counter-based Philox4x32-10
+    stream (seed = key, offset = first counter block).  Like `LuxCore.replicate(rng)` followed by
+    `rand!`, drawing n values returns a new state and leaves this one untouched."""
+    seed: int = 0
+    offset: int = 0
+
+    def advanced(self, n: int) -> "PhiloxRNG":
+        return PhiloxRNG(self.seed, self.offset + (n + 3) // 4)
+
+
+def dropout_shape(x_shape, dims):
+    """`dropout_shape(x, dims)` (impl/dropout.jl:74-78): dims is None (Julia's `:`) or the 1-based
+    dims along which the mask varies."""
+    if dims is None:
+        return tuple(x_shape)
+    return tuple(s if (i + 1) in dims else 1 for i, s in enumerate(x_shape))
+
+
+def rand_uniform(rng: PhiloxRNG, shape, dtype="f32"):
+    """`rand!(rng, similar(x, shape))`: (noise, advanced rng)."""
+    out = DeviceArray(tuple(shape), dtype)
+    _lib.call("luxhip_rand_uniform", current_stream(), out.code, out.size, rng.seed, rng.offset, out.ptr)
+    return out, rng.advanced(out.size)
+
+
+def _shape_arg(shape):
+    return (C.c_int64 * max(len(shape), 1))(*shape)
+
+
+def dropout_dot_mul(x: DeviceArray, mask: DeviceArray) -> DeviceArray:
+    """`dropout_dot_mul(x, mask)` = x .* mask (impl/dropout.jl:220), mask broadcast over its
+    singleton dims."""
+    if mask.ndim != x.ndim or any(m not in (1, sx) for m, sx in zip(mask.shape, x.shape)):
+        raise AssertionError("`mask` is not of the same size as `LuxLib.dropout_shape(x, dims)`.")   # impl/dropout.jl:49-52
+    _same_dtype(x, mask)
+    y = DeviceArray(x.shape, x.dtype)
+    _lib.call("luxhip_dropout_mul", current_stream(), x.code, x.ndim, _shape_arg(x.shape), _shape_arg(mask.shape),
+              x.ptr, mask.ptr, y.ptr)
+    return y
+
+
+def _dropout_fwd(rng, x, p, training, invp, dims, mask, update_mask):
+    if mask is not None and not update_mask:
+        if not training:
+            return x, mask, rng                                   # impl/dropout.jl:36-47
+        if tuple(mask.shape) != dropout_shape(x.shape, dims):
+            raise AssertionError("`mask` is not of the same size as `LuxLib.dropout_shape(x, dims)`.")
+        return dropout_dot_mul(x, mask), mask, rng                # impl/dropout.jl:22-34
+    if not training:
+        return x, (x if mask is None else mask), rng              # impl/dropout.jl:8
+    mshape = dropout_shape(x.shape, dims)
+    new_mask = DeviceArray(mshape, x.dtype)
+    if mshape == tuple(x.shape):
+        y = DeviceArray(x.shape, x.dtype)
+        _lib.call("luxhip_dropout_fwd", current_stream(), x.code, x.size, rng.seed, rng.offset, float(p), float(invp),
+                  x.ptr, y.ptr, new_mask.ptr)
+    else:
+        _lib.call("luxhip_dropout_fwd", current_stream(), x.code, new_mask.size, rng.seed, rng.offset, float(p), float(invp),
+                  None, None, new_mask.ptr)
+        y = dropout_dot_mul(x, new_mask)
+    return y, new_mask, rng.advanced(new_mask.size)
+
+
+def dropout(rng: PhiloxRNG, x: DeviceArray, p, training, invp, dims=None, *, mask=None, update_mask=True):
+    """`dropout(rng, x, p, training, invp, dims)` and, with `mask=`/`update_mask=`,
+    `dropout(rng, x, mask, p, training, update_mask, invp, dims)` (api/dropout.jl:40-69):
+    returns `(y, mask, rng′)`.  dims=None is Julia's `:`."""
+    return _dropout_fwd(rng, x, p, bool(training), invp, dims, mask, bool(update_mask))
+
+
+def rrule_dropout(rng, x, p, training, invp, dims=None, *, mask=None, update_mask=True):
+    """((y, mask, rng′), Δ -> (∂x,)): only dropout_dot_mul is differentiable
+    (impl/dropout.jl:222-228): ∂x = Δ .* mask; not training: ∂x = Δ."""
+    training = bool(training)
+    y, m, rng2 = _dropout_fwd(rng, x, p, training, invp, dims, mask, bool(update_mask))
+
+    def back(delta: DeviceArray):
+        return (dropout_dot_mul(delta, m) if training else delta,)
+
+    return (y, m, rng2), back
+
+
+def _alpha_coefficients(p, alpha, A, B):
+    if alpha is None:                                             # impl/dropout.jl:57-62
+        alpha = -1.7580993408473766
+        A = 1.0 / math.sqrt((1 - p) * (1 + p * alpha ** 2))
+        B = -A * alpha * p
+    return float(alpha), float(A), float(B)
+
+
+def alpha_dropout(rng: PhiloxRNG, x: DeviceArray, p, training, alpha=None, A=None, B=None):
+    """`alpha_dropout(rng, x, p, training[, α, A, B])` (api/dropout.jl:107-115): `(y, rng′)`."""
+    return rrule_alpha_dropout(rng, x, p, training, alpha, A, B)[0]
+
+
+def rrule_alpha_dropout(rng, x, p, training, alpha=None, A=None, B=None):
+    """((y, rng′), Δ -> (∂x,)); ∂x = Δ · (noise > p) · A (impl/dropout.jl:137-150)."""
+    if not bool(training):
+        return (x, rng), (lambda delta: (delta,))                 # impl/dropout.jl:71
+    alpha, A, B = _alpha_coefficients(float(p), alpha, A, B)
+    noise, rng2 = rand_uniform(rng, x.shape, x.dtype)             # generate_alpha_dropout_noise, impl/dropout.jl:171-177
+    y = DeviceArray(x.shape, x.dtype)
+    _lib.call("luxhip_alpha_dropout_fwd", current_stream(), x.code, x.size, noise.ptr, float(p), x.ptr, alpha, A, B, y.ptr)
+
+    def back(delta: DeviceArray):
+        dx = DeviceArray(x.shape, x.dtype)
+        _lib.call("luxhip_alpha_dropout_bwd", current_stream(), x.code, x.size, noise.ptr, float(p), delta.ptr, A, dx.ptr)
+        return (dx,)
+
+    return (y, rng2), back
 
 
 # ------------------------------------------------------------------------------- dense
@@ -451,57 +567,60 @@ def rrule_layernorm(x, scale, bias, act="identity", dims=DEFAULT_DIMS, epsilon=N
 # ------------------------------------------------------------------------------- conv
 @dataclass
 class DenseConvDims:
-    """The fields of NNlib.DenseConvDims this path consumes (2 spatial dims).
-    padding = (w_lo, w_hi, h_lo, h_hi); flipkernel=False is true convolution."""
-    x_shape: Tuple[int, int, int, int]
-    w_shape: Tuple[int, int, int, int]
-    stride: Tuple[int, int] = (1, 1)
-    padding: Tuple[int, int, int, int] = (0, 0, 0, 0)
-    dilation: Tuple[int, int] = (1, 1)
+    """The fields of NNlib.DenseConvDims this path consumes (1 or 2 spatial dims: x (W, C, N) or
+    (W, H, C, N)).  padding = (w_lo, w_hi[, h_lo, h_hi]); flipkernel=False is true convolution."""
+    x_shape: Tuple[int, ...]
+    w_shape: Tuple[int, ...]
+    stride: Tuple[int, ...] = 1
+    padding: Tuple[int, ...] = 0
+    dilation: Tuple[int, ...] = 1
     groups: int = 1
     flipkernel: bool = False
     _c: Optional[_lib.ConvDimsStruct] = field(default=None, repr=False, compare=False)
 
     def __post_init__(self):
-        if isinstance(self.stride, int):
-            self.stride = (self.stride,) * 2
-        if isinstance(self.dilation, int):
-            self.dilation = (self.dilation,) * 2
-        if isinstance(self.padding, int):
-            self.padding = (self.padding,) * 4
-        elif len(self.padding) == 2:
-            self.padding = (self.padding[0], self.padding[0], self.padding[1], self.padding[1])
         self.x_shape, self.w_shape = tuple(self.x_shape), tuple(self.w_shape)
-        if len(self.x_shape) != 4 or len(self.w_shape) != 4:
-            raise _lib.Unsupported(_lib.UNSUPPORTED, "only 2 spatial dimensions are handled on the device")
-        W, H, Cin, N = self.x_shape
-        kW, kH, Cg, Cout = self.w_shape
+        if len(self.x_shape) != len(self.w_shape) or len(self.x_shape) not in (3, 4):
+            raise _lib.Unsupported(_lib.UNSUPPORTED, "only 1 or 2 spatial dimensions are handled on the device")
+        self.spatial = len(self.x_shape) - 2
+        one = self.spatial == 1           # (W, C, N): the same memory as (W, 1, C, N), a 2-d problem of height 1
+        if isinstance(self.stride, int):
+            self.stride = (self.stride,) * self.spatial
+        if isinstance(self.dilation, int):
+            self.dilation = (self.dilation,) * self.spatial
+        if isinstance(self.padding, int):
+            self.padding = (self.padding,) * (2 * self.spatial)
+        elif len(self.padding) == self.spatial:
+            self.padding = tuple(p for q in self.padding for p in (q, q))
+        self.stride, self.dilation, self.padding = tuple(self.stride), tuple(self.dilation), tuple(self.padding)
+        if len(self.stride) != self.spatial or len(self.dilation) != self.spatial or len(self.padding) != 2 * self.spatial:
+            raise DimensionMismatch("stride, dilation and padding must match the number of spatial dimensions")
+        stride, dil, pad = ((self.stride + (1,), self.dilation + (1,), self.padding + (0, 0)) if one
+                            else (self.stride, self.dilation, self.padding))
+        W, H, Cin, N = (self.x_shape[0], 1) + self.x_shape[1:] if one else self.x_shape
+        kW, kH, Cg, Cout = (self.w_shape[0], 1) + self.w_shape[1:] if one else self.w_shape
         if Cg * self.groups != Cin:
             raise DimensionMismatch(f"input channels {Cin} != weight channels {Cg} x groups {self.groups}")
         if Cout % self.groups != 0:
             raise DimensionMismatch("output channels must be divisible by groups")
-        self._c = _lib.ConvDimsStruct(W, H, Cin, N, kW, kH, Cout, self.stride[0], self.stride[1], *self.padding,
-                                      self.dilation[0], self.dilation[1], self.groups, int(self.flipkernel))
+        self._c = _lib.ConvDimsStruct(W, H, Cin, N, kW, kH, Cout, stride[0], stride[1], *pad,
+                                      dil[0], dil[1], self.groups, int(self.flipkernel))
 
     @property
     def out_spatial(self):
-        W, H = self.x_shape[:2]
-        kW, kH = self.w_shape[:2]
-        ow = (W + self.padding[0] + self.padding[1] - self.dilation[0] * (kW - 1) - 1) // self.stride[0] + 1
-        oh = (H + self.padding[2] + self.padding[3] - self.dilation[1] * (kH - 1) - 1) // self.stride[1] + 1
-        return ow, oh
+        return tuple((self.x_shape[d] + self.padding[2 * d] + self.padding[2 * d + 1]
+                      - self.dilation[d] * (self.w_shape[d] - 1) - 1) // self.stride[d] + 1 for d in range(self.spatial))
 
     @property
     def y_shape(self):
-        ow, oh = self.out_spatial
-        return (ow, oh, self.w_shape[3], self.x_shape[3])
+        return self.out_spatial + (self.w_shape[-1], self.x_shape[-1])
 
 
 def _check_conv(weight, x, b, cdims):
     if tuple(x.shape) != cdims.x_shape or tuple(weight.shape) != cdims.w_shape:
         raise DimensionMismatch(f"x {x.shape} / weight {weight.shape} do not match cdims {cdims.x_shape} / {cdims.w_shape}")
     if b is not None:
-        assert b.ndim == 1 and b.shape[0] == cdims.w_shape[3], "length(bias) must equal the number of output channels"
+        assert b.ndim == 1 and b.shape[0] == cdims.w_shape[-1], "length(bias) must equal the number of output channels"
 
 
 def fused_conv_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b, cdims: DenseConvDims) -> DeviceArray:
@@ -562,6 +681,8 @@ _RRULES = {
     groupnorm: rrule_groupnorm,
     instancenorm: rrule_instancenorm,
     fast_activation: rrule_fast_activation,
+    dropout: rrule_dropout,
+    alpha_dropout: rrule_alpha_dropout,
     layernorm: rrule_layernorm,
     fused_conv_bias_activation: rrule_fused_conv_bias_activation,
 }

@@ -22,6 +22,9 @@ tests/test_oracle_*.py):
                                         torch F.batch_norm autograd, finite differences
   * groupnorm (+bwd) .................. torch F.group_norm autograd, finite differences
   * layernorm (+bwd) .................. mean~0/std~1 invariant, torch F.layer_norm autograd
+  * dropout / alpha_dropout ........... closed forms; the Philox4x32-10 noise stream against
+                                        the Random123 known-answer vectors and uniformity
+                                        statistics (Julia's own rng streams are out of reach)
   * instancenorm (+running stats, bwd)  torch F.instance_norm (values, running statistics,
                                         autograd), groupnorm with G = C, finite differences
   * conv / dgrad / wgrad .............. reference known answers (impulse response,
@@ -499,6 +502,93 @@ def instancenorm_pullback(x, gamma, beta, act: str, eps, delta, *, training=True
 
 
 # --------------------------------------------------------------------------------------
+# dropout / alpha_dropout  (api/dropout.jl, impl/dropout.jl).  The reference draws its noise
+# with `rand!(rng, y)` from Julia's generators, whose streams cannot be reproduced without
+# Julia; the arithmetic that follows the noise is restated here, and the noise itself comes
+# from Philox4x32-10 (Salmon et al., SC'11; the Random123 library's known-answer vectors pin it).
+# --------------------------------------------------------------------------------------
+_PHILOX_M0, _PHILOX_M1 = 0xD2511F53, 0xCD9E8D57
+_PHILOX_W0, _PHILOX_W1 = 0x9E3779B9, 0xBB67AE85
+
+
+def philox4x32_10(counter, key):
+    """counter: (..., 4) uint32, key: (2,) uint32 -> (..., 4) uint32."""
+    c = [np.asarray(counter)[..., i].astype(np.uint64) for i in range(4)]
+    k0, k1 = int(key[0]), int(key[1])
+    mask = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0 = np.uint64(_PHILOX_M0) * c[0]
+        p1 = np.uint64(_PHILOX_M1) * c[2]
+        hi0, lo0, hi1, lo1 = p0 >> np.uint64(32), p0 & mask, p1 >> np.uint64(32), p1 & mask
+        c = [hi1 ^ c[1] ^ np.uint64(k0), lo1, hi0 ^ c[3] ^ np.uint64(k1), lo0]
+        k0, k1 = (k0 + _PHILOX_W0) & 0xFFFFFFFF, (k1 + _PHILOX_W1) & 0xFFFFFFFF
+    return np.stack(c, axis=-1).astype(np.uint32)
+
+
+def rand_uniform(n, seed, offset, bf16=False):
+    """The first n values of the stream (seed, offset): element e = lane e % 4 of the block with
+    counter (offset + e // 4, 0) under the key (seed mod 2^32, seed div 2^32); a word u becomes
+    (u >> 8) 2^-24, or (u >> 24) 2^-8 for bf16 storage.  float32 values in [0, 1)."""
+    nb = (n + 3) // 4
+    ctr = (np.arange(nb, dtype=np.uint64) + np.uint64(offset))
+    counter = np.zeros((nb, 4), np.uint32)
+    counter[:, 0] = (ctr & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    counter[:, 1] = (ctr >> np.uint64(32)).astype(np.uint32)
+    u = philox4x32_10(counter, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)).reshape(-1)[:n]
+    if bf16:
+        return (u >> np.uint32(24)).astype(np.float32) * np.float32(2.0 ** -8)
+    return (u >> np.uint32(8)).astype(np.float32) * np.float32(2.0 ** -24)
+
+
+def dropout_shape(x_shape, dims):
+    """impl/dropout.jl:74-78; dims: None (Julia's `:`) or 1-based dims that keep their extent."""
+    if dims is None:
+        return tuple(x_shape)
+    return tuple(s if (i + 1) in dims else 1 for i, s in enumerate(x_shape))
+
+
+def generate_dropout_mask(noise, p, invp):
+    """(noise > T(p)) * T(invp) in noise's dtype T (impl/dropout.jl:200-218)."""
+    T = noise.dtype.type
+    return (noise > T(p)).astype(noise.dtype) * T(invp)
+
+
+def dropout(noise, x, p, training, invp, mask=None, update_mask=True):
+    """(y, mask) of api/dropout.jl:40-69 / impl/dropout.jl:3-47 given the uniform noise (an array
+    of dropout_shape(x, dims), column-major order of draws) that `rand!` would have produced.
+    Not training: (x, x) without a mask argument (the returned mask is meaningless), (x, mask)
+    with one."""
+    if mask is not None and not update_mask:
+        if not training:
+            return x, mask
+        assert all(m in (1, s) for m, s in zip(mask.shape, x.shape)) and mask.ndim == x.ndim, \
+            "`mask` is not of the same size as `LuxLib.dropout_shape(x, dims)`."
+        return x * mask, mask
+    if not training:
+        return x, (x if mask is None else mask)
+    m = generate_dropout_mask(noise, p, invp)
+    return x * m, m
+
+
+def alpha_dropout_coefficients(p):
+    """impl/dropout.jl:57-62."""
+    alpha = -1.7580993408473766
+    A = 1.0 / math.sqrt((1 - p) * (1 + p * alpha ** 2))
+    return alpha, A, -A * alpha * p
+
+
+def alpha_dropout(noise, p, x, alpha, A, B):
+    """muladd(ifelse(noise > p, x, α), A, B) with α, A, B in x's dtype (impl/dropout.jl:84-89)."""
+    T = x.dtype.type
+    return np.where(noise > p, x, T(alpha)) * T(A) + T(B)
+
+
+def alpha_dropout_pullback(noise, p, delta, A):
+    """∂x = Δ · (noise > p) · A (impl/dropout.jl:137-150)."""
+    return delta * (noise > p) * delta.dtype.type(A)
+
+
+# --------------------------------------------------------------------------------------
 # layernorm  (api/layernorm.jl:32-43, impl/layernorm.jl:3-51, impl/normalization.jl:3-17)
 # --------------------------------------------------------------------------------------
 def layernorm(x, gamma, beta, act: str = "identity", dims=None, eps=None):
@@ -586,6 +676,18 @@ class ConvDims:
             raise DimensionMismatch("input channels do not match weight channels x groups")
         if Cout % self.groups != 0:
             raise DimensionMismatch("output channels must be divisible by groups")
+
+    @classmethod
+    def one_spatial_dim(cls, x_shape, w_shape, stride=1, padding=(0, 0), dilation=1, groups=1, flipkernel=False):
+        """x (W, C, N), w (K, C/groups, Cout): the problem of height 1 over x (W, 1, C, N) that NNlib
+        itself reduces fewer-than-3-d convolutions to (it inserts singleton spatial dims).
+        padding = (lo, hi) or one int."""
+        if isinstance(padding, int):
+            padding = (padding, padding)
+        W, C, N = x_shape
+        K, Cg, Cout = w_shape
+        return cls((W, 1, C, N), (K, 1, Cg, Cout), (int(np.ravel(stride)[0]), 1), tuple(padding) + (0, 0),
+                   (int(np.ravel(dilation)[0]), 1), groups, flipkernel)
 
     @property
     def out_spatial(self):

@@ -109,6 +109,36 @@ def test_fused_conv_pullback(gpu, dtype, act):
                 assert gb is None
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("xs,ws,stride,pad,dil,groups,flip", [
+    ((12, 4, 2), (3, 4, 6), 1, (1, 1), 1, 1, False), ((13, 6, 3), (4, 3, 4), 2, (0, 2), 2, 2, False),
+    ((9, 2, 2), (2, 2, 3), 1, (1, 0), 1, 1, True), ((200, 64, 4), (5, 64, 96), 1, 2, 1, 1, False)])
+def test_one_spatial_dim(gpu, dtype, xs, ws, stride, pad, dil, groups, flip):
+    """x (W, C, N), w (K, C/groups, Cout) (lib/LuxLib/test/common_ops/conv_tests.jl runs 1-d cases too)."""
+    rng = np.random.default_rng(stable_seed(dtype, xs, ws))
+    gd = gpu.DenseConvDims(xs, ws, stride=stride, padding=pad, dilation=dil, groups=groups, flipkernel=flip)
+    od = O.ConvDims.one_spatial_dim(xs, ws, stride, pad, dil, groups, flip)
+    assert gd.y_shape == (od.y_shape()[0],) + od.y_shape()[2:]
+    x, w, b, delta = host_inputs(dtype, rng.normal(size=xs), rng.normal(size=ws) * np.sqrt(2.0 / (ws[0] * ws[1])),
+                                 rng.normal(size=ws[2]) * 0.1, rng.normal(size=gd.y_shape))
+    y, back = gpu.pullback(gpu.fused_conv_bias_activation, "tanh", dev(gpu, w, dtype), dev(gpu, x, dtype), dev(gpu, b, dtype), gd)
+    x4, w4, d4 = f64(x).reshape(od.x_shape), f64(w).reshape(od.w_shape), f64(delta).reshape(od.y_shape())
+    wy, wdw, wdx, wdb = O.fused_conv_pullback("tanh", w4, x4, f64(b), od, d4)
+    assert_close(y.to_numpy(), wy.reshape(gd.y_shape), dtype, "1-d y")
+    gw, gx, gb = back(dev(gpu, delta, dtype))
+    if dtype == "bf16":                      # y and dz are stored in bf16 between the passes
+        yq = f64(O.round_to_bf16(wy.astype(np.float32)))
+        dzx = O.grad_activation(d4, yq, "tanh", None)
+        dz = f64(O.round_to_bf16(dzx.astype(np.float32)))
+        wdw, wdx, wdb = O.conv_filter_grad(x4, dz, od), O.conv_data_grad(dz, w4, od), O.grad_bias_add(b, dzx)
+    assert gw.shape == tuple(ws) and gx.shape == tuple(xs)
+    assert_close(gw.to_numpy(), wdw.reshape(ws), dtype, "1-d dw", scale=np.sqrt(np.prod(gd.y_shape) / ws[2]) * rms(delta) * rms(x) * 0.5)
+    assert_close(gx.to_numpy(), wdx.reshape(xs), dtype, "1-d dx", scale=np.sqrt(ws[0] * ws[2] / groups) * rms(delta) * rms(w) * 0.5)
+    assert_close(gb.to_numpy(), wdb, dtype, "1-d db", rel=None if dtype == "f32" else 2e-2)
+    with pytest.raises(gpu.Unsupported):
+        gpu.DenseConvDims((4, 4, 4, 2, 1), (2, 2, 2, 2, 3))
+
+
 def test_dimension_mismatch(gpu):
     with pytest.raises(gpu.DimensionMismatch):
         gpu.DenseConvDims((8, 8, 4, 2), (3, 3, 3, 6))

@@ -411,6 +411,28 @@ def test_conv_vs_bruteforce_and_torch(xs, ws, stride, pad, dil, groups, flip):
     np.testing.assert_allclose(dw, twg if flip else twg[::-1, ::-1], rtol=1e-10, atol=1e-11)
 
 
+@pytest.mark.parametrize("xs,ws,stride,pad,dil,groups,flip", [
+    ((12, 4, 2), (3, 4, 6), 1, (1, 1), 1, 1, False), ((13, 6, 3), (4, 3, 4), 2, (0, 2), 2, 2, False),
+    ((9, 2, 2), (2, 2, 3), 1, (1, 0), 1, 1, True)])
+def test_conv_one_spatial_dim_vs_torch(xs, ws, stride, pad, dil, groups, flip):
+    """(W, C, N) inputs as a height-1 problem against torch conv1d (cross-correlation over NCW)."""
+    x, w = RNG.normal(size=xs), RNG.normal(size=ws)
+    cd = O.ConvDims.one_spatial_dim(xs, ws, stride, pad, dil, groups, flip)
+    x4, w4 = x.reshape(cd.x_shape), w.reshape(cd.w_shape)
+    y = O.conv(x4, w4, cd)
+    tx = torch.tensor(np.transpose(x, (2, 1, 0)).copy(), requires_grad=True)
+    tw = torch.tensor(np.transpose(w if flip else w[::-1], (2, 1, 0)).copy(), requires_grad=True)
+    ty = F.conv1d(F.pad(tx, pad), tw, None, stride=stride, dilation=dil, groups=groups)
+    assert y.shape[1] == 1
+    np.testing.assert_allclose(y[:, 0], np.transpose(ty.detach().numpy(), (2, 1, 0)), rtol=1e-11, atol=1e-11)
+    delta = RNG.normal(size=y.shape)
+    ty.backward(torch.tensor(np.transpose(delta[:, 0], (2, 1, 0)).copy()))
+    np.testing.assert_allclose(O.conv_data_grad(delta, w4, cd)[:, 0], np.transpose(tx.grad.numpy(), (2, 1, 0)),
+                               rtol=1e-10, atol=1e-11)
+    twg = np.transpose(tw.grad.numpy(), (2, 1, 0))
+    np.testing.assert_allclose(O.conv_filter_grad(x4, delta, cd)[:, 0], twg if flip else twg[::-1], rtol=1e-10, atol=1e-11)
+
+
 def test_fused_conv_pullback_finite_differences():
     xs, ws = (5, 4, 2, 2), (3, 3, 2, 3)
     x, w, b = RNG.normal(size=xs), RNG.normal(size=ws), RNG.normal(size=3)
