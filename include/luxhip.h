@@ -237,6 +237,19 @@ int luxhip_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t 
                   const void* A, int64_t lda, const void* B, int64_t ldb, const void* bias, void* C,
                   int64_t ldc);
 
+/* Impl.batched_matmul!(z, opmode, x, y) (src/impl/batched_mul.jl:204-212; NNlib.batched_mul! on
+ * 3-d arrays): C_b (M x N) = op(A_b) op(B_b) for b < batch, matrix b of an operand starting
+ * b * stride elements after the first; a stride of 0 shares one matrix among all products
+ * (batch dims of extent 1, :171-174, 255-268).  transA / transB as in luxhip_matmul: the pullback
+ * multiplies by the batched adjoints (batched_mul.jl rrule: dx = dz y', dy = x' dz). */
+int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                          int64_t batch, const void* A, int64_t lda, int64_t strideA, const void* B, int64_t ldb,
+                          int64_t strideB, void* C, int64_t ldc, int64_t strideC);
+
+/* `sum(tmp; dims=3)` of the batched_matmul pullback when an operand was shared among the
+ * products (src/impl/batched_mul.jl:324-330): out[i] = sum_b in[i + b n], i < n, in batch order. */
+int luxhip_batch_sum(luxhip_stream_t s, int dtype, int64_t n, int64_t batch, const void* in, void* out);
+
 /* y (M x N) = act.(W (M x K) * x (K x N) .+ bias).  Stands behind
  * Impl.fused_dense!(y, ::GPUBroadcastOp, act, W, x, b) (src/impl/dense.jl:46-69; precedent
  * cublasLt_fused_dense!, ext/CUDAExt/cublaslt.jl:351-403).  If pre != NULL (M x N, ld =

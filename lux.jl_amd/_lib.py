@@ -76,6 +76,8 @@ SIGNATURES = {
     "luxhip_layernorm_fwd": [_vp, _i, _i, _i64, _i64, _vp, _vp, _vp, _d, _vp, _fp, _fp],
     "luxhip_layernorm_bwd": [_vp, _i, _i, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _vp, _vp, _vp],
     "luxhip_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64],
+    "luxhip_batched_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64],
+    "luxhip_batch_sum": [_vp, _i, _i64, _i64, _vp, _vp],
     "luxhip_fused_dense_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp],
     "luxhip_fused_dense_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp],
     "luxhip_conv_fwd": [_vp, _i, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp, _vp, _vp],

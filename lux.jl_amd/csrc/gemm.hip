@@ -37,6 +37,70 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
     return launch_layout<T, false, false>(s, a);
 }
 
+// C_b = op(A_b) op(B_b) for b < batch; a batch stride of 0 shares one matrix among all products
+template <typename T>
+static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, const T* A,
+                        int64_t lda, int64_t strideA, const T* B, int64_t ldb, int64_t strideB, T* C, int64_t ldc,
+                        int64_t strideC) {
+    DenseArgs<T> a;
+    const bool a_kmajor = transA != 0, b_kmajor = transB == 0;
+    a.A.p = A;
+    a.A.sr = a_kmajor ? lda : 1;
+    a.A.sk = a_kmajor ? 1 : lda;
+    a.A.rows = (int)M;
+    a.A.vec_ok = aligned16(A) && (lda * sizeof(T)) % 16 == 0 && (strideA * sizeof(T)) % 16 == 0;
+    a.B.p = B;
+    a.B.sr = b_kmajor ? ldb : 1;
+    a.B.sk = b_kmajor ? 1 : ldb;
+    a.B.rows = (int)N;
+    a.B.vec_ok = aligned16(B) && (ldb * sizeof(T)) % 16 == 0 && (strideB * sizeof(T)) % 16 == 0;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.C = C; a.ldc = ldc; a.bias = nullptr; a.pre = nullptr; a.act = LUXHIP_ACT_IDENTITY;
+    a.batch = (int)batch; a.bsA = strideA; a.bsB = strideB; a.bsC = strideC;
+    if (a_kmajor && b_kmajor) return launch_batched_layout<T, true, true>(s, a);
+    if (a_kmajor) return launch_batched_layout<T, true, false>(s, a);
+    if (b_kmajor) return launch_batched_layout<T, false, true>(s, a);
+    return launch_batched_layout<T, false, false>(s, a);
+}
+
+// out[i] = sum_b in[i + b n]: `sum(tmp; dims=3)` of a stack of matrices, accumulated in fp32 in batch order
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void batch_sum_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t n, int batch,
+                                                        int64_t first, int64_t nvec) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const int64_t e = first + i * VEC;
+        float acc[VEC] = {};
+        for (int b = 0; b < batch; ++b) {
+            float v[VEC];
+            if constexpr (VEC == 1) v[0] = ld(in + e + (int64_t)b * n);
+            else Vec<T>::load(in + e + (int64_t)b * n, v);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] += v[k];
+        }
+        if constexpr (VEC == 1) st(out + e, acc[0]);
+        else Vec<T>::store(out + e, acc);
+    }
+}
+
+template <typename T>
+static int batch_sum_impl(hipStream_t s, int64_t n, int64_t batch, const T* in, T* out) {
+    constexpr int V = Vec<T>::N;
+    const bool vec = aligned16(in) && aligned16(out) && (n * sizeof(T)) % 16 == 0;
+    const int64_t nvec = vec ? n / V : 0;
+    ProfScope ps("batch_sum_kernel", s);
+    const unsigned cap = (unsigned)(num_cus() > 0 ? num_cus() : 256) * 16;
+    if (nvec > 0) {
+        batch_sum_kernel<T, V><<<std::min((unsigned)ceil_div(nvec, 256), cap), 256, 0, s>>>(in, out, n, (int)batch, 0, nvec);
+        LUX_CHECK_LAUNCH();
+    }
+    if (nvec * V < n) {
+        const int64_t rest = n - nvec * V;
+        batch_sum_kernel<T, 1><<<std::min((unsigned)ceil_div(rest, 256), cap), 256, 0, s>>>(in, out, n, (int)batch, nvec * V, rest);
+        LUX_CHECK_LAUNCH();
+    }
+    return LUXHIP_OK;
+}
+
 static int gemm_check(int dtype, int act, int64_t M, int64_t N, int64_t K) {
     LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
     LUX_UNSUPPORTED_IF(act < 0 || act >= LUXHIP_ACT_COUNT, "unsupported activation id %d", act);
@@ -72,6 +136,37 @@ int luxhip_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t 
     if (rc != LUXHIP_OK) return rc;
     return gemm_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, A, lda, B, ldb, bias, C, ldc, nullptr,
                          LUXHIP_ACT_IDENTITY);
+}
+
+int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                          int64_t batch, const void* A, int64_t lda, int64_t strideA, const void* B, int64_t ldb,
+                          int64_t strideB, void* C, int64_t ldc, int64_t strideC) {
+    LUX_REQUIRE_INIT();
+    int rc = gemm_check(dtype, 0, M, N, K);
+    if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF(batch < 0 || strideA < 0 || strideB < 0 || strideC < 0, "batched_matmul: negative batch or stride");
+    LUX_UNSUPPORTED_IF(batch >= (1ll << 31), "batched_matmul: batch of 2^31 or more");
+    if (M == 0 || N == 0 || batch == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(C == nullptr, "batched_matmul: C must not be NULL");
+    LUX_INVALID_IF(K > 0 && (A == nullptr || B == nullptr), "batched_matmul: A and B must not be NULL");
+    LUX_INVALID_IF(lda < (transA ? K : M) || ldb < (transB ? N : K) || ldc < M, "batched_matmul: leading dimension too small");
+    LUX_INVALID_IF(batch > 1 && strideC < ldc * (N - 1) + M, "batched_matmul: the results would overlap");
+    if (dtype == LUXHIP_F32)
+        return batched_impl<float>((hipStream_t)s, transA, transB, M, N, K, batch, (const float*)A, lda, strideA,
+                                   (const float*)B, ldb, strideB, (float*)C, ldc, strideC);
+    return batched_impl<bf16_t>((hipStream_t)s, transA, transB, M, N, K, batch, (const bf16_t*)A, lda, strideA,
+                                (const bf16_t*)B, ldb, strideB, (bf16_t*)C, ldc, strideC);
+}
+
+int luxhip_batch_sum(luxhip_stream_t s, int dtype, int64_t n, int64_t batch, const void* in, void* out) {
+    LUX_REQUIRE_INIT();
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_INVALID_IF(n < 0 || batch < 1, "batch_sum: invalid extent");
+    LUX_UNSUPPORTED_IF(batch >= (1ll << 31), "batch_sum: batch of 2^31 or more");
+    if (n == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(in == nullptr || out == nullptr, "batch_sum: in and out must not be NULL");
+    if (dtype == LUXHIP_F32) return batch_sum_impl<float>((hipStream_t)s, n, batch, (const float*)in, (float*)out);
+    return batch_sum_impl<bf16_t>((hipStream_t)s, n, batch, (const bf16_t*)in, (bf16_t*)out);
 }
 
 int luxhip_fused_dense_fwd(luxhip_stream_t s, int dtype, int act, int64_t M, int64_t K, int64_t N, const void* W,

@@ -195,4 +195,62 @@ int launch_layout(hipStream_t s, DenseArgs<T>& a) {
     return launch_cfg<T, 1, 1, AK, BKM>(s, a);
 }
 
+// Batched products: grid.x walks the tiles of one product, grid.y the batch.
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
+__global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<T> a) {
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM>;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T* lds = reinterpret_cast<T*>(lds_raw);
+    int tm, tn;
+    tile_coords(blockIdx.x, a.tiles_m, a.tiles_n, tm, tn);
+    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
+    for (int b = blockIdx.y; b < a.batch; b += gridDim.y) {
+        DenseArgs<T> ab = a;
+        ab.A.p = a.A.p + (int64_t)b * a.bsA;
+        ab.B.p = a.B.p + (int64_t)b * a.bsB;
+        ab.C = a.C + (int64_t)b * a.bsC;
+        f32x16_v acc[WM][WN];
+        if constexpr (ML::DIRECT) {
+            DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(ab.A, m0);
+            DirectLoader<B_KMAJOR, ML::TILE_N, ML::THREADS> lb(ab.B, n0);
+            ML::pipeline_fill(la, lb, a.K, lds);
+            ML::pipeline_loop(la, lb, a.K, lds, acc);
+        } else {
+            ML::run(ab.A, ab.B, a.K, m0, n0, lds, acc);
+        }
+        dense_epilogue<ML, T, WM, WN, FULL>(acc, ab, m0, n0);
+        __syncthreads();   // every wave is done with the LDS stages before the next product refills them
+    }
+}
+
+template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL>
+int launch_batched_cfg(hipStream_t s, DenseArgs<T>& a) {
+    using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL, 2, 0, 2>;
+    a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
+    a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
+    auto kernel = batched_gemm_kernel<T, WM, WN, AK, BKM, FULL, 2, 2>;
+    static bool prepared = false;
+    if (!prepared) {
+        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)ML::LDS_BYTES));
+        prepared = true;
+    }
+    ProfScope ps(sizeof(T) == 2 ? "batched_gemm_kernel<bf16>" : "batched_gemm_kernel<f32>", s);
+    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)std::min(a.batch, 65535)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T, bool AK, bool BKM>
+int launch_batched_layout(hipStream_t s, DenseArgs<T>& a) {
+    // 128 x 128 tiles when a product has at least one whole tile of them, 64 x 64 otherwise;
+    // the variant without bounds checks when every product is made of whole, aligned tiles
+    const bool strides_ok = (a.bsA * sizeof(T)) % 16 == 0 && (a.bsB * sizeof(T)) % 16 == 0;
+    if (a.M >= 128 && a.N >= 128) {
+        if (strides_ok && whole_tiles<T, 128, 128>(a)) return launch_batched_cfg<T, 2, 2, AK, BKM, true>(s, a);
+        return launch_batched_cfg<T, 2, 2, AK, BKM, false>(s, a);
+    }
+    return launch_batched_cfg<T, 1, 1, AK, BKM, false>(s, a);
+}
+
 }  // namespace luxhip

@@ -328,6 +328,92 @@ def matmul(A: DeviceArray, B: DeviceArray, bias: Optional[DeviceArray] = None, t
     return out
 
 
+# ------------------------------------------------------------------------------- batched_matmul
+def _as_batched(a: DeviceArray, what: str):
+    """(rows, cols, batch, batch_shape) of an N-d operand whose batching dims are the trailing ones."""
+    if a.ndim < 3:
+        raise ArgumentError(f"{what}: N must be at least 3")       # impl/batched_mul.jl:127
+    b = 1
+    for sdim in a.shape[2:]:
+        b *= sdim
+    return a.shape[0], a.shape[1], b, tuple(a.shape[2:])
+
+
+def _bmm(A, tA, B, tB, M, N, K, batch, sA, sB, dtype):
+    out = DeviceArray((M, N, batch), dtype)
+    _lib.call("luxhip_batched_matmul", current_stream(), out.code, int(tA), int(tB), M, N, K, batch,
+              A.ptr, max(A.shape[0], 1), sA, B.ptr, max(B.shape[0], 1), sB, out.ptr, max(M, 1), M * N)
+    return out
+
+
+def _batched_geometry(x, y, lhs_contracting_dim, rhs_contracting_dim):
+    if x.ndim == 2 and y.ndim >= 3:
+        x = x.reshape(x.shape + (1,) * (y.ndim - 2))               # expand_batchdim, api/batched_mul.jl
+    if y.ndim == 2 and x.ndim >= 3:
+        y = y.reshape(y.shape + (1,) * (x.ndim - 2))
+    if x.ndim != y.ndim:
+        raise ArgumentError("batched_matmul: x and y must have the same number of dims")
+    if lhs_contracting_dim not in (1, 2) or rhs_contracting_dim not in (1, 2):
+        raise _lib.Unsupported(_lib.UNSUPPORTED, "batched_matmul: the batching dims must be the trailing ones")
+    xr, xc, xb, xbs = _as_batched(x, "x")
+    yr, yc, yb, ybs = _as_batched(y, "y")
+    for a_, b_ in zip(xbs, ybs):
+        if a_ != b_ and a_ != 1 and b_ != 1:
+            raise DimensionMismatch(f"Batching dimensions mismatch: {xbs} vs {ybs}")      # impl/batched_mul.jl:133-141
+    bshape = tuple(max(a_, b_) for a_, b_ in zip(xbs, ybs))
+    batch = 1
+    for sdim in bshape:
+        batch *= sdim
+    if not (xb in (1, batch) and yb in (1, batch)):
+        raise _lib.Unsupported(_lib.UNSUPPORTED, "batched_matmul: batch dims that repeat only some of several dims")
+    tA, tB = lhs_contracting_dim == 1, rhs_contracting_dim == 2
+    M, Kx = (xc, xr) if tA else (xr, xc)
+    Ky, N = (yc, yr) if tB else (yr, yc)
+    if Kx != Ky:
+        raise DimensionMismatch(f"size(x) = {x.shape}, size(y) = {y.shape} inconsistent for batched_matmul.")
+    return x, y, tA, tB, M, N, Kx, batch, xb, yb, bshape
+
+
+def batched_matmul(x: DeviceArray, y: DeviceArray, lhs_contracting_dim: int = 2, rhs_contracting_dim: int = 1):
+    """`batched_matmul(x, y; lhs_contracting_dim, rhs_contracting_dim)` (api/batched_mul.jl,
+    impl/batched_mul.jl:2-58) with the default (trailing) batching dims: z[:, :, b...] =
+    op(x[:, :, b...]) op(y[:, :, b...]); batch dims of extent 1 are shared among the products."""
+    return rrule_batched_matmul(x, y, lhs_contracting_dim, rhs_contracting_dim, _need_back=False)[0]
+
+
+def rrule_batched_matmul(x, y, lhs_contracting_dim=2, rhs_contracting_dim=1, _need_back=True):
+    """CRC.rrule(batched_matmul_fallback) (impl/batched_mul.jl:320-334): (z, Δ -> (∂x, ∂y)) with
+    ∂x = Δ ⊠ adjoint(y), ∂y = adjoint(x) ⊠ Δ, summed over the batch for a shared operand."""
+    x_shape, y_shape = x.shape, y.shape
+    dt = _same_dtype(x, y)
+    x, y, tA, tB, M, N, K, batch, xb, yb, bshape = _batched_geometry(x, y, lhs_contracting_dim, rhs_contracting_dim)
+    sx, sy = (x.shape[0] * x.shape[1] if xb > 1 else 0), (y.shape[0] * y.shape[1] if yb > 1 else 0)
+    z = _bmm(x, tA, y, tB, M, N, K, batch, sx, sy, dt).reshape((M, N) + bshape)
+
+    def back(delta: DeviceArray):
+        g = delta.reshape((M, N, batch))
+        # ∂(op(x)) = Δ op(y)ᵀ, stored as x is: transposed when x is contracted along dim 1
+        if not tA:
+            dx = _bmm(g, False, y, not tB, M, K, N, batch, M * N, sy, dt)
+        else:
+            dx = _bmm(y, tB, g, True, K, M, N, batch, sy, M * N, dt)
+        if not tB:
+            dy = _bmm(x, not tA, g, False, K, N, M, batch, sx, M * N, dt)
+        else:
+            dy = _bmm(g, True, x, tA, N, K, M, batch, M * N, sx, dt)
+        out = []
+        for grad, shared, shape in ((dx, xb == 1 and batch > 1, x_shape), (dy, yb == 1 and batch > 1, y_shape)):
+            if shared:
+                n = grad.shape[0] * grad.shape[1]
+                red = DeviceArray((grad.shape[0], grad.shape[1], 1), dt)
+                _lib.call("luxhip_batch_sum", current_stream(), grad.code, n, batch, grad.ptr, red.ptr)
+                grad = red
+            out.append(grad.reshape(shape))
+        return tuple(out)
+
+    return z, back
+
+
 # ------------------------------------------------------------------------------- batchnorm
 def batchnorm(x: DeviceArray, scale, bias, running_mean, running_var, training, act: str = "identity",
               momentum: float = 0.1, epsilon: Optional[float] = None):
@@ -682,6 +768,7 @@ _RRULES = {
     instancenorm: rrule_instancenorm,
     fast_activation: rrule_fast_activation,
     dropout: rrule_dropout,
+    batched_matmul: rrule_batched_matmul,
     alpha_dropout: rrule_alpha_dropout,
     layernorm: rrule_layernorm,
     fused_conv_bias_activation: rrule_fused_conv_bias_activation,

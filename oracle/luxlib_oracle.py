@@ -22,6 +22,7 @@ tests/test_oracle_*.py):
                                         torch F.batch_norm autograd, finite differences
   * groupnorm (+bwd) .................. torch F.group_norm autograd, finite differences
   * layernorm (+bwd) .................. mean~0/std~1 invariant, torch F.layer_norm autograd
+  * batched_matmul (+pullback) ........ torch.matmul over a batch + autograd
   * dropout / alpha_dropout ........... closed forms; the Philox4x32-10 noise stream against
                                         the Random123 known-answer vectors and uniformity
                                         statistics (Julia's own rng streams are out of reach)
@@ -499,6 +500,53 @@ def instancenorm_pullback(x, gamma, beta, act: str, eps, delta, *, training=True
         dvar = -(dx * xmu).sum(axis=axes, keepdims=True) * T(0.5) * idenom * idenom
         dx = dx + mean_var_pullback(x, mu, axes, dmu, dvar)
     return dx, (None if gamma is None else dgamma), (None if beta is None else dbeta)
+
+
+# --------------------------------------------------------------------------------------
+# batched_matmul  (api/batched_mul.jl, impl/batched_mul.jl:2-58, 171-334) with the default
+# (trailing) batching dims
+# --------------------------------------------------------------------------------------
+def _bmm_operands(x, y, lhs_contracting_dim, rhs_contracting_dim):
+    x, y = np.asarray(x), np.asarray(y)
+    if x.ndim == 2 and y.ndim >= 3:
+        x = x.reshape(x.shape + (1,) * (y.ndim - 2))        # expand_batchdim
+    if y.ndim == 2 and x.ndim >= 3:
+        y = y.reshape(y.shape + (1,) * (x.ndim - 2))
+    if x.ndim < 3 or x.ndim != y.ndim:
+        raise ArgumentError("N must be at least 3")
+    for a, b in zip(x.shape[2:], y.shape[2:]):
+        if a != b and a != 1 and b != 1:
+            raise DimensionMismatch("Batching dimensions mismatch")
+    xo = x if lhs_contracting_dim == 2 else np.swapaxes(x, 0, 1)      # (M, K, b...)
+    yo = y if rhs_contracting_dim == 1 else np.swapaxes(y, 0, 1)      # (K, N, b...)
+    if xo.shape[1] != yo.shape[0]:
+        raise DimensionMismatch("inconsistent for batched_matmul")
+    return x, y, xo, yo
+
+
+def batched_matmul(x, y, lhs_contracting_dim=2, rhs_contracting_dim=1):
+    """z[:, :, b...] = op(x[:, :, b...]) op(y[:, :, b...]); batch dims of extent 1 repeat
+    (impl/batched_mul.jl:76-110, 255-268)."""
+    _, _, xo, yo = _bmm_operands(x, y, lhs_contracting_dim, rhs_contracting_dim)
+    return np.einsum("mk...,kn...->mn...", xo, yo)
+
+
+def batched_matmul_pullback(x, y, delta, lhs_contracting_dim=2, rhs_contracting_dim=1):
+    """(∂x, ∂y): ∂x = Δ ⊠ adjoint(y), ∂y = adjoint(x) ⊠ Δ, summed over the batch dims along which
+    the operand was repeated (impl/batched_mul.jl:320-334), in the operand's own layout."""
+    x0, y0 = np.asarray(x), np.asarray(y)
+    x, y, xo, yo = _bmm_operands(x, y, lhs_contracting_dim, rhs_contracting_dim)
+    delta = np.asarray(delta)
+    dxo = np.einsum("mn...,kn...->mk...", delta, np.broadcast_to(yo, yo.shape[:2] + delta.shape[2:]))
+    dyo = np.einsum("mk...,mn...->kn...", np.broadcast_to(xo, xo.shape[:2] + delta.shape[2:]), delta)
+    dx = dxo if lhs_contracting_dim == 2 else np.swapaxes(dxo, 0, 1)
+    dy = dyo if rhs_contracting_dim == 1 else np.swapaxes(dyo, 0, 1)
+    for ax in range(2, delta.ndim):
+        if x.shape[ax] == 1 and delta.shape[ax] != 1:
+            dx = dx.sum(axis=ax, keepdims=True)
+        if y.shape[ax] == 1 and delta.shape[ax] != 1:
+            dy = dy.sum(axis=ax, keepdims=True)
+    return dx.reshape(x0.shape), dy.reshape(y0.shape)
 
 
 # --------------------------------------------------------------------------------------

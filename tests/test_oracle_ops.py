@@ -465,3 +465,42 @@ def test_bf16_round_trip_is_rne():
 def test_default_epsilon():
     # utils.jl:130: eps(T)^(5/7)
     assert abs(O.default_epsilon(np.float32) - (2.0 ** -23) ** (5 / 7)) < 1e-12
+
+
+# ----------------------------------------------------------------------------- batched_matmul
+@pytest.mark.parametrize("xs,ys,lc,rc", [
+    ((4, 5, 3), (5, 6, 3), 2, 1), ((4, 5, 1), (5, 6, 3), 2, 1), ((4, 5, 3), (5, 6, 1), 2, 1),
+    ((5, 4, 3), (5, 6, 3), 1, 1), ((4, 5, 3), (6, 5, 3), 2, 2), ((5, 4, 2, 3), (6, 5, 2, 3), 1, 2),
+    ((4, 5), (5, 6, 3), 2, 1), ((4, 5, 3), (5, 6), 2, 1)])
+def test_batched_matmul_vs_torch(xs, ys, lc, rc):
+    # lib/LuxLib/test/common_ops/bmm_tests.jl compares with a loop of `*`; here torch.matmul + autograd
+    x, y = RNG.normal(size=xs), RNG.normal(size=ys)
+    z = O.batched_matmul(x, y, lc, rc)
+    tx, ty = torch.tensor(x, requires_grad=True), torch.tensor(y, requires_grad=True)
+    bx = tx if tx.ndim > 2 else tx.reshape(tx.shape + (1,) * (ty.ndim - 2))
+    by = ty if ty.ndim > 2 else ty.reshape(ty.shape + (1,) * (tx.ndim - 2))
+    nd = bx.ndim
+    to_batch_first = tuple(range(nd - 1, 1, -1)) + (0, 1)
+    ax = bx.permute(to_batch_first)
+    ay = by.permute(to_batch_first)
+    if lc == 1:
+        ax = ax.transpose(-1, -2)
+    if rc == 2:
+        ay = ay.transpose(-1, -2)
+    tz = torch.matmul(ax, ay)
+    back_perm = (nd - 2, nd - 1) + tuple(range(nd - 3, -1, -1))
+    np.testing.assert_allclose(z, tz.permute(back_perm).detach().numpy(), rtol=1e-12, atol=1e-12)
+    delta = RNG.normal(size=z.shape)
+    tz.backward(torch.tensor(delta).permute(to_batch_first).contiguous())
+    dx, dy = O.batched_matmul_pullback(x, y, delta, lc, rc)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(dy, ty.grad.numpy(), rtol=1e-11, atol=1e-12)
+
+
+def test_batched_matmul_errors():
+    with pytest.raises(O.DimensionMismatch):
+        O.batched_matmul(np.ones((4, 5, 3)), np.ones((5, 6, 2)))
+    with pytest.raises(O.DimensionMismatch):
+        O.batched_matmul(np.ones((4, 5, 3)), np.ones((4, 6, 3)))
+    with pytest.raises(O.ArgumentError):
+        O.batched_matmul(np.ones((4, 5)), np.ones((5, 6)))
