@@ -180,6 +180,28 @@ int luxhip_instancenorm_running_stats(luxhip_stream_t s, int dtype, int64_t I, i
                                       double momentum, const void* rmean, const void* rvar, void* rmean_out,
                                       void* rvar_out);
 
+/* ---------------------------------------------------------------- attention ----------
+ * scaled_dot_product_attention (src/impl/attention.jl:5-117) = batched_matmul(k, q .* scale) ->
+ * apply_attention_mask_bias -> softmax over the key positions -> batched_matmul(v, probs).  The two
+ * products are luxhip_batched_matmul_strided calls; these are the passes between them.
+ * logits, probs, dprobs, dlogits: (S, L, H, B) column-major, S = key positions. */
+
+/* probs[:, l, h, b] = softmax_s(scale * logits[s, l, h, b] + bias[s, l, h, b], -inf where masked)
+ * (apply_attention_mask_bias, src/impl/attention.jl:119-128; NNlib.softmax(...; dims=1), :94-104).
+ * The scale multiplies the logits here instead of q before the product (:98).  causal != 0: keep
+ * s <= l (make_causal_mask, :130-134).  mask: bytes, non-zero = keep, or NULL; bias: storage dtype
+ * or NULL; both (S, L, H or 1, B or 1): the strides (in elements) along h and b are 0 where the
+ * extent is 1. */
+int luxhip_attention_softmax_fwd(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t H, int64_t B,
+                                 const void* logits, double scale, int causal, const uint8_t* mask,
+                                 int64_t mask_stride_h, int64_t mask_stride_b, const void* bias,
+                                 int64_t bias_stride_h, int64_t bias_stride_b, void* probs);
+
+/* Pullback of the same (the softmax rule of NNlib, reached by AD in the reference):
+ * dlogits = scale * probs .* (dprobs - sum_s dprobs .* probs); cols = L * H * B. */
+int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t cols, const void* dprobs,
+                                 const void* probs, double scale, void* dlogits);
+
 /* ---------------------------------------------------------------- dropout ----------
  * The reference draws its noise with `rand!(rng, y)` from the array package's generator
  * (src/impl/dropout.jl:171-190); here a counter-based Philox4x32-10 stream stands in for it:
@@ -245,6 +267,16 @@ int luxhip_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t 
 int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
                           int64_t batch, const void* A, int64_t lda, int64_t strideA, const void* B, int64_t ldb,
                           int64_t strideB, void* C, int64_t ldc, int64_t strideC);
+
+/* The same over up to three nested batch dims (batch_dims[0] innermost) with one stride per dim and
+ * operand: the products of permuted / repeated operands without copies, e.g. the (heads, batch)
+ * dims of scaled_dot_product_attention's [E, H, L, B] tensors and the key/value groups that
+ * repeat_inner_gqa (src/impl/attention.jl:1-3, 44-48) would materialise (stride 0 along the repeat).
+ * The caller lays out C so that the products do not overlap. */
+int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N,
+                                  int64_t K, const int64_t* batch_dims, const void* A, int64_t lda,
+                                  const int64_t* stridesA, const void* B, int64_t ldb, const int64_t* stridesB,
+                                  void* C, int64_t ldc, const int64_t* stridesC);
 
 /* `sum(tmp; dims=3)` of the batched_matmul pullback when an operand was shared among the
  * products (src/impl/batched_mul.jl:324-330): out[i] = sum_b in[i + b n], i < n, in batch order. */

@@ -37,6 +37,7 @@ class ConvDimsStruct(C.Structure):
 
 _vp, _i, _i64, _d, _sz, _u64 = C.c_void_p, C.c_int, C.c_int64, C.c_double, C.c_size_t, C.c_uint64
 _fp = C.c_void_p  # float* passed as raw address
+_ip64 = C.POINTER(C.c_int64)
 
 # name -> argtypes; every function returns int
 SIGNATURES = {
@@ -67,16 +68,19 @@ SIGNATURES = {
     "luxhip_groupnorm_fwd": [_vp, _i, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _d, _vp, _fp, _fp],
     "luxhip_groupnorm_bwd": [_vp, _i, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _vp, _vp, _vp],
     "luxhip_instancenorm_running_stats": [_vp, _i, _i64, _i64, _i64, _fp, _fp, _d, _d, _vp, _vp, _vp, _vp],
+    "luxhip_attention_softmax_fwd": [_vp, _i, _i64, _i64, _i64, _i64, _vp, _d, _i, _vp, _i64, _i64, _vp, _i64, _i64, _vp],
+    "luxhip_attention_softmax_bwd": [_vp, _i, _i64, _i64, _vp, _vp, _d, _vp],
     "luxhip_rand_uniform": [_vp, _i, _i64, _u64, _u64, _vp],
     "luxhip_dropout_fwd": [_vp, _i, _i64, _u64, _u64, _d, _d, _vp, _vp, _vp],
     "luxhip_dropout_mask": [_vp, _i, _i64, _d, _d, _vp],
-    "luxhip_dropout_mul": [_vp, _i, _i, C.POINTER(C.c_int64), C.POINTER(C.c_int64), _vp, _vp, _vp],
+    "luxhip_dropout_mul": [_vp, _i, _i, _ip64, _ip64, _vp, _vp, _vp],
     "luxhip_alpha_dropout_fwd": [_vp, _i, _i64, _vp, _d, _vp, _d, _d, _d, _vp],
     "luxhip_alpha_dropout_bwd": [_vp, _i, _i64, _vp, _d, _vp, _d, _vp],
     "luxhip_layernorm_fwd": [_vp, _i, _i, _i64, _i64, _vp, _vp, _vp, _d, _vp, _fp, _fp],
     "luxhip_layernorm_bwd": [_vp, _i, _i, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _vp, _vp, _vp],
     "luxhip_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64],
     "luxhip_batched_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64],
+    "luxhip_batched_matmul_strided": [_vp, _i, _i, _i, _i64, _i64, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64],
     "luxhip_batch_sum": [_vp, _i, _i64, _i64, _vp, _vp],
     "luxhip_fused_dense_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp],
     "luxhip_fused_dense_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp],

@@ -7,7 +7,8 @@ import numpy as np
 
 from . import _lib
 
-DTYPES = {"f32": (_lib.F32, 4), "bf16": (_lib.BF16, 2)}
+# "u8": boolean masks (one byte per element, non-zero = true); no arithmetic entry point takes it as a storage type
+DTYPES = {"f32": (_lib.F32, 4), "bf16": (_lib.BF16, 2), "u8": (-1, 1)}
 
 _stream = C.c_void_p(None)
 
@@ -38,7 +39,7 @@ class DeviceArray:
 
     def __init__(self, shape, dtype="f32", ptr=None, base=None):
         if dtype not in DTYPES:
-            raise TypeError(f"unsupported dtype {dtype!r} (use 'f32' or 'bf16')")
+            raise TypeError(f"unsupported dtype {dtype!r} (use 'f32' or 'bf16'; 'u8' for masks)")
         self.shape = tuple(int(s) for s in shape)
         self.dtype = dtype
         self._base = base
@@ -80,7 +81,10 @@ class DeviceArray:
     def from_numpy(cls, a, dtype="f32") -> "DeviceArray":
         a = np.asarray(a)
         out = cls(a.shape, dtype)
-        host = np.ascontiguousarray(np.asarray(a, dtype=np.float32).ravel(order="F"))
+        if dtype == "u8":
+            host = np.ascontiguousarray((a != 0).astype(np.uint8).ravel(order="F"))
+        else:
+            host = np.ascontiguousarray(np.asarray(a, dtype=np.float32).ravel(order="F"))
         if dtype == "bf16":
             host = _to_bf16_bits(host)
         if host.nbytes:
@@ -88,8 +92,8 @@ class DeviceArray:
         return out
 
     def to_numpy(self) -> np.ndarray:
-        """float32 numpy array with the logical shape (bf16 is widened exactly)."""
-        host = np.empty(self.size, dtype=np.float32 if self.dtype == "f32" else np.uint16)
+        """float32 numpy array with the logical shape (bf16 is widened exactly; masks stay bytes)."""
+        host = np.empty(self.size, dtype={"f32": np.float32, "bf16": np.uint16, "u8": np.uint8}[self.dtype])
         if host.nbytes:
             _lib.call("luxhip_memcpy_d2h", host.ctypes.data, self.ptr, host.nbytes, current_stream())
         if self.dtype == "bf16":

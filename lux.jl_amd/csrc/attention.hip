@@ -1,0 +1,225 @@
+// The softmax of scaled_dot_product_attention: scale, additive bias, boolean / causal mask and the
+// softmax over the key positions in one pass over the logits, and its pullback.  The two batched
+// products around it run on the batched MFMA GEMM.
+//
+// logits, probs: (S, L, H, B) column-major, S = key positions (softmax axis), L = query positions.
+// One wavefront owns one column of S values; columns of up to 64 * 16 values stay in registers
+// between the passes, longer ones are read again (they sit in the cache by then).
+#include <algorithm>
+
+#include "common.h"
+
+namespace luxhip {
+
+constexpr int kAttnWaves = 4;
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+__device__ __forceinline__ float wave_add(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+template <typename T>
+struct SoftmaxCol {
+    const T* x;
+    const T* bias;
+    const uint8_t* mask;
+    float scale;
+    int limit;      // positions s > limit are masked (causal); S - 1 otherwise
+    __device__ __forceinline__ float logit(int s) const {
+        float z = ld(x + s) * scale;
+        if (bias) z += ld(bias + s);
+        const bool keep = s <= limit && (mask == nullptr || mask[s] != 0);
+        return keep ? z : -INFINITY;
+    }
+};
+
+// NV > 0: the column (S <= 64 NV) is held in registers; NV == 0: any S, re-read per pass
+template <typename T, int NV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_kernel(const T* __restrict__ logits, T* __restrict__ probs,
+                                                                           int S, int L, int H, int64_t cols, float scale,
+                                                                           int causal, const uint8_t* __restrict__ mask,
+                                                                           int64_t mask_sh, int64_t mask_sb,
+                                                                           const T* __restrict__ bias, int64_t bias_sh,
+                                                                           int64_t bias_sb) {
+    const int lane = threadIdx.x & 63;
+    const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
+    if (col >= cols) return;            // whole wavefronts leave; nothing below synchronises across waves
+    const int l = (int)(col % L);
+    const int64_t hb = col / L;
+    const int h = (int)(hb % H);
+    const int64_t b = hb / H;
+    SoftmaxCol<T> c;
+    c.x = logits + col * S;
+    c.bias = bias ? bias + (int64_t)l * S + h * bias_sh + b * bias_sb : nullptr;
+    c.mask = mask ? mask + (int64_t)l * S + h * mask_sh + b * mask_sb : nullptr;
+    c.scale = scale;
+    c.limit = causal ? l : S - 1;       // make_causal_mask: keep key s for query l where s <= l
+    T* y = probs + col * S;
+    if constexpr (NV > 0) {
+        float z[NV];
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int s = lane + 64 * i;
+            z[i] = s < S ? c.logit(s) : -INFINITY;
+            m = fmaxf(m, z[i]);
+        }
+        m = wave_max(m);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            z[i] = __expf(z[i] - m);
+            sum += z[i];
+        }
+        const float inv = 1.f / wave_add(sum);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int s = lane + 64 * i;
+            if (s < S) st(y + s, z[i] * inv);
+        }
+    } else {
+        float m = -INFINITY;
+        for (int s = lane; s < S; s += 64) m = fmaxf(m, c.logit(s));
+        m = wave_max(m);
+        float sum = 0.f;
+        for (int s = lane; s < S; s += 64) sum += __expf(c.logit(s) - m);
+        const float inv = 1.f / wave_add(sum);
+        for (int s = lane; s < S; s += 64) st(y + s, __expf(c.logit(s) - m) * inv);
+    }
+}
+
+// dlogits = scale * probs .* (dprobs - sum_s dprobs .* probs)
+template <typename T, int NV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_kernel(const T* __restrict__ dprobs,
+                                                                           const T* __restrict__ probs, T* __restrict__ dlogits,
+                                                                           int S, int64_t cols, float scale) {
+    const int lane = threadIdx.x & 63;
+    const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
+    if (col >= cols) return;
+    const T* dy = dprobs + col * S;
+    const T* y = probs + col * S;
+    T* dx = dlogits + col * S;
+    if constexpr (NV > 0) {
+        float yv[NV], dv[NV];
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int s = lane + 64 * i;
+            yv[i] = s < S ? ld(y + s) : 0.f;
+            dv[i] = s < S ? ld(dy + s) : 0.f;
+            dot += yv[i] * dv[i];
+        }
+        dot = wave_add(dot);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int s = lane + 64 * i;
+            if (s < S) st(dx + s, scale * yv[i] * (dv[i] - dot));
+        }
+    } else {
+        float dot = 0.f;
+        for (int s = lane; s < S; s += 64) dot += ld(y + s) * ld(dy + s);
+        dot = wave_add(dot);
+        for (int s = lane; s < S; s += 64) st(dx + s, scale * ld(y + s) * (ld(dy + s) - dot));
+    }
+}
+
+static inline int cached_vectors(int64_t S) {
+    for (int nv : {1, 2, 4, 8, 16})
+        if (S <= 64 * nv) return nv;
+    return 0;
+}
+
+template <typename T>
+static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int64_t B, const T* logits, float scale, int causal,
+                            const uint8_t* mask, int64_t mask_sh, int64_t mask_sb, const T* bias, int64_t bias_sh,
+                            int64_t bias_sb, T* probs) {
+    const int64_t cols = L * H * B;
+    const unsigned grid = (unsigned)ceil_div(cols, kAttnWaves);
+    ProfScope ps("attn_softmax_fwd_kernel", s);
+#define LUX_SOFTMAX_FWD(NV)                                                                                                   \
+    attn_softmax_fwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
+                                                                    mask, mask_sh, mask_sb, bias, bias_sh, bias_sb)
+    switch (cached_vectors(S)) {
+        case 1: LUX_SOFTMAX_FWD(1); break;
+        case 2: LUX_SOFTMAX_FWD(2); break;
+        case 4: LUX_SOFTMAX_FWD(4); break;
+        case 8: LUX_SOFTMAX_FWD(8); break;
+        case 16: LUX_SOFTMAX_FWD(16); break;
+        default: LUX_SOFTMAX_FWD(0); break;
+    }
+#undef LUX_SOFTMAX_FWD
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+template <typename T>
+static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t cols, const T* dprobs, const T* probs, float scale, T* dlogits) {
+    const unsigned grid = (unsigned)ceil_div(cols, kAttnWaves);
+    ProfScope ps("attn_softmax_bwd_kernel", s);
+#define LUX_SOFTMAX_BWD(NV) attn_softmax_bwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, cols, scale)
+    switch (cached_vectors(S)) {
+        case 1: LUX_SOFTMAX_BWD(1); break;
+        case 2: LUX_SOFTMAX_BWD(2); break;
+        case 4: LUX_SOFTMAX_BWD(4); break;
+        case 8: LUX_SOFTMAX_BWD(8); break;
+        case 16: LUX_SOFTMAX_BWD(16); break;
+        default: LUX_SOFTMAX_BWD(0); break;
+    }
+#undef LUX_SOFTMAX_BWD
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+static int softmax_check(int dtype, int64_t S, int64_t cols) {
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_INVALID_IF(S < 0 || cols < 0, "invalid dimension");
+    LUX_UNSUPPORTED_IF(S >= (1ll << 31) || cols >= (1ll << 33), "attention softmax: dimension too large");
+    return LUXHIP_OK;
+}
+
+}  // namespace luxhip
+
+using namespace luxhip;
+
+extern "C" {
+
+int luxhip_attention_softmax_fwd(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t H, int64_t B, const void* logits,
+                                 double scale, int causal, const uint8_t* mask, int64_t mask_stride_h, int64_t mask_stride_b,
+                                 const void* bias, int64_t bias_stride_h, int64_t bias_stride_b, void* probs) {
+    LUX_REQUIRE_INIT();
+    LUX_INVALID_IF(L < 0 || H < 0 || B < 0, "invalid dimension");
+    int rc = softmax_check(dtype, S, L * H * B);
+    if (rc != LUXHIP_OK) return rc;
+    if (S * L * H * B == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(logits == nullptr || probs == nullptr, "attention_softmax_fwd: logits and probs must not be NULL");
+    LUX_INVALID_IF(mask_stride_h < 0 || mask_stride_b < 0 || bias_stride_h < 0 || bias_stride_b < 0, "negative stride");
+    LUX_INVALID_IF(causal != 0 && mask != nullptr, "`mask` and `is_causal` cannot both be specified");
+    if (dtype == LUXHIP_F32)
+        return softmax_fwd_impl<float>((hipStream_t)s, S, L, H, B, (const float*)logits, (float)scale, causal, mask, mask_stride_h,
+                                       mask_stride_b, (const float*)bias, bias_stride_h, bias_stride_b, (float*)probs);
+    return softmax_fwd_impl<bf16_t>((hipStream_t)s, S, L, H, B, (const bf16_t*)logits, (float)scale, causal, mask, mask_stride_h,
+                                    mask_stride_b, (const bf16_t*)bias, bias_stride_h, bias_stride_b, (bf16_t*)probs);
+}
+
+int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t cols, const void* dprobs, const void* probs,
+                                 double scale, void* dlogits) {
+    LUX_REQUIRE_INIT();
+    int rc = softmax_check(dtype, S, cols);
+    if (rc != LUXHIP_OK) return rc;
+    if (S * cols == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(dprobs == nullptr || probs == nullptr || dlogits == nullptr,
+                   "attention_softmax_bwd: dprobs, probs and dlogits must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return softmax_bwd_impl<float>((hipStream_t)s, S, cols, (const float*)dprobs, (const float*)probs, (float)scale,
+                                       (float*)dlogits);
+    return softmax_bwd_impl<bf16_t>((hipStream_t)s, S, cols, (const bf16_t*)dprobs, (const bf16_t*)probs, (float)scale,
+                                    (bf16_t*)dlogits);
+}
+
+}  // extern "C"

@@ -37,30 +37,57 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
     return launch_layout<T, false, false>(s, a);
 }
 
-// C_b = op(A_b) op(B_b) for b < batch; a batch stride of 0 shares one matrix among all products
+// C_b = op(A_b) op(B_b) over up to three nested batch dims; a stride of 0 shares one matrix
 template <typename T>
-static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, const T* A,
-                        int64_t lda, int64_t strideA, const T* B, int64_t ldb, int64_t strideB, T* C, int64_t ldc,
-                        int64_t strideC) {
+static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const int64_t* bdim, const T* A,
+                        int64_t lda, const int64_t* sA, const T* B, int64_t ldb, const int64_t* sB, T* C, int64_t ldc,
+                        const int64_t* sC) {
     DenseArgs<T> a;
     const bool a_kmajor = transA != 0, b_kmajor = transB == 0;
     a.A.p = A;
     a.A.sr = a_kmajor ? lda : 1;
     a.A.sk = a_kmajor ? 1 : lda;
     a.A.rows = (int)M;
-    a.A.vec_ok = aligned16(A) && (lda * sizeof(T)) % 16 == 0 && (strideA * sizeof(T)) % 16 == 0;
+    a.A.vec_ok = aligned16(A) && (lda * sizeof(T)) % 16 == 0;
     a.B.p = B;
     a.B.sr = b_kmajor ? ldb : 1;
     a.B.sk = b_kmajor ? 1 : ldb;
     a.B.rows = (int)N;
-    a.B.vec_ok = aligned16(B) && (ldb * sizeof(T)) % 16 == 0 && (strideB * sizeof(T)) % 16 == 0;
+    a.B.vec_ok = aligned16(B) && (ldb * sizeof(T)) % 16 == 0;
+    a.batch = 1;
+    for (int d = 0; d < 3; ++d) {
+        a.bdim[d] = (int)bdim[d];
+        a.batch *= (int)bdim[d];
+        a.bsA[d] = sA[d]; a.bsB[d] = sB[d]; a.bsC[d] = sC[d];
+        a.A.vec_ok = a.A.vec_ok && (sA[d] * sizeof(T)) % 16 == 0;
+        a.B.vec_ok = a.B.vec_ok && (sB[d] * sizeof(T)) % 16 == 0;
+    }
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.C = C; a.ldc = ldc; a.bias = nullptr; a.pre = nullptr; a.act = LUXHIP_ACT_IDENTITY;
-    a.batch = (int)batch; a.bsA = strideA; a.bsB = strideB; a.bsC = strideC;
     if (a_kmajor && b_kmajor) return launch_batched_layout<T, true, true>(s, a);
     if (a_kmajor) return launch_batched_layout<T, true, false>(s, a);
     if (b_kmajor) return launch_batched_layout<T, false, true>(s, a);
     return launch_batched_layout<T, false, false>(s, a);
+}
+
+static int batched_dispatch(hipStream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                            const int64_t* bdim, const void* A, int64_t lda, const int64_t* sA, const void* B, int64_t ldb,
+                            const int64_t* sB, void* C, int64_t ldc, const int64_t* sC) {
+    int64_t batch = 1;
+    for (int d = 0; d < 3; ++d) {
+        LUX_INVALID_IF(bdim[d] < 0 || sA[d] < 0 || sB[d] < 0 || sC[d] < 0, "batched_matmul: negative batch extent or stride");
+        batch *= bdim[d];
+        LUX_UNSUPPORTED_IF(batch >= (1ll << 31), "batched_matmul: batch of 2^31 or more");
+    }
+    if (M == 0 || N == 0 || batch == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(C == nullptr, "batched_matmul: C must not be NULL");
+    LUX_INVALID_IF(K > 0 && (A == nullptr || B == nullptr), "batched_matmul: A and B must not be NULL");
+    LUX_INVALID_IF(lda < (transA ? K : M) || ldb < (transB ? N : K) || ldc < M, "batched_matmul: leading dimension too small");
+    if (dtype == LUXHIP_F32)
+        return batched_impl<float>(s, transA, transB, M, N, K, bdim, (const float*)A, lda, sA, (const float*)B, ldb, sB, (float*)C,
+                                   ldc, sC);
+    return batched_impl<bf16_t>(s, transA, transB, M, N, K, bdim, (const bf16_t*)A, lda, sA, (const bf16_t*)B, ldb, sB,
+                                (bf16_t*)C, ldc, sC);
 }
 
 // out[i] = sum_b in[i + b n]: `sum(tmp; dims=3)` of a stack of matrices, accumulated in fp32 in batch order
@@ -144,18 +171,21 @@ int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, 
     LUX_REQUIRE_INIT();
     int rc = gemm_check(dtype, 0, M, N, K);
     if (rc != LUXHIP_OK) return rc;
-    LUX_INVALID_IF(batch < 0 || strideA < 0 || strideB < 0 || strideC < 0, "batched_matmul: negative batch or stride");
-    LUX_UNSUPPORTED_IF(batch >= (1ll << 31), "batched_matmul: batch of 2^31 or more");
-    if (M == 0 || N == 0 || batch == 0) return LUXHIP_OK;
-    LUX_INVALID_IF(C == nullptr, "batched_matmul: C must not be NULL");
-    LUX_INVALID_IF(K > 0 && (A == nullptr || B == nullptr), "batched_matmul: A and B must not be NULL");
-    LUX_INVALID_IF(lda < (transA ? K : M) || ldb < (transB ? N : K) || ldc < M, "batched_matmul: leading dimension too small");
-    LUX_INVALID_IF(batch > 1 && strideC < ldc * (N - 1) + M, "batched_matmul: the results would overlap");
-    if (dtype == LUXHIP_F32)
-        return batched_impl<float>((hipStream_t)s, transA, transB, M, N, K, batch, (const float*)A, lda, strideA,
-                                   (const float*)B, ldb, strideB, (float*)C, ldc, strideC);
-    return batched_impl<bf16_t>((hipStream_t)s, transA, transB, M, N, K, batch, (const bf16_t*)A, lda, strideA,
-                                (const bf16_t*)B, ldb, strideB, (bf16_t*)C, ldc, strideC);
+    LUX_INVALID_IF(batch > 1 && M > 0 && N > 0 && strideC < ldc * (N - 1) + M, "batched_matmul: the results would overlap");
+    const int64_t bdim[3] = {batch, 1, 1}, sA[3] = {strideA, 0, 0}, sB[3] = {strideB, 0, 0}, sC[3] = {strideC, 0, 0};
+    return batched_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, bdim, A, lda, sA, B, ldb, sB, C, ldc, sC);
+}
+
+int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
+                                  const int64_t* batch_dims, const void* A, int64_t lda, const int64_t* stridesA, const void* B,
+                                  int64_t ldb, const int64_t* stridesB, void* C, int64_t ldc, const int64_t* stridesC) {
+    LUX_REQUIRE_INIT();
+    int rc = gemm_check(dtype, 0, M, N, K);
+    if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF(batch_dims == nullptr || stridesA == nullptr || stridesB == nullptr || stridesC == nullptr,
+                   "batched_matmul_strided: batch extents and strides must not be NULL");
+    return batched_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, batch_dims, A, lda, stridesA, B, ldb, stridesB, C, ldc,
+                            stridesC);
 }
 
 int luxhip_batch_sum(luxhip_stream_t s, int dtype, int64_t n, int64_t batch, const void* in, void* out) {

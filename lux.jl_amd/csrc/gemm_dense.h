@@ -206,9 +206,11 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
     const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
     for (int b = blockIdx.y; b < a.batch; b += gridDim.y) {
         DenseArgs<T> ab = a;
-        ab.A.p = a.A.p + (int64_t)b * a.bsA;
-        ab.B.p = a.B.p + (int64_t)b * a.bsB;
-        ab.C = a.C + (int64_t)b * a.bsC;
+        const int i0 = b % a.bdim[0], r0 = b / a.bdim[0];
+        const int i1 = r0 % a.bdim[1], i2 = r0 / a.bdim[1];
+        ab.A.p = a.A.p + i0 * a.bsA[0] + i1 * a.bsA[1] + i2 * a.bsA[2];
+        ab.B.p = a.B.p + i0 * a.bsB[0] + i1 * a.bsB[1] + i2 * a.bsB[2];
+        ab.C = a.C + i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
         f32x16_v acc[WM][WN];
         if constexpr (ML::DIRECT) {
             DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(ab.A, m0);
@@ -245,9 +247,8 @@ template <typename T, bool AK, bool BKM>
 int launch_batched_layout(hipStream_t s, DenseArgs<T>& a) {
     // 128 x 128 tiles when a product has at least one whole tile of them, 64 x 64 otherwise;
     // the variant without bounds checks when every product is made of whole, aligned tiles
-    const bool strides_ok = (a.bsA * sizeof(T)) % 16 == 0 && (a.bsB * sizeof(T)) % 16 == 0;
     if (a.M >= 128 && a.N >= 128) {
-        if (strides_ok && whole_tiles<T, 128, 128>(a)) return launch_batched_cfg<T, 2, 2, AK, BKM, true>(s, a);
+        if (whole_tiles<T, 128, 128>(a)) return launch_batched_cfg<T, 2, 2, AK, BKM, true>(s, a);
         return launch_batched_cfg<T, 2, 2, AK, BKM, false>(s, a);
     }
     return launch_batched_cfg<T, 1, 1, AK, BKM, false>(s, a);

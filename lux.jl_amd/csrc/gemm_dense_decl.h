@@ -16,9 +16,11 @@ struct DenseArgs {
     T* pre;          // same layout as C, may be null
     int act;
     int tiles_m, tiles_n;
-    // batched products: matrix b of each operand starts b * stride elements after the first (0: shared)
+    // batched products: the batch index runs over up to three nested dims (bdim[0] innermost); along
+    // dim d the matrices of an operand lie stride[d] elements apart (0: one matrix shared by all)
     int batch = 1;
-    int64_t bsA = 0, bsB = 0, bsC = 0;
+    int bdim[3] = {1, 1, 1};
+    int64_t bsA[3] = {0, 0, 0}, bsB[3] = {0, 0, 0}, bsC[3] = {0, 0, 0};
 };
 
 template <typename T, bool A_KMAJOR, bool B_KMAJOR>

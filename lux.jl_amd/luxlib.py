@@ -414,6 +414,117 @@ def rrule_batched_matmul(x, y, lhs_contracting_dim=2, rhs_contracting_dim=1, _ne
     return z, back
 
 
+# ------------------------------------------------------------------------------- attention
+def _i64x3(v):
+    return (C.c_int64 * 3)(*v)
+
+
+def _bmm_strided(tA, tB, M, N, K, bdims, A, lda, sA, B, ldb, sB, Cm, ldc, sC):
+    _lib.call("luxhip_batched_matmul_strided", current_stream(), Cm.code, int(tA), int(tB), M, N, K, _i64x3(bdims),
+              A.ptr, max(lda, 1), _i64x3(sA), B.ptr, max(ldb, 1), _i64x3(sB), Cm.ptr, max(ldc, 1), _i64x3(sC))
+
+
+class _AttnLayout:
+    """Strides (elements) of an attention operand whose embedding dim is the first: token / heads
+    dims are 2 and 3 in either order, everything after is one flattened batch dim."""
+
+    def __init__(self, a: DeviceArray, token_dim: int):
+        self.E, d2, d3 = a.shape[0], a.shape[1], a.shape[2]
+        self.tokens, self.heads = (d2, d3) if token_dim == 2 else (d3, d2)
+        self.st, self.sh = (self.E, self.E * d2) if token_dim == 2 else (self.E * d2, self.E)
+        self.sb = self.E * d2 * d3
+        self.batch = a.size // self.sb if self.sb else 0
+
+
+def scaled_dot_product_attention(q: DeviceArray, k: DeviceArray, v: DeviceArray, head_dim: int = 1, token_dim: int = 3,
+                                 scale=None, mask=None, is_causal=None, bias=None):
+    """`scaled_dot_product_attention(q, k, v; head_dim, token_dim, scale, mask, is_causal, bias)`
+    (api/attention.jl, impl/attention.jl:5-117): returns `(output [Ev, H, L, B...], attention weights
+    [S, L, H, B...])`.  `mask` / `bias`: host arrays or DeviceArrays of shape [S, L, H or 1, B or 1]."""
+    return rrule_scaled_dot_product_attention(q, k, v, head_dim, token_dim, scale, mask, is_causal, bias)[0]
+
+
+def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=None, mask=None, is_causal=None, bias=None):
+    """((output, weights), (Δoutput[, Δweights]) -> (∂q, ∂k, ∂v)): the pullbacks of the two batched
+    products (impl/batched_mul.jl:320-334), of NNlib.softmax and of repeat_inner_gqa, composed as the
+    reference's AD does.  The gradient of `bias` is not computed."""
+    N = q.ndim
+    # impl/attention.jl:16-43
+    assert N >= 4 and k.ndim == N and v.ndim == N, "N must be at least 4"
+    assert 1 <= head_dim <= 3 and 1 <= token_dim <= 3 and head_dim != token_dim, "head_dim and token_dim must differ, in 1:3"
+    assert q.shape[head_dim - 1] == k.shape[head_dim - 1], "`q` and `k` must have the same number of heads."
+    for i in range(3, N):
+        if not (q.shape[i] == k.shape[i] == v.shape[i]):
+            raise DimensionMismatch("All dimensions (except first 3) of q, k, v must be the same.")
+    if head_dim != 1:
+        raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: the embedding dim must be the first one on the device")
+    dt = _same_dtype(q, k, v)
+    lq, lk, lv = _AttnLayout(q, token_dim), _AttnLayout(k, token_dim), _AttnLayout(v, token_dim)
+    assert lv.tokens == lk.tokens, "`v` and `k` must have the same number of tokens."
+    assert lk.heads == lv.heads and lq.heads % max(lk.heads, 1) == 0, "num_heads must be divisible by num_kv_groups"
+    if mask is not None and is_causal is not None:
+        raise AssertionError("`mask` and `is_causal` cannot both be specified")
+    E, Ev, H, G, L, S, B = lq.E, lv.E, lq.heads, lk.heads, lq.tokens, lk.tokens, lq.batch
+    r = H // G if G else 1
+    bshape = tuple(q.shape[3:])
+    scale_inv = 1.0 / (math.sqrt(E) if scale is None else float(scale))      # impl/attention.jl:50-51
+    bdims = (r, G, B)
+
+    def side(arr, what, kind):
+        if arr is None:
+            return None, 0, 0
+        if not isinstance(arr, DeviceArray):
+            arr = DeviceArray.from_numpy(np.asarray(arr, np.uint8 if kind == "mask" else np.float32),
+                                         "u8" if kind == "mask" else dt)
+        shp = tuple(arr.shape) + (1,) * (4 - arr.ndim) if arr.ndim < 4 else (arr.shape[0], arr.shape[1], arr.shape[2],
+                                                                              int(np.prod(arr.shape[3:])))
+        if shp[0] != S or shp[1] != L or shp[2] not in (1, H) or shp[3] not in (1, B):
+            raise DimensionMismatch(f"{what} of shape {arr.shape} does not broadcast to the logits {(S, L, H) + bshape}")
+        return arr, (S * L if shp[2] == H and H > 1 else 0), (S * L * shp[2] if shp[3] == B and B > 1 else 0)
+
+    mask_a, mask_sh, mask_sb = side(mask, "mask", "mask")
+    bias_a, bias_sh, bias_sb = side(bias, "bias", "bias")
+    logits = DeviceArray((S, L, H) + bshape, dt)
+    sC = (S * L, S * L * r, S * L * H)
+    _bmm_strided(True, False, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, (lq.sh, lq.sh * r, lq.sb), logits, S, sC)
+    probs = DeviceArray((S, L, H) + bshape, dt)
+    _lib.call("luxhip_attention_softmax_fwd", current_stream(), probs.code, S, L, H, B, logits.ptr, scale_inv,
+              int(bool(is_causal)), _p(mask_a), mask_sh, mask_sb, _p(bias_a), bias_sh, bias_sb, probs.ptr)
+    out = DeviceArray((Ev, H, L) + bshape, dt)
+    so = (Ev, Ev * r, Ev * H * L)
+    _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so)
+
+    def back(d_out: DeviceArray, d_probs: Optional[DeviceArray] = None):
+        dp = DeviceArray(probs.shape, dt)
+        _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC)
+        if d_probs is not None:
+            raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: a cotangent for the returned weights")
+        dlogits = logits                                              # the logits are no longer needed
+        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L * H * B, dp.ptr, probs.ptr, scale_inv,
+                  dlogits.ptr)
+        dq = DeviceArray(q.shape, dt)
+        _bmm_strided(False, False, E, L, S, bdims, k, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, dq, lq.st,
+                     (lq.sh, lq.sh * r, lq.sb))
+
+        def kv_grad(like, lay, A, lda, sA, Bm):
+            # (rows of `like`) x S = A (rows x L) * Bm' (L x S), one product per head; the heads that share
+            # a key/value group are summed afterwards (pullback of repeat_inner_gqa)
+            full = DeviceArray(((r,) if r > 1 else ()) + tuple(like.shape), dt)
+            _bmm_strided(False, True, lay.E, S, L, bdims, A, lda, sA, Bm, S, sC, full, lay.st,
+                         (like.size if r > 1 else 0, lay.sh, lay.sb))
+            if r == 1:
+                return full
+            red = DeviceArray(like.shape, dt)
+            _lib.call("luxhip_batch_sum", current_stream(), red.code, like.size, r, full.ptr, red.ptr)
+            return red
+
+        dv = kv_grad(v, lv, d_out, Ev * H, so, probs)
+        dk = kv_grad(k, lk, q, lq.st, (lq.sh, lq.sh * r, lq.sb), dlogits)
+        return dq, dk, dv
+
+    return (out, probs), back
+
+
 # ------------------------------------------------------------------------------- batchnorm
 def batchnorm(x: DeviceArray, scale, bias, running_mean, running_var, training, act: str = "identity",
               momentum: float = 0.1, epsilon: Optional[float] = None):
@@ -769,6 +880,7 @@ _RRULES = {
     fast_activation: rrule_fast_activation,
     dropout: rrule_dropout,
     batched_matmul: rrule_batched_matmul,
+    scaled_dot_product_attention: rrule_scaled_dot_product_attention,
     alpha_dropout: rrule_alpha_dropout,
     layernorm: rrule_layernorm,
     fused_conv_bias_activation: rrule_fused_conv_bias_activation,

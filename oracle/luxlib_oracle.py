@@ -22,6 +22,8 @@ tests/test_oracle_*.py):
                                         torch F.batch_norm autograd, finite differences
   * groupnorm (+bwd) .................. torch F.group_norm autograd, finite differences
   * layernorm (+bwd) .................. mean~0/std~1 invariant, torch F.layer_norm autograd
+  * scaled_dot_product_attention ...... torch F.scaled_dot_product_attention (values, causal and
+                                        boolean masks, additive bias, grouped heads) + autograd
   * batched_matmul (+pullback) ........ torch.matmul over a batch + autograd
   * dropout / alpha_dropout ........... closed forms; the Philox4x32-10 noise stream against
                                         the Random123 known-answer vectors and uniformity
@@ -547,6 +549,74 @@ def batched_matmul_pullback(x, y, delta, lhs_contracting_dim=2, rhs_contracting_
         if y.shape[ax] == 1 and delta.shape[ax] != 1:
             dy = dy.sum(axis=ax, keepdims=True)
     return dx.reshape(x0.shape), dy.reshape(y0.shape)
+
+
+# --------------------------------------------------------------------------------------
+# scaled_dot_product_attention  (api/attention.jl, impl/attention.jl:5-134), head_dim = 1
+# --------------------------------------------------------------------------------------
+def _attn_canonical(a, token_dim):
+    """[E, heads, tokens, B] view (B = the flattened trailing dims) of an operand whose token dim is 2 or 3."""
+    a = np.asarray(a)
+    a4 = a.reshape(a.shape[:3] + (-1,))
+    return a4 if token_dim == 3 else np.swapaxes(a4, 1, 2)
+
+
+def scaled_dot_product_attention(q, k, v, token_dim=3, scale=None, mask=None, is_causal=None, bias=None):
+    """Returns (output [Ev, H, L, B...], weights [S, L, H, B...]).
+    logits[s,l,h,b] = (1/scale) Σ_d k[d,h,s,b] q[d,h,l,b] (+ bias), -inf where the mask is false
+    (impl/attention.jl:90-104, 119-128); weights = softmax over s; output[e,h,l,b] =
+    Σ_s v[e,h,s,b] weights[s,l,h,b] (:107-117).  Fewer key/value heads than query heads: each is
+    used by H/G consecutive query heads (repeat_inner_gqa, :1-3, 44-48).  scale defaults to
+    sqrt(E) (:50-51).  is_causal keeps s <= l (make_causal_mask: triu!, :130-134)."""
+    assert not (mask is not None and is_causal is not None), "`mask` and `is_causal` cannot both be specified"
+    tail = np.asarray(q).shape[3:]
+    q4, k4, v4 = (_attn_canonical(a, token_dim) for a in (q, k, v))
+    E, H, L, B = q4.shape
+    G, S = k4.shape[1], k4.shape[2]
+    assert H % G == 0, "num_heads must be divisible by num_kv_groups"
+    k4, v4 = np.repeat(k4, H // G, axis=1), np.repeat(v4, H // G, axis=1)
+    T = q4.dtype.type
+    inv = T(1) / (np.sqrt(T(E)) if scale is None else T(scale))
+    logits = np.einsum("dhsb,dhlb->slhb", k4, q4 * inv)
+    if bias is not None:
+        logits = logits + np.asarray(bias).reshape(np.asarray(bias).shape[:3] + (-1,))
+    if is_causal:
+        mask = np.triu(np.ones((S, L), bool))
+    if mask is not None:
+        m = np.asarray(mask, bool)
+        m = m.reshape(m.shape + (1,) * (4 - m.ndim)) if m.ndim < 4 else m.reshape(m.shape[:3] + (-1,))
+        logits = np.where(m, logits, -np.inf)
+    z = logits - logits.max(axis=0, keepdims=True)
+    w = np.exp(z)
+    w = w / w.sum(axis=0, keepdims=True)
+    out = np.einsum("ehsb,slhb->ehlb", v4, w)
+    return out.reshape(out.shape[:3] + tail), w.reshape(w.shape[:3] + tail)
+
+
+def scaled_dot_product_attention_pullback(q, k, v, d_out, token_dim=3, scale=None, mask=None, is_causal=None, bias=None):
+    """(∂q, ∂k, ∂v) for a cotangent of the output only: the chain of the batched_matmul rrules
+    (impl/batched_mul.jl:320-334), the softmax rule dS = W ∘ (dW - Σ_s dW ∘ W), the scale, and the
+    sum over the query heads that share a key/value head."""
+    q0, k0, v0 = np.asarray(q), np.asarray(k), np.asarray(v)
+    q4, k4, v4 = (_attn_canonical(a, token_dim) for a in (q0, k0, v0))
+    E, H, L, B = q4.shape
+    G, S = k4.shape[1], k4.shape[2]
+    r = H // G
+    kr, vr = np.repeat(k4, r, axis=1), np.repeat(v4, r, axis=1)
+    T = q4.dtype.type
+    inv = T(1) / (np.sqrt(T(E)) if scale is None else T(scale))
+    _, w = scaled_dot_product_attention(q, k, v, token_dim, scale, mask, is_causal, bias)
+    w = w.reshape(w.shape[:3] + (-1,))
+    do = np.asarray(d_out).reshape(np.asarray(d_out).shape[:3] + (-1,))       # [Ev, H, L, B]
+    dw = np.einsum("ehsb,ehlb->slhb", vr, do)
+    dvr = np.einsum("ehlb,slhb->ehsb", do, w)
+    ds = w * (dw - (dw * w).sum(axis=0, keepdims=True)) * inv
+    dq4 = np.einsum("dhsb,slhb->dhlb", kr, ds)
+    dkr = np.einsum("dhlb,slhb->dhsb", q4, ds)
+    dk4 = dkr.reshape(E, G, r, S, B).sum(axis=2)
+    dv4 = dvr.reshape(v4.shape[0], G, r, S, B).sum(axis=2)
+    back = (lambda a, like: (a if token_dim == 3 else np.swapaxes(a, 1, 2)).reshape(like.shape))
+    return back(dq4, q0), back(dk4, k0), back(dv4, v0)
 
 
 # --------------------------------------------------------------------------------------

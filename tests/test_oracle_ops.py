@@ -504,3 +504,56 @@ def test_batched_matmul_errors():
         O.batched_matmul(np.ones((4, 5, 3)), np.ones((4, 6, 3)))
     with pytest.raises(O.ArgumentError):
         O.batched_matmul(np.ones((4, 5)), np.ones((5, 6)))
+
+
+# ----------------------------------------------------------------------------- attention
+@pytest.mark.parametrize("E,Ev,H,G,L,S,B,token_dim,kind", [
+    (8, 8, 4, 4, 5, 5, 2, 3, "plain"), (8, 6, 4, 2, 5, 7, 2, 3, "plain"), (4, 4, 2, 2, 6, 6, 3, 3, "causal"),
+    (4, 4, 2, 1, 6, 6, 1, 2, "causal"), (8, 8, 2, 2, 4, 6, 2, 3, "mask"), (8, 8, 2, 2, 4, 6, 2, 2, "bias"),
+    (8, 8, 3, 3, 4, 6, 2, 3, "mask+bias")])
+def test_attention_vs_torch(E, Ev, H, G, L, S, B, token_dim, kind):
+    # lib/LuxLib/test/common_ops/attention_tests.jl compares with NNlib.dot_product_attention; here the
+    # torch library routine on [B, H, L, E] tensors
+    shape = (lambda e, h, t: (e, h, t, B) if token_dim == 3 else (e, t, h, B))
+    q, k, v = RNG.normal(size=shape(E, H, L)), RNG.normal(size=shape(E, G, S)), RNG.normal(size=shape(Ev, G, S))
+    mask = (RNG.uniform(size=(S, L, 1, B)) > 0.3) if "mask" in kind else None
+    if mask is not None:
+        mask[0] = True                                              # no fully masked query
+    bias = RNG.normal(size=(S, L, H, 1)) if "bias" in kind else None
+    causal = True if kind == "causal" else None
+    out, w = O.scaled_dot_product_attention(q, k, v, token_dim, None, mask, causal, bias)
+    canon = lambda a: torch.tensor(np.transpose(a if token_dim == 3 else np.swapaxes(a, 1, 2), (3, 1, 2, 0)).copy(),
+                                   requires_grad=True)           # [B, H, T, E]
+    tq, tk, tv = canon(q), canon(k), canon(v)
+    tkr, tvr = tk.repeat_interleave(H // G, dim=1), tv.repeat_interleave(H // G, dim=1)
+    am = None
+    if bias is not None or mask is not None:
+        am = torch.zeros(B, H, L, S, dtype=torch.float64)
+        if bias is not None:
+            am = am + torch.tensor(np.transpose(np.broadcast_to(bias, (S, L, H, B)), (3, 2, 1, 0)).copy())
+        if mask is not None:
+            am = am.masked_fill(~torch.tensor(np.transpose(np.broadcast_to(mask, (S, L, H, B)), (3, 2, 1, 0)).copy()), -np.inf)
+    if causal:
+        # the reference keeps key s for query l where s <= l, for any S and L (triu! of an S x L matrix)
+        am = torch.zeros(L, S, dtype=torch.float64).masked_fill(~torch.tensor(np.triu(np.ones((S, L), bool)).T.copy()), -np.inf)
+    to = F.scaled_dot_product_attention(tq, tkr, tvr, attn_mask=am)
+    assert out.shape == (Ev, H, L, B) and w.shape == (S, L, H, B)
+    np.testing.assert_allclose(out, np.transpose(to.detach().numpy(), (3, 1, 2, 0)), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(w.sum(axis=0), 1.0, rtol=1e-12)
+    d_out = RNG.normal(size=out.shape)
+    to.backward(torch.tensor(np.transpose(d_out, (3, 1, 2, 0)).copy()))
+    dq, dk, dv = O.scaled_dot_product_attention_pullback(q, k, v, d_out, token_dim, None, mask, causal, bias)
+    uncanon = lambda t: (lambda a: a if token_dim == 3 else np.swapaxes(a, 1, 2))(np.transpose(t.grad.numpy(), (3, 1, 2, 0)))
+    np.testing.assert_allclose(dq, uncanon(tq), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(dk, uncanon(tk), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(dv, uncanon(tv), rtol=1e-9, atol=1e-11)
+
+
+def test_attention_scale_and_trailing_batch_dims():
+    q, k, v = RNG.normal(size=(4, 2, 3, 2, 2)), RNG.normal(size=(4, 2, 5, 2, 2)), RNG.normal(size=(6, 2, 5, 2, 2))
+    out, w = O.scaled_dot_product_attention(q, k, v, scale=2.0)
+    assert out.shape == (6, 2, 3, 2, 2) and w.shape == (5, 3, 2, 2, 2)
+    logits = np.einsum("dhsab,dhlab->slhab", k, q) / 2.0
+    e = np.exp(logits)
+    np.testing.assert_allclose(w, e / e.sum(axis=0), rtol=1e-12)
+    np.testing.assert_allclose(out, np.einsum("ehsab,slhab->ehlab", v, w), rtol=1e-12)
