@@ -335,7 +335,79 @@ class C5Conv(_ApiWorkload):
         return {f"conv_fprop_kernel<{t}>": f, f"conv_dgrad_kernel<{t}>": f, f"conv_wgrad_kernel<{t}>": f}
 
 
-WORKLOADS = {"C1": C1Dense, "C2": C2BatchnormBiasAct, "C3": lambda: C3Groupnorm("f32"), "C3bf16": lambda: C3Groupnorm("bf16"),
+class InstanceNorm(_ApiWorkload):
+    """instancenorm (training, running statistics updated) + relu, x 64x64x256x16 fp32: one slice per channel and sample."""
+    name, bound, dtype = "IN", "hbm", "f32"
+    shape = (64, 64, 256, 16)
+    description = "instancenorm(train, running stats, relu) fwd+bwd, x 64x64x256x16 f32"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1010)
+        self.x = self.d(rng.standard_normal(size=self.shape, dtype=np.float32))
+        self.g = self.d(rng.uniform(0.8, 1.2, 256).astype(np.float32))
+        self.b = self.d((0.05 * rng.standard_normal(256)).astype(np.float32))
+        self.rm, self.rv = self.d(np.zeros(256, np.float32)), self.d(np.ones(256, np.float32))
+        self.delta = self.d(rng.standard_normal(size=self.shape, dtype=np.float32))
+
+    def step(self):
+        _, back = self.lux.pullback(self.lux.instancenorm, self.x, self.g, self.b, self.rm, self.rv, True, "relu", 0.1, 1e-5)
+        back(self.delta)
+
+    def work_per_step(self):
+        return 5 * 4 * int(np.prod(self.shape))
+
+    def kernel_work(self):
+        E = 4 * int(np.prod(self.shape))
+        return {"gn_fwd_kernel": 2 * E, "gn_bwd_kernel": 3 * E}
+
+
+class Dropout(_ApiWorkload):
+    """dropout(p = 0.5) with a full-size mask, forward (x in, y and mask out) + pullback (delta, mask in, dx out)."""
+    name, bound, dtype = "DROPOUT", "hbm", "f32"
+    shape = (32, 32, 64, 128)
+    description = "dropout(p=0.5, dims=:) fwd+bwd, x 32x32x64x128 f32"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1011)
+        self.x = self.d(rng.standard_normal(size=self.shape, dtype=np.float32))
+        self.delta = self.d(rng.standard_normal(size=self.shape, dtype=np.float32))
+        self.rng = lux.PhiloxRNG(1, 0)
+
+    def step(self):
+        (_, _, self.rng), back = self.lux.pullback(self.lux.dropout, self.rng, self.x, 0.5, True, 2.0)
+        back(self.delta)
+
+    def work_per_step(self):
+        return 6 * 4 * int(np.prod(self.shape))
+
+    def kernel_work(self):
+        E = 4 * int(np.prod(self.shape))
+        return {"dropout_fwd_kernel": 3 * E, "dropout_mul_kernel": 3 * E}
+
+
+class Attention(_ApiWorkload):
+    """scaled_dot_product_attention, causal, 32 heads of width 128 over 2048 positions, batch 4, bf16, fwd+bwd."""
+    name, bound, dtype = "SDPA", "mfma", "bf16"
+    E, H, L, B = 128, 32, 2048, 4
+    description = "scaled_dot_product_attention(causal) fwd+bwd, q/k/v 128x32x2048x4 bf16"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1012)
+        shp = (self.E, self.H, self.L, self.B)
+        self.q, self.k, self.v, self.do = (self.d(rng.standard_normal(size=shp, dtype=np.float32)) for _ in range(4))
+
+    def step(self):
+        _, back = self.lux.pullback(self.lux.scaled_dot_product_attention, self.q, self.k, self.v, 1, 3, None, None, True, None)
+        back(self.do)
+
+    def work_per_step(self):
+        return 6 * 2.0 * self.E * self.L * self.L * self.H * self.B     # six batched products (all positions computed)
+
+    def kernel_work(self):
+        return {"batched_gemm_kernel<bf16>": 2.0 * self.E * self.L * self.L * self.H * self.B}
+
+
+WORKLOADS = {"IN": InstanceNorm, "DROPOUT": Dropout, "SDPA": Attention, "C1": C1Dense, "C2": C2BatchnormBiasAct, "C3": lambda: C3Groupnorm("f32"), "C3bf16": lambda: C3Groupnorm("bf16"),
              "C4": C4TransformerMLP, "C5": lambda: C5Conv("f32"), "C5bf16": lambda: C5Conv("bf16")}
 
 
@@ -391,7 +463,7 @@ def main():
         name, _, val = opt.partition("=")
         lux.set_option(name, int(val))
     wl = WORKLOADS[args.workload]()
-    heavy = args.workload in ("C4", "C5", "C5bf16")
+    heavy = args.workload in ("C4", "C5", "C5bf16", "SDPA")
     if args.steps is None:
         args.steps = 20 if heavy else 200
     if args.warmup is None:

@@ -3,8 +3,9 @@
 // products around it run on the batched MFMA GEMM.
 //
 // logits, probs: (S, L, H, B) column-major, S = key positions (softmax axis), L = query positions.
-// One wavefront owns one column of S values; columns of up to 64 * 16 values stay in registers
-// between the passes, longer ones are read again (they sit in the cache by then).
+// One wavefront owns one column of S values and keeps it in registers between the passes (16-byte
+// accesses when S is a multiple of the vector width, up to 64 * 8 vectors; otherwise scalar accesses,
+// up to 64 * 16 values); longer columns are read again per pass (they sit in the cache by then).
 #include <algorithm>
 
 #include "common.h"
@@ -129,6 +130,115 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_kernel(const
     }
 }
 
+// The same with 16-byte accesses: lane j owns the vectors j, j + 64, ... of the column
+// (S a multiple of the vector width, S <= 64 VEC NVV, every pointer 16-byte aligned).
+template <typename T, int NVV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_vec_kernel(
+    const T* __restrict__ logits, T* __restrict__ probs, int S, int L, int H, int64_t cols, float scale, int causal,
+    const uint8_t* __restrict__ mask, int64_t mask_sh, int64_t mask_sb, const T* __restrict__ bias, int64_t bias_sh,
+    int64_t bias_sb) {
+    constexpr int VEC = Vec<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
+    if (col >= cols) return;
+    const int l = (int)(col % L);
+    const int64_t hb = col / L;
+    const int h = (int)(hb % H);
+    const int64_t b = hb / H;
+    const T* x = logits + col * S;
+    const T* bp = bias ? bias + (int64_t)l * S + h * bias_sh + b * bias_sb : nullptr;
+    const uint8_t* mp = mask ? mask + (int64_t)l * S + h * mask_sh + b * mask_sb : nullptr;
+    const int limit = causal ? l : S - 1;
+    float z[NVV][VEC];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NVV; ++i) {
+        const int s0 = (lane + 64 * i) * VEC;
+        if (s0 < S && s0 <= limit) {            // vectors past the causal limit are never read
+            Vec<T>::load(x + s0, z[i]);
+            float bv[VEC];
+            if (bp) Vec<T>::load(bp + s0, bv);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float v = z[i][k] * scale;
+                if (bp) v += bv[k];
+                const bool keep = s0 + k <= limit && (mp == nullptr || mp[s0 + k] != 0);
+                z[i][k] = keep ? v : -INFINITY;
+                m = fmaxf(m, z[i][k]);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) z[i][k] = -INFINITY;
+        }
+    }
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NVV; ++i)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            z[i][k] = __expf(z[i][k] - m);
+            sum += z[i][k];
+        }
+    const float inv = 1.f / wave_add(sum);
+    T* y = probs + col * S;
+#pragma unroll
+    for (int i = 0; i < NVV; ++i) {
+        const int s0 = (lane + 64 * i) * VEC;
+        if (s0 < S) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) z[i][k] *= inv;
+            Vec<T>::store(y + s0, z[i]);
+        }
+    }
+}
+
+template <typename T, int NVV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(const T* __restrict__ dprobs,
+                                                                               const T* __restrict__ probs,
+                                                                               T* __restrict__ dlogits, int S, int64_t cols,
+                                                                               float scale) {
+    constexpr int VEC = Vec<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
+    if (col >= cols) return;
+    const T* dy = dprobs + col * S;
+    const T* y = probs + col * S;
+    float yv[NVV][VEC], dv[NVV][VEC];
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < NVV; ++i) {
+        const int s0 = (lane + 64 * i) * VEC;
+        if (s0 < S) {
+            Vec<T>::load(y + s0, yv[i]);
+            Vec<T>::load(dy + s0, dv[i]);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) dot += yv[i][k] * dv[i][k];
+        }
+    }
+    dot = wave_add(dot);
+    T* dx = dlogits + col * S;
+#pragma unroll
+    for (int i = 0; i < NVV; ++i) {
+        const int s0 = (lane + 64 * i) * VEC;
+        if (s0 < S) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) yv[i][k] = scale * yv[i][k] * (dv[i][k] - dot);
+            Vec<T>::store(dx + s0, yv[i]);
+        }
+    }
+}
+
+// 16-byte vectors per lane for a column of S values, 0 when the vector kernels do not apply
+template <typename T>
+static inline int lane_vectors(int64_t S, bool aligned) {
+    constexpr int V = Vec<T>::N;
+    if (!aligned || S % V != 0) return 0;
+    for (int nvv : {1, 2, 4, 8})
+        if (S <= (int64_t)64 * V * nvv) return nvv;
+    return 0;
+}
+
 static inline int cached_vectors(int64_t S) {
     for (int nv : {1, 2, 4, 8, 16})
         if (S <= 64 * nv) return nv;
@@ -142,6 +252,19 @@ static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int6
     const int64_t cols = L * H * B;
     const unsigned grid = (unsigned)ceil_div(cols, kAttnWaves);
     ProfScope ps("attn_softmax_fwd_kernel", s);
+    const bool aligned = aligned16(logits) && aligned16(probs) && (bias == nullptr || aligned16(bias)) &&
+                         (mask == nullptr || (reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
+#define LUX_SOFTMAX_FWD_VEC(NVV)                                                                                                \
+    attn_softmax_fwd_vec_kernel<T, NVV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
+                                                                         mask, mask_sh, mask_sb, bias, bias_sh, bias_sb)
+    switch (lane_vectors<T>(S, aligned)) {
+        case 1: LUX_SOFTMAX_FWD_VEC(1); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        case 2: LUX_SOFTMAX_FWD_VEC(2); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        case 4: LUX_SOFTMAX_FWD_VEC(4); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        case 8: LUX_SOFTMAX_FWD_VEC(8); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        default: break;
+    }
+#undef LUX_SOFTMAX_FWD_VEC
 #define LUX_SOFTMAX_FWD(NV)                                                                                                   \
     attn_softmax_fwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
                                                                     mask, mask_sh, mask_sb, bias, bias_sh, bias_sb)
@@ -162,6 +285,16 @@ template <typename T>
 static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t cols, const T* dprobs, const T* probs, float scale, T* dlogits) {
     const unsigned grid = (unsigned)ceil_div(cols, kAttnWaves);
     ProfScope ps("attn_softmax_bwd_kernel", s);
+#define LUX_SOFTMAX_BWD_VEC(NVV) \
+    attn_softmax_bwd_vec_kernel<T, NVV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, cols, scale)
+    switch (lane_vectors<T>(S, aligned16(dprobs) && aligned16(probs) && aligned16(dlogits))) {
+        case 1: LUX_SOFTMAX_BWD_VEC(1); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        case 2: LUX_SOFTMAX_BWD_VEC(2); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        case 4: LUX_SOFTMAX_BWD_VEC(4); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        case 8: LUX_SOFTMAX_BWD_VEC(8); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
+        default: break;
+    }
+#undef LUX_SOFTMAX_BWD_VEC
 #define LUX_SOFTMAX_BWD(NV) attn_softmax_bwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, cols, scale)
     switch (cached_vectors(S)) {
         case 1: LUX_SOFTMAX_BWD(1); break;

@@ -195,33 +195,73 @@ int launch_layout(hipStream_t s, DenseArgs<T>& a) {
     return launch_cfg<T, 1, 1, AK, BKM>(s, a);
 }
 
-// Batched products: grid.x walks the tiles of one product, grid.y the batch.
+// Batched products, persistent like dense_gemm_kernel: the tiles of all products form one
+// sequence (the tiles of one product are neighbours, so its operands stay in the L2 caches);
+// workgroup w handles tiles w, w + gridDim.x, ...
+template <typename T>
+struct BatchTile {
+    Operand<T> A, B;
+    T* C;
+    int m0, n0;
+};
+template <typename T, int TILE_M, int TILE_N>
+__device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t, int tiles) {
+    const int b = t / tiles;
+    int tm, tn;
+    tile_coords(t - b * tiles, a.tiles_m, a.tiles_n, tm, tn);
+    const int i0 = b % a.bdim[0], r0 = b / a.bdim[0];
+    const int i1 = r0 % a.bdim[1], i2 = r0 / a.bdim[1];
+    BatchTile<T> bt;
+    bt.A = a.A;
+    bt.B = a.B;
+    bt.A.p = a.A.p + i0 * a.bsA[0] + i1 * a.bsA[1] + i2 * a.bsA[2];
+    bt.B.p = a.B.p + i0 * a.bsB[0] + i1 * a.bsB[1] + i2 * a.bsB[2];
+    bt.C = a.C + i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
+    bt.m0 = tm * TILE_M;
+    bt.n0 = tn * TILE_N;
+    return bt;
+}
+
 template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
 __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<T> a) {
     using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
-    int tm, tn;
-    tile_coords(blockIdx.x, a.tiles_m, a.tiles_n, tm, tn);
-    const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
-    for (int b = blockIdx.y; b < a.batch; b += gridDim.y) {
-        DenseArgs<T> ab = a;
-        const int i0 = b % a.bdim[0], r0 = b / a.bdim[0];
-        const int i1 = r0 % a.bdim[1], i2 = r0 / a.bdim[1];
-        ab.A.p = a.A.p + i0 * a.bsA[0] + i1 * a.bsA[1] + i2 * a.bsA[2];
-        ab.B.p = a.B.p + i0 * a.bsB[0] + i1 * a.bsB[1] + i2 * a.bsB[2];
-        ab.C = a.C + i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
-        f32x16_v acc[WM][WN];
-        if constexpr (ML::DIRECT) {
-            DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(ab.A, m0);
-            DirectLoader<B_KMAJOR, ML::TILE_N, ML::THREADS> lb(ab.B, n0);
-            ML::pipeline_fill(la, lb, a.K, lds);
+    const int tiles = a.tiles_m * a.tiles_n;
+    const int total = tiles * a.batch;
+    f32x16_v acc[WM][WN];
+    if constexpr (ML::DIRECT) {
+        int t = blockIdx.x;
+        BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
+        DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(cur.A, cur.m0);
+        DirectLoader<B_KMAJOR, ML::TILE_N, ML::THREADS> lb(cur.B, cur.n0);
+        ML::pipeline_fill(la, lb, a.K, lds);
+        for (;;) {
             ML::pipeline_loop(la, lb, a.K, lds, acc);
-        } else {
-            ML::run(ab.A, ab.B, a.K, m0, n0, lds, acc);
+            const int tnext = t + gridDim.x;
+            DenseArgs<T> out = a;
+            out.C = cur.C;
+            const int m0 = cur.m0, n0 = cur.n0;
+            if (tnext < total) {
+                cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, tnext, tiles);
+                la.move_to(cur.A, cur.m0);
+                lb.move_to(cur.B, cur.n0);
+                ML::pipeline_drain();
+                ML::pipeline_fill(la, lb, a.K, lds);
+            }
+            dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
+            if (tnext >= total) break;
+            t = tnext;
         }
-        dense_epilogue<ML, T, WM, WN, FULL>(acc, ab, m0, n0);
-        __syncthreads();   // every wave is done with the LDS stages before the next product refills them
+    } else {
+        for (int t = blockIdx.x; t < total; t += gridDim.x) {
+            const BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
+            ML::run(cur.A, cur.B, a.K, cur.m0, cur.n0, lds, acc);
+            DenseArgs<T> out = a;
+            out.C = cur.C;
+            dense_epilogue<ML, T, WM, WN, FULL>(acc, out, cur.m0, cur.n0);
+            __syncthreads();   // every wave is done with the LDS stages before the next tile refills them
+        }
     }
 }
 
@@ -230,15 +270,17 @@ int launch_batched_cfg(hipStream_t s, DenseArgs<T>& a) {
     using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL, 2, 0, 2>;
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
+    const int64_t total = (int64_t)a.tiles_m * a.tiles_n * a.batch;
+    LUX_UNSUPPORTED_IF(total >= (1ll << 31), "batched_matmul: too many tiles");
     auto kernel = batched_gemm_kernel<T, WM, WN, AK, BKM, FULL, 2, 2>;
-    static bool prepared = false;
-    if (!prepared) {
+    static int resident = 0;
+    if (resident == 0) {
         LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)ML::LDS_BYTES));
-        prepared = true;
+        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
     }
     ProfScope ps(sizeof(T) == 2 ? "batched_gemm_kernel<bf16>" : "batched_gemm_kernel<f32>", s);
-    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)std::min(a.batch, 65535)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
+    kernel<<<dim3((unsigned)std::min<int64_t>(total, resident)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

@@ -520,19 +520,26 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
 // instancenorm's running statistics: the statistics of the (channel, sample) slices averaged over
 // the batch, the variance with the n / (n - 1) correction of a slice of n = I values.
 template <typename T>
-__global__ void in_running_stats_kernel(const float* __restrict__ mean, const float* __restrict__ invstd, int C, int N,
-                                        float eps, float momentum, float corrected, const T* __restrict__ rmean,
-                                        const T* __restrict__ rvar, T* __restrict__ rmean_out, T* __restrict__ rvar_out) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(256) void in_running_stats_kernel(const float* __restrict__ mean, const float* __restrict__ invstd,
+                                                               int C, int N, float eps, float momentum, float corrected,
+                                                               const T* __restrict__ rmean, const T* __restrict__ rvar,
+                                                               T* __restrict__ rmean_out, T* __restrict__ rvar_out) {
+    // one wavefront per channel, the lanes stride over the samples
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (c >= C) return;
+    const int lane = threadIdx.x & 63;
     float sm = 0.f, sv = 0.f;
-    for (int n = 0; n < N; ++n) {
+    for (int n = lane; n < N; n += 64) {
         const float is = invstd[c + (size_t)C * n];
         sm += mean[c + (size_t)C * n];
         sv += 1.f / (is * is) - eps;
     }
-    st<T>(rmean_out + c, (1.f - momentum) * ld<T>(rmean + c) + momentum * (sm / (float)N));
-    st<T>(rvar_out + c, (1.f - momentum) * ld<T>(rvar + c) + corrected * (sv / (float)N));
+    sm = wave_sum(sm);
+    sv = wave_sum(sv);
+    if (lane == 0) {
+        st<T>(rmean_out + c, (1.f - momentum) * ld<T>(rmean + c) + momentum * (sm / (float)N));
+        st<T>(rvar_out + c, (1.f - momentum) * ld<T>(rvar + c) + corrected * (sv / (float)N));
+    }
 }
 
 template <typename T>
@@ -541,7 +548,7 @@ static int in_running_stats_impl(hipStream_t s, int64_t I, int64_t C, int64_t N,
     const float m = (float)I;
     const float corrected = momentum * m / (m - 1.f);            // update_normalization_statistics
     ProfScope ps("in_running_stats_kernel", s);
-    in_running_stats_kernel<T><<<dim3((unsigned)ceil_div(C, 256)), dim3(256), 0, s>>>(mean, invstd, (int)C, (int)N, eps, momentum,
+    in_running_stats_kernel<T><<<dim3((unsigned)ceil_div(C, 4)), dim3(256), 0, s>>>(mean, invstd, (int)C, (int)N, eps, momentum,
                                                                                       corrected, rmean, rvar, rmean_out, rvar_out);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
