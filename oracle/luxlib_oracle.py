@@ -33,6 +33,8 @@ tests/test_oracle_*.py):
   * conv / dgrad / wgrad .............. reference known answers (impulse response,
                                         asymmetric-pad counts), brute-force 7-loop direct
                                         convolution, torch conv2d with flipped kernel
+  * PARITY UNPINNED: the bit pattern of the reference's dropout masks (drawn from Julia's rng,
+    which cannot run here); `rand_uniform` is a Philox stream of the same distribution.
   * NNlib's `tanh_fast`/`sigmoid_fast` rational approximations, exact `gelu` constants and
     Julia's summation order are NOT reproducible without Julia: parity for those is pinned
     to tolerance only (few-ulp effects), not bit-for-bit.
