@@ -21,6 +21,7 @@ using NNlib: NNlib, DenseConvDims
 using MLDataDevices: MLDataDevices, AbstractGPUDevice
 using Static: True, False, StaticBool, known
 using LinearAlgebra: Adjoint, Transpose
+using Random: Random
 
 const CRC = ChainRulesCore
 const libluxhip = get(ENV, "LIBLUXHIP", joinpath(@__DIR__, "..", "libluxhip.so"))
@@ -303,5 +304,106 @@ function Impl.∇conv_filter(x::HIPArray{T,4}, dy::HIPArray{T,4}, cdims::DenseCo
         stream(), dtype_code(T), d, optr(x), optr(dy), optr(dw))) || return NNlib.∇conv_filter(x, dy, cdims)
     return dw
 end
+
+# ---------------------------------------------------------------------------------------------
+# batched_matmul: Impl.batched_matmul!(z, opmode, x, y)  (impl/batched_mul.jl:204-212) and the
+# products of the rrule (:320-334), which arrive as NNlib.BatchedAdjoint wrappers
+# ---------------------------------------------------------------------------------------------
+bunwrap(a::HIPArray{T,3}) where {T} = (a, Cint(0))
+bunwrap(a::Union{NNlib.BatchedAdjoint{<:Any,<:HIPArray},NNlib.BatchedTranspose{<:Any,<:HIPArray}}) = (parent(a), Cint(1))
+bstride(a::HIPArray{T,3}) where {T} = size(a, 3) == 1 ? 0 : size(a, 1) * size(a, 2)      # extent 1 = shared by all products
+
+function Impl.batched_matmul!(z::HIPArray{T,3}, ::HIPOp, x::AbstractArray{T,3}, y::AbstractArray{T,3}) where {T<:HIPFloat}
+    (xp, tx), (yp, ty) = bunwrap(x), bunwrap(y)
+    M, N, B = size(z)
+    K = size(x, 2)
+    check(ccall((:luxhip_batched_matmul, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Int64, Int64, Ptr{Cvoid}, Int64, Int64,
+         Ptr{Cvoid}, Int64, Int64),
+        stream(), dtype_code(T), tx, ty, M, N, K, B, optr(xp), max(1, size(xp, 1)), bstride(xp), optr(yp), max(1, size(yp, 1)),
+        bstride(yp), optr(z), max(1, M), M * N)) || NNlib.batched_mul!(z, x, y)
+    return nothing
+end
+
+# `sum(tmp; dims=3)` of the rrule when an operand was shared among the products
+function batch_sum(tmp::HIPArray{T,3}) where {T<:HIPFloat}
+    out = similar(tmp, T, (size(tmp, 1), size(tmp, 2), 1))
+    check(ccall((:luxhip_batch_sum, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), size(tmp, 1) * size(tmp, 2), size(tmp, 3), optr(tmp), optr(out))) || return sum(tmp; dims=3)
+    return out
+end
+
+# ---------------------------------------------------------------------------------------------
+# dropout: the device generator stands in for `rand!(rng, y)`  (impl/dropout.jl:171-228)
+# ---------------------------------------------------------------------------------------------
+mutable struct PhiloxRNG <: Random.AbstractRNG      # what LuxCore.replicate copies
+    seed::UInt64
+    offset::UInt64
+end
+Base.copy(r::PhiloxRNG) = PhiloxRNG(r.seed, r.offset)
+
+function Random.rand!(rng::PhiloxRNG, y::HIPArray{T}) where {T<:HIPFloat}
+    check(ccall((:luxhip_rand_uniform, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, UInt64, UInt64, Ptr{Cvoid}),
+        stream(), dtype_code(T), length(y), rng.seed, rng.offset, optr(y))) || error(last_error())
+    rng.offset += cld(length(y), 4)
+    return y
+end
+
+function Impl.generate_dropout_mask!(y::HIPArray{T}, ::HIPOp, p, invp) where {T<:HIPFloat}
+    check(ccall((:luxhip_dropout_mask, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, Cdouble, Cdouble, Ptr{Cvoid}),
+        stream(), dtype_code(T), length(y), Float64(p), Float64(invp), optr(y))) || (y .= (y .> T(p)) .* T(invp))
+    return nothing
+end
+
+function Impl.dropout_dot_mul(x::HIPArray{T,N}, mask::HIPArray{T,N}) where {T<:HIPFloat,N}
+    y = similar(x)
+    xs, ms = Int64[size(x)...], Int64[size(mask)...]
+    check(ccall((:luxhip_dropout_mul, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), N, xs, ms, optr(x), optr(mask), optr(y))) || return x .* mask
+    return y
+end
+
+# full-size masks: noise, mask and product in one pass (impl/dropout.jl:3-6 with dims = :)
+function Impl.dropout(rng::PhiloxRNG, x::HIPArray{T}, p::P, ::True, invp::P, ::Colon) where {T<:HIPFloat,P}
+    rngₙ = copy(rng)
+    y, mask = similar(x), similar(x)
+    check(ccall((:luxhip_dropout_fwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Int64, UInt64, UInt64, Cdouble, Cdouble, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), length(x), rngₙ.seed, rngₙ.offset, Float64(p), Float64(invp), optr(x), optr(y), optr(mask))) ||
+        error(last_error())
+    rngₙ.offset += cld(length(x), 4)
+    return y, mask, rngₙ
+end
+# its pullback is dropout_dot_mul(Δ, mask), as in the reference's rrule (impl/dropout.jl:222-228)
+
+function Impl.alpha_dropout(::HIPOp, noise::HIPArray{T}, p, x::HIPArray{T}, α, A, B) where {T<:HIPFloat}
+    y = similar(x)
+    check(ccall((:luxhip_alpha_dropout_fwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Int64, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Cdouble, Cdouble, Cdouble, Ptr{Cvoid}),
+        stream(), dtype_code(T), length(x), optr(noise), Float64(p), optr(x), Float64(α), Float64(A), Float64(B), optr(y))) ||
+        return @. muladd(ifelse(noise > p, x, T(α)), T(A), T(B))
+    return y
+end
+function CRC.rrule(::typeof(Impl.alpha_dropout), op::HIPOp, noise::HIPArray{T}, p, x::HIPArray{T}, α, A, B) where {T<:HIPFloat}
+    y = Impl.alpha_dropout(op, noise, p, x, α, A, B)
+    function ∇alpha_dropout_hip(Δ′)
+        Δ = CRC.unthunk(Δ′)
+        ∂x = similar(x)
+        check(ccall((:luxhip_alpha_dropout_bwd, libluxhip), Cint,
+            (Ptr{Cvoid}, Cint, Int64, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}),
+            stream(), dtype_code(T), length(x), optr(noise), Float64(p), optr(Δ), Float64(A), optr(∂x))) ||
+            (∂x = Δ .* (noise .> p) .* T(A))
+        return (ntuple(Returns(NoTangent()), 4)..., ∂x, ntuple(Returns(NoTangent()), 3)...)
+    end
+    return y, ∇alpha_dropout_hip
+end
+
+# instancenorm (impl/normalization.jl:191-208) is Impl.groupnorm with G = C, followed in training
+# with running statistics by luxhip_instancenorm_running_stats on the saved (C, N) statistics;
+# scaled_dot_product_attention (impl/attention.jl:70-117) is two luxhip_batched_matmul_strided
+# calls around luxhip_attention_softmax_fwd, its rrule four products around
+# luxhip_attention_softmax_bwd.  (lux.jl_amd/luxlib.py: rrule_instancenorm,
+# rrule_scaled_dot_product_attention spell out the strides.)
 
 end # module
