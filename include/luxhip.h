@@ -86,6 +86,8 @@ int luxhip_profile_enable(int on);
  *   "bn_spin_limit" polls after which a resident batchnorm workgroup stops waiting for its peer
  *                   workgroups and recomputes their share itself (default 2^22; 0 = never wait)
  *   "gemm_tile"     0 automatic (default), 82 | 42 | 22 | 11 force a GEMM tile shape
+ *   "gemm_pretranspose" 1 (default) / 0: large bf16 matmul operands that are contiguous along m or n
+ *                   are first copied into the k-contiguous layout the fastest kernel reads
  *   "conv_tile"     0 automatic (default); bf16 whole-tap convolution kernels: 82 = 256x256 tile on
  *                   8 waves, 84 / 83 = 512x128 on 8 waves with 4 / 3 LDS stages, 42 = 256x128 on 4 waves */
 int luxhip_set_option(const char* name, int64_t value);

@@ -18,6 +18,7 @@ int num_cus();
 int64_t option_bn_resident();     // 1: single-pass batchnorm kernels for tensors that fit the register file
 int64_t option_bn_spin_limit();   // polls before a resident workgroup stops waiting for its peers
 int64_t option_gemm_tile();       // 0 automatic, else 82 | 42 | 22 | 11
+int64_t option_gemm_pretranspose();   // 1: large M/N-major bf16 operands are copied into the K-major layout first
 int64_t option_conv_tile();       // 0 automatic, else a tile code of the bf16 whole-tap convolution kernels
 
 // Per-stream scratch owned by the library (partial results of the reduction kernels,

@@ -184,6 +184,13 @@ static int transpose_to_cwhn(hipStream_t s, const T* in, T* out, int P, int C, i
     return LUXHIP_OK;
 }
 
+// out (C x P, C contiguous) = transpose of in (P x C, P contiguous); for the GEMM dispatch, which
+// turns large operands into the K-major layout its fastest kernel reads
+int transpose_matrix_bf16(hipStream_t s, const bf16_t* in, bf16_t* out, int64_t P, int64_t C) {
+    LUX_UNSUPPORTED_IF(P >= (1ll << 31) || C >= (1ll << 31), "matrix too large for the layout transform");
+    return transpose_to_cwhn<bf16_t>(s, in, out, (int)P, (int)C, 1);
+}
+
 template <typename T>
 static int pack_filter(hipStream_t s, const T* w, T* out, const ConvGeom& g, int for_dgrad) {
     ProfScope ps("pack_filter_kernel", s);

@@ -12,13 +12,48 @@ namespace luxhip {
 int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* delta,
                           const void* out, const void* pre, void* dx, void* dbias);   // elementwise.hip
 
+int transpose_matrix_bf16(hipStream_t s, const bf16_t* in, bf16_t* out, int64_t P, int64_t C);   // conv.hip
+
 int gemm_tile_override() { return (int)option_gemm_tile(); }
+
+// The 256 x 256 bf16 kernel reads K-major operands from LDS at twice the rate of M/N-major ones
+// (plain 16-byte reads against transposing reads): 1090-1190 TFLOP/s against 800-950 measured on
+// 4096..11008-sized problems.  A large M/N-major operand is therefore copied into the K-major
+// layout first (a pass at HBM rate: 90 MB in ~37 us, against ~200 us saved), when the other
+// dimension is long enough for the copy to pay (threshold from those measurements).
+template <typename T>
+static bool pretranspose_pays(int64_t M, int64_t N, int64_t K, int64_t other, int64_t ld, int64_t rows, const T* p) {
+    if constexpr (sizeof(T) != 2) return false;
+    return option_gemm_pretranspose() != 0 && gemm_tile_override() == 0 && M % 256 == 0 && N % 256 == 0 && K % 32 == 0 &&
+           (M / 256) * (N / 256) >= 128 && K >= 1024 && other >= 4096 && ld == rows && aligned16(p);
+}
 
 template <typename T>
 static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const T* A, int64_t lda,
                      const T* B, int64_t ldb, const T* bias, T* C, int64_t ldc, T* pre, int act) {
     DenseArgs<T> a;
-    const bool a_kmajor = transA != 0, b_kmajor = transB == 0;
+    bool a_kmajor = transA != 0, b_kmajor = transB == 0;
+    if constexpr (sizeof(T) == 2) {
+        const bool ta = !a_kmajor && pretranspose_pays<T>(M, N, K, N, lda, M, A);
+        const bool tb = !b_kmajor && pretranspose_pays<T>(M, N, K, M, ldb, N, B);
+        if (ta || tb) {
+            const size_t ab = ta ? (((size_t)M * K * sizeof(T) + 255) & ~size_t(255)) : 0;
+            const size_t bb = tb ? (size_t)N * K * sizeof(T) : 0;
+            Workspace ws;
+            int rc = get_workspace(s, ab + bb, &ws);
+            if (rc != LUXHIP_OK) return rc;
+            if (ta) {
+                T* At = reinterpret_cast<T*>(ws.data);
+                if ((rc = transpose_matrix_bf16(s, A, At, M, K)) != LUXHIP_OK) return rc;
+                A = At; lda = K; a_kmajor = true;
+            }
+            if (tb) {
+                T* Bt = reinterpret_cast<T*>(ws.data + ab);
+                if ((rc = transpose_matrix_bf16(s, B, Bt, N, K)) != LUXHIP_OK) return rc;
+                B = Bt; ldb = K; b_kmajor = true;
+            }
+        }
+    }
     a.A.p = A;
     a.A.sr = a_kmajor ? lda : 1;
     a.A.sk = a_kmajor ? 1 : lda;

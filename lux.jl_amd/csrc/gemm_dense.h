@@ -113,7 +113,8 @@ int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
         resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
     }
     const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
-    ProfScope ps(sizeof(T) == 2 ? "dense_gemm_kernel<bf16>" : "dense_gemm_kernel<f32>", s);
+    ProfScope ps(sizeof(T) == 2 ? (a.tail ? "dense_gemm_kernel<bf16>+tail" : "dense_gemm_kernel<bf16>")
+                                : (a.tail ? "dense_gemm_kernel<f32>+tail" : "dense_gemm_kernel<f32>"), s);
     kernel<<<dim3((unsigned)grid), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
@@ -181,6 +182,7 @@ int launch_layout(hipStream_t s, DenseArgs<T>& a) {
                         if (a.pre) rest.pre = a.pre + cut * a.ldc;
                     }
                     big.A.rows = big.M; big.B.rows = big.N;
+                    rest.tail = 1;
                     rest.A.rows = rest.M; rest.B.rows = rest.N;
                     int rc = launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, big);
                     if (rc != LUXHIP_OK) return rc;

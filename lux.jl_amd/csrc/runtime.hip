@@ -93,11 +93,13 @@ bool initialized() { return g_init; }
 int num_cus() { return g_cus; }
 
 namespace {
-std::atomic<int64_t> g_opt_bn_resident{1}, g_opt_bn_spin_limit{int64_t(1) << 22}, g_opt_gemm_tile{-1}, g_opt_conv_tile{0};
+std::atomic<int64_t> g_opt_bn_resident{1}, g_opt_bn_spin_limit{int64_t(1) << 22}, g_opt_gemm_tile{-1}, g_opt_conv_tile{0},
+    g_opt_gemm_pretranspose{1};
 }
 int64_t option_bn_resident() { return g_opt_bn_resident.load(); }
 int64_t option_bn_spin_limit() { return g_opt_bn_spin_limit.load(); }
 int64_t option_conv_tile() { return g_opt_conv_tile.load(); }
+int64_t option_gemm_pretranspose() { return g_opt_gemm_pretranspose.load(); }
 int64_t option_gemm_tile() {
     int64_t v = g_opt_gemm_tile.load();
     if (v < 0) {   // not set through the API: the environment variable LUXHIP_GEMM_TILE, read once
@@ -212,6 +214,9 @@ int luxhip_set_option(const char* name, int64_t value) {
         LUX_INVALID_IF(value != 0 && value != 82 && value != 83 && value != 84 && value != 42,
                        "set_option: conv_tile must be 0, 82, 83, 84 or 42");
         g_opt_conv_tile.store(value);
+    } else if (strcmp(name, "gemm_pretranspose") == 0) {
+        LUX_INVALID_IF(value != 0 && value != 1, "set_option: gemm_pretranspose must be 0 or 1");
+        g_opt_gemm_pretranspose.store(value);
     } else {
         return set_error(LUXHIP_INVALID, "set_option: unknown option '%s'", name);
     }

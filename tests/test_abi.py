@@ -60,10 +60,13 @@ def test_tuning_switches_validate_their_arguments(lux):
         lux.set_option("no_such_switch", 1)
     with pytest.raises(lux.LuxHipError, match="gemm_tile"):
         lux.set_option("gemm_tile", 7)
+    with pytest.raises(lux.LuxHipError, match="gemm_pretranspose"):
+        lux.set_option("gemm_pretranspose", 2)
     with pytest.raises(lux.LuxHipError, match="bn_spin_limit"):
         lux.set_option("bn_spin_limit", -1)
     for name, value in (("bn_resident", 0), ("bn_resident", 1), ("bn_spin_limit", 0), ("bn_spin_limit", 1 << 22),
-                        ("gemm_tile", 82), ("gemm_tile", 0), ("conv_tile", 84), ("conv_tile", 0)):
+                        ("gemm_tile", 82), ("gemm_tile", 0), ("conv_tile", 84), ("conv_tile", 0),
+                        ("gemm_pretranspose", 0), ("gemm_pretranspose", 1)):
         lux.set_option(name, value)
 
 

@@ -184,3 +184,24 @@ def test_ragged_tile_rounds_bf16(gpu, ragged):
         assert_close(got[edge], want(edge, full), "bf16", "ragged m rows")
     else:
         assert_close(got[:, edge], want(full, edge), "bf16", "ragged n cols")
+
+
+@pytest.mark.parametrize("transA,transB", [(False, False), (False, True), (True, True)])
+@pytest.mark.parametrize("pretranspose", [1, 0])
+def test_large_bf16_operand_layouts(gpu, transA, transB, pretranspose):
+    """Large bf16 products whose operands are contiguous along m or n: by default such operands are
+    first copied into the k-contiguous layout (switch gemm_pretranspose); both routes against the
+    fp64 oracle on a band of rows and columns."""
+    rng = np.random.default_rng(78)
+    M, N, K = 4096, 4096, 1024
+    A, B, bias = host_inputs("bf16", rng.normal(size=(K, M) if transA else (M, K)), rng.normal(size=(N, K) if transB else (K, N)),
+                             rng.normal(size=M))
+    gpu.set_option("gemm_pretranspose", pretranspose)
+    try:
+        got = gpu.matmul(dev(gpu, A, "bf16"), dev(gpu, B, "bf16"), dev(gpu, bias, "bf16"), transA=transA, transB=transB).to_numpy()
+    finally:
+        gpu.set_option("gemm_pretranspose", 1)
+    Am, Bm = (f64(A).T if transA else f64(A)), (f64(B).T if transB else f64(B))
+    rows = np.r_[0:130, 2040:2060, M - 130:M]
+    assert_close(got[rows], Am[rows] @ Bm + f64(bias[rows])[:, None], "bf16", "rows", scale=np.sqrt(K))
+    assert_close(got[:, rows], Am @ Bm[:, rows] + f64(bias)[:, None], "bf16", "cols", scale=np.sqrt(K))
