@@ -34,8 +34,11 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
     DenseArgs<T> a;
     bool a_kmajor = transA != 0, b_kmajor = transB == 0;
     if constexpr (sizeof(T) == 2) {
-        const bool ta = !a_kmajor && pretranspose_pays<T>(M, N, K, N, lda, M, A);
-        const bool tb = !b_kmajor && pretranspose_pays<T>(M, N, K, M, ldb, N, B);
+        bool ta = !a_kmajor && pretranspose_pays<T>(M, N, K, N, lda, M, A);
+        bool tb = !b_kmajor && pretranspose_pays<T>(M, N, K, M, ldb, N, B);
+        // only the kernel with both operands K-major is faster (a mixed pair is not), and two copies
+        // need a longer K to pay than one (measured: 4096 x 4096 x 1024 loses, x 4096 wins)
+        if (!((a_kmajor || ta) && (b_kmajor || tb)) || (ta && tb && K < 2048)) ta = tb = false;
         if (ta || tb) {
             const size_t ab = ta ? (((size_t)M * K * sizeof(T) + 255) & ~size_t(255)) : 0;
             const size_t bb = tb ? (size_t)N * K * sizeof(T) : 0;

@@ -193,7 +193,7 @@ def test_large_bf16_operand_layouts(gpu, transA, transB, pretranspose):
     first copied into the k-contiguous layout (switch gemm_pretranspose); both routes against the
     fp64 oracle on a band of rows and columns."""
     rng = np.random.default_rng(78)
-    M, N, K = 4096, 4096, 1024
+    M, N, K = 4096, 4096, 2048
     A, B, bias = host_inputs("bf16", rng.normal(size=(K, M) if transA else (M, K)), rng.normal(size=(N, K) if transB else (K, N)),
                              rng.normal(size=M))
     gpu.set_option("gemm_pretranspose", pretranspose)
