@@ -69,6 +69,7 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
     a.B.vec_ok = aligned16(B) && (ldb * sizeof(T)) % 16 == 0;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.C = C; a.ldc = ldc; a.bias = bias; a.pre = pre; a.act = act;
+    a.c_vec = (reinterpret_cast<uintptr_t>(C) & 7u) == 0 && (reinterpret_cast<uintptr_t>(pre) & 7u) == 0 && ldc % 4 == 0;
     if (a_kmajor && b_kmajor) return launch_layout<T, true, true>(s, a);
     if (a_kmajor) return launch_layout<T, true, false>(s, a);
     if (b_kmajor) return launch_layout<T, false, true>(s, a);
@@ -102,6 +103,7 @@ static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_
     }
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.C = C; a.ldc = ldc; a.bias = nullptr; a.pre = nullptr; a.act = LUXHIP_ACT_IDENTITY;
+    a.c_vec = (reinterpret_cast<uintptr_t>(C) & 7u) == 0 && ldc % 4 == 0 && sC[0] % 4 == 0 && sC[1] % 4 == 0 && sC[2] % 4 == 0;
     if (a_kmajor && b_kmajor) return launch_batched_layout<T, true, true>(s, a);
     if (a_kmajor) return launch_batched_layout<T, true, false>(s, a);
     if (b_kmajor) return launch_batched_layout<T, false, true>(s, a);

@@ -210,7 +210,11 @@ struct TileLoader {
 // stage linearly (lane i -> byte 16*i after a wave-uniform base); lane i therefore fetches the
 // global chunk whose swizzled home is that slot.  BOUNDED: rows at or past op.rows read from
 // `zero` (16 zero bytes somewhere in device memory) instead, so partial tiles need no branch.
-template <bool KMAJOR_, int ROWS, int THREADS = kGemmThreads, bool BOUNDED = false>
+// PERM_WM > 0 (K-major only): the rows are permuted inside groups of 32 * PERM_WM: LDS row
+// 32*i + j of a group holds global row PERM_WM*j + i.  A lane of the MFMA then owns PERM_WM
+// consecutive rows of the result instead of rows 32 apart, and the epilogue stores them with one
+// instruction.  The LDS layout and the fragment reads do not change.
+template <bool KMAJOR_, int ROWS, int THREADS = kGemmThreads, bool BOUNDED = false, int PERM_WM = 0>
 struct DirectLoader {
     using T = bf16_t;
     static constexpr bool KMAJOR = KMAJOR_;
@@ -220,6 +224,13 @@ struct DirectLoader {
     static_assert(INSTR >= 1 && (ROWS * BK / 8) % THREADS == 0, "stage must split evenly over the workgroup");
     static constexpr int STEP = THREADS / CPR;                // LDS rows covered per instruction of the workgroup
     static_assert(!BOUNDED || KMAJOR, "row bounds are implemented for K-major operands");
+    static_assert(PERM_WM == 0 || (KMAJOR && STEP % (32 * PERM_WM) == 0), "row permutation: whole groups per instruction");
+    __device__ __forceinline__ static int global_row(int lds_row) {
+        if constexpr (PERM_WM == 0) return lds_row;
+        constexpr int G = 32 * PERM_WM;
+        const int o = lds_row % G;
+        return lds_row - o + (o % 32) * PERM_WM + o / 32;
+    }
     const char* base;      // uniform: first element of the tile (row r0, k = 0)
     const char* zero;      // BOUNDED only
     int64_t step_bytes;    // uniform: global distance between consecutive instructions of a thread
@@ -232,7 +243,7 @@ struct DirectLoader {
         const int row = q / CPR, slot = q % CPR;
         if constexpr (KMAJOR) {
             const int chunk = slot ^ ((row >> 2) & 3);
-            voff = (uint32_t)(((int64_t)row * op.sr + chunk * 8) * 2);
+            voff = (uint32_t)(((int64_t)global_row(row) * op.sr + chunk * 8) * 2);
             step_bytes = (int64_t)STEP * op.sr * 2;
             k_bytes = 2;
         } else {
@@ -248,7 +259,7 @@ struct DirectLoader {
     // tile that starts at row r0 of the same operand
     __device__ __forceinline__ void move_to(const Operand<T>& op, int r0) {
         base = reinterpret_cast<const char*>(op.p + (KMAJOR ? (int64_t)r0 * op.sr : (int64_t)r0));
-        rows_left = op.rows - r0 - (int)threadIdx.x / CPR;
+        rows_left = op.rows - r0 - global_row((int)threadIdx.x / CPR);
     }
     // stage starting at k0 -> tile at `lds_tile` (uniform)
     __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
@@ -337,8 +348,10 @@ inline int persistent_grid(Kernel kernel, int threads, size_t lds_bytes, int64_t
 // Accumulates the (2*WM*32) x (2*WN*32) tile at (m0, n0).  acc[wm][wn][r] of lane l belongs to
 //   m = m0 + wave_m*WM*32 + wm*32 + l%32,   n = n0 + wave_n*WN*32 + wn*32 + 8*(r/4) + 4*(l/32) + r%4.
 // NWM x NWN waves per workgroup (along m, along n); wave w sits at (w % NWM, w / NWM).
+// PERMUTE: on the direct-to-LDS path with a K-major A, the A rows of each wave are permuted
+// (DirectLoader PERM_WM = WM) so that a lane owns WM consecutive m: m = lane_m + i.
 template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL = false, int NWN = 2, int NSTAGES = 0,
-          int NWM = 2>
+          int NWM = 2, bool PERMUTE = false>
 struct GemmMainloop {
     using Tr = GemmTraits<T>;
     static constexpr int THREADS = NWM * NWN * 64;
@@ -351,6 +364,10 @@ struct GemmMainloop {
     static constexpr bool DIRECT = FULL && sizeof(T) == 2;     // global -> LDS without registers
     static constexpr int NST = NSTAGES > 0 ? NSTAGES : (DIRECT ? 4 : 2);   // LDS stages
     static constexpr size_t LDS_BYTES = NST * (size_t)STAGE_ELEMS * sizeof(T);
+    static constexpr int PERM_A = (PERMUTE && DIRECT && A_KMAJOR && WM > 1 && (THREADS / 4) % (32 * WM) == 0) ? WM : 0;
+    static constexpr int M_STEP = PERM_A ? 1 : 32;            // distance in m between acc[i] and acc[i + 1] of a lane
+    using DirectLoaderA = DirectLoader<A_KMAJOR, TILE_M, THREADS, false, PERM_A>;
+    using DirectLoaderB = DirectLoader<B_KMAJOR, TILE_N, THREADS>;
 
     __device__ __forceinline__ static void run(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0, T* lds,
                                                f32x16_v (&acc)[WM][WN]) {
@@ -399,8 +416,8 @@ struct GemmMainloop {
     // registers, no ds_write).
     __device__ __forceinline__ static void run_direct(const Operand<T>& A, const Operand<T>& B, int K, int m0, int n0,
                                                       T* lds, f32x16_v (&acc)[WM][WN]) {
-        DirectLoader<A_KMAJOR, TILE_M, THREADS> la(A, m0);
-        DirectLoader<B_KMAJOR, TILE_N, THREADS> lb(B, n0);
+        DirectLoaderA la(A, m0);
+        DirectLoaderB lb(B, n0);
         run_pipeline(la, lb, K, lds, acc);
     }
 
@@ -546,9 +563,9 @@ struct GemmMainloop {
     }
 
     // First m and n of this lane inside the tile at (m0, n0); element acc[i][j][r] belongs to
-    // m = lane_m + 32*i,  n = lane_n + 32*j + 8*(r/4) + r%4.
+    // m = lane_m + M_STEP*i,  n = lane_n + 32*j + 8*(r/4) + r%4.
     __device__ __forceinline__ static int lane_m(int m0) {
-        return m0 + ((threadIdx.x >> 6) % NWM) * (WM * 32) + (threadIdx.x & 31);
+        return m0 + ((threadIdx.x >> 6) % NWM) * (WM * 32) + (threadIdx.x & 31) * (PERM_A ? WM : 1);
     }
     __device__ __forceinline__ static int lane_n(int n0) {
         return n0 + ((threadIdx.x >> 6) / NWM) * (WN * 32) + (((threadIdx.x & 63) >> 5) << 2);
@@ -558,14 +575,14 @@ struct GemmMainloop {
     template <typename F>
     __device__ __forceinline__ static void for_each(const f32x16_v (&acc)[WM][WN], int m0, int n0, F&& f) {
         const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
-        const int mb = m0 + (w % NWM) * (WM * 32) + (l & 31);
+        const int mb = lane_m(m0);
         const int nb = n0 + (w / NWM) * (WN * 32) + ((l >> 5) << 2);
 #pragma unroll
         for (int i = 0; i < WM; ++i)
 #pragma unroll
             for (int j = 0; j < WN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) f(mb + i * 32, nb + j * 32 + ((r >> 2) << 3) + (r & 3), acc[i][j][r]);
+                for (int r = 0; r < 16; ++r) f(mb + i * M_STEP, nb + j * 32 + ((r >> 2) << 3) + (r & 3), acc[i][j][r]);
     }
 };
 

@@ -14,13 +14,37 @@ namespace luxhip {
 
 // Epilogue of one tile: C = act(acc + bias), optional pre-activation copy.  CHECK: bounds tests;
 // the activation mode and HAS_PRE are resolved once per tile, so the common cases have no branch per element.
+// WM consecutive values of one column -> memory; one store when the lane's rows are consecutive
+// (ML::M_STEP == 1), the storage type is bf16 and the destination allows it
+template <class ML, typename T, int WM, bool CHECK>
+__device__ __forceinline__ void store_column(T* col, const float (&v)[WM], int mb, int M, bool vec) {
+    if constexpr (ML::M_STEP == 1 && sizeof(T) == 2 && !CHECK && (WM == 2 || WM == 4)) {
+        if (vec) {
+            if constexpr (WM == 4) {
+                uint2 w;
+                w.x = f32x2_to_bf16x2(v[0], v[1]);
+                w.y = f32x2_to_bf16x2(v[2], v[3]);
+                *reinterpret_cast<uint2*>(col) = w;
+            } else {
+                *reinterpret_cast<uint32_t*>(col) = f32x2_to_bf16x2(v[0], v[1]);
+            }
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+        if (!CHECK || mb + i * ML::M_STEP < M) st(col + i * ML::M_STEP, v[i]);
+}
+
 template <class ML, typename T, int WM, int WN, bool CHECK, int ACT_MODE, bool HAS_PRE>
 __device__ __forceinline__ void dense_epilogue_as(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int m0, int n0) {
     const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
     float bv[WM];
 #pragma unroll
-    for (int i = 0; i < WM; ++i) bv[i] = (a.bias && (!CHECK || mb + i * 32 < a.M)) ? ld(a.bias + mb + i * 32) : 0.0f;
+    for (int i = 0; i < WM; ++i)
+        bv[i] = (a.bias && (!CHECK || mb + i * ML::M_STEP < a.M)) ? ld(a.bias + mb + i * ML::M_STEP) : 0.0f;
     const int act = a.act;
+    const bool vec = a.c_vec != 0;
     static_for<WN * 16>([&](auto JR) {
         {
             constexpr int j = decltype(JR)::value / 16, r = decltype(JR)::value % 16;
@@ -29,18 +53,10 @@ __device__ __forceinline__ void dense_epilogue_as(const f32x16_v (&acc)[WM][WN],
                 float v[WM];
 #pragma unroll
                 for (int i = 0; i < WM; ++i) v[i] = acc[i][j][r] + bv[i];
-                if constexpr (HAS_PRE) {
-                    T* pcol = a.pre + (int64_t)n * a.ldc + mb;
-#pragma unroll
-                    for (int i = 0; i < WM; ++i)
-                        if (!CHECK || mb + i * 32 < a.M) st(pcol + i * 32, v[i]);
-                }
+                if constexpr (HAS_PRE) store_column<ML, T, WM, CHECK>(a.pre + (int64_t)n * a.ldc + mb, v, mb, a.M, vec);
                 if constexpr (ACT_MODE == 1) act_vec_as<LUXHIP_ACT_RELU>(v);
                 else if constexpr (ACT_MODE == 2) act_vec(act, v);
-                T* ccol = a.C + (int64_t)n * a.ldc + mb;
-#pragma unroll
-                for (int i = 0; i < WM; ++i)
-                    if (!CHECK || mb + i * 32 < a.M) st(ccol + i * 32, v[i]);
+                store_column<ML, T, WM, CHECK>(a.C + (int64_t)n * a.ldc + mb, v, mb, a.M, vec);
             }
         }
     });
@@ -59,7 +75,7 @@ __device__ __forceinline__ void dense_epilogue(const f32x16_v (&acc)[WM][WN], co
 // stores overlap with the loads.
 template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
 __global__ __launch_bounds__(NWM * NWN * 64) void dense_gemm_kernel(DenseArgs<T> a) {
-    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM>;
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM, true>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
     const int total = a.tiles_m * a.tiles_n;
@@ -69,8 +85,8 @@ __global__ __launch_bounds__(NWM * NWN * 64) void dense_gemm_kernel(DenseArgs<T>
         int t = blockIdx.x;
         tile_coords(t, a.tiles_m, a.tiles_n, tm, tn);
         int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
-        DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(a.A, m0);
-        DirectLoader<B_KMAJOR, ML::TILE_N, ML::THREADS> lb(a.B, n0);
+        typename ML::DirectLoaderA la(a.A, m0);
+        typename ML::DirectLoaderB lb(a.B, n0);
         ML::pipeline_fill(la, lb, a.K, lds);
         for (;;) {
             ML::pipeline_loop(la, lb, a.K, lds, acc);
@@ -226,7 +242,7 @@ __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t,
 
 template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
 __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<T> a) {
-    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM>;
+    using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM, true>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
     const int tiles = a.tiles_m * a.tiles_n;
@@ -235,8 +251,8 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
     if constexpr (ML::DIRECT) {
         int t = blockIdx.x;
         BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
-        DirectLoader<A_KMAJOR, ML::TILE_M, ML::THREADS> la(cur.A, cur.m0);
-        DirectLoader<B_KMAJOR, ML::TILE_N, ML::THREADS> lb(cur.B, cur.n0);
+        typename ML::DirectLoaderA la(cur.A, cur.m0);
+        typename ML::DirectLoaderB lb(cur.B, cur.n0);
         ML::pipeline_fill(la, lb, a.K, lds);
         for (;;) {
             ML::pipeline_loop(la, lb, a.K, lds, acc);
