@@ -306,7 +306,7 @@ class C4TransformerMLP(_ApiWorkload):
     def kernel_bytes(self):
         """HBM-bound kernels of this workload: name -> algorithmic bytes of one launch."""
         E, H = 2 * self.D * self.Ntok, 2 * self.F * self.Ntok      # bytes of a (D, tokens) / (F, tokens) bf16 tensor
-        return {"ln_fwd_kernel": 2 * E, "ln_bwd_dx_kernel": 3 * E, "ln_param_grad_kernel": 2 * E,
+        return {"ln_fwd_kernel": 2 * E, "ln_bwd_fused_kernel": 3 * E, "ln_bwd_dx_kernel": 3 * E, "ln_param_grad_kernel": 2 * E,
                 "whcn_to_cwhn_kernel": None,                         # operand copies: sizes differ per launch
                 "bias_act_bwd_plane_kernel": None}
 

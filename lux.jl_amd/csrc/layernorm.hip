@@ -8,6 +8,7 @@
 //             ln_param_grad_kernel: dgamma[l] = sum_r dy*xhat, dbeta[l] = sum_r dy as a column
 //             reduction (threads along l, coalesced; R split into slices, partials combined
 //             in a fixed order by ln_param_finalize_kernel).
+//             ln_bwd_fused_kernel: both in one pass for columns that one wavefront holds.
 #include <algorithm>
 
 #include "common.h"
@@ -227,6 +228,111 @@ __global__ __launch_bounds__(WAVE ? 256 : 1024) void ln_bwd_dx_kernel(const T* _
     }
 }
 
+// ------------------------------------------------------------------------------- pullback: dx, dgamma, dbeta in one pass
+// Columns of up to 64 * kLnCache vectors with affine parameters.  Two wavefronts share a column
+// (half of its vectors each, so that the per-position sums fit the register file next to the
+// column itself); a pair walks over columns r = pair, pair + P, ... (P pairs in the grid) with
+// delta and x of the current column in registers, as ln_bwd_dx_kernel does, and keeps dy * xhat
+// and dy of its positions l summed over its columns.  The two pairs of a workgroup add their sums
+// in pair order through LDS; row `blockIdx.x` of pg / pb receives the result and
+// ln_param_finalize_kernel adds the rows in order.  delta and x are read once.
+constexpr int kLnFusedCache = kLnCache / 2;
+template <typename T, int ACT, int VEC>
+__global__ __launch_bounds__(256) void ln_bwd_fused_kernel(const T* __restrict__ delta, const T* __restrict__ x,
+                                                           const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                           const float* __restrict__ save_mean,
+                                                           const float* __restrict__ save_invstd, T* dx, float* pg, float* pb,
+                                                           uint32_t nvec, uint32_t R, float inv_L) {
+    __shared__ float red[2][2][128 * VEC];
+    __shared__ float colsum[2][2][2];                  // [pair][wave of the pair][s1, s2]
+    const uint32_t w = threadIdx.x >> 6, pair = w >> 1, half = w & 1u;
+    const uint32_t t = half * 64u + (threadIdx.x & 63u);          // 0..127 inside the pair
+    const uint32_t pairs = gridDim.x * 2u;
+    using K = Kept<T, VEC>;
+    float ag[kLnFusedCache][VEC], ab[kLnFusedCache][VEC];
+#pragma unroll
+    for (int u = 0; u < kLnFusedCache; ++u)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { ag[u][e] = 0.0f; ab[u][e] = 0.0f; }
+    const uint32_t rounds = (R + pairs - 1) / pairs;              // the same for every wavefront: barriers inside
+    for (uint32_t it = 0; it < rounds; ++it) {
+        const uint32_t r = it * pairs + blockIdx.x * 2u + pair;
+        const bool live = r < R;                                  // uniform per wavefront
+        const uint32_t rc = live ? r : R - 1;
+        const size_t base = (size_t)rc * nvec * VEC;
+        const float mean = save_mean[rc], invstd = save_invstd[rc];
+        typename K::type kd[kLnFusedCache], kv[kLnFusedCache];
+#pragma unroll
+        for (int u = 0; u < kLnFusedCache; ++u) {
+            const size_t off = base + (size_t)min(u * 128u + t, nvec - 1) * VEC;   // past the end: the last vector again
+            kd[u] = K::load(delta, off);
+            kv[u] = K::load(x, off);
+        }
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kLnFusedCache; ++u) {
+            const uint32_t q = u * 128u + t;
+            if (q < nvec && live) {
+                float d[VEC], v[VEC], dy[VEC], gm[VEC];
+                K::get(kd[u], d);
+                K::get(kv[u], v);
+                ln_dy<T, ACT, VEC>(gamma, beta, q, mean, invstd, d, v, dy, gm);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float xh = (v[e] - mean) * invstd;
+                    const float g = gm[e] * dy[e];
+                    s1 += g;
+                    s2 = fmaf(g, xh, s2);
+                    ag[u][e] = fmaf(dy[e], xh, ag[u][e]);
+                    ab[u][e] += dy[e];
+                }
+            }
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        if ((threadIdx.x & 63u) == 0) { colsum[pair][half][0] = s1; colsum[pair][half][1] = s2; }
+        __syncthreads();
+        s1 = (colsum[pair][0][0] + colsum[pair][1][0]) * inv_L;
+        s2 = (colsum[pair][0][1] + colsum[pair][1][1]) * inv_L;
+        __syncthreads();                                          // colsum is rewritten in the next round
+#pragma unroll
+        for (int u = 0; u < kLnFusedCache; ++u) {
+            const uint32_t q = u * 128u + t;
+            if (q < nvec && live) {
+                float d[VEC], v[VEC], dy[VEC], gm[VEC], o[VEC];
+                K::get(kd[u], d);
+                K::get(kv[u], v);
+                ln_dy<T, ACT, VEC>(gamma, beta, q, mean, invstd, d, v, dy, gm);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float xh = (v[e] - mean) * invstd;
+                    o[e] = invstd * (gm[e] * dy[e] - s1 - xh * s2);
+                }
+                ln_store<T, VEC>(dx, base + (size_t)q * VEC, o);
+            }
+        }
+    }
+    // sums of the two pairs, in pair order, one cached vector at a time
+    const size_t row = (size_t)blockIdx.x * nvec * VEC;
+#pragma unroll
+    for (int u = 0; u < kLnFusedCache; ++u) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            red[0][pair][t * VEC + e] = ag[u][e];
+            red[1][pair][t * VEC + e] = ab[u][e];
+        }
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < 128u * VEC; i += 256u) {
+            const uint32_t l = u * 128u * VEC + i;
+            if (l < nvec * VEC) {
+                pg[row + l] = red[0][0][i] + red[0][1][i];
+                pb[row + l] = red[1][0][i] + red[1][1][i];
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // ------------------------------------------------------------------------------- pullback: dgamma, dbeta
 // grid (ceil(nvec / 64), S): a thread owns one vector of positions l and walks over the
 // columns of slice s; partial sums go to pg/pb[s][l].
@@ -273,27 +379,40 @@ __global__ __launch_bounds__(64) void ln_param_grad_kernel(const T* __restrict__
     for (int e = 0; e < VEC; ++e) { pg[o + e] = ag[e]; pb[o + e] = ab[e]; }
 }
 
-// dgamma[l] = sum_s pg[s][l], dbeta likewise.  Workgroup of 64 positions x 16 slice groups:
-// group g adds slices g, g+16, ... and the 16 group sums are added in group order.
+// dgamma[l] = sum_s pg[s][l], dbeta likewise.  Workgroup of LW positions x (1024 / LW) slice groups:
+// group g adds slices g, g + G, ... and the G group sums are added in group order.  LW = 32 gives
+// L / 32 workgroups (128-byte row segments): enough of them to fill the device for L of a few thousand.
+constexpr int kLnFinalizeWidth = 32;
 template <typename T>
 __global__ __launch_bounds__(1024) void ln_param_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb,
                                                                  T* dgamma, T* dbeta, uint32_t L, uint32_t S) {
-    __shared__ float sg[16][64], sb[16][64];
-    const uint32_t lx = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const uint32_t l = blockIdx.x * 64 + lx;
+    constexpr int LW = kLnFinalizeWidth, G = 1024 / LW;
+    __shared__ float sg[G][LW], sb[G][LW];
+    const uint32_t lx = threadIdx.x % LW, grp = threadIdx.x / LW;
+    const uint32_t l = blockIdx.x * LW + lx;
     float tg = 0.0f, tb = 0.0f;
-    if (l < L)
-        for (uint32_t s = grp; s < S; s += 16) {
+    if (l < L) {
+        uint32_t s = grp;
+        for (; s + 3 * G < S; s += 4 * G) {          // four independent loads in flight
+            const float g0 = pg[(size_t)s * L + l], g1 = pg[(size_t)(s + G) * L + l];
+            const float g2 = pg[(size_t)(s + 2 * G) * L + l], g3 = pg[(size_t)(s + 3 * G) * L + l];
+            const float b0 = pb[(size_t)s * L + l], b1 = pb[(size_t)(s + G) * L + l];
+            const float b2 = pb[(size_t)(s + 2 * G) * L + l], b3 = pb[(size_t)(s + 3 * G) * L + l];
+            tg = (((tg + g0) + g1) + g2) + g3;
+            tb = (((tb + b0) + b1) + b2) + b3;
+        }
+        for (; s < S; s += G) {
             tg += pg[(size_t)s * L + l];
             tb += pb[(size_t)s * L + l];
         }
+    }
     sg[grp][lx] = tg;
     sb[grp][lx] = tb;
     __syncthreads();
     if (grp == 0 && l < L) {
         tg = 0.0f; tb = 0.0f;
 #pragma unroll
-        for (int g = 0; g < 16; ++g) { tg += sg[g][lx]; tb += sb[g][lx]; }
+        for (int g = 0; g < G; ++g) { tg += sg[g][lx]; tb += sb[g][lx]; }
         if (dgamma) st(dgamma + l, tg);
         if (dbeta) st(dbeta + l, tb);
     }
@@ -371,6 +490,26 @@ static int ln_bwd_impl(hipStream_t s, int act, int64_t L, int64_t R, const T* de
                         (gamma == nullptr || (aligned16(gamma) && aligned16(beta)));
     LnPlan p = ln_plan<T>(L, R, ptr_ok);
     const float inv_L = 1.0f / (float)L;
+    if (p.vec && p.wave && gamma != nullptr && (dgamma != nullptr || dbeta != nullptr) && R >= 64) {
+        // one pass over delta and x: dx and the per-position sums of every workgroup
+        const int64_t blocks = std::min<int64_t>(ceil_div(R, 2), 3 * (int64_t)(num_cus() > 0 ? num_cus() : 256));
+        Workspace ws;
+        int rc = get_workspace(s, (size_t)2 * blocks * L * sizeof(float), &ws);
+        if (rc != LUXHIP_OK) return rc;
+        float* pg = reinterpret_cast<float*>(ws.data);
+        float* pb = pg + (size_t)blocks * L;
+        {
+            ProfScope ps("ln_bwd_fused_kernel", s);
+#define LN_FUSED(A) ln_bwd_fused_kernel<T, A, V><<<(unsigned)blocks, 256, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pg, pb, p.nvec, (uint32_t)R, inv_L)
+            LUX_DISPATCH_ACT(act, LN_FUSED);
+#undef LN_FUSED
+        }
+        LUX_CHECK_LAUNCH();
+        ProfScope ps2("ln_param_finalize_kernel", s);
+        ln_param_finalize_kernel<T><<<(unsigned)ceil_div(L, kLnFinalizeWidth), 1024, 0, s>>>(pg, pb, dgamma, dbeta, (uint32_t)L, (uint32_t)blocks);
+        LUX_CHECK_LAUNCH();
+        return LUXHIP_OK;
+    }
     {
         ProfScope ps("ln_bwd_dx_kernel", s);
 #define LN_BWD(A) LN_VARIANTS(ln_bwd_dx_kernel, A, delta, x, gamma, beta, save_mean, save_invstd, dx, p.nvec, (uint32_t)R, inv_L)
@@ -402,7 +541,7 @@ static int ln_bwd_impl(hipStream_t s, int act, int64_t L, int64_t R, const T* de
         }
         LUX_CHECK_LAUNCH();
         ProfScope ps2("ln_param_finalize_kernel", s);
-        ln_param_finalize_kernel<T><<<(unsigned)ceil_div(L, 64), 1024, 0, s>>>(pg, pb, dgamma, dbeta, (uint32_t)L, (uint32_t)S);
+        ln_param_finalize_kernel<T><<<(unsigned)ceil_div(L, kLnFinalizeWidth), 1024, 0, s>>>(pg, pb, dgamma, dbeta, (uint32_t)L, (uint32_t)S);
         LUX_CHECK_LAUNCH();
     }
     return LUXHIP_OK;
