@@ -10,7 +10,10 @@ pytestmark = pytest.mark.gpu
 
 # (shape, number of leading normalised dims)
 CASES = [((4, 4, 6, 2), 3), ((6, 3), 1), ((16, 5), 1), ((3, 4, 5), 1), ((3, 4, 5), 2), ((512, 9), 1), ((1000, 7), 1),
-         ((4096, 6), 1), ((20000, 3), 1), ((24, 24, 8, 5), 3)]
+         ((4096, 6), 1), ((20000, 3), 1), ((24, 24, 8, 5), 3),
+         # 64 columns or more of at most 512 vectors: the pullback that reads delta and x once (an odd
+         # number of columns, more columns than wavefront pairs in the grid, a ragged last round)
+         ((256, 67), 1), ((4096, 70), 1), ((520, 1601), 1), ((24, 8, 200), 2)]
 
 
 def test_invariants_without_affine(gpu):
