@@ -200,9 +200,13 @@ int luxhip_attention_softmax_fwd(luxhip_stream_t s, int dtype, int64_t S, int64_
                                  int64_t bias_stride_h, int64_t bias_stride_b, void* probs);
 
 /* Pullback of the same (the softmax rule of NNlib, reached by AD in the reference):
- * dlogits = scale * probs .* (dprobs - sum_s dprobs .* probs); cols = L * H * B. */
-int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t cols, const void* dprobs,
-                                 const void* probs, double scale, void* dlogits);
+ * dlogits = scale * probs .* (dprobs - sum_s dprobs .* probs); cols = L * H * B.  causal != 0:
+ * 16-byte vectors of a column that lie wholly past s = l are neither read from dprobs / probs
+ * (tiles of dprobs that structure 1 left untouched) nor computed: zeros are stored up to the end of
+ * the block of 128 key positions that holds s = l, which is as far as the products with structure
+ * 2 or 3 read; dlogits past that block is left untouched. */
+int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t cols, int causal,
+                                 const void* dprobs, const void* probs, double scale, void* dlogits);
 
 /* ---------------------------------------------------------------- dropout ----------
  * The reference draws its noise with `rand!(rng, y)` from the array package's generator
@@ -274,11 +278,19 @@ int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, 
  * operand: the products of permuted / repeated operands without copies, e.g. the (heads, batch)
  * dims of scaled_dot_product_attention's [E, H, L, B] tensors and the key/value groups that
  * repeat_inner_gqa (src/impl/attention.jl:1-3, 44-48) would materialise (stride 0 along the repeat).
- * The caller lays out C so that the products do not overlap. */
+ * The caller lays out C so that the products do not overlap.
+ * structure: what a causal mask (keep key s for query l where s <= l, make_causal_mask,
+ * src/impl/attention.jl:130-134) lets the products of attention skip; 0 for a plain product.
+ *   1: the elements of C with m > n are not needed (logits[s, l], and their cotangent): tiles
+ *      that hold only such elements are left untouched;
+ *   2: op(B)[k, n] is zero for k > n (weights and their cotangent as the right operand, contracted
+ *      over s): the contraction of a tile stops at its last column;
+ *   3: op(B)[k, n] is zero for k < n (the same matrices transposed, contracted over l): it starts
+ *      at the tile's first column. */
 int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N,
                                   int64_t K, const int64_t* batch_dims, const void* A, int64_t lda,
                                   const int64_t* stridesA, const void* B, int64_t ldb, const int64_t* stridesB,
-                                  void* C, int64_t ldc, const int64_t* stridesC);
+                                  void* C, int64_t ldc, const int64_t* stridesC, int structure);
 
 /* `sum(tmp; dims=3)` of the batched_matmul pullback when an operand was shared among the
  * products (src/impl/batched_mul.jl:324-330): out[i] = sum_b in[i + b n], i < n, in batch order. */

@@ -69,7 +69,7 @@ SIGNATURES = {
     "luxhip_groupnorm_bwd": [_vp, _i, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _vp, _vp, _vp],
     "luxhip_instancenorm_running_stats": [_vp, _i, _i64, _i64, _i64, _fp, _fp, _d, _d, _vp, _vp, _vp, _vp],
     "luxhip_attention_softmax_fwd": [_vp, _i, _i64, _i64, _i64, _i64, _vp, _d, _i, _vp, _i64, _i64, _vp, _i64, _i64, _vp],
-    "luxhip_attention_softmax_bwd": [_vp, _i, _i64, _i64, _vp, _vp, _d, _vp],
+    "luxhip_attention_softmax_bwd": [_vp, _i, _i64, _i64, _i64, _i, _vp, _vp, _d, _vp],
     "luxhip_rand_uniform": [_vp, _i, _i64, _u64, _u64, _vp],
     "luxhip_dropout_fwd": [_vp, _i, _i64, _u64, _u64, _d, _d, _vp, _vp, _vp],
     "luxhip_dropout_mask": [_vp, _i, _i64, _d, _d, _vp],
@@ -80,7 +80,7 @@ SIGNATURES = {
     "luxhip_layernorm_bwd": [_vp, _i, _i, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _vp, _vp, _vp],
     "luxhip_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64],
     "luxhip_batched_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64],
-    "luxhip_batched_matmul_strided": [_vp, _i, _i, _i, _i64, _i64, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64],
+    "luxhip_batched_matmul_strided": [_vp, _i, _i, _i, _i64, _i64, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64, _i],
     "luxhip_batch_sum": [_vp, _i, _i64, _i64, _vp, _vp],
     "luxhip_fused_dense_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp],
     "luxhip_fused_dense_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp],

@@ -99,34 +99,39 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_kernel(const
 template <typename T, int NV>
 __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_kernel(const T* __restrict__ dprobs,
                                                                            const T* __restrict__ probs, T* __restrict__ dlogits,
-                                                                           int S, int64_t cols, float scale) {
+                                                                           int S, int L, int causal, int64_t cols, float scale) {
     const int lane = threadIdx.x & 63;
     const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
     if (col >= cols) return;
     const T* dy = dprobs + col * S;
     const T* y = probs + col * S;
     T* dx = dlogits + col * S;
+    const int limit = causal ? (int)(col % L) : S - 1;      // positions past it: weight 0, cotangent not read
+    // causal: zeros are stored up to the end of the 128-block of s that holds the limit (what the
+    // products with a triangular structure read); the rest of the column is left untouched
+    const int wend = causal ? min(S, ((limit >> 7) + 1) << 7) : S;
     if constexpr (NV > 0) {
         float yv[NV], dv[NV];
         float dot = 0.f;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int s = lane + 64 * i;
-            yv[i] = s < S ? ld(y + s) : 0.f;
-            dv[i] = s < S ? ld(dy + s) : 0.f;
+            const bool in = s < S && s <= limit;
+            yv[i] = in ? ld(y + s) : 0.f;
+            dv[i] = in ? ld(dy + s) : 0.f;
             dot += yv[i] * dv[i];
         }
         dot = wave_add(dot);
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int s = lane + 64 * i;
-            if (s < S) st(dx + s, scale * yv[i] * (dv[i] - dot));
+            if (s < wend) st(dx + s, scale * yv[i] * (dv[i] - dot));
         }
     } else {
         float dot = 0.f;
-        for (int s = lane; s < S; s += 64) dot += ld(y + s) * ld(dy + s);
+        for (int s = lane; s < S && s <= limit; s += 64) dot += ld(y + s) * ld(dy + s);
         dot = wave_add(dot);
-        for (int s = lane; s < S; s += 64) st(dx + s, scale * ld(y + s) * (ld(dy + s) - dot));
+        for (int s = lane; s < wend; s += 64) st(dx + s, s <= limit ? scale * ld(y + s) * (ld(dy + s) - dot) : 0.f);
     }
 }
 
@@ -196,24 +201,29 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_vec_kernel(
 template <typename T, int NVV>
 __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(const T* __restrict__ dprobs,
                                                                                const T* __restrict__ probs,
-                                                                               T* __restrict__ dlogits, int S, int64_t cols,
-                                                                               float scale) {
+                                                                               T* __restrict__ dlogits, int S, int L, int causal,
+                                                                               int64_t cols, float scale) {
     constexpr int VEC = Vec<T>::N;
     const int lane = threadIdx.x & 63;
     const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
     if (col >= cols) return;
     const T* dy = dprobs + col * S;
     const T* y = probs + col * S;
+    const int limit = causal ? (int)(col % L) : S - 1;
+    const int wend = causal ? min(S, ((limit >> 7) + 1) << 7) : S;       // see attn_softmax_bwd_kernel
     float yv[NVV][VEC], dv[NVV][VEC];
     float dot = 0.f;
 #pragma unroll
     for (int i = 0; i < NVV; ++i) {
         const int s0 = (lane + 64 * i) * VEC;
-        if (s0 < S) {
+        if (s0 < S && s0 <= limit) {            // vectors wholly past the limit: weights are 0, nothing is read
             Vec<T>::load(y + s0, yv[i]);
             Vec<T>::load(dy + s0, dv[i]);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) dot += yv[i][k] * dv[i][k];
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) { yv[i][k] = 0.f; dv[i][k] = 0.f; }
         }
     }
     dot = wave_add(dot);
@@ -221,7 +231,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(c
 #pragma unroll
     for (int i = 0; i < NVV; ++i) {
         const int s0 = (lane + 64 * i) * VEC;
-        if (s0 < S) {
+        if (s0 < wend) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) yv[i][k] = scale * yv[i][k] * (dv[i][k] - dot);
             Vec<T>::store(dx + s0, yv[i]);
@@ -282,11 +292,12 @@ static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int6
 }
 
 template <typename T>
-static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t cols, const T* dprobs, const T* probs, float scale, T* dlogits) {
+static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t L, int causal, int64_t cols, const T* dprobs, const T* probs,
+                            float scale, T* dlogits) {
     const unsigned grid = (unsigned)ceil_div(cols, kAttnWaves);
     ProfScope ps("attn_softmax_bwd_kernel", s);
 #define LUX_SOFTMAX_BWD_VEC(NVV) \
-    attn_softmax_bwd_vec_kernel<T, NVV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, cols, scale)
+    attn_softmax_bwd_vec_kernel<T, NVV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, (int)L, causal, cols, scale)
     switch (lane_vectors<T>(S, aligned16(dprobs) && aligned16(probs) && aligned16(dlogits))) {
         case 1: LUX_SOFTMAX_BWD_VEC(1); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
         case 2: LUX_SOFTMAX_BWD_VEC(2); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
@@ -295,7 +306,7 @@ static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t cols, const T* dpr
         default: break;
     }
 #undef LUX_SOFTMAX_BWD_VEC
-#define LUX_SOFTMAX_BWD(NV) attn_softmax_bwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, cols, scale)
+#define LUX_SOFTMAX_BWD(NV) attn_softmax_bwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, (int)L, causal, cols, scale)
     switch (cached_vectors(S)) {
         case 1: LUX_SOFTMAX_BWD(1); break;
         case 2: LUX_SOFTMAX_BWD(2); break;
@@ -340,18 +351,19 @@ int luxhip_attention_softmax_fwd(luxhip_stream_t s, int dtype, int64_t S, int64_
                                     mask_stride_b, (const bf16_t*)bias, bias_stride_h, bias_stride_b, (bf16_t*)probs);
 }
 
-int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t cols, const void* dprobs, const void* probs,
-                                 double scale, void* dlogits) {
+int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t cols, int causal, const void* dprobs,
+                                 const void* probs, double scale, void* dlogits) {
     LUX_REQUIRE_INIT();
     int rc = softmax_check(dtype, S, cols);
     if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF(L <= 0 && cols > 0, "attention_softmax_bwd: L must be positive");
     if (S * cols == 0) return LUXHIP_OK;
     LUX_INVALID_IF(dprobs == nullptr || probs == nullptr || dlogits == nullptr,
                    "attention_softmax_bwd: dprobs, probs and dlogits must not be NULL");
     if (dtype == LUXHIP_F32)
-        return softmax_bwd_impl<float>((hipStream_t)s, S, cols, (const float*)dprobs, (const float*)probs, (float)scale,
+        return softmax_bwd_impl<float>((hipStream_t)s, S, L, causal, cols, (const float*)dprobs, (const float*)probs, (float)scale,
                                        (float*)dlogits);
-    return softmax_bwd_impl<bf16_t>((hipStream_t)s, S, cols, (const bf16_t*)dprobs, (const bf16_t*)probs, (float)scale,
+    return softmax_bwd_impl<bf16_t>((hipStream_t)s, S, L, causal, cols, (const bf16_t*)dprobs, (const bf16_t*)probs, (float)scale,
                                     (bf16_t*)dlogits);
 }
 

@@ -80,8 +80,9 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
 template <typename T>
 static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const int64_t* bdim, const T* A,
                         int64_t lda, const int64_t* sA, const T* B, int64_t ldb, const int64_t* sB, T* C, int64_t ldc,
-                        const int64_t* sC) {
+                        const int64_t* sC, int structure) {
     DenseArgs<T> a;
+    a.structure = structure;
     const bool a_kmajor = transA != 0, b_kmajor = transB == 0;
     a.A.p = A;
     a.A.sr = a_kmajor ? lda : 1;
@@ -112,7 +113,8 @@ static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_
 
 static int batched_dispatch(hipStream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
                             const int64_t* bdim, const void* A, int64_t lda, const int64_t* sA, const void* B, int64_t ldb,
-                            const int64_t* sB, void* C, int64_t ldc, const int64_t* sC) {
+                            const int64_t* sB, void* C, int64_t ldc, const int64_t* sC, int structure) {
+    LUX_INVALID_IF(structure < 0 || structure > 3, "batched_matmul: structure must be 0..3");
     int64_t batch = 1;
     for (int d = 0; d < 3; ++d) {
         LUX_INVALID_IF(bdim[d] < 0 || sA[d] < 0 || sB[d] < 0 || sC[d] < 0, "batched_matmul: negative batch extent or stride");
@@ -125,9 +127,9 @@ static int batched_dispatch(hipStream_t s, int dtype, int transA, int transB, in
     LUX_INVALID_IF(lda < (transA ? K : M) || ldb < (transB ? N : K) || ldc < M, "batched_matmul: leading dimension too small");
     if (dtype == LUXHIP_F32)
         return batched_impl<float>(s, transA, transB, M, N, K, bdim, (const float*)A, lda, sA, (const float*)B, ldb, sB, (float*)C,
-                                   ldc, sC);
+                                   ldc, sC, structure);
     return batched_impl<bf16_t>(s, transA, transB, M, N, K, bdim, (const bf16_t*)A, lda, sA, (const bf16_t*)B, ldb, sB,
-                                (bf16_t*)C, ldc, sC);
+                                (bf16_t*)C, ldc, sC, structure);
 }
 
 // out[i] = sum_b in[i + b n]: `sum(tmp; dims=3)` of a stack of matrices, accumulated in fp32 in batch order
@@ -213,19 +215,20 @@ int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, 
     if (rc != LUXHIP_OK) return rc;
     LUX_INVALID_IF(batch > 1 && M > 0 && N > 0 && strideC < ldc * (N - 1) + M, "batched_matmul: the results would overlap");
     const int64_t bdim[3] = {batch, 1, 1}, sA[3] = {strideA, 0, 0}, sB[3] = {strideB, 0, 0}, sC[3] = {strideC, 0, 0};
-    return batched_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, bdim, A, lda, sA, B, ldb, sB, C, ldc, sC);
+    return batched_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, bdim, A, lda, sA, B, ldb, sB, C, ldc, sC, 0);
 }
 
 int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K,
                                   const int64_t* batch_dims, const void* A, int64_t lda, const int64_t* stridesA, const void* B,
-                                  int64_t ldb, const int64_t* stridesB, void* C, int64_t ldc, const int64_t* stridesC) {
+                                  int64_t ldb, const int64_t* stridesB, void* C, int64_t ldc, const int64_t* stridesC,
+                                  int structure) {
     LUX_REQUIRE_INIT();
     int rc = gemm_check(dtype, 0, M, N, K);
     if (rc != LUXHIP_OK) return rc;
     LUX_INVALID_IF(batch_dims == nullptr || stridesA == nullptr || stridesB == nullptr || stridesC == nullptr,
                    "batched_matmul_strided: batch extents and strides must not be NULL");
     return batched_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, batch_dims, A, lda, stridesA, B, ldb, stridesB, C, ldc,
-                            stridesC);
+                            stridesC, structure);
 }
 
 int luxhip_batch_sum(luxhip_stream_t s, int dtype, int64_t n, int64_t batch, const void* in, void* out) {

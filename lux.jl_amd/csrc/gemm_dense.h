@@ -221,12 +221,19 @@ struct BatchTile {
     Operand<T> A, B;
     T* C;
     int m0, n0;
+    int K;          // extent of the contraction for this tile (a.structure may shorten it)
+    bool store;     // false: the tile is not computed (a.structure == 1, every m > n)
 };
 template <typename T, int TILE_M, int TILE_N>
 __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t, int tiles) {
     const int b = t / tiles;
+    int ti = t - b * tiles;
+    // with a triangular structure the tiles of a product differ in cost: the walk through a product
+    // starts at a different tile for every product, so that a workgroup (which takes every
+    // gridDim.x-th tile of the sequence) does not land on the same tile position each time
+    if (a.structure != 0) ti = (ti + (int)(((int64_t)b * 97) % tiles)) % tiles;
     int tm, tn;
-    tile_coords(t - b * tiles, a.tiles_m, a.tiles_n, tm, tn);
+    tile_coords(ti, a.tiles_m, a.tiles_n, tm, tn);
     const int i0 = b % a.bdim[0], r0 = b / a.bdim[0];
     const int i1 = r0 % a.bdim[1], i2 = r0 / a.bdim[1];
     BatchTile<T> bt;
@@ -237,6 +244,18 @@ __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t,
     bt.C = a.C + i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
     bt.m0 = tm * TILE_M;
     bt.n0 = tn * TILE_N;
+    bt.K = a.K;
+    bt.store = true;
+    if (a.structure == 1) {
+        if (bt.m0 >= bt.n0 + TILE_N) { bt.store = false; bt.K = 0; }
+    } else if (a.structure == 2) {
+        bt.K = min(a.K, bt.n0 + TILE_N);
+    } else if (a.structure == 3) {
+        const int k_lo = min(bt.n0, a.K);        // n0 is a multiple of the tile width, hence of the stage depth
+        bt.A.p += (int64_t)k_lo * a.A.sk;
+        bt.B.p += (int64_t)k_lo * a.B.sk;
+        bt.K = a.K - k_lo;
+    }
     return bt;
 }
 
@@ -253,28 +272,30 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
         BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
         typename ML::DirectLoaderA la(cur.A, cur.m0);
         typename ML::DirectLoaderB lb(cur.B, cur.n0);
-        ML::pipeline_fill(la, lb, a.K, lds);
+        ML::pipeline_fill(la, lb, cur.K, lds);
         for (;;) {
-            ML::pipeline_loop(la, lb, a.K, lds, acc);
+            ML::pipeline_loop(la, lb, cur.K, lds, acc);
             const int tnext = t + gridDim.x;
             DenseArgs<T> out = a;
             out.C = cur.C;
             const int m0 = cur.m0, n0 = cur.n0;
+            const bool store = cur.store;
             if (tnext < total) {
                 cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, tnext, tiles);
                 la.move_to(cur.A, cur.m0);
                 lb.move_to(cur.B, cur.n0);
                 ML::pipeline_drain();
-                ML::pipeline_fill(la, lb, a.K, lds);
+                ML::pipeline_fill(la, lb, cur.K, lds);
             }
-            dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
+            if (store) dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
             if (tnext >= total) break;
             t = tnext;
         }
     } else {
         for (int t = blockIdx.x; t < total; t += gridDim.x) {
             const BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
-            ML::run(cur.A, cur.B, a.K, cur.m0, cur.n0, lds, acc);
+            if (!cur.store) continue;          // uniform
+            ML::run(cur.A, cur.B, cur.K, cur.m0, cur.n0, lds, acc);
             DenseArgs<T> out = a;
             out.C = cur.C;
             dense_epilogue<ML, T, WM, WN, FULL>(acc, out, cur.m0, cur.n0);

@@ -23,6 +23,10 @@ struct DenseArgs {
     int batch = 1;
     int bdim[3] = {1, 1, 1};
     int64_t bsA[3] = {0, 0, 0}, bsB[3] = {0, 0, 0}, bsC[3] = {0, 0, 0};
+    // batched products with a triangular operand or result (causal attention), see luxhip_batched_matmul_strided:
+    // 0 none; 1 tiles of C with every m > n are left untouched; 2 op(B)[k, n] = 0 for k > n: the
+    // contraction stops at the tile's last column; 3 op(B)[k, n] = 0 for k < n: it starts at the tile's first column
+    int structure = 0;
 };
 
 template <typename T, bool A_KMAJOR, bool B_KMAJOR>

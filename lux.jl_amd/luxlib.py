@@ -419,9 +419,9 @@ def _i64x3(v):
     return (C.c_int64 * 3)(*v)
 
 
-def _bmm_strided(tA, tB, M, N, K, bdims, A, lda, sA, B, ldb, sB, Cm, ldc, sC):
+def _bmm_strided(tA, tB, M, N, K, bdims, A, lda, sA, B, ldb, sB, Cm, ldc, sC, structure=0):
     _lib.call("luxhip_batched_matmul_strided", current_stream(), Cm.code, int(tA), int(tB), M, N, K, _i64x3(bdims),
-              A.ptr, max(lda, 1), _i64x3(sA), B.ptr, max(ldb, 1), _i64x3(sB), Cm.ptr, max(ldc, 1), _i64x3(sC))
+              A.ptr, max(lda, 1), _i64x3(sA), B.ptr, max(ldb, 1), _i64x3(sB), Cm.ptr, max(ldc, 1), _i64x3(sC), int(structure))
 
 
 class _AttnLayout:
@@ -486,32 +486,36 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
     bias_a, bias_sh, bias_sb = side(bias, "bias", "bias")
     logits = DeviceArray((S, L, H) + bshape, dt)
     sC = (S * L, S * L * r, S * L * H)
-    _bmm_strided(True, False, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, (lq.sh, lq.sh * r, lq.sb), logits, S, sC)
+    # a causal mask (keep s <= l) leaves whole tiles of the logits unused and makes the weights and every
+    # cotangent of the same shape triangular: the products skip what is known to be zero or unused
+    causal = bool(is_causal)
+    _bmm_strided(True, False, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, (lq.sh, lq.sh * r, lq.sb), logits, S, sC,
+                 1 if causal else 0)
     probs = DeviceArray((S, L, H) + bshape, dt)
     _lib.call("luxhip_attention_softmax_fwd", current_stream(), probs.code, S, L, H, B, logits.ptr, scale_inv,
-              int(bool(is_causal)), _p(mask_a), mask_sh, mask_sb, _p(bias_a), bias_sh, bias_sb, probs.ptr)
+              int(causal), _p(mask_a), mask_sh, mask_sb, _p(bias_a), bias_sh, bias_sb, probs.ptr)
     out = DeviceArray((Ev, H, L) + bshape, dt)
     so = (Ev, Ev * r, Ev * H * L)
-    _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so)
+    _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so, 2 if causal else 0)
 
     def back(d_out: DeviceArray, d_probs: Optional[DeviceArray] = None):
         dp = DeviceArray(probs.shape, dt)
-        _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC)
+        _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC, 1 if causal else 0)
         if d_probs is not None:
             raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: a cotangent for the returned weights")
         dlogits = logits                                              # the logits are no longer needed
-        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L * H * B, dp.ptr, probs.ptr, scale_inv,
-                  dlogits.ptr)
+        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L, L * H * B, int(causal), dp.ptr, probs.ptr,
+                  scale_inv, dlogits.ptr)
         dq = DeviceArray(q.shape, dt)
         _bmm_strided(False, False, E, L, S, bdims, k, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, dq, lq.st,
-                     (lq.sh, lq.sh * r, lq.sb))
+                     (lq.sh, lq.sh * r, lq.sb), 2 if causal else 0)
 
         def kv_grad(like, lay, A, lda, sA, Bm):
             # (rows of `like`) x S = A (rows x L) * Bm' (L x S), one product per head; the heads that share
             # a key/value group are summed afterwards (pullback of repeat_inner_gqa)
             full = DeviceArray(((r,) if r > 1 else ()) + tuple(like.shape), dt)
             _bmm_strided(False, True, lay.E, S, L, bdims, A, lda, sA, Bm, S, sC, full, lay.st,
-                         (like.size if r > 1 else 0, lay.sh, lay.sb))
+                         (like.size if r > 1 else 0, lay.sh, lay.sb), 3 if causal else 0)
             if r == 1:
                 return full
             red = DeviceArray(like.shape, dt)

@@ -16,6 +16,9 @@ CASES = [
     (8, 8, 3, 3, 4, 6, (2,), 3, "mask+bias"), (16, 24, 2, 2, 9, 11, (2, 3), 3, "plain"),
     (64, 64, 8, 2, 128, 128, (2,), 3, "causal"), (64, 64, 4, 4, 130, 257, (1,), 3, "plain"),
     (32, 32, 2, 2, 40, 1100, (1,), 3, "bias"), (64, 128, 4, 4, 256, 256, (2,), 2, "plain"),
+    # causal masks over several tiles: the products skip tiles and parts of the contraction
+    (64, 64, 2, 2, 512, 512, (2,), 3, "causal"), (64, 32, 4, 2, 300, 520, (1,), 3, "causal"),
+    (32, 64, 2, 1, 520, 300, (1,), 2, "causal"),
 ]
 
 
