@@ -231,7 +231,7 @@ __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t,
     // with a triangular structure the tiles of a product differ in cost: the walk through a product
     // starts at a different tile for every product, so that a workgroup (which takes every
     // gridDim.x-th tile of the sequence) does not land on the same tile position each time
-    if (a.structure != 0) ti = (ti + (int)(((int64_t)b * 97) % tiles)) % tiles;
+    if (a.structure != 0) ti = (ti + (int)((((uint32_t)b * 2654435761u) >> 12) % (uint32_t)tiles)) % tiles;   // multiplicative hash of the product index
     int tm, tn;
     tile_coords(ti, a.tiles_m, a.tiles_n, tm, tn);
     const int i0 = b % a.bdim[0], r0 = b / a.bdim[0];
