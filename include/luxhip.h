@@ -331,9 +331,11 @@ typedef struct luxhip_conv_dims {
 
 /* y = act.(conv(x, w) .+ bias[cout]).  Stands behind Impl.conv!(y, ::Type{Dev}, x, w, cdims)
  * (bias == NULL, act identity) and Impl.conv_bias_act(::Type{Dev}, x, w, cdims, bias, act)
- * (src/impl/conv.jl:29-60,138-166).  pre (optional) receives conv .+ bias. */
+ * (src/impl/conv.jl:29-60,138-166).  pre (optional) receives conv .+ bias.  xt_keep (optional, as
+ * large as x): receives the channel-contiguous copy of x that the kernels read; an rrule keeps it
+ * next to x and hands it to luxhip_fused_conv_bwd, which then does not make it again. */
 int luxhip_conv_fwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d, const void* x,
-                    const void* w, const void* bias, void* y, void* pre);
+                    const void* w, const void* bias, void* y, void* pre, void* xt_keep);
 /* dx = ∇conv_data(dy, w, cdims) (src/impl/conv.jl:128-131). */
 int luxhip_conv_bwd_data(luxhip_stream_t s, int dtype, const luxhip_conv_dims_t* d, const void* dy,
                          const void* w, void* dx);
@@ -342,10 +344,10 @@ int luxhip_conv_bwd_filter(luxhip_stream_t s, int dtype, const luxhip_conv_dims_
                            const void* dy, void* dw);
 /* ∇fused_conv (src/impl/conv.jl:261-275): dz = delta .* act'(y, pre); dbias = sum_{w,h,n} dz;
  * dw = ∇conv_filter(x, dz); dx = ∇conv_data(dz, w).  dz: caller scratch like
- * luxhip_fused_dense_bwd. */
+ * luxhip_fused_dense_bwd.  xt_kept (optional): what luxhip_conv_fwd wrote to xt_keep for the same x. */
 int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d,
                           const void* delta, const void* y, const void* pre, const void* x, const void* w,
-                          void* dz, void* dw, void* dx, void* dbias);
+                          void* dz, void* dw, void* dx, void* dbias, const void* xt_kept);
 
 #ifdef __cplusplus
 }

@@ -84,10 +84,10 @@ SIGNATURES = {
     "luxhip_batch_sum": [_vp, _i, _i64, _i64, _vp, _vp],
     "luxhip_fused_dense_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp],
     "luxhip_fused_dense_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp],
-    "luxhip_conv_fwd": [_vp, _i, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp, _vp, _vp],
+    "luxhip_conv_fwd": [_vp, _i, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp, _vp, _vp, _vp],
     "luxhip_conv_bwd_data": [_vp, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp],
     "luxhip_conv_bwd_filter": [_vp, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp],
-    "luxhip_fused_conv_bwd": [_vp, _i, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "luxhip_fused_conv_bwd": [_vp, _i, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
 }
 
 _lib = None

@@ -367,13 +367,15 @@ static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy,
 
 // ----------------------------------------------------------------------------- typed entry points
 template <typename T>
-static int conv_fwd_t(hipStream_t s, int act, const ConvGeom& g, const T* x, const T* w, const T* bias, T* y, T* pre) {
-    const size_t xb = align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
+static int conv_fwd_t(hipStream_t s, int act, const ConvGeom& g, const T* x, const T* w, const T* bias, T* y, T* pre,
+                      T* xt_keep) {
+    // xt_keep: caller's buffer of x's size that keeps the channel-contiguous copy of x for the pullback
+    const size_t xb = xt_keep ? 0 : align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
     const size_t wb = align256((size_t)g.kW * g.kH * g.Cin_g * g.Cout * sizeof(T));
     Workspace ws;
     int rc = get_workspace(s, xb + wb, &ws);
     if (rc != LUXHIP_OK) return rc;
-    T* xT = reinterpret_cast<T*>(ws.data);
+    T* xT = xt_keep ? xt_keep : reinterpret_cast<T*>(ws.data);
     T* wF = reinterpret_cast<T*>(ws.data + xb);
     if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
     if ((rc = pack_filter<T>(s, w, wF, g, 0)) != LUXHIP_OK) return rc;
@@ -414,8 +416,8 @@ static int conv_bwd_filter_t(hipStream_t s, const ConvGeom& g, const T* x, const
 
 template <typename T>
 static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g, const T* delta, const T* y,
-                            const T* pre, const T* x, const T* w, T* dz, T* dw, T* dx, T* dbias) {
-    const size_t xb = align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
+                            const T* pre, const T* x, const T* w, T* dz, T* dw, T* dx, T* dbias, const T* xt_kept) {
+    const size_t xb = xt_kept ? 0 : align256((size_t)g.W * g.H * g.Cin * g.N * sizeof(T));
     const size_t yb = align256((size_t)g.OW * g.OH * g.Cout * g.N * sizeof(T));
     const size_t wb = align256((size_t)g.kW * g.kH * g.Cin_g * g.Cout * sizeof(T));
     const size_t pb = wgrad_partial_bytes<T>(g);
@@ -432,7 +434,7 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
         if (dz_out) dzp = dz_out;
     }
     if (dw == nullptr && dx == nullptr) return LUXHIP_OK;
-    T* xT = reinterpret_cast<T*>(ws.data);
+    const T* xT = xt_kept ? xt_kept : reinterpret_cast<const T*>(ws.data);
     T* dzT = reinterpret_cast<T*>(ws.data + xb);
     T* wD = reinterpret_cast<T*>(ws.data + xb + yb);
     float* partial = reinterpret_cast<float*>(ws.data + xb + yb + wb);
@@ -442,7 +444,8 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
         if ((rc = run_conv_gemm<T>(s, g, true, dzT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY, ws.zeros)) != LUXHIP_OK) return rc;
     }
     if (dw != nullptr) {
-        if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
+        if (!xt_kept && (rc = transpose_to_cwhn<T>(s, x, reinterpret_cast<T*>(ws.data), g.W * g.H, g.Cin, g.N)) != LUXHIP_OK)
+            return rc;
         if ((rc = run_wgrad<T>(s, g, xT, dzp, dzT, partial, dw, ws.zeros)) != LUXHIP_OK) return rc;
     }
     return LUXHIP_OK;
@@ -461,7 +464,7 @@ using namespace luxhip;
 extern "C" {
 
 int luxhip_conv_fwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d, const void* x, const void* w,
-                    const void* bias, void* y, void* pre) {
+                    const void* bias, void* y, void* pre, void* xt_keep) {
     LUX_REQUIRE_INIT();
     int rc = conv_check(dtype, act);
     if (rc != LUXHIP_OK) return rc;
@@ -470,8 +473,10 @@ int luxhip_conv_fwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dim
     if (g.N == 0) return LUXHIP_OK;
     LUX_INVALID_IF(x == nullptr || w == nullptr || y == nullptr, "conv_fwd: x, w and y must not be NULL");
     if (dtype == LUXHIP_F32)
-        return conv_fwd_t<float>((hipStream_t)s, act, g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, (float*)pre);
-    return conv_fwd_t<bf16_t>((hipStream_t)s, act, g, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, (bf16_t*)pre);
+        return conv_fwd_t<float>((hipStream_t)s, act, g, (const float*)x, (const float*)w, (const float*)bias, (float*)y, (float*)pre,
+                                 (float*)xt_keep);
+    return conv_fwd_t<bf16_t>((hipStream_t)s, act, g, (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, (bf16_t*)y, (bf16_t*)pre,
+                              (bf16_t*)xt_keep);
 }
 
 int luxhip_conv_bwd_data(luxhip_stream_t s, int dtype, const luxhip_conv_dims_t* d, const void* dy, const void* w, void* dx) {
@@ -501,7 +506,7 @@ int luxhip_conv_bwd_filter(luxhip_stream_t s, int dtype, const luxhip_conv_dims_
 
 int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_conv_dims_t* d, const void* delta,
                           const void* y, const void* pre, const void* x, const void* w, void* dz, void* dw, void* dx,
-                          void* dbias) {
+                          void* dbias, const void* xt_kept) {
     LUX_REQUIRE_INIT();
     int rc = conv_check(dtype, act);
     if (rc != LUXHIP_OK) return rc;
@@ -517,12 +522,14 @@ int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_co
     LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && dz == nullptr, "fused_conv_bwd: dz scratch is required");
     LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && !act_needs_pre(act) && y == nullptr, "fused_conv_bwd: activation %d needs y", act);
     LUX_INVALID_IF(act_needs_pre(act) && pre == nullptr, "fused_conv_bwd: activation %d needs the pre-activation", act);
-    LUX_INVALID_IF((dw != nullptr && x == nullptr) || (dx != nullptr && w == nullptr), "fused_conv_bwd: x / w must not be NULL");
+    LUX_INVALID_IF((dw != nullptr && x == nullptr && xt_kept == nullptr) || (dx != nullptr && w == nullptr), "fused_conv_bwd: x / w must not be NULL");
     if (dtype == LUXHIP_F32)
         return fused_conv_bwd_t<float>((hipStream_t)s, dtype, act, g, (const float*)delta, (const float*)y, (const float*)pre,
-                                       (const float*)x, (const float*)w, (float*)dz, (float*)dw, (float*)dx, (float*)dbias);
+                                       (const float*)x, (const float*)w, (float*)dz, (float*)dw, (float*)dx, (float*)dbias,
+                                       (const float*)xt_kept);
     return fused_conv_bwd_t<bf16_t>((hipStream_t)s, dtype, act, g, (const bf16_t*)delta, (const bf16_t*)y, (const bf16_t*)pre,
-                                    (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)dz, (bf16_t*)dw, (bf16_t*)dx, (bf16_t*)dbias);
+                                    (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)dz, (bf16_t*)dw, (bf16_t*)dx, (bf16_t*)dbias,
+                                    (const bf16_t*)xt_kept);
 }
 
 }  // extern "C"

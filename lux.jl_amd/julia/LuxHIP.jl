@@ -278,16 +278,16 @@ function Impl.conv_bias_act(::Type{LuxHIPDevice}, x::HIPArray{T,4}, w::HIPArray{
     y = similar(x, T, (NNlib.output_size(cdims)..., NNlib.channels_out(cdims), size(x, 4)))
     d = Ref(ConvDimsC(cdims, size(x, 4)))
     ok = id !== nothing && check(ccall((:luxhip_conv_fwd, libluxhip), Cint,
-        (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), id, d, optr(x), optr(w), optr(bias), optr(y), C_NULL))
+        (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), id, d, optr(x), optr(w), optr(bias), optr(y), C_NULL, C_NULL))
     ok || return invoke(Impl.conv_bias_act, Tuple{Type,Any,Any,Any,Any,Any}, Nothing, x, w, cdims, bias, act)
     return y
 end
 function Impl.conv!(y::HIPArray{T,4}, ::Type{LuxHIPDevice}, x::HIPArray{T,4}, w::HIPArray{T,4}, cdims::DenseConvDims{2}) where {T<:HIPFloat}
     d = Ref(ConvDimsC(cdims, size(x, 4)))
     check(ccall((:luxhip_conv_fwd, libluxhip), Cint,
-        (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), Cint(0), d, optr(x), optr(w), C_NULL, optr(y), C_NULL)) || NNlib.conv!(y, x, w, cdims)
+        (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), Cint(0), d, optr(x), optr(w), C_NULL, optr(y), C_NULL, C_NULL)) || NNlib.conv!(y, x, w, cdims)
     return nothing
 end
 function Impl.∇conv_data(dy::HIPArray{T,4}, w::HIPArray{T,4}, cdims::DenseConvDims{2}) where {T<:HIPFloat}

@@ -830,7 +830,7 @@ def fused_conv_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b,
     dt = _same_dtype(weight, x, b)
     y = DeviceArray(cdims.y_shape, dt)
     _lib.call("luxhip_conv_fwd", current_stream(), y.code, _act_id(act), C.byref(cdims._c), x.ptr, weight.ptr, _p(b),
-              y.ptr, None)
+              y.ptr, None, None)
     return y
 
 
@@ -841,7 +841,9 @@ def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDim
     dt = _same_dtype(weight, x, b)
     y = DeviceArray(cdims.y_shape, dt)
     pre = DeviceArray(cdims.y_shape, dt) if aid in _NEEDS_PRE else None
-    _lib.call("luxhip_conv_fwd", current_stream(), y.code, aid, C.byref(cdims._c), x.ptr, weight.ptr, _p(b), y.ptr, _p(pre))
+    xt = DeviceArray(x.shape, dt)      # the channel-contiguous copy of x, kept for the filter gradient
+    _lib.call("luxhip_conv_fwd", current_stream(), y.code, aid, C.byref(cdims._c), x.ptr, weight.ptr, _p(b), y.ptr, _p(pre),
+              xt.ptr)
 
     def back(delta):
         dw = DeviceArray(weight.shape, dt)
@@ -849,7 +851,7 @@ def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDim
         db = None if b is None else DeviceArray(b.shape, dt)
         dz = None if aid == 0 else DeviceArray(cdims.y_shape, dt)
         _lib.call("luxhip_fused_conv_bwd", current_stream(), y.code, aid, C.byref(cdims._c), delta.ptr, y.ptr, _p(pre),
-                  x.ptr, weight.ptr, _p(dz), dw.ptr, dx.ptr, _p(db))
+                  x.ptr, weight.ptr, _p(dz), dw.ptr, dx.ptr, _p(db), xt.ptr)
         return dw, dx, db
 
     return y, back
