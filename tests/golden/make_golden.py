@@ -73,6 +73,33 @@ def main():
     y, dw, dx, db = O.fused_conv_pullback("sigmoid", cw, cx, cb, cd, cdelta)
     g.update(conv_x=cx, conv_w=cw, conv_b=cb, conv_delta=cdelta, conv_y=y, conv_dw=dw, conv_dx=dx, conv_db=db)
 
+    # --- instancenorm (instancenorm_tests.jl shape (4,4,6,2)), training with running statistics, relu
+    y, rm2, rv2 = O.instancenorm(x, gm, bt, rm, rv, True, "relu", 0.1, 1e-5)
+    dx, dg, dbt = O.instancenorm_pullback(x, gm, bt, "relu", 1e-5, delta)
+    g.update(in_y=y, in_rmean_out=rm2, in_rvar_out=rv2, in_dx=dx, in_dgamma=dg, in_dbeta=dbt)
+
+    # --- batched_matmul (bmm_tests.jl: a shared left operand, the right one contracted along its second dim)
+    bx, by = fixed((4, 5, 1), 0.5), fixed((6, 5, 3), 0.5, 2.0)
+    bz = O.batched_matmul(bx, by, 2, 2)
+    bdelta = np.cos(np.arange(bz.size)).reshape(bz.shape, order="F")
+    bdx, bdy = O.batched_matmul_pullback(bx, by, bdelta, 2, 2)
+    g.update(bmm_x=bx, bmm_y=by, bmm_z=bz, bmm_delta=bdelta, bmm_dx=bdx, bmm_dy=bdy)
+
+    # --- scaled_dot_product_attention (attention_tests.jl): 4 query heads on 2 key/value heads, causal
+    aq, ak, av = fixed((8, 4, 5, 2), 0.5, 2.0), fixed((8, 2, 5, 2), 0.5, 2.0), fixed((6, 2, 5, 2), 0.5)
+    ao, aw = O.scaled_dot_product_attention(aq, ak, av, 3, None, None, True, None)
+    adelta = np.sin(np.arange(ao.size)).reshape(ao.shape, order="F")
+    adq, adk, adv = O.scaled_dot_product_attention_pullback(aq, ak, av, adelta, 3, None, None, True, None)
+    g.update(attn_q=aq, attn_k=ak, attn_v=av, attn_out=ao, attn_weights=aw, attn_delta=adelta, attn_dq=adq, attn_dk=adk,
+             attn_dv=adv)
+
+    # --- dropout: the first 24 values of the noise stream (seed 7, offset 2; the Philox4x32-10 known-answer
+    #     vectors themselves are checked in tests/test_oracle_dropout.py), the mask and the product for p = 0.25
+    dnoise = O.rand_uniform(24, 7, 2).astype(np.float64).reshape((4, 3, 2), order="F")
+    dxin = fixed((4, 3, 2), 0.5, 2.0)
+    dy_, dmask = O.dropout(dnoise.astype(np.float32), dxin.astype(np.float32), 0.25, True, 1.0 / 0.75)
+    g.update(drop_noise=dnoise, drop_x=dxin, drop_mask=dmask, drop_y=dy_)
+
     np.savez_compressed(OUT, **{k: np.asarray(v, dtype=np.float64) for k, v in g.items()})
     print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(g), "arrays")
 

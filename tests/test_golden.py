@@ -27,6 +27,14 @@ def test_oracle_reproduces_golden_vectors():
     y, dw, dx, db = O.fused_conv_pullback("sigmoid", G["conv_w"], G["conv_x"], G["conv_b"], cd, G["conv_delta"])
     for got, k in ((y, "conv_y"), (dw, "conv_dw"), (dx, "conv_dx"), (db, "conv_db")):
         np.testing.assert_allclose(got, G[k], rtol=1e-12, atol=1e-13)
+    y, rm, rv = O.instancenorm(G["bn_x"], G["bn_gamma"], G["bn_beta"], G["bn_rmean"], G["bn_rvar"], True, "relu", 0.1, 1e-5)
+    for got, k in ((y, "in_y"), (rm, "in_rmean_out"), (rv, "in_rvar_out")):
+        np.testing.assert_allclose(got, G[k], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(O.batched_matmul(G["bmm_x"], G["bmm_y"], 2, 2), G["bmm_z"], rtol=1e-13, atol=1e-14)
+    out, w = O.scaled_dot_product_attention(G["attn_q"], G["attn_k"], G["attn_v"], 3, None, None, True, None)
+    np.testing.assert_allclose(out, G["attn_out"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(w, G["attn_weights"], rtol=1e-12, atol=1e-14)
+    np.testing.assert_array_equal(O.rand_uniform(24, 7, 2).reshape((4, 3, 2), order="F"), G["drop_noise"].astype(np.float32))
 
 
 @pytest.mark.gpu
@@ -61,3 +69,23 @@ def test_hip_path_matches_golden_vectors(gpu):
     np.testing.assert_allclose(yk.to_numpy(), G["kat_bn_y"], atol=1e-5)
     np.testing.assert_allclose(stk["running_mean"].to_numpy(), G["kat_bn_running_mean"], rtol=1e-6)
     np.testing.assert_allclose(stk["running_var"].to_numpy(), G["kat_bn_running_var"], rtol=1e-6)
+    # the widened operators
+    (y, st), back = gpu.pullback(gpu.instancenorm, d("bn_x"), d("bn_gamma"), d("bn_beta"), d("bn_rmean"), d("bn_rvar"), True,
+                                 "relu", 0.1, 1e-5)
+    dx, dg, dbt = back(d("bn_delta"))
+    chk(y, "in_y"); chk(st["running_mean"], "in_rmean_out"); chk(st["running_var"], "in_rvar_out")
+    chk(dx, "in_dx", scale=2.0); chk(dg, "in_dgamma", scale=1.0); chk(dbt, "in_dbeta", scale=1.0)
+    z, back = gpu.pullback(gpu.batched_matmul, d("bmm_x"), d("bmm_y"), 2, 2)
+    dx, dy = back(d("bmm_delta"))
+    chk(z, "bmm_z", scale=1.0); chk(dx, "bmm_dx", scale=2.0); chk(dy, "bmm_dy", scale=1.0)
+    (out, w), back = gpu.pullback(gpu.scaled_dot_product_attention, d("attn_q"), d("attn_k"), d("attn_v"), 1, 3, None, None, True,
+                                  None)
+    dq, dk, dv = back(d("attn_delta"))
+    chk(out, "attn_out"); chk(w, "attn_weights"); chk(dq, "attn_dq", scale=0.5); chk(dk, "attn_dk", scale=0.5)
+    chk(dv, "attn_dv", scale=0.5)
+    rng = gpu.PhiloxRNG(7, 2)
+    noise, _ = gpu.rand_uniform(rng, (4, 3, 2))
+    np.testing.assert_array_equal(noise.to_numpy(), G["drop_noise"].astype(np.float32))
+    y, mask, _ = gpu.dropout(rng, d("drop_x"), 0.25, True, 1.0 / 0.75)
+    np.testing.assert_array_equal(mask.to_numpy(), G["drop_mask"].astype(np.float32))
+    np.testing.assert_array_equal(y.to_numpy(), G["drop_y"].astype(np.float32))
