@@ -28,12 +28,20 @@ from __graft_entry__ import load_package  # noqa: E402
 PEAK_HBM_GBS = 8000.0                 # MI355X HBM3E
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
-# size (profiles/c2_hbm_traffic_pmc.md holds the commands and the raw counter values).
+# size (profiles/*_hbm_traffic_pmc.md hold the commands and the raw counter values).
 MEASURED_TRAFFIC = {
     ("C2", "bn_fwd_resident_kernel"): 67764601,
     ("C2", "bias_act_fwd_kernel"): 67138039,
     ("C2", "bias_act_bwd_channel_kernel"): 100918103,
     ("C2", "bn_bwd_resident_kernel"): 100979652,
+    ("C3", "gn_fwd_kernel"): 134324931,
+    ("C3", "gn_bwd_kernel"): 202195147,
+    ("C3bf16", "gn_fwd_kernel"): 67290712,
+    ("C3bf16", "gn_bwd_kernel"): 101301450,
+    ("IN", "gn_fwd_kernel"): 134569817,
+    ("IN", "gn_bwd_kernel"): 202845995,
+    ("DROPOUT", "dropout_fwd_kernel"): 100695712,      # dropout_rng_kernel<float, 4, 2> in the trace
+    ("DROPOUT", "dropout_mul_kernel"): 100691762,
 }
 METRIC = "fwd+bwd TFLOP/s & HBM GB/s (% MI355X roofline) per LuxLib fused op, 1 GPU"
 
