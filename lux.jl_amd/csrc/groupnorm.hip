@@ -584,7 +584,12 @@ int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64
     int rc = gn_check(dtype, act, I, C, G, N);
     if (rc != LUXHIP_OK) return rc;
     LUX_INVALID_IF((gamma == nullptr) != (beta == nullptr), "groupnorm_bwd: gamma and beta must be given together");
-    if (I * C * N == 0) return LUXHIP_OK;
+    if (I * C * N == 0) {   // nothing to read: the parameter gradients are empty sums
+        const size_t bytes = (size_t)C * (dtype == LUXHIP_F32 ? 4 : 2);
+        if (C > 0 && dgamma) { rc = luxhip_fill_zero(dgamma, bytes, s); if (rc) return rc; }
+        if (C > 0 && dbeta) { rc = luxhip_fill_zero(dbeta, bytes, s); if (rc) return rc; }
+        return LUXHIP_OK;
+    }
     LUX_INVALID_IF(delta == nullptr || x == nullptr || dx == nullptr || save_mean == nullptr || save_invstd == nullptr,
                    "groupnorm_bwd: delta, x, dx, save_mean and save_invstd must not be NULL");
     if (dtype == LUXHIP_F32)
