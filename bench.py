@@ -350,6 +350,38 @@ class C5Conv(_ApiWorkload):
         return {f"conv_fprop_kernel<{t}>": f, f"conv_dgrad_kernel<{t}>": f, f"conv_wgrad_kernel<{t}>": f}
 
 
+class Conv3d(_ApiWorkload):
+    """fused_conv_bias_activation with three spatial dims: 3x3x3, 64->128, volumes 32x32x16, batch 8, pad 1, relu.
+    Runs as the two-dimensional problem on the depth-unfolded input (192 channels, 128 samples)."""
+    bound = "mfma"
+    xs, ws = (32, 32, 16, 64, 8), (3, 3, 3, 64, 128)
+
+    def __init__(self, dtype="bf16"):
+        self.dtype = dtype
+        self.name = "CONV3D" if dtype == "bf16" else "CONV3Df32"
+        self.description = f"fused_conv_bias_activation(relu) 3x3x3 64->128, x 32x32x16x64x8, pad 1, fwd+bwd {dtype}"
+
+    def build(self, lux):
+        rng = np.random.default_rng(1013)
+        self.cd = lux.DenseConvDims(self.xs, self.ws, padding=1)
+        self.x = self.d(rng.standard_normal(size=self.xs, dtype=np.float32))
+        self.w = self.d(np.sqrt(2.0 / 1728) * rng.standard_normal(size=self.ws, dtype=np.float32))
+        self.b = self.d((0.01 * rng.standard_normal(128)).astype(np.float32))
+        self.delta = self.d(rng.standard_normal(size=self.cd.y_shape, dtype=np.float32))
+
+    def step(self):
+        y, back = self.lux.pullback(self.lux.fused_conv_bias_activation, "relu", self.w, self.x, self.b, self.cd)
+        back(self.delta)
+
+    def work_per_step(self):
+        return 3 * 2.0 * (32 * 32 * 16 * 8) * 128 * 1728
+
+    def kernel_work(self):
+        f = 2.0 * (32 * 32 * 16 * 8) * 128 * 1728
+        t = "bf16" if self.dtype == "bf16" else "f32"
+        return {f"conv_fprop_kernel<{t}>": f, f"conv_dgrad_kernel<{t}>": f, f"conv_wgrad_kernel<{t}>": f}
+
+
 class InstanceNorm(_ApiWorkload):
     """instancenorm (training, running statistics updated) + relu, x 64x64x256x16 fp32: one slice per channel and sample."""
     name, bound, dtype = "IN", "hbm", "f32"
@@ -423,7 +455,8 @@ class Attention(_ApiWorkload):
 
 
 WORKLOADS = {"IN": InstanceNorm, "DROPOUT": Dropout, "SDPA": Attention, "C1": C1Dense, "C2": C2BatchnormBiasAct, "C3": lambda: C3Groupnorm("f32"), "C3bf16": lambda: C3Groupnorm("bf16"),
-             "C4": C4TransformerMLP, "C5": lambda: C5Conv("f32"), "C5bf16": lambda: C5Conv("bf16")}
+             "C4": C4TransformerMLP, "C5": lambda: C5Conv("f32"), "C5bf16": lambda: C5Conv("bf16"),
+             "CONV3D": lambda: Conv3d("bf16"), "CONV3Df32": lambda: Conv3d("f32")}
 
 
 # ----------------------------------------------------------------------------- timing

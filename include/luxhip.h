@@ -349,6 +349,27 @@ int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_co
                           const void* delta, const void* y, const void* pre, const void* x, const void* w,
                           void* dz, void* dw, void* dx, void* dbias, const void* xt_kept);
 
+/* Convolutions with three spatial dims (x (W, H, D, C, N), w (kW, kH, kD, C/groups, Cout)): the
+ * reference hands them to the same NNlib.conv / ∇conv_data / ∇conv_filter calls as the
+ * two-dimensional ones (src/impl/conv.jl:29-60,128-136).  Here they run as the two-dimensional
+ * problem on the depth-unfolded input: xu (W, H, kD*C, Dout*N), channel kd + kD*c of sample
+ * od + Dout*n = depth slice od*stride_d + tap*dil_d - pad_d_lo of x (zeros outside), tap = kD-1-kd
+ * for true convolution and kd with flipkernel; the weight read as (kW, kH, kD*C/groups, Cout) needs
+ * no copy.  plane = W*H. */
+int luxhip_conv_depth_unfold(luxhip_stream_t s, int dtype, int64_t plane, int64_t D, int64_t C, int64_t N, int64_t KD,
+                             int64_t Dout, int64_t stride_d, int64_t pad_d_lo, int64_t dil_d, int flipkernel, const void* x,
+                             void* xu);
+/* The adjoint of luxhip_conv_depth_unfold: dx (plane, D, C, N) gathers, in a fixed order, the terms
+ * of dxu (plane, kD*C, Dout, N) that the unfolding copied from it (∇conv_data of a three-dimensional
+ * problem = this applied to the two-dimensional ∇conv_data). */
+int luxhip_conv_depth_fold(luxhip_stream_t s, int dtype, int64_t plane, int64_t D, int64_t C, int64_t N, int64_t KD,
+                           int64_t Dout, int64_t stride_d, int64_t pad_d_lo, int64_t dil_d, int flipkernel, const void* dxu,
+                           void* dx);
+/* out (inner, B, A, outer) = permutedims(in (inner, A, B, outer), (1, 3, 2, 4)): between the output
+ * of the two-dimensional problem, (OW*OH, Cout, Dout, N), and the caller's (OW*OH, Dout, Cout, N). */
+int luxhip_swap_middle_dims(luxhip_stream_t s, int dtype, int64_t inner, int64_t A, int64_t B, int64_t outer, const void* in,
+                            void* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,9 @@ SIGNATURES = {
     "luxhip_conv_bwd_data": [_vp, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp],
     "luxhip_conv_bwd_filter": [_vp, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp],
     "luxhip_fused_conv_bwd": [_vp, _i, _i, C.POINTER(ConvDimsStruct), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "luxhip_conv_depth_unfold": [_vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp],
+    "luxhip_conv_depth_fold": [_vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp],
+    "luxhip_swap_middle_dims": [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp],
 }
 
 _lib = None

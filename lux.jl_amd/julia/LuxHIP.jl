@@ -305,6 +305,69 @@ function Impl.∇conv_filter(x::HIPArray{T,4}, dy::HIPArray{T,4}, cdims::DenseCo
     return dw
 end
 
+# Three spatial dims (x (W, H, D, C, N), DenseConvDims{3}): the two-dimensional problem on the
+# depth-unfolded input.  `inner2d` is the DenseConvDims{2} over (W, H, kD*C, Dout*N); the weight is
+# reshaped, not copied.
+function inner2d(c::DenseConvDims{3}, N::Integer)
+    (W, H, D), (kW, kH, kD) = NNlib.input_size(c), NNlib.kernel_size(c)
+    Dout = NNlib.output_size(c)[3]
+    g = NNlib.groupcount(c)
+    return DenseConvDims((W, H, kD * NNlib.channels_in(c), Dout * N), (kW, kH, kD * (NNlib.channels_in(c) ÷ g), NNlib.channels_out(c));
+        stride=NNlib.stride(c)[1:2], padding=NNlib.padding(c)[1:4], dilation=NNlib.dilation(c)[1:2], groups=g,
+        flipkernel=NNlib.flipkernel(c))
+end
+depth_args(c::DenseConvDims{3}, N::Integer) = (Int64(prod(NNlib.input_size(c)[1:2])), Int64(NNlib.input_size(c)[3]),
+    Int64(NNlib.channels_in(c)), Int64(N), Int64(NNlib.kernel_size(c)[3]), Int64(NNlib.output_size(c)[3]),
+    Int64(NNlib.stride(c)[3]), Int64(NNlib.padding(c)[5]), Int64(NNlib.dilation(c)[3]), Cint(NNlib.flipkernel(c)))
+const DepthSig = (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid})
+function depth_unfold(x::HIPArray{T,5}, c::DenseConvDims{3}) where {T<:HIPFloat}
+    c2 = inner2d(c, size(x, 5))
+    xu = similar(x, T, (NNlib.input_size(c2)..., NNlib.channels_in(c2), NNlib.output_size(c)[3] * size(x, 5)))
+    check(ccall((:luxhip_conv_depth_unfold, libluxhip), Cint, DepthSig, stream(), dtype_code(T), depth_args(c, size(x, 5))..., optr(x), optr(xu))) ||
+        error("luxhip_conv_depth_unfold")
+    return xu, c2
+end
+function depth_fold(dxu::HIPArray{T,4}, c::DenseConvDims{3}, N::Integer) where {T<:HIPFloat}
+    dx = similar(dxu, T, (NNlib.input_size(c)..., NNlib.channels_in(c), N))
+    check(ccall((:luxhip_conv_depth_fold, libluxhip), Cint, DepthSig, stream(), dtype_code(T), depth_args(c, N)..., optr(dxu), optr(dx))) ||
+        error("luxhip_conv_depth_fold")
+    return dx
+end
+function swap_middle(a::HIPArray{T}, inner, A, B, outer, shape) where {T<:HIPFloat}
+    out = similar(a, T, shape)
+    check(ccall((:luxhip_swap_middle_dims, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), inner, A, B, outer, optr(a), optr(out))) || error("luxhip_swap_middle_dims")
+    return out
+end
+function from_inner(y2::HIPArray{T,4}, c::DenseConvDims{3}, N) where {T}     # (OW, OH, Cout, Dout*N) -> (OW, OH, Dout, Cout, N)
+    (ow, oh, od), co = NNlib.output_size(c), NNlib.channels_out(c)
+    return swap_middle(y2, ow * oh, co, od, N, (ow, oh, od, co, N))
+end
+function to_inner(dy::HIPArray{T,5}, c::DenseConvDims{3}) where {T}          # the inverse
+    (ow, oh, od), co, N = NNlib.output_size(c), NNlib.channels_out(c), size(dy, 5)
+    return swap_middle(dy, ow * oh, od, co, N, (ow, oh, co, od * N))
+end
+w2d(w::HIPArray{T,5}) where {T} = reshape(w, size(w, 1), size(w, 2), size(w, 3) * size(w, 4), size(w, 5))
+
+function Impl.conv_bias_act(::Type{LuxHIPDevice}, x::HIPArray{T,5}, w::HIPArray{T,5}, cdims::DenseConvDims{3}, bias, act::F) where {F,T<:HIPFloat}
+    xu, c2 = depth_unfold(x, cdims)
+    return from_inner(Impl.conv_bias_act(LuxHIPDevice, xu, w2d(w), c2, bias, act), cdims, size(x, 5))
+end
+function Impl.conv!(y::HIPArray{T,5}, ::Type{LuxHIPDevice}, x::HIPArray{T,5}, w::HIPArray{T,5}, cdims::DenseConvDims{3}) where {T<:HIPFloat}
+    xu, c2 = depth_unfold(x, cdims)
+    y2 = similar(y, T, (NNlib.output_size(c2)..., NNlib.channels_out(c2), size(xu, 4)))
+    Impl.conv!(y2, LuxHIPDevice, xu, w2d(w), c2)
+    copyto!(y, from_inner(y2, cdims, size(x, 5)))
+    return nothing
+end
+Impl.∇conv_data(dy::HIPArray{T,5}, w::HIPArray{T,5}, cdims::DenseConvDims{3}) where {T<:HIPFloat} =
+    depth_fold(Impl.∇conv_data(to_inner(dy, cdims), w2d(w), inner2d(cdims, size(dy, 5))), cdims, size(dy, 5))
+function Impl.∇conv_filter(x::HIPArray{T,5}, dy::HIPArray{T,5}, cdims::DenseConvDims{3}) where {T<:HIPFloat}
+    xu, c2 = depth_unfold(x, cdims)
+    return reshape(Impl.∇conv_filter(xu, to_inner(dy, cdims), c2), NNlib.kernel_size(cdims)...,
+        NNlib.channels_in(cdims) ÷ NNlib.groupcount(cdims), NNlib.channels_out(cdims))
+end
+
 # ---------------------------------------------------------------------------------------------
 # batched_matmul: Impl.batched_matmul!(z, opmode, x, y)  (impl/batched_mul.jl:204-212) and the
 # products of the rrule (:320-334), which arrive as NNlib.BatchedAdjoint wrappers

@@ -768,8 +768,10 @@ def rrule_layernorm(x, scale, bias, act="identity", dims=DEFAULT_DIMS, epsilon=N
 # ------------------------------------------------------------------------------- conv
 @dataclass
 class DenseConvDims:
-    """The fields of NNlib.DenseConvDims this path consumes (1 or 2 spatial dims: x (W, C, N) or
-    (W, H, C, N)).  padding = (w_lo, w_hi[, h_lo, h_hi]); flipkernel=False is true convolution."""
+    """The fields of NNlib.DenseConvDims this path consumes (1, 2 or 3 spatial dims: x (W, C, N),
+    (W, H, C, N) or (W, H, D, C, N)).  padding = (w_lo, w_hi[, h_lo, h_hi[, d_lo, d_hi]]);
+    flipkernel=False is true convolution.  Three spatial dims run as the two-dimensional problem
+    `inner` on the depth-unfolded input (kD*C channels, Dout*N samples)."""
     x_shape: Tuple[int, ...]
     w_shape: Tuple[int, ...]
     stride: Tuple[int, ...] = 1
@@ -781,8 +783,8 @@ class DenseConvDims:
 
     def __post_init__(self):
         self.x_shape, self.w_shape = tuple(self.x_shape), tuple(self.w_shape)
-        if len(self.x_shape) != len(self.w_shape) or len(self.x_shape) not in (3, 4):
-            raise _lib.Unsupported(_lib.UNSUPPORTED, "only 1 or 2 spatial dimensions are handled on the device")
+        if len(self.x_shape) != len(self.w_shape) or len(self.x_shape) not in (3, 4, 5):
+            raise _lib.Unsupported(_lib.UNSUPPORTED, "only 1, 2 or 3 spatial dimensions are handled on the device")
         self.spatial = len(self.x_shape) - 2
         one = self.spatial == 1           # (W, C, N): the same memory as (W, 1, C, N), a 2-d problem of height 1
         if isinstance(self.stride, int):
@@ -796,6 +798,16 @@ class DenseConvDims:
         self.stride, self.dilation, self.padding = tuple(self.stride), tuple(self.dilation), tuple(self.padding)
         if len(self.stride) != self.spatial or len(self.dilation) != self.spatial or len(self.padding) != 2 * self.spatial:
             raise DimensionMismatch("stride, dilation and padding must match the number of spatial dimensions")
+        self.inner = None
+        if self.spatial == 3:
+            W, H, D, Cin, N = self.x_shape
+            kW, kH, kD, Cg, Cout = self.w_shape
+            if Cg * self.groups != Cin:
+                raise DimensionMismatch(f"input channels {Cin} != weight channels {Cg} x groups {self.groups}")
+            dout = self.out_spatial[2]
+            self.inner = DenseConvDims((W, H, kD * Cin, dout * N), (kW, kH, kD * Cg, Cout), self.stride[:2], self.padding[:4],
+                                       self.dilation[:2], self.groups, self.flipkernel)
+            return
         stride, dil, pad = ((self.stride + (1,), self.dilation + (1,), self.padding + (0, 0)) if one
                             else (self.stride, self.dilation, self.padding))
         W, H, Cin, N = (self.x_shape[0], 1) + self.x_shape[1:] if one else self.x_shape
@@ -828,10 +840,54 @@ def fused_conv_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b,
     """`fused_conv_bias_activation(σ, weight, x, b, cdims)` (api/conv.jl:30-38)."""
     _check_conv(weight, x, b, cdims)
     dt = _same_dtype(weight, x, b)
+    if cdims.inner is not None:
+        return _from_inner_output(cdims, fused_conv_bias_activation(act, _inner_weight(cdims, weight), _depth_unfold(cdims, x), b,
+                                                                    cdims.inner))
     y = DeviceArray(cdims.y_shape, dt)
     _lib.call("luxhip_conv_fwd", current_stream(), y.code, _act_id(act), C.byref(cdims._c), x.ptr, weight.ptr, _p(b),
               y.ptr, None, None)
     return y
+
+
+# Three spatial dims: the depth-unfolded two-dimensional problem.
+def _depth_args(cdims, N):
+    W, H, D, Cin, _ = cdims.x_shape
+    return (W * H, D, Cin, N, cdims.w_shape[2], cdims.out_spatial[2], cdims.stride[2], cdims.padding[4], cdims.dilation[2],
+            int(cdims.flipkernel))
+
+
+def _depth_unfold(cdims, x):
+    xu = DeviceArray(cdims.inner.x_shape, x.dtype)
+    _lib.call("luxhip_conv_depth_unfold", current_stream(), x.code, *_depth_args(cdims, x.shape[-1]), x.ptr, xu.ptr)
+    return xu
+
+
+def _depth_fold(cdims, dxu):
+    dx = DeviceArray(cdims.x_shape, dxu.dtype)
+    _lib.call("luxhip_conv_depth_fold", current_stream(), dx.code, *_depth_args(cdims, cdims.x_shape[-1]), dxu.ptr, dx.ptr)
+    return dx
+
+
+def _inner_weight(cdims, weight):
+    return weight.reshape(cdims.inner.w_shape)        # the same memory: channel kd + kD*c
+
+
+def _from_inner_output(cdims, y2):
+    """(OW, OH, Cout, Dout*N) of the inner problem -> (OW, OH, Dout, Cout, N)."""
+    ow, oh, dout = cdims.out_spatial
+    cout, n = cdims.w_shape[-1], cdims.x_shape[-1]
+    y = DeviceArray((ow, oh, dout, cout, n), y2.dtype)
+    _lib.call("luxhip_swap_middle_dims", current_stream(), y.code, ow * oh, cout, dout, n, y2.ptr, y.ptr)
+    return y
+
+
+def _to_inner_output(cdims, dy):
+    """(OW, OH, Dout, Cout, N) -> (OW, OH, Cout, Dout*N)."""
+    ow, oh, dout = cdims.out_spatial
+    cout, n = cdims.w_shape[-1], cdims.x_shape[-1]
+    d2 = DeviceArray((ow, oh, cout, dout * n), dy.dtype)
+    _lib.call("luxhip_swap_middle_dims", current_stream(), dy.code, ow * oh, dout, cout, n, dy.ptr, d2.ptr)
+    return d2
 
 
 def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDims):
@@ -839,6 +895,14 @@ def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDim
     _check_conv(weight, x, b, cdims)
     aid = _act_id(act)
     dt = _same_dtype(weight, x, b)
+    if cdims.inner is not None:
+        y2, back2 = rrule_fused_conv_bias_activation(act, _inner_weight(cdims, weight), _depth_unfold(cdims, x), b, cdims.inner)
+
+        def back3(delta):
+            dw2, dxu, db = back2(_to_inner_output(cdims, delta))
+            return dw2.reshape(cdims.w_shape), _depth_fold(cdims, dxu), db
+
+        return _from_inner_output(cdims, y2), back3
     y = DeviceArray(cdims.y_shape, dt)
     pre = DeviceArray(cdims.y_shape, dt) if aid in _NEEDS_PRE else None
     xt = DeviceArray(x.shape, dt)      # the channel-contiguous copy of x, kept for the filter gradient
@@ -864,6 +928,8 @@ def conv(x, weight, cdims):
 
 def conv_data_grad(dy, weight, cdims):
     """`Impl.∇conv_data` (impl/conv.jl:128-131)."""
+    if cdims.inner is not None:
+        return _depth_fold(cdims, conv_data_grad(_to_inner_output(cdims, dy), _inner_weight(cdims, weight), cdims.inner))
     dx = DeviceArray(cdims.x_shape, dy.dtype)
     _lib.call("luxhip_conv_bwd_data", current_stream(), dy.code, C.byref(cdims._c), dy.ptr, weight.ptr, dx.ptr)
     return dx
@@ -871,6 +937,8 @@ def conv_data_grad(dy, weight, cdims):
 
 def conv_filter_grad(x, dy, cdims):
     """`Impl.∇conv_filter` (impl/conv.jl:133-136)."""
+    if cdims.inner is not None:
+        return conv_filter_grad(_depth_unfold(cdims, x), _to_inner_output(cdims, dy), cdims.inner).reshape(cdims.w_shape)
     dw = DeviceArray(cdims.w_shape, x.dtype)
     _lib.call("luxhip_conv_bwd_filter", current_stream(), x.code, C.byref(cdims._c), x.ptr, dy.ptr, dw.ptr)
     return dw

@@ -33,6 +33,10 @@ tests/test_oracle_*.py):
   * conv / dgrad / wgrad .............. reference known answers (impulse response,
                                         asymmetric-pad counts), brute-force 7-loop direct
                                         convolution, torch conv2d with flipped kernel
+  * conv_nd / its gradients (k dims) .. the 2-d functions above at k = 2; scipy.signal
+                                        convolve / correlate ('valid') at k = 3; an
+                                        element-by-element definition with strides, asymmetric
+                                        padding, dilation and groups; adjoint identities
   * PARITY UNPINNED: the bit pattern of the reference's dropout masks (drawn from Julia's rng,
     which cannot run here); `rand_uniform` is a Philox stream of the same distribution.
   * NNlib's `tanh_fast`/`sigmoid_fast` rational approximations, exact `gelu` constants and
@@ -918,6 +922,101 @@ def fused_conv_pullback(act: str, w, x, b, cd: ConvDims, delta):
     dy = grad_activation(delta, y, act, pre)
     db = grad_bias_add(b, dy)
     return y, conv_filter_grad(x, dy, cd), conv_data_grad(dy, w, cd), db
+
+
+# --------------------------------------------------------------------------------------
+# convolutions with any number of spatial dims (the reference passes 1-, 2- and 3-d problems to the
+# same NNlib calls, impl/conv.jl:29-60,128-136): x (S1..Sk, C, N), w (K1..Kk, C/groups, Cout)
+# --------------------------------------------------------------------------------------
+class ConvDimsND:
+    """The fields of NNlib.DenseConvDims for k spatial dims.  padding = (lo1, hi1, lo2, hi2, ...)."""
+
+    def __init__(self, x_shape, w_shape, stride=1, padding=0, dilation=1, groups=1, flipkernel=False):
+        k = len(x_shape) - 2
+        self.k = k
+        self.x_shape, self.w_shape = tuple(x_shape), tuple(w_shape)
+        self.stride = (stride,) * k if isinstance(stride, int) else tuple(stride)
+        self.dilation = (dilation,) * k if isinstance(dilation, int) else tuple(dilation)
+        if isinstance(padding, int):
+            padding = (padding,) * (2 * k)
+        elif len(padding) == k:
+            padding = tuple(p for q in padding for p in (q, q))
+        self.padding = tuple(padding)
+        self.groups, self.flipkernel = int(groups), bool(flipkernel)
+        if self.w_shape[k] * self.groups != self.x_shape[k]:
+            raise DimensionMismatch("input channels do not match weight channels x groups")
+        if self.w_shape[k + 1] % self.groups != 0:
+            raise DimensionMismatch("output channels must be divisible by groups")
+
+    @property
+    def out_spatial(self):
+        return tuple((self.x_shape[d] + self.padding[2 * d] + self.padding[2 * d + 1]
+                      - self.dilation[d] * (self.w_shape[d] - 1) - 1) // self.stride[d] + 1 for d in range(self.k))
+
+
+def _tap_slices_nd(cd: ConvDimsND, tap):
+    """Per spatial dim: (output slice, input slice) for weight index `tap`, or None when the tap
+    never meets the input.  Input position = o*stride + koff*dil - pad_lo with koff = K-1-t for true
+    convolution and t for flipkernel (the rule of _tap_slices)."""
+    res = []
+    O = cd.out_spatial
+    for d in range(cd.k):
+        L, K, s, dl, plo, t = cd.x_shape[d], cd.w_shape[d], cd.stride[d], cd.dilation[d], cd.padding[2 * d], tap[d]
+        koff = t if cd.flipkernel else (K - 1 - t)
+        base = koff * dl - plo
+        o_lo = 0 if base >= 0 else (-base + s - 1) // s
+        o_hi = min(O[d] - 1, (L - 1 - base) // s) if (L - 1 - base) >= 0 else -1
+        if o_hi < o_lo:
+            return None
+        res.append((slice(o_lo, o_hi + 1), slice(base + o_lo * s, base + o_hi * s + 1, s)))
+    return res
+
+
+def _conv_nd_terms(cd: ConvDimsND):
+    k = cd.k
+    Cin_g, Cout = cd.w_shape[k], cd.w_shape[k + 1]
+    Cout_g = Cout // cd.groups
+    for tap in np.ndindex(*cd.w_shape[:k]):
+        sl = _tap_slices_nd(cd, tap)
+        if sl is None:
+            continue
+        osl = tuple(s[0] for s in sl)
+        isl = tuple(s[1] for s in sl)
+        for g in range(cd.groups):
+            yield tap, osl, isl, slice(g * Cin_g, (g + 1) * Cin_g), slice(g * Cout_g, (g + 1) * Cout_g)
+
+
+def conv_nd(x, w, cd: ConvDimsND):
+    x, w = np.asarray(x), np.asarray(w)
+    y = np.zeros(cd.out_spatial + (cd.w_shape[-1], x.shape[-1]), dtype=np.result_type(x, w))
+    for tap, osl, isl, cs, os_ in _conv_nd_terms(cd):
+        y[osl + (os_, slice(None))] += np.einsum("...cn,co->...on", x[isl + (cs, slice(None))], w[tap + (slice(None), os_)])
+    return y
+
+
+def conv_nd_data_grad(dy, w, cd: ConvDimsND):
+    dy, w = np.asarray(dy), np.asarray(w)
+    dx = np.zeros(cd.x_shape[:-1] + (dy.shape[-1],), dtype=np.result_type(dy, w))
+    for tap, osl, isl, cs, os_ in _conv_nd_terms(cd):
+        dx[isl + (cs, slice(None))] += np.einsum("...on,co->...cn", dy[osl + (os_, slice(None))], w[tap + (slice(None), os_)])
+    return dx
+
+
+def conv_nd_filter_grad(x, dy, cd: ConvDimsND):
+    x, dy = np.asarray(x), np.asarray(dy)
+    dw = np.zeros(cd.w_shape, dtype=np.result_type(x, dy))
+    for tap, osl, isl, cs, os_ in _conv_nd_terms(cd):
+        xs, ds = x[isl + (cs, slice(None))], dy[osl + (os_, slice(None))]
+        dw[tap + (slice(None), os_)] = np.einsum("scn,son->co", xs.reshape((-1,) + xs.shape[-2:]), ds.reshape((-1,) + ds.shape[-2:]))
+    return dw
+
+
+def fused_conv_nd_pullback(act: str, w, x, b, cd: ConvDimsND, delta):
+    """(y, ∂w, ∂x, ∂b) as fused_conv_pullback, for k spatial dims."""
+    pre = bias_add(conv_nd(x, w, cd), b)
+    y = act_value(act, pre)
+    dy = grad_activation(delta, y, act, pre)
+    return y, conv_nd_filter_grad(x, dy, cd), conv_nd_data_grad(dy, w, cd), grad_bias_add(b, dy)
 
 
 # --------------------------------------------------------------------------------------

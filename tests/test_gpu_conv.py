@@ -136,7 +136,7 @@ def test_one_spatial_dim(gpu, dtype, xs, ws, stride, pad, dil, groups, flip):
     assert_close(gx.to_numpy(), wdx.reshape(xs), dtype, "1-d dx", scale=np.sqrt(ws[0] * ws[2] / groups) * rms(delta) * rms(w) * 0.5)
     assert_close(gb.to_numpy(), wdb, dtype, "1-d db", rel=None if dtype == "f32" else 2e-2)
     with pytest.raises(gpu.Unsupported):
-        gpu.DenseConvDims((4, 4, 4, 2, 1), (2, 2, 2, 2, 3))
+        gpu.DenseConvDims((4, 4, 4, 4, 2, 1), (2, 2, 2, 2, 2, 3))       # four spatial dims
 
 
 def test_dimension_mismatch(gpu):

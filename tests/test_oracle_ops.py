@@ -557,3 +557,72 @@ def test_attention_scale_and_trailing_batch_dims():
     e = np.exp(logits)
     np.testing.assert_allclose(w, e / e.sum(axis=0), rtol=1e-12)
     np.testing.assert_allclose(out, np.einsum("ehsab,slhab->ehlab", v, w), rtol=1e-12)
+
+
+# ------------------------------------------------------------------ convolutions with k spatial dims
+def _conv_nd_brute(x, w, cd):
+    """Element-by-element definition: y[o, co, n] = sum_{t, c} w[t, c, co] x[o*s + koff(t)*d - p, c, n]."""
+    k = cd.k
+    Cg, Cout = cd.w_shape[k], cd.w_shape[k + 1]
+    Cout_g = Cout // cd.groups
+    y = np.zeros(cd.out_spatial + (Cout, x.shape[-1]))
+    for o in np.ndindex(*cd.out_spatial):
+        for t in np.ndindex(*cd.w_shape[:k]):
+            pos = []
+            for d in range(k):
+                koff = t[d] if cd.flipkernel else cd.w_shape[d] - 1 - t[d]
+                pos.append(o[d] * cd.stride[d] + koff * cd.dilation[d] - cd.padding[2 * d])
+            if any(p < 0 or p >= cd.x_shape[d] for d, p in enumerate(pos)):
+                continue
+            for co in range(Cout):
+                g = co // Cout_g
+                for c in range(Cg):
+                    y[o + (co,)] += w[t + (c, co)] * x[tuple(pos) + (g * Cg + c,)]
+    return y
+
+
+def test_conv_nd_equals_the_two_dimensional_oracle():
+    rng = np.random.default_rng(60)
+    for stride, pad, dil, groups, flip in [((1, 1), (0, 0, 0, 0), (1, 1), 1, False), ((2, 1), (1, 2, 0, 1), (1, 2), 2, False),
+                                           ((1, 2), (2, 2, 1, 1), (2, 1), 1, True)]:
+        x = rng.normal(size=(9, 8, 4, 3))
+        w = rng.normal(size=(3, 2, 4 // groups, 6))
+        cd2 = O.ConvDims(x.shape, w.shape, stride, pad, dil, groups, flip)
+        cdn = O.ConvDimsND(x.shape, w.shape, stride, pad, dil, groups, flip)
+        y = O.conv(x, w, cd2)
+        np.testing.assert_allclose(O.conv_nd(x, w, cdn), y, rtol=1e-12, atol=1e-12)
+        dy = rng.normal(size=y.shape)
+        np.testing.assert_allclose(O.conv_nd_data_grad(dy, w, cdn), O.conv_data_grad(dy, w, cd2), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(O.conv_nd_filter_grad(x, dy, cdn), O.conv_filter_grad(x, dy, cd2), rtol=1e-12, atol=1e-12)
+
+
+def test_conv_3d_against_scipy_and_brute_force():
+    from scipy import signal
+    rng = np.random.default_rng(61)
+    # one channel, stride 1, no padding: true convolution is scipy's N-d 'valid' convolution and
+    # flipkernel is its correlation
+    x = rng.normal(size=(7, 6, 5, 1, 1))
+    w = rng.normal(size=(3, 2, 3, 1, 1))
+    got = O.conv_nd(x, w, O.ConvDimsND(x.shape, w.shape))
+    np.testing.assert_allclose(got[..., 0, 0], signal.convolve(x[..., 0, 0], w[..., 0, 0], mode="valid"), rtol=1e-12, atol=1e-12)
+    got = O.conv_nd(x, w, O.ConvDimsND(x.shape, w.shape, flipkernel=True))
+    np.testing.assert_allclose(got[..., 0, 0], signal.correlate(x[..., 0, 0], w[..., 0, 0], mode="valid"), rtol=1e-12, atol=1e-12)
+    # strides, asymmetric padding, dilation and groups against the element-by-element definition
+    for flip in (False, True):
+        x = rng.normal(size=(5, 4, 6, 4, 2))
+        w = rng.normal(size=(2, 3, 2, 2, 4))
+        cd = O.ConvDimsND(x.shape, w.shape, (1, 2, 2), (1, 0, 2, 1, 1, 2), (2, 1, 2), 2, flip)
+        np.testing.assert_allclose(O.conv_nd(x, w, cd), _conv_nd_brute(x, w, cd), rtol=1e-12, atol=1e-12)
+
+
+def test_conv_3d_gradients_are_the_adjoints():
+    rng = np.random.default_rng(62)
+    x = rng.normal(size=(5, 4, 6, 4, 2))
+    w = rng.normal(size=(2, 3, 2, 2, 4))
+    cd = O.ConvDimsND(x.shape, w.shape, (1, 2, 2), (1, 0, 2, 1, 1, 2), (2, 1, 2), 2)
+    y = O.conv_nd(x, w, cd)
+    dy = rng.normal(size=y.shape)
+    x2, w2 = rng.normal(size=x.shape), rng.normal(size=w.shape)
+    # <dy, conv(x2, w)> = <conv_data_grad(dy, w), x2>;  <dy, conv(x, w2)> = <conv_filter_grad(x, dy), w2>
+    np.testing.assert_allclose(np.vdot(dy, O.conv_nd(x2, w, cd)), np.vdot(O.conv_nd_data_grad(dy, w, cd), x2), rtol=1e-10)
+    np.testing.assert_allclose(np.vdot(dy, O.conv_nd(x, w2, cd)), np.vdot(O.conv_nd_filter_grad(x, dy, cd), w2), rtol=1e-10)
