@@ -692,76 +692,116 @@ def rrule_instancenorm(x, scale, bias, running_mean, running_var, training, act=
 
 
 # ------------------------------------------------------------------------------- layernorm
+COLON = ":"                 # Julia's `Colon()` as a `dims` argument: every dim
+DEFAULT_DIMS = "1:(N-1)"
+
+
 def _layernorm_geometry(x, scale, bias, dims):
-    """Returns (L, R) when the normalised dims are the leading ones and scale/bias (if any)
-    span exactly those dims; raises Unsupported otherwise (the host would fall back to the
-    generic broadcast path, impl/layernorm.jl:3-14)."""
+    """Returns (L, R, channel_view): statistics run over the L elements of the leading dims, R
+    columns.  channel_view is None when scale/bias span exactly the normalised dims (one fused
+    kernel), else the (I, C, N) view of x in which the expanded scale/bias vary along C only (the
+    affine part then runs as a per-channel pass after the normalisation).  Other layouts raise
+    Unsupported (the host would fall back to the generic broadcast path, impl/layernorm.jl:3-14)."""
     if scale is None and bias is None and dims is None:
         raise ArgumentError("`dims` must be passed explicitly if `scale` and `bias` are `nothing`")
     if (scale is None) != (bias is None):
         raise ArgumentError("scale and bias must be given together")
     nd = x.ndim
+    pshape = None if scale is None else tuple(scale.shape)
+    if scale is not None and tuple(bias.shape) != pshape:
+        raise DimensionMismatch("scale and bias must have the same shape")
     if dims is None:
-        # compute_layernorm_dims (impl/layernorm.jl:21-28): 1:(N - M)
+        # compute_layernorm_dims / expand_layernorm_dims (impl/layernorm.jl:21-28,40-46): dims = 1:(N - M),
+        # parameters reshaped to (size(γ)..., 1, ..., 1)
         assert nd > scale.ndim, "`x` must have more dimensions than `scale` and `bias` when `dims` is `nothing`"
         dims = tuple(range(1, nd - scale.ndim + 1))
-        raise _lib.Unsupported(_lib.UNSUPPORTED, "layernorm with dims=nothing and trailing-dim affine parameters")
+        pshape = pshape + (1,) * (nd - scale.ndim)
+    elif isinstance(dims, str) and dims == COLON:
+        dims = tuple(range(1, nd + 1))
+    elif isinstance(dims, str) and dims == DEFAULT_DIMS:
+        dims = tuple(range(1, nd))
     if isinstance(dims, int):
         dims = (dims,)
     dims = tuple(sorted(dims))
     if dims != tuple(range(1, len(dims) + 1)):
         raise _lib.Unsupported(_lib.UNSUPPORTED, f"layernorm over non-leading dims {dims}")
+    k = len(dims)
     L = 1
     for d in dims:
         L *= x.shape[d - 1]
     R = x.size // max(L, 1)
-    if scale is not None:
-        want = tuple(x.shape[:len(dims)]) + (1,) * (nd - len(dims))
-        if scale.ndim != nd or bias.ndim != nd:
-            raise ArgumentError("scale and bias must have the same number of dimensions as x when dims is given")
-        if tuple(scale.shape) != want or tuple(bias.shape) != want:
-            raise _lib.Unsupported(_lib.UNSUPPORTED, f"layernorm affine parameters of shape {scale.shape} (want {want})")
-    return L, R
-
-
-DEFAULT_DIMS = "1:(N-1)"
+    if scale is None:
+        return L, R, None
+    if len(pshape) != nd:
+        raise ArgumentError("scale and bias must have the same number of dimensions as x when dims is given")
+    if any(g not in (1, sx) for g, sx in zip(pshape, x.shape)):
+        raise DimensionMismatch(f"scale/bias of shape {pshape} do not broadcast against x {x.shape}")
+    if pshape == tuple(x.shape[:k]) + (1,) * (nd - k):
+        return L, R, None
+    # the dims along which the parameters vary must be one contiguous run
+    varying = [d for d in range(nd) if pshape[d] != 1]
+    a, b = (varying[0], varying[-1] + 1) if varying else (nd, nd)
+    if any(pshape[d] != x.shape[d] for d in range(a, b)):
+        raise _lib.Unsupported(_lib.UNSUPPORTED, f"layernorm affine parameters of shape {pshape} for x {x.shape}")
+    prod = lambda t: int(np.prod(t, dtype=np.int64)) if len(t) else 1
+    return L, R, (prod(x.shape[:a]), prod(x.shape[a:b]), prod(x.shape[b:]))
 
 
 def layernorm(x: DeviceArray, scale, bias, act: str = "identity", dims=DEFAULT_DIMS, epsilon: Optional[float] = None):
     """`layernorm(x, scale, bias, σ, dims, epsilon)` (api/layernorm.jl:32-43).  `dims` uses
-    Julia's 1-based numbering; the default is 1:(N-1); `None` is Julia's `nothing`."""
+    Julia's 1-based numbering; the default is 1:(N-1); `None` is Julia's `nothing` (dims inferred
+    from the parameters' rank), `COLON` is `Colon()`."""
     return _layernorm_fwd(x, scale, bias, act, dims, epsilon, False)[0]
 
 
 def _layernorm_fwd(x, scale, bias, act, dims, epsilon, save):
-    if isinstance(dims, str) and dims == DEFAULT_DIMS:
-        dims = tuple(range(1, x.ndim))
-    L, R = _layernorm_geometry(x, scale, bias, dims)
+    L, R, view = _layernorm_geometry(x, scale, bias, dims)
     dt = _same_dtype(x, scale, bias)
     if epsilon is None:
         epsilon = default_epsilon(dt)
     y = DeviceArray(x.shape, dt)
     sm = StatArray(R) if save else None
     si = StatArray(R) if save else None
-    _lib.call("luxhip_layernorm_fwd", current_stream(), x.code, _act_id(act), L, R, x.ptr, _p(scale), _p(bias),
-              float(epsilon), y.ptr, _p(sm), _p(si))
-    return y, (sm, si, L, R)
+    if view is None:
+        _lib.call("luxhip_layernorm_fwd", current_stream(), x.code, _act_id(act), L, R, x.ptr, _p(scale), _p(bias),
+                  float(epsilon), y.ptr, _p(sm), _p(si))
+        return y, (sm, si, L, R, None)
+    # parameters that vary along other dims than the normalised ones: x̂ first, then the per-channel
+    # affine transform and activation as a batchnorm in inference mode with mean 0, variance 1, ε = 0
+    _lib.call("luxhip_layernorm_fwd", current_stream(), x.code, 0, L, R, x.ptr, None, None, float(epsilon), y.ptr, _p(sm), _p(si))
+    I, Cc, Nn = view
+    zeros = DeviceArray.from_numpy(np.zeros(Cc, np.float32), dt)
+    ones = DeviceArray.from_numpy(np.ones(Cc, np.float32), dt)
+    args = (y.reshape(I, Cc, Nn), scale.reshape(Cc), bias.reshape(Cc), zeros, ones, False, act, 0.1, 0.0)
+    if save:
+        (out, _), affine_back = rrule_batchnorm(*args)
+    else:
+        (out, _), affine_back = batchnorm(*args), None
+    return out.reshape(x.shape), (sm, si, L, R, affine_back)
 
 
 def rrule_layernorm(x, scale, bias, act="identity", dims=DEFAULT_DIMS, epsilon=None):
     """Pullback of layernorm: the chain AD derives from impl/normalization.jl:11-17 and the
-    mean_var rrule (impl/common_ops.jl:45-61), as one fused device pass."""
-    y, (sm, si, L, R) = _layernorm_fwd(x, scale, bias, act, dims, epsilon, True)
+    mean_var rrule (impl/common_ops.jl:45-61), as one fused device pass (two when the parameters
+    vary along other dims than the normalised ones)."""
+    y, (sm, si, L, R, affine_back) = _layernorm_fwd(x, scale, bias, act, dims, epsilon, True)
     aid = _act_id(act)
 
     def back(delta):
         dx = DeviceArray(x.shape, x.dtype)
+        if affine_back is not None:
+            dxhat, dg, db = affine_back(delta.reshape(dxhat_shape))
+            _lib.call("luxhip_layernorm_bwd", current_stream(), x.code, 0, L, R, dxhat.ptr, x.ptr, None, None,
+                      sm.ptr, si.ptr, dx.ptr, None, None)
+            return dx, dg.reshape(scale.shape), db.reshape(bias.shape)
         dg = None if scale is None else DeviceArray(scale.shape, x.dtype)
         db = None if bias is None else DeviceArray(bias.shape, x.dtype)
         _lib.call("luxhip_layernorm_bwd", current_stream(), x.code, aid, L, R, delta.ptr, x.ptr, _p(scale), _p(bias),
                   sm.ptr, si.ptr, dx.ptr, _p(dg), _p(db))
         return dx, dg, db
 
+    if affine_back is not None:
+        dxhat_shape = _layernorm_geometry(x, scale, bias, dims)[2]
     return y, back
 
 

@@ -99,3 +99,85 @@ def test_config4_layernorm_full_size(gpu):
     _, wdg, wdb = O.layernorm_pullback(f64(x), f64(g), f64(b), "identity", (0,), eps, f64(delta))
     assert_close(gg.to_numpy(), wdg, "bf16", "config4 LN dgamma", rel=3e-2, scale=rms(delta) * 90)
     assert_close(gb.to_numpy(), wdb, "bf16", "config4 LN dbeta", rel=3e-2, scale=rms(delta) * 90)
+
+
+REFERENCE_CONFIGS = [(xs, aff, act) for xs in ((3, 3, 2, 1), (2, 2, 2, 1)) for aff in (None, "channel")
+                     for act in ("identity", "sigmoid_fast", "tanh")]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("xs,aff,act", REFERENCE_CONFIGS)
+def test_reference_test_configurations(gpu, dtype, xs, aff, act):
+    """The configurations of lib/LuxLib/test/normalization/layernorm_tests.jl:80-86 on its own input
+    generator: dims = Colon() with parameters (1, 1, C, 1), and dims = nothing with parameters
+    (1, 1, C) (statistics over 1:(N - 3), :22-32).  (Its cube activation is not in the table; tanh
+    stands in.)"""
+    eps = gpu.default_epsilon(dtype)
+    x = O.generate_fixed_array(np.float32, xs)
+    cases = [(gpu.COLON, (1, 1, xs[2], 1), tuple(range(len(xs))))]
+    if aff is not None:
+        cases.append((None, (1, 1, xs[2]), (0,)))
+    for dims, pshape, axes in cases:
+        if aff is None:
+            g = b = gfull = bfull = None
+        else:
+            g, b = O.generate_fixed_array(np.float32, pshape), O.generate_fixed_array(np.float32, pshape)
+            gfull, bfull = g.reshape(pshape + (1,) * (len(xs) - len(pshape))), b.reshape(pshape + (1,) * (len(xs) - len(pshape)))
+        xq, gq, bq = host_inputs(dtype, x, g, b)
+        gfq = None if gq is None else gq.reshape(gfull.shape)
+        bfq = None if bq is None else bq.reshape(bfull.shape)
+        delta = host_inputs(dtype, np.random.default_rng(5).normal(size=xs))[0]
+        y, back = gpu.pullback(gpu.layernorm, dev(gpu, xq, dtype), dev(gpu, gq, dtype), dev(gpu, bq, dtype), act, dims, eps)
+        tag = f"{dtype} {xs} {pshape if aff else None} {act} dims={dims}"
+        want = O.layernorm(f64(xq), f64(gfq), f64(bfq), act, axes, eps)
+        assert y.shape == tuple(xs)
+        assert_close(y.to_numpy(), want, dtype, tag + " y", rel=None if dtype == "f32" else 2e-2)
+        if aff is None and act == "identity":        # :56-59
+            np.testing.assert_allclose(y.to_numpy().mean(axis=axes), 0, atol=1e-3 if dtype == "f32" else 2e-2)
+        gx, gg, gb = back(dev(gpu, delta, dtype))
+        wdx, wdg, wdb = O.layernorm_pullback(f64(xq), f64(gfq), f64(bfq), act, axes, eps, f64(delta))
+        w32 = O.layernorm_pullback(xq, gfq, bfq, act, axes, np.float32(eps), delta)
+        rel = None if dtype == "f32" else 4e-2
+        assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=rms(delta), want32=w32[0])
+        if aff is not None:
+            assert gg.shape == tuple(pshape) and gb.shape == tuple(pshape)
+            assert_close(gg.to_numpy().reshape(gfull.shape), wdg, dtype, tag + " dgamma", rel=rel, scale=rms(delta), want32=w32[1])
+            assert_close(gb.to_numpy().reshape(bfull.shape), wdb, dtype, tag + " dbeta", rel=rel, scale=rms(delta), want32=w32[2])
+        else:
+            assert gg is None and gb is None
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_channel_parameters_on_larger_shapes(gpu, dtype):
+    """Statistics over a prefix of the dims with parameters that vary along one other run of dims."""
+    rng = np.random.default_rng(8)
+    eps = 1e-5 if dtype == "f32" else 1e-3
+    for xs, dims, pshape, axes in [((16, 12, 24, 5), gpu.COLON, (1, 1, 24, 1), (0, 1, 2, 3)),
+                                   ((16, 12, 24, 5), (1, 2, 3), (1, 1, 24, 1), (0, 1, 2)),
+                                   ((16, 12, 24, 5), (1, 2), (1, 1, 24, 1), (0, 1)),
+                                   ((64, 8, 6), (1,), (1, 8, 6), (0,)),
+                                   ((32, 10, 7), None, (32, 10), (0,)),
+                                   ((8, 4, 6, 3), (1, 2), (1, 1, 1, 1), (0, 1))]:
+        full = pshape + (1,) * (len(xs) - len(pshape))
+        x, g, b, delta = host_inputs(dtype, rng.normal(size=xs) * 2 + 0.5, rng.uniform(0.5, 1.5, size=pshape), rng.normal(size=pshape),
+                                     rng.normal(size=xs))
+        for act in ("identity", "gelu"):
+            y, back = gpu.pullback(gpu.layernorm, dev(gpu, x, dtype), dev(gpu, g, dtype), dev(gpu, b, dtype), act, dims, eps)
+            tag = f"{dtype} {xs} dims={dims} params={pshape} {act}"
+            assert_close(y.to_numpy(), O.layernorm(f64(x), f64(g).reshape(full), f64(b).reshape(full), act, axes, eps), dtype, tag + " y",
+                         rel=None if dtype == "f32" else 2e-2)
+            gx, gg, gb = back(dev(gpu, delta, dtype))
+            wdx, wdg, wdb = O.layernorm_pullback(f64(x), f64(g).reshape(full), f64(b).reshape(full), act, axes, eps, f64(delta))
+            w32 = O.layernorm_pullback(x, g.reshape(full), b.reshape(full), act, axes, np.float32(eps), delta)
+            rel = None if dtype == "f32" else 4e-2
+            assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=rms(delta) * 1.5, want32=w32[0])
+            assert_close(gg.to_numpy().reshape(full), wdg, dtype, tag + " dgamma", rel=rel, scale=rms(delta) * np.sqrt(x.size / g.size), want32=w32[1])
+            assert_close(gb.to_numpy().reshape(full), wdb, dtype, tag + " dbeta", rel=rel, scale=rms(delta) * np.sqrt(x.size / g.size), want32=w32[2])
+
+
+def test_dims_nothing_assertion(gpu):
+    d = gpu.DeviceArray.from_numpy
+    x = np.random.default_rng(1).random((2, 3)).astype(np.float32)
+    sc = np.random.default_rng(2).random((2, 1)).astype(np.float32)
+    with pytest.raises(AssertionError):                      # layernorm_tests.jl:108-111
+        gpu.layernorm(d(x), d(sc), d(sc), "identity", None, 1e-5)

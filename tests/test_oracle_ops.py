@@ -319,6 +319,31 @@ def test_layernorm_vs_torch(shape, nd, act, affine):
         np.testing.assert_allclose(db, np.transpose(tb.grad.numpy().reshape(tuple(reversed(pshape))), rev), rtol=1e-9, atol=1e-11)
 
 
+@pytest.mark.parametrize("shape,nd,pshape", [((3, 3, 2, 1), 4, (1, 1, 2, 1)), ((5, 4, 6, 3), 2, (1, 1, 6, 1)), ((5, 4, 6, 3), 1, (1, 4, 6, 1))])
+@pytest.mark.parametrize("act", ["identity", "gelu"])
+def test_layernorm_with_parameters_along_other_dims_vs_torch(shape, nd, pshape, act):
+    """Statistics over the leading `nd` dims, parameters broadcast along others (the reference's own test
+    configurations: dims = Colon() with (1, 1, C, 1) parameters): torch layer_norm without affine
+    parameters, then the broadcast affine transform, differentiated by autograd."""
+    from tests.test_oracle_activations import TORCH
+    x, delta = RNG.normal(size=shape), RNG.normal(size=shape)
+    g, b = RNG.uniform(0.5, 1.5, pshape), RNG.normal(size=pshape)
+    eps = 1e-5
+    dims = tuple(range(nd))
+    y = O.layernorm(x, g, b, act, dims, eps)
+    dx, dg, db = O.layernorm_pullback(x, g, b, act, dims, eps, delta)
+    rev = tuple(reversed(range(len(shape))))
+    tx = torch.tensor(np.transpose(x, rev).copy(), requires_grad=True)
+    tg = torch.tensor(np.transpose(g, rev).copy(), requires_grad=True)
+    tb = torch.tensor(np.transpose(b, rev).copy(), requires_grad=True)
+    ty = TORCH[act](F.layer_norm(tx, tuple(reversed(shape[:nd])), None, None, eps) * tg + tb)
+    ty.backward(torch.tensor(np.transpose(delta, rev).copy()))
+    np.testing.assert_allclose(y, np.transpose(ty.detach().numpy(), rev), rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(dx, np.transpose(tx.grad.numpy(), rev), rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(dg, np.transpose(tg.grad.numpy(), rev), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(db, np.transpose(tb.grad.numpy(), rev), rtol=1e-9, atol=1e-11)
+
+
 # ----------------------------------------------------------------------------- conv
 def brute_conv(x, w, cd):
     """7-loop direct convolution straight from the index formula
