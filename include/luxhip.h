@@ -349,6 +349,13 @@ int luxhip_fused_conv_bwd(luxhip_stream_t s, int dtype, int act, const luxhip_co
                           const void* delta, const void* y, const void* pre, const void* x, const void* w,
                           void* dz, void* dw, void* dx, void* dbias, const void* xt_kept);
 
+/* out = permutedims(in, (p1, p2, p3, 4:N...)) for in of size (d1, d2, d3, outer) (p: a permutation of
+ * 1:3).  scaled_dot_product_attention accepts the embedding (`head_dim`) and token dims in any of
+ * the first three positions (src/impl/attention.jl:5-16,66-103); operands whose embedding dim is not
+ * the first are brought to (E, H, L, B...) with this, and their gradients taken back. */
+int luxhip_permute_leading3(luxhip_stream_t s, int dtype, int64_t d1, int64_t d2, int64_t d3, int64_t outer, int p1, int p2,
+                            int p3, const void* in, void* out);
+
 /* Convolutions with three spatial dims (x (W, H, D, C, N), w (kW, kH, kD, C/groups, Cout)): the
  * reference hands them to the same NNlib.conv / ∇conv_data / ∇conv_filter calls as the
  * two-dimensional ones (src/impl/conv.jl:29-60,128-136).  Here they run as the two-dimensional

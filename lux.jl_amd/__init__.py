@@ -18,7 +18,7 @@ from . import _lib
 from ._lib import LuxHipError, Unsupported
 from .array import DeviceArray, StatArray, current_stream, set_stream
 from .luxlib import (ArgumentError, PhiloxRNG, scaled_dot_product_attention, rrule_scaled_dot_product_attention, batched_matmul, rrule_batched_matmul, alpha_dropout, dropout, dropout_dot_mul, dropout_shape, rand_uniform,
-                     rrule_alpha_dropout, rrule_dropout, DenseConvDims, DimensionMismatch, DEFAULT_DIMS, COLON, batchnorm, bias_activation,
+                     rrule_alpha_dropout, rrule_dropout, attention_dropout, DenseConvDims, DimensionMismatch, DEFAULT_DIMS, COLON, batchnorm, bias_activation,
                      bias_activation_inplace, conv, conv_data_grad, conv_filter_grad, default_epsilon,
                      fast_activation, fast_activation_inplace, fused_conv_bias_activation, fused_dense_bias_activation,
                      groupnorm, instancenorm, layernorm, matmul, pullback, rrule_fast_activation, rrule_instancenorm,

@@ -327,6 +327,21 @@ static int softmax_check(int dtype, int64_t S, int64_t cols) {
     return LUXHIP_OK;
 }
 
+// permutedims of the first three dims (operands whose embedding dim is not the first are brought
+// to the (E, H, L, B...) layout and their gradients taken back): one element per thread, lanes
+// along the output's first dim.
+template <typename U>
+__global__ __launch_bounds__(256) void permute3_kernel(const U* __restrict__ in, U* __restrict__ out, uint32_t o1, uint32_t o2,
+                                                       uint32_t o3, uint32_t s1, uint32_t s2, uint32_t s3, uint32_t total) {
+    const uint32_t block = o1 * o2 * o3;
+    for (uint32_t idx = blockIdx.x * 256u + threadIdx.x; idx < total; idx += gridDim.x * 256u) {
+        const uint32_t o = idx / block, r = idx - o * block;
+        const uint32_t i3 = r / (o1 * o2), r2 = r - i3 * (o1 * o2);
+        const uint32_t i2 = r2 / o1, i1 = r2 - i2 * o1;
+        out[idx] = in[(size_t)o * block + (size_t)i1 * s1 + (size_t)i2 * s2 + (size_t)i3 * s3];
+    }
+}
+
 }  // namespace luxhip
 
 using namespace luxhip;
@@ -365,6 +380,31 @@ int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_
                                        (float*)dlogits);
     return softmax_bwd_impl<bf16_t>((hipStream_t)s, S, L, causal, cols, (const bf16_t*)dprobs, (const bf16_t*)probs, (float)scale,
                                     (bf16_t*)dlogits);
+}
+
+int luxhip_permute_leading3(luxhip_stream_t s, int dtype, int64_t d1, int64_t d2, int64_t d3, int64_t outer, int p1, int p2,
+                            int p3, const void* in, void* out) {
+    LUX_REQUIRE_INIT();
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_INVALID_IF(d1 < 0 || d2 < 0 || d3 < 0 || outer < 0, "permute_leading3: negative dimension");
+    LUX_INVALID_IF(p1 < 1 || p1 > 3 || p2 < 1 || p2 > 3 || p3 < 1 || p3 > 3 || p1 == p2 || p1 == p3 || p2 == p3,
+                   "permute_leading3: (%d, %d, %d) is not a permutation of 1:3", p1, p2, p3);
+    LUX_UNSUPPORTED_IF((long double)d1 * d2 * d3 * std::max<int64_t>(outer, 1) >= 2147483648.0L,
+                       "permute_leading3: tensors of 2^31 or more elements are not supported");
+    const int64_t total = d1 * d2 * d3 * outer;
+    if (total == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(in == nullptr || out == nullptr || in == out, "permute_leading3: in and out must be distinct buffers");
+    const int64_t d[3] = {d1, d2, d3}, st[3] = {1, d1, d1 * d2};
+    const uint32_t o1 = (uint32_t)d[p1 - 1], o2 = (uint32_t)d[p2 - 1], o3 = (uint32_t)d[p3 - 1];
+    const uint32_t s1 = (uint32_t)st[p1 - 1], s2 = (uint32_t)st[p2 - 1], s3 = (uint32_t)st[p3 - 1];
+    const unsigned blocks = (unsigned)std::min<int64_t>((total + 255) / 256, 65535 * 16);
+    ProfScope ps("permute3_kernel", (hipStream_t)s);
+    if (dtype == LUXHIP_F32)
+        permute3_kernel<uint32_t><<<blocks, 256, 0, (hipStream_t)s>>>((const uint32_t*)in, (uint32_t*)out, o1, o2, o3, s1, s2, s3, (uint32_t)total);
+    else
+        permute3_kernel<uint16_t><<<blocks, 256, 0, (hipStream_t)s>>>((const uint16_t*)in, (uint16_t*)out, o1, o2, o3, s1, s2, s3, (uint32_t)total);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
 }
 
 }  // extern "C"

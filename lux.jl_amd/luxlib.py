@@ -436,15 +436,35 @@ class _AttnLayout:
         self.batch = a.size // self.sb if self.sb else 0
 
 
+def _permute_leading3(a: DeviceArray, perm) -> DeviceArray:
+    """permutedims(a, (perm..., 4:N...))."""
+    out = DeviceArray(tuple(a.shape[p - 1] for p in perm) + tuple(a.shape[3:]), a.dtype)
+    outer = int(np.prod(a.shape[3:], dtype=np.int64)) if a.ndim > 3 else 1
+    _lib.call("luxhip_permute_leading3", current_stream(), a.code, a.shape[0], a.shape[1], a.shape[2], outer, *perm, a.ptr, out.ptr)
+    return out
+
+
+def attention_dropout(rng: "PhiloxRNG", p: float):
+    """An `fdrop` for scaled_dot_product_attention: dropout of the attention weights with rate p
+    (what `Base.Fix2(fdrop, p)` is in test/common_ops/attention_tests.jl:291-299).  Called with the
+    weights, returns (weights′, Δweights′ -> Δweights)."""
+    def fdrop(weights: DeviceArray):
+        (y, _, _), back = rrule_dropout(rng, weights, p, True, 1.0 / (1.0 - p))
+        return y, (lambda d: back(d)[0])
+    return fdrop
+
+
 def scaled_dot_product_attention(q: DeviceArray, k: DeviceArray, v: DeviceArray, head_dim: int = 1, token_dim: int = 3,
-                                 scale=None, mask=None, is_causal=None, bias=None):
-    """`scaled_dot_product_attention(q, k, v; head_dim, token_dim, scale, mask, is_causal, bias)`
+                                 scale=None, mask=None, is_causal=None, bias=None, fdrop=None):
+    """`scaled_dot_product_attention(q, k, v; head_dim, token_dim, scale, mask, is_causal, bias, fdrop)`
     (api/attention.jl, impl/attention.jl:5-117): returns `(output [Ev, H, L, B...], attention weights
-    [S, L, H, B...])`.  `mask` / `bias`: host arrays or DeviceArrays of shape [S, L, H or 1, B or 1]."""
-    return rrule_scaled_dot_product_attention(q, k, v, head_dim, token_dim, scale, mask, is_causal, bias)[0]
+    [S, L, H, B...])`.  `mask` / `bias`: host arrays or DeviceArrays of shape [S, L, H or 1, B or 1].
+    `fdrop`: None (identity) or a callable weights -> (weights′, pullback), e.g. `attention_dropout`."""
+    return rrule_scaled_dot_product_attention(q, k, v, head_dim, token_dim, scale, mask, is_causal, bias, fdrop)[0]
 
 
-def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=None, mask=None, is_causal=None, bias=None):
+def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=None, mask=None, is_causal=None, bias=None,
+                                       fdrop=None):
     """((output, weights), (Δoutput[, Δweights]) -> (∂q, ∂k, ∂v)): the pullbacks of the two batched
     products (impl/batched_mul.jl:320-334), of NNlib.softmax and of repeat_inner_gqa, composed as the
     reference's AD does.  The gradient of `bias` is not computed."""
@@ -457,7 +477,14 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
         if not (q.shape[i] == k.shape[i] == v.shape[i]):
             raise DimensionMismatch("All dimensions (except first 3) of q, k, v must be the same.")
     if head_dim != 1:
-        raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: the embedding dim must be the first one on the device")
+        # the kernels want the embedding dim first: bring the operands to (E, H, L, B...) and take the
+        # gradients back (the results' layout does not depend on the operands', impl/attention.jl:107-117)
+        heads_dim = ({1, 2, 3} - {head_dim, token_dim}).pop()
+        perm = (head_dim, heads_dim, token_dim)
+        inv = tuple(perm.index(d) + 1 for d in (1, 2, 3))
+        res, back_c = rrule_scaled_dot_product_attention(*(_permute_leading3(a, perm) for a in (q, k, v)), 1, 3, scale, mask,
+                                                         is_causal, bias, fdrop)
+        return res, (lambda d_out, d_probs=None: tuple(_permute_leading3(g, inv) for g in back_c(d_out, d_probs)))
     dt = _same_dtype(q, k, v)
     lq, lk, lv = _AttnLayout(q, token_dim), _AttnLayout(k, token_dim), _AttnLayout(v, token_dim)
     assert lv.tokens == lk.tokens, "`v` and `k` must have the same number of tokens."
@@ -489,33 +516,39 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
     # a causal mask (keep s <= l) leaves whole tiles of the logits unused and makes the weights and every
     # cotangent of the same shape triangular: the products skip what is known to be zero or unused
     causal = bool(is_causal)
+    tri = causal and fdrop is None       # an arbitrary fdrop need not keep the masked weights at zero
     _bmm_strided(True, False, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, (lq.sh, lq.sh * r, lq.sb), logits, S, sC,
                  1 if causal else 0)
     probs = DeviceArray((S, L, H) + bshape, dt)
     _lib.call("luxhip_attention_softmax_fwd", current_stream(), probs.code, S, L, H, B, logits.ptr, scale_inv,
               int(causal), _p(mask_a), mask_sh, mask_sb, _p(bias_a), bias_sh, bias_sb, probs.ptr)
+    softmax_out, fdrop_back = probs, None
+    if fdrop is not None:
+        probs, fdrop_back = fdrop(softmax_out)         # impl/attention.jl:88-104: fdrop(softmax(...))
     out = DeviceArray((Ev, H, L) + bshape, dt)
     so = (Ev, Ev * r, Ev * H * L)
-    _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so, 2 if causal else 0)
+    _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so, 2 if tri else 0)
 
     def back(d_out: DeviceArray, d_probs: Optional[DeviceArray] = None):
         dp = DeviceArray(probs.shape, dt)
-        _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC, 1 if causal else 0)
+        _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC, 1 if tri else 0)
         if d_probs is not None:
             raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: a cotangent for the returned weights")
+        if fdrop_back is not None:
+            dp = fdrop_back(dp)
         dlogits = logits                                              # the logits are no longer needed
-        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L, L * H * B, int(causal), dp.ptr, probs.ptr,
+        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L, L * H * B, int(causal), dp.ptr, softmax_out.ptr,
                   scale_inv, dlogits.ptr)
         dq = DeviceArray(q.shape, dt)
         _bmm_strided(False, False, E, L, S, bdims, k, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, dq, lq.st,
-                     (lq.sh, lq.sh * r, lq.sb), 2 if causal else 0)
+                     (lq.sh, lq.sh * r, lq.sb), 2 if tri else 0)
 
         def kv_grad(like, lay, A, lda, sA, Bm):
             # (rows of `like`) x S = A (rows x L) * Bm' (L x S), one product per head; the heads that share
             # a key/value group are summed afterwards (pullback of repeat_inner_gqa)
             full = DeviceArray(((r,) if r > 1 else ()) + tuple(like.shape), dt)
             _bmm_strided(False, True, lay.E, S, L, bdims, A, lda, sA, Bm, S, sC, full, lay.st,
-                         (like.size if r > 1 else 0, lay.sh, lay.sb), 3 if causal else 0)
+                         (like.size if r > 1 else 0, lay.sh, lay.sb), 3 if tri else 0)
             if r == 1:
                 return full
             red = DeviceArray(like.shape, dt)

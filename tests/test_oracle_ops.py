@@ -651,3 +651,16 @@ def test_conv_3d_gradients_are_the_adjoints():
     # <dy, conv(x2, w)> = <conv_data_grad(dy, w), x2>;  <dy, conv(x, w2)> = <conv_filter_grad(x, dy), w2>
     np.testing.assert_allclose(np.vdot(dy, O.conv_nd(x2, w, cd)), np.vdot(O.conv_nd_data_grad(dy, w, cd), x2), rtol=1e-10)
     np.testing.assert_allclose(np.vdot(dy, O.conv_nd(x, w2, cd)), np.vdot(O.conv_nd_filter_grad(x, dy, cd), w2), rtol=1e-10)
+
+
+def test_attention_reference_specific_results():
+    """test/common_ops/attention_tests.jl:115-170: q = k = v = reshape(1:12, 2, 2, 3, 1) ./ 12 and the
+    output and weights the reference's test holds for it."""
+    q = (np.arange(1, 13, dtype=np.float64) / 12).reshape((2, 2, 3, 1), order="F")
+    y, w = O.scaled_dot_product_attention(q, q, q)
+    ytrue = [0.429754, 0.513087, 0.613791, 0.697125, 0.46431, 0.547644, 0.647876, 0.73121, 0.49773, 0.581064, 0.680455,
+             0.763788]
+    wtrue = [0.313896, 0.332948, 0.353157, 0.264431, 0.328206, 0.407362, 0.219215, 0.31838, 0.462405, 0.288691, 0.331243,
+             0.380066, 0.241239, 0.323893, 0.434868, 0.198438, 0.311761, 0.489801]
+    np.testing.assert_allclose(y, np.reshape(ytrue, (2, 2, 3, 1), order="F"), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(w, np.reshape(wtrue, (3, 3, 2, 1), order="F"), rtol=1e-5, atol=1e-5)
