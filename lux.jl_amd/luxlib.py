@@ -374,18 +374,145 @@ def _batched_geometry(x, y, lhs_contracting_dim, rhs_contracting_dim):
     return x, y, tA, tB, M, N, Kx, batch, xb, yb, bshape
 
 
-def batched_matmul(x: DeviceArray, y: DeviceArray, lhs_contracting_dim: int = 2, rhs_contracting_dim: int = 1):
-    """`batched_matmul(x, y; lhs_contracting_dim, rhs_contracting_dim)` (api/batched_mul.jl,
-    impl/batched_mul.jl:2-58) with the default (trailing) batching dims: z[:, :, b...] =
-    op(x[:, :, b...]) op(y[:, :, b...]); batch dims of extent 1 are shared among the products."""
-    return rrule_batched_matmul(x, y, lhs_contracting_dim, rhs_contracting_dim, _need_back=False)[0]
+def batched_matmul(x: DeviceArray, y: DeviceArray, lhs_contracting_dim: int = 2, rhs_contracting_dim: int = 1,
+                   lhs_batching_dims=None, rhs_batching_dims=None):
+    """`batched_matmul(x, y; lhs_contracting_dim, rhs_contracting_dim, lhs_batching_dims, rhs_batching_dims)`
+    (api/batched_mul.jl, impl/batched_mul.jl:2-58): z[:, :, b...] = op(x[.., b...]) op(y[.., b...]); batch
+    dims of extent 1 are shared among the products.  The batching dims default to the trailing ones."""
+    return rrule_batched_matmul(x, y, lhs_contracting_dim, rhs_contracting_dim, lhs_batching_dims, rhs_batching_dims,
+                                _need_back=False)[0]
 
 
-def rrule_batched_matmul(x, y, lhs_contracting_dim=2, rhs_contracting_dim=1, _need_back=True):
+def _dense_strides(shape):
+    st, p = [], 1
+    for e in shape:
+        st.append(p)
+        p *= e
+    return st
+
+
+class _BmmOperand:
+    """One operand of the general product: where its (free x contracting) matrix and its batching dims lie."""
+
+    def __init__(self, a: DeviceArray, contracting_dim: int, batching_dims, what: str):
+        nd = a.ndim
+        if nd < 3:
+            raise ArgumentError(f"{what}: N must be at least 3")
+        bd = tuple(range(3, nd + 1)) if batching_dims is None else tuple(int(d) for d in batching_dims)
+        rest = [d for d in range(1, nd + 1) if d != contracting_dim and d not in bd]
+        if len(bd) != nd - 2 or len(set(bd)) != len(bd) or len(rest) != 1 or not 1 <= contracting_dim <= nd:
+            raise ArgumentError(f"{what}: one contracting dim, one free dim and N - 2 distinct batching dims are needed")
+        st = _dense_strides(a.shape)
+        self.a, self.bd = a, bd
+        self.F, self.K = a.shape[rest[0] - 1], a.shape[contracting_dim - 1]
+        self.sf, self.sk = st[rest[0] - 1], st[contracting_dim - 1]
+        self.bext = [a.shape[d - 1] for d in bd]
+        self.bst = [st[d - 1] for d in bd]
+        # free-major: the free index is the contiguous one
+        if self.sf == 1 or self.F == 1:
+            self.free_major, self.ld = True, (self.sk if self.K > 1 else max(self.F, 1))
+        elif self.sk == 1 or self.K == 1:
+            self.free_major, self.ld = False, (self.sf if self.F > 1 else max(self.K, 1))
+        else:
+            raise _lib.Unsupported(_lib.UNSUPPORTED, f"batched_matmul: neither matrix dim of {what} is contiguous")
+
+
+def _launch_general(tA, tB, M, N, K, pairs, A, lda, B, ldb, Cm, ldc):
+    """pairs: (extent, stride in A, stride in B, stride in C) per batch dim, innermost first."""
+    pairs = [p for p in pairs if p[0] != 1]
+    merged = []
+    for p in pairs:
+        if merged:
+            e, sa, sb, sc = merged[-1]
+            if p[1] == sa * e and p[2] == sb * e and p[3] == sc * e:
+                merged[-1] = (e * p[0], sa, sb, sc)
+                continue
+        merged.append(p)
+    if len(merged) > 3:
+        raise _lib.Unsupported(_lib.UNSUPPORTED, "batched_matmul: more than three batch dims that cannot be merged")
+    merged += [(1, 0, 0, 0)] * (3 - len(merged))
+    _bmm_strided(tA, tB, M, N, K, [p[0] for p in merged], A, lda, [p[1] for p in merged], B, ldb, [p[2] for p in merged],
+                 Cm, ldc, [p[3] for p in merged])
+
+
+def _rrule_batched_matmul_general(x, y, cx, cy, bx, by):
+    dt = _same_dtype(x, y)
+    X, Y = _BmmOperand(x, cx, bx, "x"), _BmmOperand(y, cy, by, "y")
+    if X.K != Y.K:
+        raise DimensionMismatch(f"size(x) = {x.shape}, size(y) = {y.shape} inconsistent for batched_matmul.")
+    for a_, b_ in zip(X.bext, Y.bext):
+        if a_ != b_ and a_ != 1 and b_ != 1:
+            raise DimensionMismatch(f"Batching dimensions mismatch: {X.bext} vs {Y.bext}")      # impl/batched_mul.jl:133-141
+    M, N, K = X.F, Y.F, X.K
+    ext = [max(a_, b_) if min(a_, b_) > 0 else 0 for a_, b_ in zip(X.bext, Y.bext)]
+    zst = _dense_strides((M, N) + tuple(ext))[2:]
+    sx = [st if e > 1 else 0 for st, e in zip(X.bst, X.bext)]
+    sy = [st if e > 1 else 0 for st, e in zip(Y.bst, Y.bext)]
+    tA, tB = not X.free_major, Y.free_major          # A is M x K: transposed storage = contracting-major; B is K x N
+    z = DeviceArray((M, N) + tuple(ext), dt)
+    if z.size:
+        _launch_general(tA, tB, M, N, K, list(zip(ext, sx, sy, zst)), x, X.ld, y, Y.ld, z, M)
+
+    def grad(op, other_is_y):
+        """Gradient of one operand, in its own layout."""
+        a = op.a
+        shared = [i for i in range(len(ext)) if op.bext[i] == 1 and ext[i] > 1]
+        shared_total = int(np.prod([ext[i] for i in shared], dtype=np.int64)) if shared else 1
+        target = DeviceArray(tuple(a.shape) + ((shared_total,) if shared else ()), dt)
+        # a repeated operand gets one slab in its own layout per repetition, summed afterwards (the repeated
+        # dims have extent 1 in the operand, so they do not enter its layout)
+        sc, p = [0] * len(ext), a.size
+        for i in range(len(ext)):
+            sc[i] = op.bst[i] if op.bext[i] > 1 else 0
+        for i in shared:
+            sc[i] = p
+            p *= ext[i]
+        return a, shared, shared_total, target, sc
+
+    def back(delta: DeviceArray):
+        out = []
+        for op, is_x in ((X, True), (Y, False)):
+            a, shared, shared_total, target, sc = grad(op, is_x)
+            if target.size:
+                pairs = lambda sother: list(zip(ext, zst, sother, sc))
+                if is_x:
+                    if X.free_major:        # dx (M x K) = Δ op(y)ᵀ
+                        _launch_general(False, not tB, M, K, N, pairs(sy), delta, M, y, Y.ld, target, X.ld)
+                    else:                   # stored K x M: op(y) Δᵀ
+                        _launch_general(tB, True, K, M, N, [(e, b_, a_, c_) for e, a_, b_, c_ in pairs(sy)], y, Y.ld, delta, M,
+                                        target, X.ld)
+                else:
+                    if not Y.free_major:    # dy (K x N) = op(x)ᵀ Δ
+                        _launch_general(not tA, False, K, N, M, [(e, b_, a_, c_) for e, a_, b_, c_ in pairs(sx)], x, X.ld, delta, M,
+                                        target, Y.ld)
+                    else:                   # stored N x K: Δᵀ op(x)
+                        _launch_general(True, tA, N, K, M, pairs(sx), delta, M, x, X.ld, target, Y.ld)
+            if shared:
+                red = DeviceArray(a.shape, dt)
+                _lib.call("luxhip_batch_sum", current_stream(), red.code, a.size, shared_total, target.ptr, red.ptr)
+                target = red
+            out.append(target)
+        return tuple(out)
+
+    return z, back
+
+
+def rrule_batched_matmul(x, y, lhs_contracting_dim=2, rhs_contracting_dim=1, lhs_batching_dims=None, rhs_batching_dims=None,
+                         _need_back=True):
     """CRC.rrule(batched_matmul_fallback) (impl/batched_mul.jl:320-334): (z, Δ -> (∂x, ∂y)) with
     ∂x = Δ ⊠ adjoint(y), ∂y = adjoint(x) ⊠ Δ, summed over the batch for a shared operand."""
     x_shape, y_shape = x.shape, y.shape
     dt = _same_dtype(x, y)
+    trailing = lambda a, bd: bd is None or tuple(bd) == tuple(range(3, a.ndim + 1))
+    simple = (trailing(x, lhs_batching_dims) and trailing(y, rhs_batching_dims) and lhs_contracting_dim in (1, 2)
+              and rhs_contracting_dim in (1, 2))
+    if simple and x.ndim == y.ndim and x.ndim >= 3:
+        xb_, yb_ = x.shape[2:], y.shape[2:]
+        full = tuple(max(a_, b_) for a_, b_ in zip(xb_, yb_))
+        simple = all(a_ in (b_, 1) or b_ == 1 for a_, b_ in zip(xb_, yb_)) and all(
+            tuple(o) == full or int(np.prod(o, dtype=np.int64)) == 1 for o in (xb_, yb_))
+    if not simple and x.ndim == y.ndim and x.ndim >= 3:
+        return _rrule_batched_matmul_general(x, y, lhs_contracting_dim, rhs_contracting_dim, lhs_batching_dims, rhs_batching_dims)
     x, y, tA, tB, M, N, K, batch, xb, yb, bshape = _batched_geometry(x, y, lhs_contracting_dim, rhs_contracting_dim)
     sx, sy = (x.shape[0] * x.shape[1] if xb > 1 else 0), (y.shape[0] * y.shape[1] if yb > 1 else 0)
     z = _bmm(x, tA, y, tB, M, N, K, batch, sx, sy, dt).reshape((M, N) + bshape)

@@ -557,6 +557,50 @@ def batched_matmul_pullback(x, y, delta, lhs_contracting_dim=2, rhs_contracting_
     return dx.reshape(x0.shape), dy.reshape(y0.shape)
 
 
+def _general_bmm_axes(ndim, contracting_dim, batching_dims):
+    """0-based (non-contracting axis, contracting axis, batching axes) for 1-based dims
+    (get_non_contracting_dim, impl/batched_mul.jl)."""
+    if batching_dims is None:
+        batching_dims = tuple(range(3, ndim + 1))
+    rest = [d for d in range(1, ndim + 1) if d != contracting_dim and d not in batching_dims]
+    assert len(rest) == 1 and len(batching_dims) == ndim - 2, "one contracting, one free and N-2 batching dims"
+    return rest[0] - 1, contracting_dim - 1, tuple(d - 1 for d in batching_dims)
+
+
+def batched_matmul_general(x, y, lhs_contracting_dim=2, rhs_contracting_dim=1, lhs_batching_dims=None, rhs_batching_dims=None):
+    """batched_matmul with arbitrary batching dims (api/batched_mul.jl, impl/batched_mul.jl:2-58): the
+    operands are permuted to (free, contracting, batch...) / (contracting, free, batch...), batch dims of
+    extent 1 repeat, and z = (free_x, free_y, batch...)."""
+    x, y = np.asarray(x), np.asarray(y)
+    fx, cx, bx = _general_bmm_axes(x.ndim, lhs_contracting_dim, lhs_batching_dims)
+    fy, cy, by = _general_bmm_axes(y.ndim, rhs_contracting_dim, rhs_batching_dims)
+    xp, yp = np.transpose(x, (fx, cx) + bx), np.transpose(y, (cy, fy) + by)
+    for a, b in zip(xp.shape[2:], yp.shape[2:]):
+        if a != b and a != 1 and b != 1:
+            raise DimensionMismatch("Batching dimensions mismatch")
+    return np.einsum("mk...,kn...->mn...", xp, yp)
+
+
+def batched_matmul_general_pullback(x, y, delta, lhs_contracting_dim=2, rhs_contracting_dim=1, lhs_batching_dims=None,
+                                    rhs_batching_dims=None):
+    """(∂x, ∂y) in the operands' own layouts: the rrule of the permuted product (impl/batched_mul.jl:320-334),
+    summed over repeated batch dims, taken back through the permutation."""
+    x, y, delta = np.asarray(x), np.asarray(y), np.asarray(delta)
+    fx, cx, bx = _general_bmm_axes(x.ndim, lhs_contracting_dim, lhs_batching_dims)
+    fy, cy, by = _general_bmm_axes(y.ndim, rhs_contracting_dim, rhs_batching_dims)
+    px, py = (fx, cx) + bx, (cy, fy) + by
+    xp, yp = np.transpose(x, px), np.transpose(y, py)
+    full = delta.shape[2:]
+    dxp = np.einsum("mn...,kn...->mk...", delta, np.broadcast_to(yp, yp.shape[:2] + full))
+    dyp = np.einsum("mk...,mn...->kn...", np.broadcast_to(xp, xp.shape[:2] + full), delta)
+    for ax in range(2, delta.ndim):
+        if xp.shape[ax] == 1 and delta.shape[ax] != 1:
+            dxp = dxp.sum(axis=ax, keepdims=True)
+        if yp.shape[ax] == 1 and delta.shape[ax] != 1:
+            dyp = dyp.sum(axis=ax, keepdims=True)
+    return np.transpose(dxp, np.argsort(px)), np.transpose(dyp, np.argsort(py))
+
+
 # --------------------------------------------------------------------------------------
 # scaled_dot_product_attention  (api/attention.jl, impl/attention.jl:5-134), head_dim = 1
 # --------------------------------------------------------------------------------------

@@ -75,3 +75,40 @@ def test_attention_shaped_products(gpu, dtype):
                  scale=1.0)
     shared = gpu.batched_matmul(dev(gpu, k[..., :1], dtype), dev(gpu, q, dtype), 1, 1).to_numpy()
     assert_close(shared[..., sub], O.batched_matmul(f64(k[..., :1]), f64(q[..., sub]), 1, 1), dtype, "shared scores", scale=1.0)
+
+
+GENERAL = [
+    # x shape, y shape, lhs contracting, rhs contracting, lhs batching dims, rhs batching dims
+    ((3, 4, 5, 2), (5, 4, 5, 1), 2, 2, None, None),            # generalized_bmm_tests.jl:8-22: a partly repeated operand
+    ((3, 5, 2, 4), (4, 5, 1, 5), 4, 1, (2, 3), (4, 3)),        # generalized_bmm_tests.jl:36-58: batch dims in the middle
+    ((6, 3, 4, 7), (6, 3, 5, 7), 1, 1, (2, 4), (2, 4)),        # contraction along the first dim of both
+    ((4, 2, 3, 5, 6), (1, 6, 3, 7, 5), 5, 2, (2, 3, 4), (1, 3, 5)),
+    ((33, 2, 3, 70), (70, 3, 1, 40), 4, 1, (2, 3), (3, 2)),
+    ((5, 4, 1, 1), (4, 6, 3, 2), 2, 1, None, None),
+    ((5, 2, 3, 4, 1), (4, 2, 3, 6, 2), 4, 1, (2, 3, 5), (2, 3, 5)),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("case", range(len(GENERAL)))
+def test_general_batching_dims(gpu, dtype, case):
+    xs, ys, cx, cy, bx, by = GENERAL[case]
+    rng = np.random.default_rng(stable_seed("bmm-general", case))
+    x, y = host_inputs(dtype, rng.normal(size=xs), rng.normal(size=ys))
+    want = O.batched_matmul_general(f64(x), f64(y), cx, cy, bx, by)
+    (delta,) = host_inputs(dtype, rng.normal(size=want.shape))
+    z, back = gpu.pullback(gpu.batched_matmul, dev(gpu, x, dtype), dev(gpu, y, dtype), cx, cy, bx, by)
+    assert z.shape == want.shape
+    assert_close(z.to_numpy(), want, dtype, f"case {case} z")
+    dx, dy = back(dev(gpu, delta, dtype))
+    wdx, wdy = O.batched_matmul_general_pullback(f64(x), f64(y), f64(delta), cx, cy, bx, by)
+    assert dx.shape == tuple(xs) and dy.shape == tuple(ys)
+    rel = None if dtype == "f32" else 3e-2
+    assert_close(dx.to_numpy(), wdx, dtype, f"case {case} dx", rel=rel)
+    assert_close(dy.to_numpy(), wdy, dtype, f"case {case} dy", rel=rel)
+
+
+def test_operand_without_a_contiguous_matrix_dim_is_refused(gpu):
+    d = lambda *shape: gpu.DeviceArray.from_numpy(np.ones(shape, np.float32))
+    with pytest.raises(gpu.Unsupported):          # y: contracting dim 3 (stride 6), free dim 4 (stride 36)
+        gpu.batched_matmul(d(4, 2, 3, 5, 6), d(2, 3, 6, 7, 5), 5, 3, (2, 3, 4), (1, 2, 5))

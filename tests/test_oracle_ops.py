@@ -664,3 +664,38 @@ def test_attention_reference_specific_results():
              0.380066, 0.241239, 0.323893, 0.434868, 0.198438, 0.311761, 0.489801]
     np.testing.assert_allclose(y, np.reshape(ytrue, (2, 2, 3, 1), order="F"), rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(w, np.reshape(wtrue, (3, 3, 2, 1), order="F"), rtol=1e-5, atol=1e-5)
+
+
+def _nnlib_batched_mul(a, b):
+    """NNlib.batched_mul on (M, K, B...) and (K, N, B...) arrays of equal batch dims, slice by slice."""
+    out = np.zeros((a.shape[0], b.shape[1]) + a.shape[2:])
+    for idx in np.ndindex(*a.shape[2:]):
+        out[(slice(None), slice(None)) + idx] = a[(slice(None), slice(None)) + idx] @ b[(slice(None), slice(None)) + idx]
+    return out
+
+
+def test_generalized_batched_matmul_as_the_reference_tests_it():
+    """test/others/bmm/generalized_bmm_tests.jl:8-22 and :36-58: the result equals NNlib.batched_mul on the
+    operands after permutedims + repeat."""
+    rng = np.random.default_rng(70)
+    x, y = rng.normal(size=(3, 4, 5, 2)), rng.normal(size=(5, 4, 5, 1))
+    want = _nnlib_batched_mul(x, np.tile(np.transpose(y, (1, 0, 2, 3)), (1, 1, 1, 2)))
+    np.testing.assert_allclose(O.batched_matmul_general(x, y, 2, 2), want, rtol=1e-12, atol=1e-12)
+    x, y = rng.normal(size=(3, 5, 2, 4)), rng.normal(size=(4, 5, 1, 5))
+    want = _nnlib_batched_mul(np.transpose(x, (0, 3, 1, 2)), np.tile(np.transpose(y, (0, 1, 3, 2)), (1, 1, 1, 2)))
+    got = O.batched_matmul_general(x, y, 4, 1, (2, 3), (4, 3))
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+    # gradients: finite differences of sum(z .* delta)
+    delta = rng.normal(size=got.shape)
+    dx, dy = O.batched_matmul_general_pullback(x, y, delta, 4, 1, (2, 3), (4, 3))
+    f = lambda xx, yy: float(np.sum(O.batched_matmul_general(xx, yy, 4, 1, (2, 3), (4, 3)) * delta))
+    for arr, grad, which in ((x, dx, 0), (y, dy, 1)):
+        assert grad.shape == arr.shape
+        for idx in [tuple(rng.integers(0, n) for n in arr.shape) for _ in range(6)]:
+            e = np.zeros_like(arr)
+            e[idx] = 1e-5
+            num = (f(x + e, y) - f(x - e, y)) / 2e-5 if which == 0 else (f(x, y + e) - f(x, y - e)) / 2e-5
+            np.testing.assert_allclose(grad[idx], num, rtol=1e-6, atol=1e-8)
+    # the default dims agree with the plain function
+    a, b = rng.normal(size=(4, 3, 2, 5)), rng.normal(size=(3, 6, 1, 5))
+    np.testing.assert_allclose(O.batched_matmul_general(a, b), O.batched_matmul(a, b), rtol=1e-12)
