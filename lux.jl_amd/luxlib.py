@@ -898,13 +898,38 @@ def _layernorm_geometry(x, scale, bias, dims):
         raise DimensionMismatch(f"scale/bias of shape {pshape} do not broadcast against x {x.shape}")
     if pshape == tuple(x.shape[:k]) + (1,) * (nd - k):
         return L, R, None
-    # the dims along which the parameters vary must be one contiguous run
+    # the per-channel pass wants the parameters to vary along one contiguous run of dims [a, b); parameters
+    # with gaps in between (e.g. (3, 1, 3, 1)) are first repeated along the gaps (_expand_parameters)
     varying = [d for d in range(nd) if pshape[d] != 1]
     a, b = (varying[0], varying[-1] + 1) if varying else (nd, nd)
-    if any(pshape[d] != x.shape[d] for d in range(a, b)):
-        raise _lib.Unsupported(_lib.UNSUPPORTED, f"layernorm affine parameters of shape {pshape} for x {x.shape}")
     prod = lambda t: int(np.prod(t, dtype=np.int64)) if len(t) else 1
     return L, R, (prod(x.shape[:a]), prod(x.shape[a:b]), prod(x.shape[b:]))
+
+
+def _expand_parameters(x, pshape, *params):
+    """Parameters of (expanded) shape `pshape` repeated along the dims that lie between the first and the
+    last dim they vary along, and the function that sums a gradient of the repeated shape back."""
+    nd = x.ndim
+    varying = [d for d in range(nd) if pshape[d] != 1]
+    a, b = (varying[0], varying[-1] + 1) if varying else (nd, nd)
+    gaps = [d for d in range(a, b) if pshape[d] == 1 and x.shape[d] != 1]
+    if not gaps:
+        return params, (lambda g: g)
+    full = tuple(x.shape[d] if a <= d < b else 1 for d in range(nd))
+    ones = DeviceArray.from_numpy(np.ones(full, np.float32), x.dtype)
+    expanded = tuple(dropout_dot_mul(ones, p_.reshape(pshape)) for p_ in params)
+
+    def reduce(g):
+        shape = list(full)
+        for d in gaps:                       # sum over dim d: (A, B, C) x ones(B) -> (A, 1, C)
+            A, B = int(np.prod(shape[:d], dtype=np.int64)), shape[d]
+            Cc = int(np.prod(shape[d + 1:], dtype=np.int64))
+            vec = DeviceArray.from_numpy(np.ones((B, 1, 1), np.float32), x.dtype)
+            g = batched_matmul(g.reshape(A, B, Cc), vec)
+            shape[d] = 1
+        return g.reshape(pshape)
+
+    return expanded, reduce
 
 
 def layernorm(x: DeviceArray, scale, bias, act: str = "identity", dims=DEFAULT_DIMS, epsilon: Optional[float] = None):
@@ -930,11 +955,17 @@ def _layernorm_fwd(x, scale, bias, act, dims, epsilon, save):
     # affine transform and activation as a batchnorm in inference mode with mean 0, variance 1, ε = 0
     _lib.call("luxhip_layernorm_fwd", current_stream(), x.code, 0, L, R, x.ptr, None, None, float(epsilon), y.ptr, _p(sm), _p(si))
     I, Cc, Nn = view
+    pshape = tuple(scale.shape) + (1,) * (x.ndim - scale.ndim)
+    (gam, bet), reduce = _expand_parameters(x, pshape, scale, bias)
     zeros = DeviceArray.from_numpy(np.zeros(Cc, np.float32), dt)
     ones = DeviceArray.from_numpy(np.ones(Cc, np.float32), dt)
-    args = (y.reshape(I, Cc, Nn), scale.reshape(Cc), bias.reshape(Cc), zeros, ones, False, act, 0.1, 0.0)
+    args = (y.reshape(I, Cc, Nn), gam.reshape(Cc), bet.reshape(Cc), zeros, ones, False, act, 0.1, 0.0)
     if save:
-        (out, _), affine_back = rrule_batchnorm(*args)
+        (out, _), bn_back = rrule_batchnorm(*args)
+
+        def affine_back(delta3):
+            dxhat, dg, db = bn_back(delta3)
+            return dxhat, reduce(dg), reduce(db)
     else:
         (out, _), affine_back = batchnorm(*args), None
     return out.reshape(x.shape), (sm, si, L, R, affine_back)

@@ -9,7 +9,8 @@ from tests.util import stable_seed, assert_close, dev, f64, host_inputs
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(7,), (4, 4), (5, 3, 2), (16, 16, 8, 3), (33, 65, 2), (1000, 37), (0, 3)]
+# the last four are the shapes of lib/LuxLib/test/common_ops/dropout_tests.jl:10
+SHAPES = [(7,), (4, 4), (5, 3, 2), (16, 16, 8, 3), (33, 65, 2), (1000, 37), (0, 3), (2, 3), (2, 2, 3), (2, 2, 3, 1), (2, 2, 1, 3, 1)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
@@ -34,7 +35,7 @@ def test_dropout(gpu, dtype, p):
     rng = gpu.PhiloxRNG(seed=77, offset=5)
     for shape in SHAPES:
         nd = len(shape)
-        for dims in [None, (1,), (nd,), tuple(range(1, nd)), (1, nd)][: 5 if nd > 1 else 1]:
+        for dims in [None, (1,), (nd,), tuple(range(1, nd)), (1, nd), (1, 2)][: (6 if nd > 2 else 5) if nd > 1 else 1]:
             if dims is not None and (len(dims) == 0 or len(set(dims)) != len(dims)):
                 continue
             x, delta = host_inputs(dtype, nprng.normal(size=shape), nprng.normal(size=shape))

@@ -157,7 +157,14 @@ def test_channel_parameters_on_larger_shapes(gpu, dtype):
                                    ((16, 12, 24, 5), (1, 2), (1, 1, 24, 1), (0, 1)),
                                    ((64, 8, 6), (1,), (1, 8, 6), (0,)),
                                    ((32, 10, 7), None, (32, 10), (0,)),
-                                   ((8, 4, 6, 3), (1, 2), (1, 1, 1, 1), (0, 1))]:
+                                   ((8, 4, 6, 3), (1, 2), (1, 1, 1, 1), (0, 1)),
+                                   # test/core_layers/normalize_tests.jl:279-283: LayerNorm((3, 3, 3)), ((1, 3, 1)), ((3, 1, 3)) on
+                                   # x 3x3x3x2 with the layer's dims = Colon()
+                                   ((3, 3, 3, 2), gpu.COLON, (3, 3, 3, 1), (0, 1, 2, 3)),
+                                   ((3, 3, 3, 2), gpu.COLON, (1, 3, 1, 1), (0, 1, 2, 3)),
+                                   ((3, 3, 3, 2), gpu.COLON, (3, 1, 3, 1), (0, 1, 2, 3)),
+                                   ((16, 5, 12, 4), (1, 2, 3), (16, 1, 12, 1), (0, 1, 2)),
+                                   ((6, 4, 5, 3, 2), (1, 2), (6, 1, 5, 1, 2), (0, 1))]:
         full = pshape + (1,) * (len(xs) - len(pshape))
         x, g, b, delta = host_inputs(dtype, rng.normal(size=xs) * 2 + 0.5, rng.uniform(0.5, 1.5, size=pshape), rng.normal(size=pshape),
                                      rng.normal(size=xs))
