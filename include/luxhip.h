@@ -94,7 +94,10 @@ int luxhip_set_option(const char* name, int64_t value);
 int luxhip_profile_report(char* buf, size_t len);
 
 /* Pooled device allocator (size-bucketed free lists; luxhip_free returns the block to the
- * pool, luxhip_trim releases the pool to the driver). */
+ * pool, luxhip_trim releases the pool to the driver).  A freed block can be handed out again at
+ * once: work that still uses it must have been enqueued on the stream on which the next owner will
+ * enqueue (one stream: always true), or be finished - a caller with several streams synchronises
+ * the stream that last used a block before freeing it. */
 int luxhip_malloc(void** out, size_t bytes);
 int luxhip_free(void* p);
 int luxhip_trim(void);

@@ -1,0 +1,142 @@
+"""The part of the C ABI that owns device buffers, streams and events (what the reference gets from
+its GPU array package): streams keep their work ordered and their scratch memory apart, the pooled
+allocator reuses blocks, events time a stream, the per-kernel profile names the kernels that ran,
+and errors come back as status codes with a message."""
+import ctypes as C
+import json
+
+import numpy as np
+import pytest
+
+from oracle import luxlib_oracle as O
+from tests.util import assert_close, dev, f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _new_stream(gpu):
+    s = C.c_void_p()
+    gpu._lib.call("luxhip_stream_create", C.byref(s))
+    return s
+
+
+def test_device_info(gpu):
+    info = gpu.device_info()
+    assert info["compute_units"] > 0 and info["total_mem"] > 0 and info["name"]
+
+
+def test_two_streams_keep_their_scratch_apart(gpu):
+    """batchnorm (arrival counters, exchange words, partial sums in the per-stream workspace) and
+    groupnorm pullbacks issued alternately on two streams that are not synchronised with each other:
+    every result equals the one computed alone."""
+    rng = np.random.default_rng(3)
+    main = gpu.current_stream()
+    other = _new_stream(gpu)
+    shapes = [(16, 16, 8, 4), (32, 32, 16, 8), (6, 5, 12, 3)]
+    cases = []
+    for shape in shapes:
+        Cc = shape[2]
+        x, d = rng.normal(size=shape).astype(np.float32), rng.normal(size=shape).astype(np.float32)
+        g, b = rng.uniform(0.5, 1.5, Cc).astype(np.float32), rng.normal(size=Cc).astype(np.float32)
+        cases.append((x, d, g, b))
+    results = {0: [], 1: []}
+    keep = []            # a block that goes back to the pool may be handed to the other stream at once: nothing
+    # is released before both streams have finished
+    try:
+        for rep in range(3):
+            for x, d, g, b in cases:
+                for which, stream in ((0, main), (1, other)):
+                    gpu.set_stream(stream)
+                    xs = x if which == 0 else -x          # different data per stream
+                    dx_, dd_, dg_, db_ = dev(gpu, xs, "f32"), dev(gpu, d, "f32"), dev(gpu, g, "f32"), dev(gpu, b, "f32")
+                    (y, _), back = gpu.pullback(gpu.batchnorm, dx_, dg_, db_, None, None, True, "relu", 0.1, 1e-5)
+                    grads = back(dd_)
+                    y2, back2 = gpu.pullback(gpu.groupnorm, dx_, dg_, db_, 2, "identity", 1e-5)
+                    grads2 = back2(dd_)
+                    keep.append((dx_, dd_, dg_, db_, back, back2))
+                    results[which].append((xs, d, g, b, y, grads, y2, grads2))
+        for stream in (main, other):
+            gpu._lib.call("luxhip_stream_synchronize", stream)
+    finally:
+        gpu.set_stream(main)
+    for which in (0, 1):
+        for xs, d, g, b, y, grads, y2, grads2 in results[which]:
+            want_y = O.batchnorm(f64(xs), f64(g), f64(b), None, None, True, "relu", 0.1, 1e-5)[0]
+            assert_close(y.to_numpy(), want_y, "f32", "batchnorm y", rel=1e-4)
+            assert_close(y2.to_numpy(), O.groupnorm(f64(xs), f64(g), f64(b), 2, "identity", 1e-5), "f32", "groupnorm y", rel=1e-4)
+            wg = O.groupnorm_pullback(f64(xs), f64(g), f64(b), 2, "identity", 1e-5, f64(d))
+            for got, w_, name in zip(grads2, wg, ("dx", "dgamma", "dbeta")):
+                assert_close(got.to_numpy(), w_, "f32", "groupnorm " + name, rel=1e-4, scale=float(np.abs(d).mean()) * 4)
+            # batchnorm: the same call alone on the main stream gives the same bits
+            (y_alone, _), back = gpu.pullback(gpu.batchnorm, dev(gpu, xs, "f32"), dev(gpu, g, "f32"), dev(gpu, b, "f32"),
+                                              None, None, True, "relu", 0.1, 1e-5)
+            alone = back(dev(gpu, d, "f32"))
+            np.testing.assert_array_equal(y.to_numpy(), y_alone.to_numpy())
+            for got, ref in zip(grads, alone):
+                np.testing.assert_array_equal(got.to_numpy(), ref.to_numpy())
+    gpu._lib.call("luxhip_stream_destroy", other)
+
+
+def test_pooled_allocator_reuses_blocks(gpu):
+    a = gpu.DeviceArray((1 << 20,), "f32")
+    ptr = a.ptr
+    del a
+    b = gpu.DeviceArray((1 << 20,), "f32")
+    assert b.ptr == ptr                                   # the block came back from the pool
+    del b
+    gpu._lib.call("luxhip_trim")                          # the pool goes back to the driver; the library keeps working
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    np.testing.assert_array_equal(gpu.DeviceArray.from_numpy(x).to_numpy(), x)
+    p = C.c_void_p()
+    gpu._lib.call("luxhip_malloc", C.byref(p), 0)         # zero bytes: a valid call
+    gpu._lib.call("luxhip_free", p)
+    with pytest.raises(gpu.LuxHipError):
+        gpu._lib.call("luxhip_free", C.c_void_p(0x1000))  # not a block of the pool
+
+
+def test_events_time_the_stream(gpu):
+    x = gpu.DeviceArray((1 << 24,), "f32")
+    e0, e1 = gpu.Event(), gpu.Event()
+    e0.record()
+    for _ in range(10):
+        gpu.bias_activation("relu", x.reshape(1 << 12, 1 << 12), None)
+    e1.record()
+    ms = e0.elapsed_ms(e1)
+    assert 0.0 < ms < 1000.0
+
+
+def test_profile_reports_the_kernels_that_ran(gpu):
+    rng = np.random.default_rng(1)
+    x = dev(gpu, rng.normal(size=(64, 32, 8)), "f32")
+    gpu._lib.call("luxhip_profile_enable", 1)
+    try:
+        gpu.bias_activation("relu", x, None)
+        gpu.groupnorm(x, None, None, 4)
+        buf = C.create_string_buffer(1 << 16)
+        gpu._lib.call("luxhip_profile_report", buf, len(buf))
+    finally:
+        gpu._lib.call("luxhip_profile_enable", 0)
+    rows = json.loads(buf.value.decode())
+    names = {r["kernel"] for r in rows}
+    assert "bias_act_fwd_kernel" in names and "gn_fwd_kernel" in names
+    for r in rows:
+        assert r["count"] >= 1 and 0.0 < r["min_ms"] <= r["max_ms"] and r["total_ms"] >= r["max_ms"] * 0.999
+    # the log was cleared by the report
+    buf2 = C.create_string_buffer(1 << 12)
+    gpu._lib.call("luxhip_profile_report", buf2, len(buf2))
+    assert json.loads(buf2.value.decode()) == []
+
+
+def test_errors_carry_a_status_and_a_message(gpu):
+    with pytest.raises(gpu.LuxHipError) as err:
+        gpu.set_option("no_such_option", 1)
+    assert "no_such_option" in str(err.value)
+    x = gpu.DeviceArray.from_numpy(np.ones((4, 6, 2), np.float32))
+    with pytest.raises(gpu.Unsupported) as err:
+        gpu._lib.call("luxhip_bias_activation_fwd", gpu.current_stream(), 7, 0, 4, 6, 2, x.ptr, None, x.ptr, None)   # dtype 7
+    assert err.value.status == -1 and "dtype" in str(err.value)
+    with pytest.raises(gpu.LuxHipError) as err:           # 6 channels do not divide into 4 groups
+        gpu._lib.call("luxhip_groupnorm_fwd", gpu.current_stream(), 0, 0, 4, 6, 4, 2, x.ptr, None, None, 1e-5, x.ptr, None, None)
+    assert "divisible" in str(err.value)
+    # the library is still usable after the errors
+    np.testing.assert_array_equal(gpu.bias_activation("relu", x, None).to_numpy(), np.ones((4, 6, 2), np.float32))
