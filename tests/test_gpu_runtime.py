@@ -78,6 +78,8 @@ def test_two_streams_keep_their_scratch_apart(gpu):
 
 
 def test_pooled_allocator_reuses_blocks(gpu):
+    gpu.synchronize()
+    gpu._lib.call("luxhip_trim")                          # start from an empty pool
     a = gpu.DeviceArray((1 << 20,), "f32")
     ptr = a.ptr
     del a
