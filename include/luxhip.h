@@ -88,6 +88,8 @@ int luxhip_profile_enable(int on);
  *   "gemm_tile"     0 automatic (default), 82 | 42 | 22 | 11 force a GEMM tile shape
  *   "gemm_pretranspose" 1 (default) / 0: large bf16 matmul operands that are contiguous along m or n
  *                   are first copied into the k-contiguous layout the fastest kernel reads
+ *   "workspace_epoch" (tests) the epoch from which the per-stream exchange words continue; the 32-bit
+ *                   epoch wraps after 2^32 calls, at which point the library clears those words
  *   "conv_tile"     0 automatic (default); bf16 whole-tap convolution kernels: 82 = 256x256 tile on
  *                   8 waves, 84 / 83 = 512x128 on 8 waves with 4 / 3 LDS stages, 42 = 256x128 on 4 waves */
 int luxhip_set_option(const char* name, int64_t value);

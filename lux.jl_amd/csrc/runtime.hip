@@ -110,6 +110,8 @@ int64_t option_gemm_tile() {
     return v;
 }
 
+__global__ void fill_zero_kernel(uint32_t* p, size_t nwords);
+
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     std::lock_guard<std::mutex> lk(g_mu);
     WsEntry& e = g_ws[s];
@@ -138,7 +140,14 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     out->counters = e.counters;
     out->flags = e.counters + kWorkspaceCounters;
     out->zeros = e.counters + kWorkspaceCounters + kWorkspaceFlags;
-    if (++e.epoch == 0) e.epoch = 1;   // 0 is what freshly cleared flags hold
+    if (++e.epoch == 0) {
+        // the 32-bit epoch has wrapped: words tagged during the previous cycle must not be taken for
+        // new ones, so the exchange words are cleared (on the stream, behind every kernel that used
+        // them) and the count starts again at 1; 0 is what cleared words hold
+        fill_zero_kernel<<<dim3(16), dim3(256), 0, s>>>(e.counters + kWorkspaceCounters, kWorkspaceFlags);
+        LUX_CHECK_LAUNCH();
+        e.epoch = 1;
+    }
     out->epoch = e.epoch;
     return LUXHIP_OK;
 }
@@ -217,6 +226,11 @@ int luxhip_set_option(const char* name, int64_t value) {
     } else if (strcmp(name, "gemm_pretranspose") == 0) {
         LUX_INVALID_IF(value != 0 && value != 1, "set_option: gemm_pretranspose must be 0 or 1");
         g_opt_gemm_pretranspose.store(value);
+    } else if (strcmp(name, "workspace_epoch") == 0) {
+        // for tests: the next call on every stream continues from this epoch (e.g. just below 2^32)
+        LUX_INVALID_IF(value < 0 || value > (int64_t)0xffffffffll, "set_option: workspace_epoch out of range");
+        std::lock_guard<std::mutex> lk(g_mu);
+        for (auto& kv : g_ws) kv.second.epoch = (uint32_t)value;
     } else {
         return set_error(LUXHIP_INVALID, "set_option: unknown option '%s'", name);
     }

@@ -142,3 +142,31 @@ def test_errors_carry_a_status_and_a_message(gpu):
     assert "divisible" in str(err.value)
     # the library is still usable after the errors
     np.testing.assert_array_equal(gpu.bias_activation("relu", x, None).to_numpy(), np.ones((4, 6, 2), np.float32))
+
+
+def test_exchange_word_epoch_wraps(gpu):
+    """The resident batchnorm kernels and the split groupnorm pullback tag the words they exchange with a
+    32-bit per-stream epoch.  Across the wrap (forced here through the test option) the words are
+    cleared and results stay right, call after call."""
+    rng = np.random.default_rng(21)
+    shape = (32, 32, 16, 8)
+    x, d = rng.normal(size=shape).astype(np.float32), rng.normal(size=shape).astype(np.float32)
+    g, b = rng.uniform(0.5, 1.5, 16).astype(np.float32), rng.normal(size=16).astype(np.float32)
+    want_y = O.batchnorm(f64(x), f64(g), f64(b), None, None, True, "identity", 0.1, 1e-5)[0]
+    want_g = O.batchnorm_pullback(f64(x), f64(g), f64(b), "identity", 1e-5, f64(d))
+    gshape = (64, 64, 16, 2)                                 # slices of 64*64*8 elements: split between two workgroups
+    xg, dg_ = rng.normal(size=gshape).astype(np.float32), rng.normal(size=gshape).astype(np.float32)
+    want_gn = O.groupnorm_pullback(f64(xg), f64(g), f64(b), 2, "identity", 1e-5, f64(dg_))
+    dx_, dd_, dgam, dbet = dev(gpu, x, "f32"), dev(gpu, d, "f32"), dev(gpu, g, "f32"), dev(gpu, b, "f32")
+    dxg, ddg = dev(gpu, xg, "f32"), dev(gpu, dg_, "f32")
+    gpu.bias_activation("relu", dx_, None)                  # the stream has its workspace
+    gpu.set_option("workspace_epoch", (1 << 32) - 6)
+    for it in range(12):
+        (y, _), back = gpu.pullback(gpu.batchnorm, dx_, dgam, dbet, None, None, True, "identity", 0.1, 1e-5)
+        grads = back(dd_)
+        assert_close(y.to_numpy(), want_y, "f32", f"call {it}: y", rel=1e-4)
+        for got, want, name in zip(grads, want_g, ("dx", "dgamma", "dbeta")):
+            assert_close(got.to_numpy(), want, "f32", f"call {it}: {name}", rel=1e-4, scale=1.0)
+        _, back_g = gpu.pullback(gpu.groupnorm, dxg, dgam, dbet, 2, "identity", 1e-5)
+        for got, want, name in zip(back_g(ddg), want_gn, ("dx", "dgamma", "dbeta")):
+            assert_close(got.to_numpy(), want, "f32", f"call {it}: groupnorm {name}", rel=1e-4, scale=1.0)
