@@ -476,6 +476,49 @@ def timed(lux, fn, steps, warmup):
     return ms_gpu / steps, ms_wall / steps
 
 
+def timed_graph(lux, fn, steps):
+    """One step recorded into a HIP graph on the library's stream (after the eager warm-up has sized the
+    workspace and filled the allocator's pool) and replayed `steps` times: the step without the host's
+    per-call work.  While the stream records, batchnorm and groupnorm use their two-pass kernels."""
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    stream = lux.current_stream()
+    lux.synchronize()
+    if hip.hipStreamBeginCapture(stream, 1) != 0:
+        return None
+    try:
+        fn()
+    finally:
+        graph = C.c_void_p()
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    if rc != 0 or not graph.value:
+        return None
+    gexec = C.c_void_p()
+    if hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) != 0:
+        hip.hipGraphDestroy(graph)
+        return None
+    for _ in range(3):
+        hip.hipGraphLaunch(gexec, stream)
+    lux.synchronize()
+    e0, e1 = lux.Event(), lux.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        hip.hipGraphLaunch(gexec, stream)
+    e1.record()
+    ms_gpu = e0.elapsed_ms(e1)
+    lux.synchronize()
+    ms_wall = (time.perf_counter() - t0) * 1e3
+    hip.hipGraphExecDestroy(gexec)
+    hip.hipGraphDestroy(graph)
+    return max(ms_gpu, ms_wall) / steps
+
+
 def kernel_profile(lux, fn, steps):
     """Per-kernel average duration: every launch bracketed by HIP events on its stream."""
     lux._lib.call("luxhip_profile_enable", 1)
@@ -499,6 +542,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB: a kernel of known traffic that "
                          "scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--graph", action="store_true",
+                    help="also record one step into a HIP graph and time its replays (reported as graph_replay; "
+                         "value stays the eager figure)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path is single-GPU; no collective is part of it); "
@@ -520,6 +566,7 @@ def main():
 
     ms_gpu, ms_wall = timed(lux, wl.step, args.steps, args.warmup)
     ms = max(ms_gpu, ms_wall)           # whole-job time: the slower of the device and host clocks
+    ms_graph = timed_graph(lux, wl.step, args.steps) if args.graph else None
     work = wl.work_per_step()
     if wl.bound == "hbm":
         value, unit, peak = work / (ms * 1e-3) / 1e9, "GB/s", PEAK_HBM_GBS
@@ -582,6 +629,9 @@ def main():
         "options": args.option, "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
         "ms_per_step_host_clock": round(ms_wall, 5), "roofline": roofline, "kernels": kernels,
     }
+    if ms_graph is not None:
+        out["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "speedup_over_eager": round(ms / ms_graph, 3),
+                               "note": "one step recorded into a HIP graph, replayed; batchnorm/groupnorm record their two-pass kernels"}
     if hasattr(wl, "step_fused"):
         fg, fw = timed(lux, wl.step_fused, args.steps, args.warmup)
         fms = max(fg, fw)

@@ -623,7 +623,7 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
 #define PICK_RES(A) res_kernel = reinterpret_cast<const void*>(&bn_fwd_resident_kernel<T, A>)
     LUX_DISPATCH_ACT(act, PICK_RES);
 #undef PICK_RES
-    const int64_t SR = batch_stats ? resident_slices(I, C, N, V, vec, resident_per_cu(res_kernel)) : 0;
+    const int64_t SR = batch_stats && !stream_capturing(s) ? resident_slices(I, C, N, V, vec, resident_per_cu(res_kernel)) : 0;
     if (SR > 0) {
         ChanGeom g;
         g.nq = (uint32_t)(I * N / V);
@@ -696,7 +696,7 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
 #define PICK_RES(A) res_kernel = reinterpret_cast<const void*>(&bn_bwd_resident_kernel<T, A>)
     LUX_DISPATCH_ACT(act, PICK_RES);
 #undef PICK_RES
-    const int64_t SR = resident_slices(I, C, N, V, vec, resident_per_cu(res_kernel));
+    const int64_t SR = stream_capturing(s) ? 0 : resident_slices(I, C, N, V, vec, resident_per_cu(res_kernel));
     if (SR > 0) {
         ChanGeom g;
         g.nq = (uint32_t)(I * N / V);

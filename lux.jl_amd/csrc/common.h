@@ -47,6 +47,10 @@ struct Workspace {
 };
 constexpr size_t kWorkspaceZeroBytes = 256;
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out);
+// True while `s` records into a HIP graph.  Kernels whose arguments carry the workspace epoch (the
+// resident batchnorm kernels, the split groupnorm pullback) would find their own tagged words again
+// on every replay of the graph, so the operators take their other code paths while a stream captures.
+bool stream_capturing(hipStream_t s);
 
 // Optional per-kernel timing with HIP events on the launch stream (luxhip_profile_enable).
 struct ProfScope {

@@ -461,7 +461,7 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
                        const T* gamma, const T* beta, const float* save_mean, const float* save_invstd, T* dx,
                        T* dgamma, T* dbeta) {
     constexpr int V = Vec<T>::N;
-    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(delta) && aligned16(dx), true);
+    GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(delta) && aligned16(dx), !stream_capturing(s));
     const bool affine = gamma != nullptr && (dgamma != nullptr || dbeta != nullptr);
     // LDS: 16 floats of reduction scratch + 2 * nw * Cg accumulators
     size_t lds_bytes = 64;

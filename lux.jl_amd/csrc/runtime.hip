@@ -112,6 +112,15 @@ int64_t option_gemm_tile() {
 
 __global__ void fill_zero_kernel(uint32_t* p, size_t nwords);
 
+bool stream_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     std::lock_guard<std::mutex> lk(g_mu);
     WsEntry& e = g_ws[s];
