@@ -95,7 +95,8 @@ int luxhip_profile_enable(int on);
 int luxhip_set_option(const char* name, int64_t value);
 int luxhip_profile_report(char* buf, size_t len);
 
-/* Pooled device allocator (size-bucketed free lists; luxhip_free returns the block to the
+/* Pooled device allocator, in place of the array package's pool that serves the reference's `similar`
+ * calls (e.g. the outputs of src/impl/dense.jl:46-57, src/impl/conv.jl:62-72) (size-bucketed free lists; luxhip_free returns the block to the
  * pool, luxhip_trim releases the pool to the driver).  A freed block can be handed out again at
  * once: work that still uses it must have been enqueued on the stream on which the next owner will
  * enqueue (one stream: always true), or be finished - a caller with several streams synchronises
@@ -371,13 +372,15 @@ int luxhip_permute_leading3(luxhip_stream_t s, int dtype, int64_t d1, int64_t d2
 int luxhip_conv_depth_unfold(luxhip_stream_t s, int dtype, int64_t plane, int64_t D, int64_t C, int64_t N, int64_t KD,
                              int64_t Dout, int64_t stride_d, int64_t pad_d_lo, int64_t dil_d, int flipkernel, const void* x,
                              void* xu);
-/* The adjoint of luxhip_conv_depth_unfold: dx (plane, D, C, N) gathers, in a fixed order, the terms
+/* The adjoint of luxhip_conv_depth_unfold (for NNlib.∇conv_data with three spatial dims, call site
+ * src/impl/conv.jl:128-131): dx (plane, D, C, N) gathers, in a fixed order, the terms
  * of dxu (plane, kD*C, Dout, N) that the unfolding copied from it (∇conv_data of a three-dimensional
  * problem = this applied to the two-dimensional ∇conv_data). */
 int luxhip_conv_depth_fold(luxhip_stream_t s, int dtype, int64_t plane, int64_t D, int64_t C, int64_t N, int64_t KD,
                            int64_t Dout, int64_t stride_d, int64_t pad_d_lo, int64_t dil_d, int flipkernel, const void* dxu,
                            void* dx);
-/* out (inner, B, A, outer) = permutedims(in (inner, A, B, outer), (1, 3, 2, 4)): between the output
+/* No counterpart in the reference (NNlib writes (W, H, D, C, N) outputs directly).
+ * out (inner, B, A, outer) = permutedims(in (inner, A, B, outer), (1, 3, 2, 4)): between the output
  * of the two-dimensional problem, (OW*OH, Cout, Dout, N), and the caller's (OW*OH, Dout, Cout, N). */
 int luxhip_swap_middle_dims(luxhip_stream_t s, int dtype, int64_t inner, int64_t A, int64_t B, int64_t outer, const void* in,
                             void* out);
