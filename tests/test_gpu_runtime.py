@@ -170,3 +170,15 @@ def test_exchange_word_epoch_wraps(gpu):
         _, back_g = gpu.pullback(gpu.groupnorm, dxg, dgam, dbet, 2, "identity", 1e-5)
         for got, want, name in zip(back_g(ddg), want_gn, ("dx", "dgamma", "dbeta")):
             assert_close(got.to_numpy(), want, "f32", f"call {it}: groupnorm {name}", rel=1e-4, scale=1.0)
+
+
+def test_plain_c_client_of_the_abi(gpu):
+    """lux.jl_amd/csrc/examples/c_client.c: a C program (no Python, no C++) that links the library and
+    reproduces the Dense and BatchNorm known answers of the reference's layer tests."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(gpu.__file__), "luxhip_c_client")
+    assert os.path.exists(exe), "build() compiles it next to the library"
+    gpu.synchronize()
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert res.returncode == 0 and res.stdout.strip() == "OK", res.stdout + res.stderr
