@@ -109,6 +109,12 @@ int luxhip_memcpy_d2h(void* dst, const void* src, size_t bytes, luxhip_stream_t 
 int luxhip_memcpy_d2d(void* dst, const void* src, size_t bytes, luxhip_stream_t s); /* asynchronous */
 int luxhip_fill_zero(void* dst, size_t bytes, luxhip_stream_t s);                   /* fill kernel, capturable */
 
+/* out = convert(eltype_out, in) for n elements (bf16: round to nearest even).  The reference promotes
+ * operands of mixed element types to the widest one before its fused dense and convolution kernels
+ * (ext/CUDAExt/cublaslt.jl:46-63, src/impl/conv.jl:11-19); a host layer does the same with this and
+ * takes the gradients back to each operand's own type. */
+int luxhip_convert(luxhip_stream_t s, int dtype_in, int dtype_out, int64_t n, const void* in, void* out);
+
 /* ---------------------------------------------------------------- bias_activation ----
  * x, y, pre, delta, out, dx: (I, C, N) column-major, I = product of the leading dims,
  * C = size(x, ndims-1), N = size(x, ndims).  bias, dbias: length C. */

@@ -91,6 +91,7 @@ SIGNATURES = {
     "luxhip_conv_depth_unfold": [_vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp],
     "luxhip_conv_depth_fold": [_vp, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp],
     "luxhip_swap_middle_dims": [_vp, _i, _i64, _i64, _i64, _i64, _vp, _vp],
+    "luxhip_convert": [_vp, _i, _i, _i64, _vp, _vp],
     "luxhip_permute_leading3": [_vp, _i, _i64, _i64, _i64, _i64, _i, _i, _i, _vp, _vp],
 }
 

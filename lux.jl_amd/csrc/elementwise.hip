@@ -451,6 +451,14 @@ int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t 
                                      (bf16_t*)dx, (bf16_t*)dbias);
 }
 
+
+// Storage conversion fp32 <-> bf16 (round to nearest even), for operands of mixed storage types that
+// are promoted before a fused operator and for taking their gradients back.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void convert_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) st(out + i, ld(in + i));
+}
+
 }  // namespace luxhip
 
 using namespace luxhip;
@@ -487,6 +495,26 @@ int luxhip_bias_activation_bwd(luxhip_stream_t s, int dtype, int act, int64_t I,
                                         (const float*)pre, (float*)dx, (float*)dbias);
     return bias_act_bwd_impl<bf16_t>((hipStream_t)s, act, I, C, N, (const bf16_t*)delta, (const bf16_t*)out,
                                      (const bf16_t*)pre, (bf16_t*)dx, (bf16_t*)dbias);
+}
+
+int luxhip_convert(luxhip_stream_t s, int dtype_in, int dtype_out, int64_t n, const void* in, void* out) {
+    LUX_REQUIRE_INIT();
+    LUX_UNSUPPORTED_IF((dtype_in != LUXHIP_F32 && dtype_in != LUXHIP_BF16) || (dtype_out != LUXHIP_F32 && dtype_out != LUXHIP_BF16),
+                       "convert: unsupported dtype %d -> %d", dtype_in, dtype_out);
+    LUX_INVALID_IF(n < 0, "convert: negative length");
+    if (n == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(in == nullptr || out == nullptr, "convert: in and out must not be NULL");
+    const unsigned blocks = (unsigned)std::min<int64_t>((n + 255) / 256, 65535 * 8);
+    const hipStream_t st_ = (hipStream_t)s;
+    ProfScope ps("convert_kernel", st_);
+    if (dtype_in == dtype_out)
+        return luxhip_memcpy_d2d(out, in, (size_t)n * (dtype_in == LUXHIP_F32 ? 4 : 2), s);
+    if (dtype_in == LUXHIP_BF16)
+        convert_kernel<bf16_t, float><<<blocks, 256, 0, st_>>>((const bf16_t*)in, (float*)out, (size_t)n);
+    else
+        convert_kernel<float, bf16_t><<<blocks, 256, 0, st_>>>((const float*)in, (bf16_t*)out, (size_t)n);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
 }
 
 }  // extern "C"

@@ -57,6 +57,41 @@ def _same_dtype(*arrs):
     return dts.pop()
 
 
+_warned_mixed = [False]
+
+
+def _convert(a: DeviceArray, dtype: str) -> DeviceArray:
+    out = DeviceArray(a.shape, dtype)
+    _lib.call("luxhip_convert", current_stream(), a.code, out.code, a.size, a.ptr, out.ptr)
+    return out
+
+
+def _promote(*arrs):
+    """Operands of mixed storage types are promoted to the widest one, with a warning the first time, as the
+    reference's fused dense and convolution do (ext/CUDAExt/cublaslt.jl:46-63, impl/conv.jl:11-19).  Returns
+    (operands, None) when there is nothing to do, else (promoted operands, the original types)."""
+    dts = {a.dtype for a in arrs if a is not None}
+    if len(dts) <= 1:
+        return arrs, None
+    if not _warned_mixed[0]:
+        _warned_mixed[0] = True
+        import warnings
+        warnings.warn(f"Mixed-precision operands {sorted(dts)}: promoting to f32 (this warning is shown once).")
+    return (tuple(a if a is None or a.dtype == "f32" else _convert(a, "f32") for a in arrs),
+            tuple(None if a is None else a.dtype for a in arrs))
+
+
+def _promoted_rule(rule, orig, *args):
+    """The rule on promoted operands; gradients go back to each operand's own storage type."""
+    y, back = rule(*args)
+
+    def back_cast(delta, *rest):
+        grads = back(delta if delta.dtype == "f32" else _convert(delta, "f32"), *rest)
+        return tuple(g if g is None or dt_ is None or g.dtype == dt_ else _convert(g, dt_) for g, dt_ in zip(grads, orig))
+
+    return y, back_cast
+
+
 def default_epsilon(dtype: str) -> float:
     """eps(T)^(5/7) (utils.jl:130); eps(BFloat16) = 2^-7."""
     eps = 2.0 ** -23 if dtype == "f32" else 2.0 ** -7
@@ -280,6 +315,7 @@ def _check_dense(weight, x, b):
 def fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b: Optional[DeviceArray]) -> DeviceArray:
     """`fused_dense_bias_activation(σ, weight, x, b)` (api/dense.jl:33-37): σ.(weight * x .+ b)."""
     _check_dense(weight, x, b)
+    (weight, x, b), _ = _promote(weight, x, b)
     dt = _same_dtype(weight, x, b)
     M, K = weight.shape
     N = x.shape[1]
@@ -292,6 +328,9 @@ def fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b
 def rrule_fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b: Optional[DeviceArray]):
     """CRC.rrule(fused_dense) (impl/dense.jl:71-134): (y, Δ -> (∂W, ∂x, ∂b))."""
     _check_dense(weight, x, b)
+    (pw, px, pb), orig = _promote(weight, x, b)
+    if orig is not None:
+        return _promoted_rule(lambda *a: rrule_fused_dense_bias_activation(act, *a), orig, pw, px, pb)
     aid = _act_id(act)
     dt = _same_dtype(weight, x, b)
     M, K = weight.shape
@@ -1070,6 +1109,7 @@ def _check_conv(weight, x, b, cdims):
 def fused_conv_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b, cdims: DenseConvDims) -> DeviceArray:
     """`fused_conv_bias_activation(σ, weight, x, b, cdims)` (api/conv.jl:30-38)."""
     _check_conv(weight, x, b, cdims)
+    (weight, x, b), _ = _promote(weight, x, b)
     dt = _same_dtype(weight, x, b)
     if cdims.inner is not None:
         return _from_inner_output(cdims, fused_conv_bias_activation(act, _inner_weight(cdims, weight), _depth_unfold(cdims, x), b,
@@ -1124,6 +1164,9 @@ def _to_inner_output(cdims, dy):
 def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDims):
     """CRC.rrule(fused_conv) + ∇fused_conv (impl/conv.jl:204-275): (y, Δ -> (∂w, ∂x, ∂b))."""
     _check_conv(weight, x, b, cdims)
+    (pw, px, pb), orig = _promote(weight, x, b)
+    if orig is not None:
+        return _promoted_rule(lambda *a: rrule_fused_conv_bias_activation(act, *a, cdims), orig, pw, px, pb)
     aid = _act_id(act)
     dt = _same_dtype(weight, x, b)
     if cdims.inner is not None:

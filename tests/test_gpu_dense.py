@@ -205,3 +205,44 @@ def test_large_bf16_operand_layouts(gpu, transA, transB, pretranspose):
     rows = np.r_[0:130, 2040:2060, M - 130:M]
     assert_close(got[rows], Am[rows] @ Bm + f64(bias[rows])[:, None], "bf16", "rows", scale=np.sqrt(K))
     assert_close(got[:, rows], Am @ Bm[:, rows] + f64(bias)[:, None], "bf16", "cols", scale=np.sqrt(K))
+
+
+def test_mixed_storage_types_are_promoted(gpu):
+    """A bf16 weight with fp32 activations (and the other way round): the operands are promoted to fp32, as
+    the reference promotes mixed element types (ext/CUDAExt/cublaslt.jl:46-63; dense_tests.jl:226-228 runs
+    the mixed combinations); the result is fp32 and each gradient comes back in its operand's own type."""
+    import warnings
+    rng = np.random.default_rng(41)
+    w = O.round_to_bf16(rng.normal(size=(24, 16)).astype(np.float32) / 4)
+    x = rng.normal(size=(16, 10)).astype(np.float32)
+    b = O.round_to_bf16(rng.normal(size=24).astype(np.float32))
+    delta = rng.normal(size=(24, 10)).astype(np.float32)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        y, back = gpu.pullback(gpu.fused_dense_bias_activation, "tanh", dev(gpu, w, "bf16"), dev(gpu, x, "f32"), dev(gpu, b, "bf16"))
+        y2 = gpu.fused_dense_bias_activation("tanh", dev(gpu, w, "bf16"), dev(gpu, x, "f32"), dev(gpu, b, "bf16"))
+    wy, wdw, wdx, wdb = O.fused_dense_pullback("tanh", f64(w), f64(x), f64(b), f64(delta))
+    assert y.dtype == "f32" and y2.dtype == "f32"
+    assert_close(y.to_numpy(), wy, "f32", "y")
+    np.testing.assert_array_equal(y2.to_numpy(), y.to_numpy())
+    dw, dx, db = back(dev(gpu, delta, "f32"))
+    assert (dw.dtype, dx.dtype, db.dtype) == ("bf16", "f32", "bf16")
+    assert_close(dw.to_numpy(), wdw, "bf16", "dw")
+    assert_close(dx.to_numpy(), wdx, "f32", "dx")
+    assert_close(db.to_numpy(), wdb, "bf16", "db")
+    # convolution: fp32 weight, bf16 input
+    cw = rng.normal(size=(3, 3, 4, 6)).astype(np.float32) / 6
+    cx = O.round_to_bf16(rng.normal(size=(8, 7, 4, 2)).astype(np.float32))
+    cd = gpu.DenseConvDims(cx.shape, cw.shape, padding=1)
+    od = O.ConvDims(cx.shape, cw.shape, 1, 1, 1)
+    cdelta = rng.normal(size=cd.y_shape).astype(np.float32)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        cy, cback = gpu.pullback(gpu.fused_conv_bias_activation, "relu", dev(gpu, cw, "f32"), dev(gpu, cx, "bf16"), None, cd)
+    wy, wdw, wdx, _ = O.fused_conv_pullback("relu", f64(cw), f64(cx), None, od, f64(cdelta))
+    assert cy.dtype == "f32"
+    assert_close(cy.to_numpy(), wy, "f32", "conv y")
+    gw, gx, gb = cback(dev(gpu, cdelta, "f32"))
+    assert (gw.dtype, gx.dtype, gb) == ("f32", "bf16", None)
+    assert_close(gw.to_numpy(), wdw, "f32", "conv dw", scale=1.0)
+    assert_close(gx.to_numpy(), wdx, "bf16", "conv dx", scale=1.0)
