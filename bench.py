@@ -99,18 +99,28 @@ class C2BatchnormBiasAct(Workload):
         self.I, self.C, self.N = W * H, Cc, N
         h = self.host_inputs()
         d = lux.DeviceArray.from_numpy
-        self.t = {k: d(v) for k, v in h.items()}
-        for k in ("y1", "y2", "dy1", "dx"):
-            self.t[k] = lux.DeviceArray(self.shape, "f32")
-        for k in ("rmean_out", "rvar_out", "dgamma", "dbeta", "dbias2"):
-            self.t[k] = lux.DeviceArray((Cc,), "f32")
         self.sm, self.si = lux.StatArray(Cc), lux.StatArray(Cc)
-        t, s = self.t, lux.current_stream()
+        # --rotate N: N sets of the six large tensors, used in turn, so that no step finds a tensor of the step
+        # before it in a cache (the working set becomes N x 201 MB)
+        self.sets = []
+        for _ in range(max(int(getattr(self, "rotate", 1)), 1)):
+            t = {k: d(v) for k, v in h.items()}
+            for k in ("y1", "y2", "dy1", "dx"):
+                t[k] = lux.DeviceArray(self.shape, "f32")
+            for k in ("rmean_out", "rvar_out", "dgamma", "dbeta", "dbias2"):
+                t[k] = lux.DeviceArray((Cc,), "f32")
+            self.sets.append((t,) + self._calls(lib, lux, t))
+        self.t, self.calls, self.fused_calls = self.sets[0]
+        self.turn = 0
+
+    def _calls(self, lib, lux, t):
+        s = lux.current_stream()
+        Cc = self.C
         vp = C.c_void_p
         p = lambda k: vp(t[k].ptr)
         I, Cc_, N_ = C.c_int64(self.I), C.c_int64(self.C), C.c_int64(self.N)
         f32, ident, relu = 0, 0, 1
-        self.calls = [
+        calls = [
             (lib.luxhip_batchnorm_fwd, (s, f32, ident, I, Cc_, N_, p("x"), p("gamma"), p("beta"), p("rmean"), p("rvar"), 1,
                                         C.c_double(0.1), C.c_double(1e-5), p("y1"), p("rmean_out"), p("rvar_out"),
                                         vp(self.sm.ptr), vp(self.si.ptr))),
@@ -120,15 +130,19 @@ class C2BatchnormBiasAct(Workload):
                                         vp(self.si.ptr), 1, p("dx"), p("dgamma"), p("dbeta"))),
         ]
         # fused variant: batchnorm(..., relu) forward + pullback
-        self.fused_calls = [
+        fused_calls = [
             (lib.luxhip_batchnorm_fwd, (s, f32, relu, I, Cc_, N_, p("x"), p("gamma"), p("beta"), p("rmean"), p("rvar"), 1,
                                         C.c_double(0.1), C.c_double(1e-5), p("y2"), p("rmean_out"), p("rvar_out"),
                                         vp(self.sm.ptr), vp(self.si.ptr))),
             (lib.luxhip_batchnorm_bwd, (s, f32, relu, I, Cc_, N_, p("delta"), p("x"), p("gamma"), p("beta"), vp(self.sm.ptr),
                                         vp(self.si.ptr), 1, p("dx"), p("dgamma"), p("dbeta"))),
         ]
+        return calls, fused_calls
 
     def step(self):
+        if len(self.sets) > 1:
+            self.turn = (self.turn + 1) % len(self.sets)
+            self.calls = self.sets[self.turn][1]
         for fn, args in self.calls:
             rc = fn(*args)
             if rc != 0:
@@ -542,6 +556,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB: a kernel of known traffic that "
                          "scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--rotate", type=int, default=1,
+                    help="C2 only: number of separate sets of the large tensors that the steps use in turn "
+                         "(1 = every step on the same buffers)")
     ap.add_argument("--graph", action="store_true",
                     help="also record one step into a HIP graph and time its replays (reported as graph_replay; "
                          "value stays the eager figure)")
@@ -562,6 +579,7 @@ def main():
         args.steps = 20 if heavy else 200
     if args.warmup is None:
         args.warmup = 3 if heavy else 20
+    wl.rotate = args.rotate
     wl.setup(lux)
 
     ms_gpu, ms_wall = timed(lux, wl.step, args.steps, args.warmup)
@@ -626,12 +644,24 @@ def main():
         "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype,
         "data": "synthetic", "config": {"workload": f"{wl.name}: {wl.description}"},
-        "options": args.option, "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
+        "options": args.option + ([f"rotate={args.rotate}"] if args.rotate > 1 else []), "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
         "ms_per_step_host_clock": round(ms_wall, 5), "roofline": roofline, "kernels": kernels,
     }
     if ms_graph is not None:
         out["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "speedup_over_eager": round(ms / ms_graph, 3),
                                "note": "one step recorded into a HIP graph, replayed; batchnorm/groupnorm record their two-pass kernels"}
+    if args.workload == "C2" and args.rotate == 1 and not args.option:
+        # the same chain on 8 sets of tensors used in turn: no step finds its inputs (x, delta) in the 256 MB
+        # Infinity Cache from the step before, as it does when every step runs on the same buffers
+        cold = WORKLOADS["C2"]()
+        cold.rotate = 8
+        cold.setup(lux)
+        cg, cw_ = timed(lux, cold.step, args.steps, args.warmup)
+        cms = max(cg, cw_)
+        out["cold_inputs"] = {"sets_of_tensors": 8, "ms_per_step": round(cms, 5),
+                              "value": round(work / (cms * 1e-3) / 1e9, 2), "unit": "GB/s",
+                              "frac_of_peak": round(work / (cms * 1e-3) / 1e9 / peak, 4)}
+        del cold
     if hasattr(wl, "step_fused"):
         fg, fw = timed(lux, wl.step_fused, args.steps, args.warmup)
         fms = max(fg, fw)
