@@ -30,10 +30,10 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
 # size (profiles/*_hbm_traffic_pmc.md hold the commands and the raw counter values).
 MEASURED_TRAFFIC = {
-    ("C2", "bn_fwd_resident_kernel"): 67764601,
-    ("C2", "bias_act_fwd_kernel"): 67138039,
-    ("C2", "bias_act_bwd_channel_kernel"): 100918103,
-    ("C2", "bn_bwd_resident_kernel"): 100979652,
+    ("C2", "bn_fwd_resident_kernel"): 67758714,
+    ("C2", "bias_act_fwd_kernel"): 67137042,
+    ("C2", "bias_act_bwd_channel_kernel"): 100892887,
+    ("C2", "bn_bwd_resident_kernel"): 100993602,
     ("C3", "gn_fwd_kernel"): 134324931,
     ("C3", "gn_bwd_kernel"): 202195147,
     ("C3bf16", "gn_fwd_kernel"): 67290712,
@@ -559,6 +559,9 @@ def main():
     ap.add_argument("--rotate", type=int, default=1,
                     help="C2 only: number of separate sets of the large tensors that the steps use in turn "
                          "(1 = every step on the same buffers)")
+    ap.add_argument("--cold-sets", type=int, default=8,
+                    help="C2 only: also time the chain on this many sets of tensors used in turn (reported as cold_inputs; "
+                         "0 = skip, e.g. under a profiler, where its launches would enter the per-kernel averages)")
     ap.add_argument("--graph", action="store_true",
                     help="also record one step into a HIP graph and time its replays (reported as graph_replay; "
                          "value stays the eager figure)")
@@ -650,15 +653,15 @@ def main():
     if ms_graph is not None:
         out["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "speedup_over_eager": round(ms / ms_graph, 3),
                                "note": "one step recorded into a HIP graph, replayed; batchnorm/groupnorm record their two-pass kernels"}
-    if args.workload == "C2" and args.rotate == 1 and not args.option:
+    if args.workload == "C2" and args.rotate == 1 and not args.option and args.cold_sets > 1:
         # the same chain on 8 sets of tensors used in turn: no step finds its inputs (x, delta) in the 256 MB
         # Infinity Cache from the step before, as it does when every step runs on the same buffers
         cold = WORKLOADS["C2"]()
-        cold.rotate = 8
+        cold.rotate = args.cold_sets
         cold.setup(lux)
         cg, cw_ = timed(lux, cold.step, args.steps, args.warmup)
         cms = max(cg, cw_)
-        out["cold_inputs"] = {"sets_of_tensors": 8, "ms_per_step": round(cms, 5),
+        out["cold_inputs"] = {"sets_of_tensors": args.cold_sets, "ms_per_step": round(cms, 5),
                               "value": round(work / (cms * 1e-3) / 1e9, 2), "unit": "GB/s",
                               "frac_of_peak": round(work / (cms * 1e-3) / 1e9 / peak, 4)}
         del cold
