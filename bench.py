@@ -148,6 +148,9 @@ class C2BatchnormBiasAct(Workload):
             if rc != 0:
                 raise RuntimeError(self.lux._lib.last_error())
 
+    def rotating_step(self):
+        self.step()
+
     def isolated_ops(self):
         """kernel name -> call that launches exactly that kernel (default library options)."""
         names = ["bn_fwd_resident_kernel", "bias_act_fwd_kernel", "bias_act_bwd_channel_kernel", "bn_bwd_resident_kernel"]
@@ -223,8 +226,18 @@ class _ApiWorkload(Workload):
 
     def setup(self, lux):
         self.lux = lux
-        self.build(lux)
+        # rotate > 1: that many sets of input tensors, used in turn by rotating_step()
+        self._sets = []
+        for _ in range(max(int(getattr(self, "rotate", 1)), 1)):
+            self.build(lux)
+            self._sets.append({k: v for k, v in vars(self).items() if isinstance(v, lux.DeviceArray)})
+        self._turn = 0
         self.step()               # allocate pool blocks and workspaces once
+
+    def rotating_step(self):
+        self._turn = (self._turn + 1) % len(self._sets)
+        self.__dict__.update(self._sets[self._turn])
+        self.step()
 
     def d(self, a, dtype=None):
         return self.lux.DeviceArray.from_numpy(a, dtype or self.storage)
@@ -557,10 +570,10 @@ def main():
                     help="also run three device-to-device copies of 256 MiB: a kernel of known traffic that "
                          "scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     ap.add_argument("--rotate", type=int, default=1,
-                    help="C2 only: number of separate sets of the large tensors that the steps use in turn "
+                    help="number of separate sets of the large tensors that the timed steps use in turn "
                          "(1 = every step on the same buffers)")
     ap.add_argument("--cold-sets", type=int, default=8,
-                    help="C2 only: also time the chain on this many sets of tensors used in turn (reported as cold_inputs; "
+                    help="HBM-bound workloads: also time the steps on this many sets of tensors used in turn (reported as cold_inputs; "
                          "0 = skip, e.g. under a profiler, where its launches would enter the per-kernel averages)")
     ap.add_argument("--graph", action="store_true",
                     help="also record one step into a HIP graph and time its replays (reported as graph_replay; "
@@ -585,7 +598,7 @@ def main():
     wl.rotate = args.rotate
     wl.setup(lux)
 
-    ms_gpu, ms_wall = timed(lux, wl.step, args.steps, args.warmup)
+    ms_gpu, ms_wall = timed(lux, wl.rotating_step if args.rotate > 1 and hasattr(wl, "rotating_step") else wl.step, args.steps, args.warmup)
     ms = max(ms_gpu, ms_wall)           # whole-job time: the slower of the device and host clocks
     ms_graph = timed_graph(lux, wl.step, args.steps) if args.graph else None
     work = wl.work_per_step()
@@ -653,13 +666,13 @@ def main():
     if ms_graph is not None:
         out["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "speedup_over_eager": round(ms / ms_graph, 3),
                                "note": "one step recorded into a HIP graph, replayed; batchnorm/groupnorm record their two-pass kernels"}
-    if args.workload == "C2" and args.rotate == 1 and not args.option and args.cold_sets > 1:
-        # the same chain on 8 sets of tensors used in turn: no step finds its inputs (x, delta) in the 256 MB
+    if wl.bound == "hbm" and args.rotate == 1 and not args.option and args.cold_sets > 1:
+        # the same steps on several sets of input tensors used in turn: no step finds its inputs in the 256 MB
         # Infinity Cache from the step before, as it does when every step runs on the same buffers
-        cold = WORKLOADS["C2"]()
+        cold = WORKLOADS[args.workload]()
         cold.rotate = args.cold_sets
         cold.setup(lux)
-        cg, cw_ = timed(lux, cold.step, args.steps, args.warmup)
+        cg, cw_ = timed(lux, cold.rotating_step, args.steps, args.warmup)
         cms = max(cg, cw_)
         out["cold_inputs"] = {"sets_of_tensors": args.cold_sets, "ms_per_step": round(cms, 5),
                               "value": round(work / (cms * 1e-3) / 1e9, 2), "unit": "GB/s",
