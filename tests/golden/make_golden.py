@@ -100,6 +100,39 @@ def main():
     dy_, dmask = O.dropout(dnoise.astype(np.float32), dxin.astype(np.float32), 0.25, True, 1.0 / 0.75)
     g.update(drop_noise=dnoise, drop_x=dxin, drop_mask=dmask, drop_y=dy_)
 
+    # --- the attention known answer of the reference (attention_tests.jl:115-170): q = k = v = reshape(1:12, 2, 2, 3, 1) ./ 12
+    g["kat_attn_q"] = (np.arange(1, 13, dtype=np.float64) / 12).reshape((2, 2, 3, 1), order="F")
+    g["kat_attn_y"] = np.reshape([0.429754, 0.513087, 0.613791, 0.697125, 0.46431, 0.547644, 0.647876, 0.73121, 0.49773,
+                                  0.581064, 0.680455, 0.763788], (2, 2, 3, 1), order="F")
+    g["kat_attn_w"] = np.reshape([0.313896, 0.332948, 0.353157, 0.264431, 0.328206, 0.407362, 0.219215, 0.31838, 0.462405,
+                                  0.288691, 0.331243, 0.380066, 0.241239, 0.323893, 0.434868, 0.198438, 0.311761, 0.489801],
+                                 (3, 3, 2, 1), order="F")
+
+    # --- convolution with three spatial dims: kernel (2, 3, 2), stride (1, 2, 1), pad (1, 0, 0, 1, 1, 1), groups 2, gelu
+    x, w, b = fixed((5, 6, 4, 4, 2), 0.5, 2.0), fixed((2, 3, 2, 2, 6), 0.5), fixed((6,), 0.5)
+    cd3 = O.ConvDimsND(x.shape, w.shape, (1, 2, 1), (1, 0, 0, 1, 1, 1), 1, 2)
+    delta = fixed(cd3.out_spatial + (6, 2), 0.4)
+    y, dw, dx, db = O.fused_conv_nd_pullback("gelu", w, x, b, cd3, delta)
+    g.update(conv3_x=x, conv3_w=w, conv3_b=b, conv3_delta=delta, conv3_y=y, conv3_dw=dw, conv3_dx=dx, conv3_db=db)
+
+    # --- layernorm as the reference's own test calls it (layernorm_tests.jl:22-32,80-86): dims = Colon() with
+    #     parameters (1, 1, C, 1), on its input generator
+    x = O.generate_fixed_array(np.float64, (3, 3, 2, 1))
+    gam, bet = O.generate_fixed_array(np.float64, (1, 1, 2, 1)), O.generate_fixed_array(np.float64, (1, 1, 2, 1))
+    delta = fixed((3, 3, 2, 1), 0.45)
+    eps = O.default_epsilon(np.float32)
+    y = O.layernorm(x, gam, bet, "sigmoid_fast", (0, 1, 2, 3), eps)
+    dx, dg, dbt = O.layernorm_pullback(x, gam, bet, "sigmoid_fast", (0, 1, 2, 3), eps, delta)
+    g.update(lnc_x=x, lnc_gamma=gam, lnc_beta=bet, lnc_delta=delta, lnc_eps=np.array(eps), lnc_y=y, lnc_dx=dx, lnc_dgamma=dg,
+             lnc_dbeta=dbt)
+
+    # --- batched_matmul with batching dims in the middle (generalized_bmm_tests.jl:36-58)
+    x, y_ = fixed((3, 5, 2, 4), 0.5), fixed((4, 5, 1, 5), 0.4)
+    z = O.batched_matmul_general(x, y_, 4, 1, (2, 3), (4, 3))
+    delta = fixed(z.shape, 0.3)
+    dx, dy = O.batched_matmul_general_pullback(x, y_, delta, 4, 1, (2, 3), (4, 3))
+    g.update(gbmm_x=x, gbmm_y=y_, gbmm_z=z, gbmm_delta=delta, gbmm_dx=dx, gbmm_dy=dy)
+
     np.savez_compressed(OUT, **{k: np.asarray(v, dtype=np.float64) for k, v in g.items()})
     print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(g), "arrays")
 

@@ -35,6 +35,18 @@ def test_oracle_reproduces_golden_vectors():
     np.testing.assert_allclose(out, G["attn_out"], rtol=1e-12, atol=1e-13)
     np.testing.assert_allclose(w, G["attn_weights"], rtol=1e-12, atol=1e-14)
     np.testing.assert_array_equal(O.rand_uniform(24, 7, 2).reshape((4, 3, 2), order="F"), G["drop_noise"].astype(np.float32))
+    y, w = O.scaled_dot_product_attention(G["kat_attn_q"], G["kat_attn_q"], G["kat_attn_q"])
+    np.testing.assert_allclose(y, G["kat_attn_y"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(w, G["kat_attn_w"], rtol=1e-5, atol=1e-5)
+    cd3 = O.ConvDimsND(G["conv3_x"].shape, G["conv3_w"].shape, (1, 2, 1), (1, 0, 0, 1, 1, 1), 1, 2)
+    for got, k in zip(O.fused_conv_nd_pullback("gelu", G["conv3_w"], G["conv3_x"], G["conv3_b"], cd3, G["conv3_delta"]),
+                      ("conv3_y", "conv3_dw", "conv3_dx", "conv3_db")):
+        np.testing.assert_allclose(got, G[k], rtol=1e-12, atol=1e-13)
+    eps = float(G["lnc_eps"])
+    np.testing.assert_allclose(O.layernorm(G["lnc_x"], G["lnc_gamma"], G["lnc_beta"], "sigmoid_fast", (0, 1, 2, 3), eps), G["lnc_y"],
+                               rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(O.batched_matmul_general(G["gbmm_x"], G["gbmm_y"], 4, 1, (2, 3), (4, 3)), G["gbmm_z"], rtol=1e-13,
+                               atol=1e-14)
 
 
 @pytest.mark.gpu
@@ -89,3 +101,18 @@ def test_hip_path_matches_golden_vectors(gpu):
     y, mask, _ = gpu.dropout(rng, d("drop_x"), 0.25, True, 1.0 / 0.75)
     np.testing.assert_array_equal(mask.to_numpy(), G["drop_mask"].astype(np.float32))
     np.testing.assert_array_equal(y.to_numpy(), G["drop_y"].astype(np.float32))
+    # the reference's attention known answer, three spatial dims, layernorm over every dim, batching dims in the middle
+    q = d("kat_attn_q")
+    y, w = gpu.scaled_dot_product_attention(q, q, q)
+    np.testing.assert_allclose(y.to_numpy(), G["kat_attn_y"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(w.to_numpy(), G["kat_attn_w"], rtol=1e-5, atol=1e-5)
+    cd3 = gpu.DenseConvDims(G["conv3_x"].shape, G["conv3_w"].shape, stride=(1, 2, 1), padding=(1, 0, 0, 1, 1, 1), groups=2)
+    y, back = gpu.pullback(gpu.fused_conv_bias_activation, "gelu", d("conv3_w"), d("conv3_x"), d("conv3_b"), cd3)
+    dw, dx, db = back(d("conv3_delta"))
+    chk(y, "conv3_y"); chk(dw, "conv3_dw", scale=1.0); chk(dx, "conv3_dx", scale=1.0); chk(db, "conv3_db", scale=1.0)
+    y, back = gpu.pullback(gpu.layernorm, d("lnc_x"), d("lnc_gamma"), d("lnc_beta"), "sigmoid_fast", gpu.COLON, float(G["lnc_eps"]))
+    dx, dg, dbt = back(d("lnc_delta"))
+    chk(y, "lnc_y"); chk(dx, "lnc_dx", scale=0.5); chk(dg, "lnc_dgamma", scale=0.5); chk(dbt, "lnc_dbeta", scale=0.5)
+    z, back = gpu.pullback(gpu.batched_matmul, d("gbmm_x"), d("gbmm_y"), 4, 1, (2, 3), (4, 3))
+    dx, dy = back(d("gbmm_delta"))
+    chk(z, "gbmm_z", scale=1.0); chk(dx, "gbmm_dx", scale=1.0); chk(dy, "gbmm_dy", scale=1.0)
