@@ -5,6 +5,8 @@ import ctypes
 import os
 import re
 
+import numpy as np
+
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -116,3 +118,56 @@ def test_fastdiv_matches_integer_division():
         for n in ns:
             if 0 <= n < (1 << 31):
                 assert fastdiv(n, d) == n // d, (n, d)
+
+
+class _Fake:
+    """An array stand-in for the host-side planning code (shapes only, nothing is launched)."""
+
+    def __init__(self, shape, dtype="f32"):
+        self.shape, self.dtype, self.ndim, self.ptr = tuple(shape), dtype, len(shape), 0
+        self.size = int(np.prod(shape)) if len(shape) else 1
+
+
+def test_layernorm_planning(lux):
+    """Which dims are normalised and how the parameters are applied (impl/layernorm.jl:21-46)."""
+    from lux_jl_amd import luxlib as L
+    x = _Fake((3, 3, 2, 5))
+    assert L._layernorm_geometry(x, None, None, L.DEFAULT_DIMS) == (18, 5, None)
+    assert L._layernorm_geometry(x, None, None, L.COLON) == (90, 1, None)
+    assert L._layernorm_geometry(x, _Fake((3, 3, 2, 1)), _Fake((3, 3, 2, 1)), (1, 2, 3)) == (18, 5, None)        # one fused kernel
+    # the reference's test configurations: Colon() with (1, 1, C, 1), nothing with (1, 1, C) -> dims 1:1
+    assert L._layernorm_geometry(x, _Fake((1, 1, 2, 1)), _Fake((1, 1, 2, 1)), L.COLON) == (90, 1, (9, 2, 5))
+    assert L._layernorm_geometry(x, _Fake((1, 1, 2)), _Fake((1, 1, 2)), None) == (3, 30, (9, 2, 5))
+    assert L._layernorm_geometry(x, _Fake((3, 1, 2, 1)), _Fake((3, 1, 2, 1)), L.COLON) == (90, 1, (1, 18, 5))    # a gap: repeated first
+    with pytest.raises(lux.Unsupported):
+        L._layernorm_geometry(x, None, None, (2, 3))
+    with pytest.raises(lux.DimensionMismatch):
+        L._layernorm_geometry(x, _Fake((2, 1, 1, 1)), _Fake((2, 1, 1, 1)), L.COLON)
+    with pytest.raises(AssertionError):
+        L._layernorm_geometry(_Fake((2, 3)), _Fake((2, 1)), _Fake((2, 1)), None)
+
+
+def test_batched_matmul_planning(lux):
+    """Where the matrices and the batching dims of batched_matmul's operands lie (impl/batched_mul.jl:2-58)."""
+    from lux_jl_amd import luxlib as L
+    op = L._BmmOperand(_Fake((3, 5, 2, 4)), 4, (2, 3), "x")           # generalized_bmm_tests.jl:36-58, left operand
+    assert (op.F, op.K, op.free_major, op.ld, op.bext, op.bst) == (3, 4, True, 30, [5, 2], [3, 15])
+    op = L._BmmOperand(_Fake((4, 5, 1, 5)), 1, (4, 3), "y")           # its right operand
+    assert (op.F, op.K, op.free_major, op.ld, op.bext, op.bst) == (5, 4, False, 4, [5, 1], [20, 20])
+    op = L._BmmOperand(_Fake((5, 4, 5, 1)), 2, None, "y")             # :8-22: contracted along dim 2, trailing batch dims
+    assert (op.F, op.K, op.free_major, op.ld) == (5, 4, True, 5)
+    with pytest.raises(lux.Unsupported):
+        L._BmmOperand(_Fake((2, 3, 6, 7, 5)), 3, (1, 2, 5), "y")     # neither matrix dim contiguous
+    with pytest.raises(lux.ArgumentError):
+        L._BmmOperand(_Fake((2, 3, 4)), 2, (2,), "x")                 # the contracting dim among the batching dims
+
+
+def test_conv_dims_with_three_spatial_dims(lux):
+    cd = lux.DenseConvDims((7, 6, 8, 4, 2), (2, 3, 3, 2, 6), stride=(1, 2, 2), padding=(1, 0, 2, 1, 1, 2), dilation=(2, 1, 2), groups=2)
+    assert cd.out_spatial == (6, 4, 4) and cd.y_shape == (6, 4, 4, 6, 2)
+    inner = cd.inner                                                   # the two-dimensional problem on the unfolded input
+    assert inner.x_shape == (7, 6, 3 * 4, 4 * 2) and inner.w_shape == (2, 3, 3 * 2, 6)
+    assert inner.stride == (1, 2) and inner.padding == (1, 0, 2, 1) and inner.dilation == (2, 1) and inner.groups == 2
+    assert inner.y_shape == (6, 4, 6, 4 * 2)
+    with pytest.raises(lux.Unsupported):
+        lux.DenseConvDims((4, 4, 4, 4, 2, 1), (2, 2, 2, 2, 2, 3))
