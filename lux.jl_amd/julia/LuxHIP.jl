@@ -468,5 +468,18 @@ end
 # calls around luxhip_attention_softmax_fwd, its rrule four products around
 # luxhip_attention_softmax_bwd.  (lux.jl_amd/luxlib.py: rrule_instancenorm,
 # rrule_scaled_dot_product_attention spell out the strides.)
+#
+# The same file holds the host side of what the hooks above do not cover one to one:
+#   * layernorm over 1:k with parameters that do not span exactly those dims (dims = Colon() with
+#     (1, 1, C, 1) parameters, dims = nothing): luxhip_layernorm_fwd without γ, β, then the per-channel
+#     affine transform and activation as luxhip_batchnorm_fwd in inference mode (mean 0, variance 1,
+#     ε = 0) on the (I, C, N) view; the pullback runs the two in reverse (_layernorm_fwd);
+#   * attention operands whose embedding dim is not the first: luxhip_permute_leading3 before, and on
+#     ∂q, ∂k, ∂v after; `fdrop` between the softmax and the second product (attention_dropout);
+#   * batched_matmul with lhs_batching_dims / rhs_batching_dims anywhere and partly repeated operands:
+#     the arrays' own strides go to luxhip_batched_matmul_strided, no permutedims / repeat
+#     (_rrule_batched_matmul_general);
+#   * operands of mixed element types in fused_dense / fused_conv: luxhip_convert to the widest type
+#     first (the reference's own rule, ext/CUDAExt/cublaslt.jl:46-63), gradients converted back (_promote).
 
 end # module
