@@ -34,12 +34,12 @@ MEASURED_TRAFFIC = {
     ("C2", "bias_act_fwd_kernel"): 67137042,
     ("C2", "bias_act_bwd_channel_kernel"): 100892887,
     ("C2", "bn_bwd_resident_kernel"): 100993602,
-    ("C3", "gn_fwd_kernel"): 134324931,
-    ("C3", "gn_bwd_kernel"): 202195147,
+    ("C3", "gn_fwd_kernel"): 134327510,
+    ("C3", "gn_bwd_kernel"): 202204269,
     ("C3bf16", "gn_fwd_kernel"): 67290712,
     ("C3bf16", "gn_bwd_kernel"): 101301450,
-    ("IN", "gn_fwd_kernel"): 134569817,
-    ("IN", "gn_bwd_kernel"): 202845995,
+    ("IN", "gn_fwd_kernel"): 135315416,
+    ("IN", "gn_bwd_kernel"): 202833217,
     ("DROPOUT", "dropout_fwd_kernel"): 100695712,      # dropout_rng_kernel<float, 4, 2> in the trace
     ("DROPOUT", "dropout_mul_kernel"): 100691762,
 }

@@ -182,6 +182,13 @@ int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64
                          const float* save_mean, const float* save_invstd, void* dx, void* dgamma,
                          void* dbeta);
 
+/* instancenorm in training mode with running statistics in one launch: luxhip_groupnorm_fwd with G = C whose
+ * workgroups also make the update that luxhip_instancenorm_running_stats describes (the workgroup of a
+ * channel that finishes last averages the channel's N slice statistics, in sample order).  save_mean,
+ * save_invstd: (C, N) fp32, required. */
+int luxhip_instancenorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* x,
+                            const void* gamma, const void* beta, double eps, void* y, float* save_mean, float* save_invstd,
+                            double momentum, const void* rmean, const void* rvar, void* rmean_out, void* rvar_out);
 /* instancenorm = the groupnorm kernels with G = C (statistics per channel and sample,
  * src/impl/normalization.jl:191-208) plus, in training with running statistics, this update
  * (update_normalization_statistics, src/impl/normalization.jl:91-110, reduce dims 1..N-2):

@@ -67,6 +67,7 @@ SIGNATURES = {
     "luxhip_batchnorm_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _i, _vp, _vp, _vp],
     "luxhip_groupnorm_fwd": [_vp, _i, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _d, _vp, _fp, _fp],
     "luxhip_groupnorm_bwd": [_vp, _i, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _vp, _vp, _vp],
+    "luxhip_instancenorm_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _d, _vp, _fp, _fp, _d, _vp, _vp, _vp, _vp],
     "luxhip_instancenorm_running_stats": [_vp, _i, _i64, _i64, _i64, _fp, _fp, _d, _d, _vp, _vp, _vp, _vp],
     "luxhip_attention_softmax_fwd": [_vp, _i, _i64, _i64, _i64, _i64, _vp, _d, _i, _vp, _i64, _i64, _vp, _i64, _i64, _vp],
     "luxhip_attention_softmax_bwd": [_vp, _i, _i64, _i64, _i64, _i, _vp, _vp, _d, _vp],

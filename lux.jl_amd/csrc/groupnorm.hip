@@ -47,10 +47,25 @@ struct GnExchange {
     uint32_t epoch, spin_limit;
 };
 
+// instancenorm's running statistics, updated by the forward kernel itself (G == C: slice = n*C + c): the
+// workgroup of a channel that arrives last averages the channel's N slice statistics, in sample order.
+// out_mean == nullptr: no update.
+template <typename T>
+struct InRunning {
+    const T* rmean;
+    const T* rvar;
+    T* out_mean;
+    T* out_var;
+    uint32_t* counters;
+    uint32_t cstride, N;
+    float momentum, corrected;     // corrected = momentum * I / (I - 1)
+};
+
 template <typename T, int ACT, int VEC, bool CACHED>
 __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta, T* y,
-                              float* save_mean, float* save_invstd, GnGeom g, float eps) {
+                              float* save_mean, float* save_invstd, GnGeom g, float eps, InRunning<T> rs) {
     __shared__ float sm[16];
+    __shared__ uint32_t last_flag;
     const uint32_t slice = blockIdx.x;              // = n*G + k
     const uint32_t k = slice % g.G;
     const size_t base = (size_t)slice * g.nvec * VEC;
@@ -102,7 +117,27 @@ __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
     }
     const float var = block_sum(dev, sm) * g.inv_m;
     const float invstd = 1.0f / sqrtf(var + eps);
-    if (threadIdx.x == 0) {
+    if (rs.out_mean != nullptr) {                     // uniform over the grid
+        if (threadIdx.x == 0) {
+            publish(reinterpret_cast<uint32_t*>(save_mean + slice), __float_as_uint(mean));
+            publish(reinterpret_cast<uint32_t*>(save_invstd + slice), __float_as_uint(invstd));
+            publish_done();
+        }
+        if (arrive_last(rs.counters + (size_t)k * rs.cstride, rs.N, &last_flag)) {
+            float tm = 0.0f, tv = 0.0f;
+            for (uint32_t n = threadIdx.x; n < rs.N; n += T_) {
+                const float is = __uint_as_float(fetch(reinterpret_cast<const uint32_t*>(save_invstd + k + (size_t)g.G * n)));
+                tm += __uint_as_float(fetch(reinterpret_cast<const uint32_t*>(save_mean + k + (size_t)g.G * n)));
+                tv += 1.0f / (is * is) - eps;
+            }
+            tm = block_sum(tm, sm);
+            tv = block_sum(tv, sm);
+            if (threadIdx.x == 0) {
+                st<T>(rs.out_mean + k, (1.0f - rs.momentum) * ld<T>(rs.rmean + k) + rs.momentum * (tm / (float)rs.N));
+                st<T>(rs.out_var + k, (1.0f - rs.momentum) * ld<T>(rs.rvar + k) + rs.corrected * (tv / (float)rs.N));
+            }
+        }
+    } else if (threadIdx.x == 0) {
         if (save_mean) save_mean[slice] = mean;
         if (save_invstd) save_invstd[slice] = invstd;
     }
@@ -439,16 +474,25 @@ static int gn_exchange(hipStream_t s, GnExchange* ex) {
 
 template <typename T>
 static int gn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, int64_t N, const T* x, const T* gamma,
-                       const T* beta, float eps, T* y, float* save_mean, float* save_invstd) {
+                       const T* beta, float eps, T* y, float* save_mean, float* save_invstd, InRunning<T> rs = InRunning<T>{}) {
     constexpr int V = Vec<T>::N;
     GnLaunch L = gn_plan<T>(I, C, G, N, aligned16(x) && aligned16(y), false);
+    if (rs.out_mean != nullptr) {
+        LUX_UNSUPPORTED_IF((size_t)C > kWorkspaceCounters, "instancenorm: more than %zu channels", kWorkspaceCounters);
+        Workspace ws;
+        int rc = get_workspace(s, 0, &ws);
+        if (rc != LUXHIP_OK) return rc;
+        rs.counters = ws.counters;
+        rs.cstride = counter_stride(C);
+        rs.N = (uint32_t)N;
+    }
     ProfScope ps("gn_fwd_kernel", s);
 #define GN_FWD(A)                                                                                                     \
     do {                                                                                                              \
-        if (L.vec && L.cached) gn_fwd_kernel<T, A, V, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);   \
-        else if (L.vec) gn_fwd_kernel<T, A, V, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);        \
-        else if (L.cached) gn_fwd_kernel<T, A, 1, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);      \
-        else gn_fwd_kernel<T, A, 1, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps);                   \
+        if (L.vec && L.cached) gn_fwd_kernel<T, A, V, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);   \
+        else if (L.vec) gn_fwd_kernel<T, A, V, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);        \
+        else if (L.cached) gn_fwd_kernel<T, A, 1, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);      \
+        else gn_fwd_kernel<T, A, 1, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);                   \
     } while (0)
     LUX_DISPATCH_ACT(act, GN_FWD);
 #undef GN_FWD
@@ -554,6 +598,17 @@ static int in_running_stats_impl(hipStream_t s, int64_t I, int64_t C, int64_t N,
     return LUXHIP_OK;
 }
 
+template <typename T>
+static int in_fwd_t(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, const void* x, const void* gamma, const void* beta,
+                    float eps, void* y, float* save_mean, float* save_invstd, float momentum, const void* rmean,
+                    const void* rvar, void* rmean_out, void* rvar_out) {
+    InRunning<T> rs{};
+    rs.rmean = (const T*)rmean; rs.rvar = (const T*)rvar; rs.out_mean = (T*)rmean_out; rs.out_var = (T*)rvar_out;
+    rs.momentum = momentum;
+    rs.corrected = momentum * (float)I / ((float)I - 1.0f);        // update_normalization_statistics
+    return gn_fwd_impl<T>(s, act, I, C, C, N, (const T*)x, (const T*)gamma, (const T*)beta, eps, (T*)y, save_mean, save_invstd, rs);
+}
+
 }  // namespace luxhip
 
 
@@ -575,6 +630,24 @@ int luxhip_groupnorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64
                                   (float)eps, (float*)y, save_mean, save_invstd);
     return gn_fwd_impl<bf16_t>((hipStream_t)s, act, I, C, G, N, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta,
                                (float)eps, (bf16_t*)y, save_mean, save_invstd);
+}
+
+int luxhip_instancenorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N, const void* x,
+                            const void* gamma, const void* beta, double eps, void* y, float* save_mean, float* save_invstd,
+                            double momentum, const void* rmean, const void* rvar, void* rmean_out, void* rvar_out) {
+    LUX_REQUIRE_INIT();
+    int rc = gn_check(dtype, act, I, C, C > 0 ? C : 1, N);
+    if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF((gamma == nullptr) != (beta == nullptr), "instancenorm_fwd: gamma and beta must be given together");
+    if (I * C * N == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(x == nullptr || y == nullptr || save_mean == nullptr || save_invstd == nullptr || rmean == nullptr ||
+                       rvar == nullptr || rmean_out == nullptr || rvar_out == nullptr,
+                   "instancenorm_fwd: x, y, the saved statistics and the running statistics must not be NULL");
+    if (dtype == LUXHIP_F32)
+        return in_fwd_t<float>((hipStream_t)s, act, I, C, N, x, gamma, beta, (float)eps, y, save_mean, save_invstd, (float)momentum,
+                               rmean, rvar, rmean_out, rvar_out);
+    return in_fwd_t<bf16_t>((hipStream_t)s, act, I, C, N, x, gamma, beta, (float)eps, y, save_mean, save_invstd, (float)momentum,
+                            rmean, rvar, rmean_out, rvar_out);
 }
 
 int luxhip_groupnorm_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t G, int64_t N,

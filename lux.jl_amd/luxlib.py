@@ -848,6 +848,14 @@ def _instancenorm_fwd(x, scale, bias, rmean, rvar, training, act, momentum, epsi
         y, stats, saved = _batchnorm_fwd(x, scale, bias, rmean, rvar, False, act, 0.0, epsilon, save)
         return y, stats, ("running",) + tuple(saved)
     upd = training and rmean is not None
+    if upd and x.size:
+        # one launch: the groupnorm forward kernel with G = C, whose workgroups also update the running statistics
+        y = DeviceArray(x.shape, dt)
+        sm, si = StatArray(Cc * N), StatArray(Cc * N)
+        rm_out, rv_out = DeviceArray((Cc,), dt), DeviceArray((Cc,), dt)
+        _lib.call("luxhip_instancenorm_fwd", current_stream(), x.code, _act_id(act), I, Cc, N, x.ptr, _p(scale), _p(bias),
+                  float(epsilon), y.ptr, sm.ptr, si.ptr, float(momentum), rmean.ptr, rvar.ptr, rm_out.ptr, rv_out.ptr)
+        return y, {"running_mean": rm_out, "running_var": rv_out}, ("sample", sm, si, float(epsilon))
     y, (sm, si) = _groupnorm_fwd(x, scale, bias, Cc, act, epsilon, save or upd)
     stats = {"running_mean": rmean, "running_var": rvar}
     if upd:
