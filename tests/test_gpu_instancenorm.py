@@ -99,3 +99,28 @@ def test_fast_activation(gpu, dtype, act):
         yq = f64(O.round_to_bf16(want.astype(np.float32))) if dtype == "bf16" else want
         assert_close(dx.to_numpy(), O.grad_activation(f64(delta), yq, act, f64(x)), dtype, f"{act} {shape} dx",
                      rel=None if dtype == "f32" else 2e-2)
+
+
+def test_separate_running_statistics_call_matches_the_fused_forward(gpu):
+    """luxhip_groupnorm_fwd with G = C followed by luxhip_instancenorm_running_stats (the two-call form of the C
+    ABI) gives the running statistics that luxhip_instancenorm_fwd computes in its own launch."""
+    rng = np.random.default_rng(77)
+    shape = (9, 7, 12, 5)
+    I, Cc, N = 63, 12, 5
+    x = rng.normal(size=shape).astype(np.float32) * 2 + 0.3
+    rm, rv = rng.normal(size=Cc).astype(np.float32), rng.uniform(0.5, 2.0, Cc).astype(np.float32)
+    d = gpu.DeviceArray.from_numpy
+    dx_, drm, drv = d(x), d(rm), d(rv)
+    (y, stats) = gpu.instancenorm(dx_, None, None, drm, drv, True, "identity", 0.2, 1e-5)
+    y2 = gpu.DeviceArray(shape, "f32")
+    sm, si = gpu.StatArray(Cc * N), gpu.StatArray(Cc * N)
+    s = gpu.current_stream()
+    gpu._lib.call("luxhip_groupnorm_fwd", s, 0, 0, I, Cc, Cc, N, dx_.ptr, None, None, 1e-5, y2.ptr, sm.ptr, si.ptr)
+    rm2, rv2 = gpu.DeviceArray((Cc,), "f32"), gpu.DeviceArray((Cc,), "f32")
+    gpu._lib.call("luxhip_instancenorm_running_stats", s, 0, I, Cc, N, sm.ptr, si.ptr, 1e-5, 0.2, drm.ptr, drv.ptr, rm2.ptr, rv2.ptr)
+    np.testing.assert_array_equal(y2.to_numpy(), y.to_numpy())
+    np.testing.assert_allclose(rm2.to_numpy(), stats["running_mean"].to_numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(rv2.to_numpy(), stats["running_var"].to_numpy(), rtol=1e-6)
+    want = O.instancenorm(x.astype(np.float64), None, None, rm.astype(np.float64), rv.astype(np.float64), True, "identity", 0.2, 1e-5)
+    np.testing.assert_allclose(rm2.to_numpy(), want[1], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(rv2.to_numpy(), want[2], rtol=1e-5)
