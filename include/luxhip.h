@@ -71,6 +71,15 @@ int luxhip_stream_create(luxhip_stream_t* out);
 int luxhip_stream_synchronize(luxhip_stream_t s);
 int luxhip_stream_destroy(luxhip_stream_t s);
 
+/* Sizes the stream's scratch memory (reduction partials, operand copies of the contractions) to at
+ * least `bytes` ahead of time.  Operators grow it on demand without making the host wait for the
+ * device (the outgrown block is retired behind an event on the stream), but not while the stream
+ * records a HIP graph: there a call that finds it too small returns LUXHIP_INVALID.  A caller that
+ * records graphs runs each operator once eagerly before, or reserves here.  No counterpart in the
+ * reference, whose vendor wrappers allocate their scratch arrays per call
+ * (ext/cuDNNExt/batchnorm.jl:17-18). */
+int luxhip_reserve(luxhip_stream_t s, size_t bytes);
+
 int luxhip_event_create(luxhip_event_t* out);
 int luxhip_event_record(luxhip_event_t e, luxhip_stream_t s);
 int luxhip_event_elapsed_ms(float* ms, luxhip_event_t start, luxhip_event_t stop); /* waits for stop */
@@ -193,7 +202,8 @@ int luxhip_instancenorm_fwd(luxhip_stream_t s, int dtype, int act, int64_t I, in
  * src/impl/normalization.jl:191-208) plus, in training with running statistics, this update
  * (update_normalization_statistics, src/impl/normalization.jl:91-110, reduce dims 1..N-2):
  *   rmean_out[c] = (1-m) rmean[c] + m mean_n(mu[c,n]),
- *   rvar_out[c]  = (1-m) rvar[c]  + m I/(I-1) mean_n(var[c,n]),   var = 1/invstd^2 - eps.
+ *   rvar_out[c]  = (1-m) rvar[c]  + m I/(I-1) mean_n(var[c,n]),   var = max(1/invstd^2 - eps, 0)
+ * (luxhip_instancenorm_fwd uses the slice variances themselves, which stay exact where var << eps).
  * save_mean, save_invstd: (C, N) fp32 as written by luxhip_groupnorm_fwd with G = C and the same
  * eps; rmean, rvar, rmean_out, rvar_out: length C in the storage dtype. */
 int luxhip_instancenorm_running_stats(luxhip_stream_t s, int dtype, int64_t I, int64_t C, int64_t N,

@@ -47,6 +47,7 @@ SIGNATURES = {
     "luxhip_stream_create": [C.POINTER(_vp)],
     "luxhip_stream_synchronize": [_vp],
     "luxhip_stream_destroy": [_vp],
+    "luxhip_reserve": [_vp, _sz],
     "luxhip_event_create": [C.POINTER(_vp)],
     "luxhip_event_record": [_vp, _vp],
     "luxhip_event_elapsed_ms": [C.POINTER(C.c_float), _vp, _vp],

@@ -632,8 +632,12 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         g.rowdiv = FastDiv(g.vec_per_row);
         g.chunk = (uint32_t)ceil_div(g.nq, SR);
         const int64_t S = ceil_div(g.nq, g.chunk);
+        // sized for the two-pass kernels as well, which the same call takes while a stream records a graph
+        // (where the workspace cannot grow): an eager call then prepares the recorded one
+        int64_t S2 = 1;
+        (void)make_geom(I, C, N, vv, &S2);
         Workspace ws;
-        int rc = get_workspace(s, 0, &ws);
+        int rc = get_workspace(s, (size_t)C * (2 + 3 * S2) * sizeof(float), &ws);
         if (rc != LUXHIP_OK) return rc;
         uint64_t* words = reinterpret_cast<uint64_t*>(ws.flags);
         const uint32_t spin = (uint32_t)option_bn_spin_limit();
@@ -705,8 +709,10 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         g.rowdiv = FastDiv(g.vec_per_row);
         g.chunk = (uint32_t)ceil_div(g.nq, SR);
         const int64_t S = ceil_div(g.nq, g.chunk);
+        int64_t S2 = 1;                      // the two-pass kernels' share, as in the forward pass
+        (void)make_geom(I, C, N, vv, &S2);
         Workspace ws;
-        int rc = get_workspace(s, 0, &ws);
+        int rc = get_workspace(s, (size_t)C * (3 + 2 * S2) * sizeof(float), &ws);
         if (rc != LUXHIP_OK) return rc;
         uint64_t* words = reinterpret_cast<uint64_t*>(ws.flags);
         const uint32_t spin = (uint32_t)option_bn_spin_limit();

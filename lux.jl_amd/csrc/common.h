@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "../../include/luxhip.h"
@@ -51,6 +52,20 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out);
 // resident batchnorm kernels, the split groupnorm pullback) would find their own tagged words again
 // on every replay of the graph, so the operators take their other code paths while a stream captures.
 bool stream_capturing(hipStream_t s);
+
+// What a persistent kernel needs to know once per process: its dynamic LDS limit raised and the
+// number of its workgroups that the device holds at once.  Host threads may race to the first
+// launch of a kernel: std::call_once lets one of them do the set-up while the others wait.
+struct ResidentOnce {
+    std::once_flag once;
+    int resident = 0;        // 0: the set-up failed (`error` says why)
+    hipError_t error = hipSuccess;
+    template <typename F>
+    int get(F&& setup) {     // setup(hipError_t&) -> workgroups resident at once
+        std::call_once(once, [&] { resident = setup(error); });
+        return resident;
+    }
+};
 
 // Optional per-kernel timing with HIP events on the launch stream (luxhip_profile_enable).
 struct ProfScope {

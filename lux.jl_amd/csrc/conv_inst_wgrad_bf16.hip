@@ -12,12 +12,12 @@ int launch_conv_wgrad_direct(hipStream_t s, ConvWgradDirectArgs& a, int slices) 
     a.tiles_m = (int)ceil_div(a.A.Mrows, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.B.Ncols, ML::TILE_N);
     auto kernel = conv_wgrad_direct_kernel<2, 2, 2, 4, 2>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)ML::LDS_BYTES));
-        attr_set = true;
-    }
+    static ResidentOnce ro;   // here only the one-time raise of the dynamic LDS limit
+    ro.get([&](hipError_t& err) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
+        return 1;
+    });
+    LUX_CHECK_HIP(ro.error);
     ProfScope ps("conv_wgrad_kernel<bf16>", s);
     kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)slices), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();

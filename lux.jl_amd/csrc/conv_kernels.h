@@ -218,12 +218,12 @@ int launch_conv_gemm(hipStream_t s, ConvGemmArgs<T>& a) {
     a.tiles_m = (int)ceil_div(a.gather.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.Ncols, ML::TILE_N);
     auto kernel = conv_gemm_kernel<T, WM, WN>;
-    static int resident = 0;   // workgroups that fit the device at once
-    if (resident == 0) {
-        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)ML::LDS_BYTES));
-        resident = persistent_grid(kernel, kGemmThreads, ML::LDS_BYTES, int64_t(1) << 40);
-    }
+    static ResidentOnce ro;    // workgroups that fit the device at once
+    const int resident = ro.get([&](hipError_t& err) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
+        return err == hipSuccess ? persistent_grid(kernel, kGemmThreads, ML::LDS_BYTES, int64_t(1) << 40) : 0;
+    });
+    LUX_CHECK_HIP(ro.error);
     const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
     ProfScope ps(a.gather.dgrad ? (sizeof(T) == 2 ? "conv_dgrad_kernel<bf16>" : "conv_dgrad_kernel<f32>")
                                 : (sizeof(T) == 2 ? "conv_fprop_kernel<bf16>" : "conv_fprop_kernel<f32>"), s);
@@ -431,15 +431,12 @@ __global__ __launch_bounds__(NWM * NWN * 64) void conv_tap_kernel(ConvTapArgs<T>
 template <typename T, int WM, int WN, int NWN, int NST, int NWM = 2>
 int conv_tap_resident() {
     using ML = GemmMainloop<T, WM, WN, true, true, sizeof(T) == 2, NWN, NST, NWM>;
-    static int resident = 0;
-    if (resident == 0) {
+    static ResidentOnce ro;
+    return ro.get([&](hipError_t& err) {
         auto kernel = conv_tap_kernel<T, WM, WN, NWN, NST, NWM>;
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)ML::LDS_BYTES) != hipSuccess)
-            return 0;
-        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
-    }
-    return resident;
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
+        return err == hipSuccess ? persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40) : 0;
+    });
 }
 
 template <typename T, int WM, int WN, int NWN, int NST, int NWM = 2>
@@ -584,12 +581,12 @@ int launch_conv_wgrad(hipStream_t s, ConvWgradArgs<T>& a, int slices) {
     a.tiles_m = (int)ceil_div(a.gather.Mrows, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.Cout_g, ML::TILE_N);
     auto kernel = conv_wgrad_kernel<T, WM, WN>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)ML::LDS_BYTES));
-        attr_set = true;
-    }
+    static ResidentOnce ro;   // here only the one-time raise of the dynamic LDS limit
+    ro.get([&](hipError_t& err) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
+        return 1;
+    });
+    LUX_CHECK_HIP(ro.error);
     ProfScope ps(sizeof(T) == 2 ? "conv_wgrad_kernel<bf16>" : "conv_wgrad_kernel<f32>", s);
     kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)slices), dim3(kGemmThreads), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();

@@ -122,12 +122,12 @@ int launch_cfg_full(hipStream_t s, DenseArgs<T>& a) {
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
     auto kernel = dense_gemm_kernel<T, WM, WN, AK, BKM, FULL, NWN, NWM>;
-    static int resident = 0;   // workgroups that fit the device at once
-    if (resident == 0) {
-        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)ML::LDS_BYTES));
-        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
-    }
+    static ResidentOnce ro;    // workgroups that fit the device at once
+    const int resident = ro.get([&](hipError_t& err) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
+        return err == hipSuccess ? persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40) : 0;
+    });
+    LUX_CHECK_HIP(ro.error);
     const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, resident);
     ProfScope ps(sizeof(T) == 2 ? (a.tail ? "dense_gemm_kernel<bf16>+tail" : "dense_gemm_kernel<bf16>")
                                 : (a.tail ? "dense_gemm_kernel<f32>+tail" : "dense_gemm_kernel<f32>"), s);
@@ -312,12 +312,12 @@ int launch_batched_cfg(hipStream_t s, DenseArgs<T>& a) {
     const int64_t total = (int64_t)a.tiles_m * a.tiles_n * a.batch;
     LUX_UNSUPPORTED_IF(total >= (1ll << 31), "batched_matmul: too many tiles");
     auto kernel = batched_gemm_kernel<T, WM, WN, AK, BKM, FULL, 2, 2>;
-    static int resident = 0;
-    if (resident == 0) {
-        LUX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)ML::LDS_BYTES));
-        resident = persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40);
-    }
+    static ResidentOnce ro;
+    const int resident = ro.get([&](hipError_t& err) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
+        return err == hipSuccess ? persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40) : 0;
+    });
+    LUX_CHECK_HIP(ro.error);
     ProfScope ps(sizeof(T) == 2 ? "batched_gemm_kernel<bf16>" : "batched_gemm_kernel<f32>", s);
     kernel<<<dim3((unsigned)std::min<int64_t>(total, resident)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();

@@ -57,6 +57,8 @@ struct InRunning {
     T* out_mean;
     T* out_var;
     uint32_t* counters;
+    float* var;                    // (C, N) words of workspace: the slice variances themselves (1/invstd^2 - eps would
+                                   // cancel for channels whose variance is far below eps)
     uint32_t cstride, N;
     float momentum, corrected;     // corrected = momentum * I / (I - 1)
 };
@@ -121,14 +123,14 @@ __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
         if (threadIdx.x == 0) {
             publish(reinterpret_cast<uint32_t*>(save_mean + slice), __float_as_uint(mean));
             publish(reinterpret_cast<uint32_t*>(save_invstd + slice), __float_as_uint(invstd));
+            publish(reinterpret_cast<uint32_t*>(rs.var + slice), __float_as_uint(var));
             publish_done();
         }
         if (arrive_last(rs.counters + (size_t)k * rs.cstride, rs.N, &last_flag)) {
             float tm = 0.0f, tv = 0.0f;
             for (uint32_t n = threadIdx.x; n < rs.N; n += T_) {
-                const float is = __uint_as_float(fetch(reinterpret_cast<const uint32_t*>(save_invstd + k + (size_t)g.G * n)));
                 tm += __uint_as_float(fetch(reinterpret_cast<const uint32_t*>(save_mean + k + (size_t)g.G * n)));
-                tv += 1.0f / (is * is) - eps;
+                tv += __uint_as_float(fetch(reinterpret_cast<const uint32_t*>(rs.var + k + (size_t)g.G * n)));
             }
             tm = block_sum(tm, sm);
             tv = block_sum(tv, sm);
@@ -480,9 +482,10 @@ static int gn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
     if (rs.out_mean != nullptr) {
         LUX_UNSUPPORTED_IF((size_t)C > kWorkspaceCounters, "instancenorm: more than %zu channels", kWorkspaceCounters);
         Workspace ws;
-        int rc = get_workspace(s, 0, &ws);
+        int rc = get_workspace(s, (size_t)C * N * sizeof(float), &ws);
         if (rc != LUXHIP_OK) return rc;
         rs.counters = ws.counters;
+        rs.var = reinterpret_cast<float*>(ws.data);
         rs.cstride = counter_stride(C);
         rs.N = (uint32_t)N;
     }
@@ -576,7 +579,7 @@ __global__ __launch_bounds__(256) void in_running_stats_kernel(const float* __re
     for (int n = lane; n < N; n += 64) {
         const float is = invstd[c + (size_t)C * n];
         sm += mean[c + (size_t)C * n];
-        sv += 1.f / (is * is) - eps;
+        sv += fmaxf(1.f / (is * is) - eps, 0.f);   // rounding can take the difference below zero when var << eps
     }
     sm = wave_sum(sm);
     sv = wave_sum(sv);

@@ -28,11 +28,19 @@ struct Pool {
     std::unordered_map<void*, size_t> live;         // block -> rounded size
 } g_pool;
 
+// A workspace block that has been replaced by a larger one: kernels queued before the switch may
+// still use it until `done` has passed.
+struct RetiredBlock {
+    void* p;
+    size_t bytes;
+    hipEvent_t done;
+};
 struct WsEntry {
     void* base = nullptr;
     size_t data_bytes = 0;
     uint32_t* counters = nullptr;   // kWorkspaceCounters words, zero between kernels, then kWorkspaceFlags words
     uint32_t epoch = 0;
+    std::vector<RetiredBlock> retired;
 };
 std::map<hipStream_t, WsEntry> g_ws;
 
@@ -121,19 +129,57 @@ bool stream_capturing(hipStream_t s) {
     return st != hipStreamCaptureStatusNone;
 }
 
+// Retired blocks whose last kernels have finished go to the allocator's pool: no wait and no hipFree
+// (which would synchronise the device) on an operator's path.  g_mu held.
+static void collect_retired(WsEntry& e, bool wait) {
+    for (size_t i = 0; i < e.retired.size();) {
+        RetiredBlock& r = e.retired[i];
+        if (wait) (void)hipEventSynchronize(r.done);
+        if (wait || hipEventQuery(r.done) == hipSuccess) {
+            (void)hipEventDestroy(r.done);
+            g_pool.free_blocks.emplace(r.bytes, r.p);
+            e.retired[i] = e.retired.back();
+            e.retired.pop_back();
+        } else {
+            (void)hipGetLastError();   // hipErrorNotReady is not an error here
+            ++i;
+        }
+    }
+}
+
+// The workspace never makes the host wait for the device: a block that has become too small is
+// retired behind an event on the stream and a new one is taken from the pool or the driver.  While
+// the stream records a graph nothing may be allocated (and an allocation inside a recording would
+// be replayed as a stale pointer): the caller sizes the workspace before, with one eager call of
+// the operator or luxhip_reserve.
 int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     std::lock_guard<std::mutex> lk(g_mu);
     WsEntry& e = g_ws[s];
-    if (e.base == nullptr || e.data_bytes < bytes) {
-        size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : round_size(bytes);
+    if (!e.retired.empty()) collect_retired(e, false);
+    const bool grow = e.base == nullptr || e.data_bytes < bytes;
+    if ((grow || e.counters == nullptr) && stream_capturing(s))
+        return set_error(LUXHIP_INVALID,
+                         "the stream is recording a graph and its workspace (%zu bytes) is smaller than the %zu bytes this call "
+                         "needs: call luxhip_reserve(stream, bytes) or run the operator once eagerly before recording",
+                         e.data_bytes, bytes);
+    if (grow) {
+        const size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : round_size(bytes);
+        void* p = nullptr;
+        auto it = g_pool.free_blocks.find(want);
+        if (it != g_pool.free_blocks.end()) {
+            p = it->second;
+            g_pool.free_blocks.erase(it);
+        } else {
+            LUX_CHECK_HIP(hipMalloc(&p, want));
+        }
         if (e.base != nullptr) {
             // the old block may still be in use by kernels queued on this stream
-            LUX_CHECK_HIP(hipStreamSynchronize(s));
-            LUX_CHECK_HIP(hipFree(e.base));
-            e.base = nullptr;
+            hipEvent_t done;
+            hipError_t rc = hipEventCreateWithFlags(&done, hipEventDisableTiming);
+            if (rc == hipSuccess) rc = hipEventRecord(done, s);
+            if (rc != hipSuccess) { g_pool.free_blocks.emplace(want, p); LUX_CHECK_HIP(rc); }
+            e.retired.push_back(RetiredBlock{e.base, e.data_bytes, done});
         }
-        void* p = nullptr;
-        LUX_CHECK_HIP(hipMalloc(&p, want));
         e.base = p;
         e.data_bytes = want;
     }
@@ -141,7 +187,8 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
         void* c = nullptr;
         constexpr size_t words = kWorkspaceCounters + kWorkspaceFlags + kWorkspaceZeroBytes / 4;
         LUX_CHECK_HIP(hipMalloc(&c, words * sizeof(uint32_t)));
-        hipError_t rc = hipMemsetAsync(c, 0, words * sizeof(uint32_t), s);
+        fill_zero_kernel<<<dim3(64), dim3(256), 0, s>>>(reinterpret_cast<uint32_t*>(c), words);
+        hipError_t rc = hipGetLastError();
         if (rc != hipSuccess) { (void)hipFree(c); LUX_CHECK_HIP(rc); }
         e.counters = reinterpret_cast<uint32_t*>(c);
     }
@@ -202,6 +249,7 @@ int luxhip_shutdown(void) {
     if (!g_init) return LUXHIP_OK;
     (void)hipDeviceSynchronize();
     for (auto& kv : g_ws) {
+        collect_retired(kv.second, true);       // into the pool, which is released below
         if (kv.second.base) (void)hipFree(kv.second.base);
         if (kv.second.counters) (void)hipFree(kv.second.counters);
     }
@@ -277,6 +325,7 @@ int luxhip_stream_destroy(luxhip_stream_t s) {
         std::lock_guard<std::mutex> lk(g_mu);
         auto it = g_ws.find((hipStream_t)s);
         if (it != g_ws.end()) {
+            collect_retired(it->second, true);  // the stream has been synchronised: into the pool
             if (it->second.base) (void)hipFree(it->second.base);
             if (it->second.counters) (void)hipFree(it->second.counters);
             g_ws.erase(it);
@@ -284,6 +333,12 @@ int luxhip_stream_destroy(luxhip_stream_t s) {
     }
     LUX_CHECK_HIP(hipStreamDestroy((hipStream_t)s));
     return LUXHIP_OK;
+}
+
+int luxhip_reserve(luxhip_stream_t s, size_t bytes) {
+    LUX_REQUIRE_INIT();
+    Workspace ws;
+    return get_workspace((hipStream_t)s, bytes, &ws);
 }
 
 int luxhip_event_create(luxhip_event_t* out) {

@@ -703,7 +703,10 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
         if fdrop_back is not None:
             dp = fdrop_back(dp)
         dlogits = logits                                              # the logits are no longer needed
-        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L, L * H * B, int(causal), dp.ptr, softmax_out.ptr,
+        # the causal shortcut of the softmax pullback leaves dlogits beyond the diagonal block untouched, which
+        # only the triangular products that follow tolerate: with an fdrop those run in full, so the whole
+        # column is computed (masked weights are zero, hence so is their dlogits)
+        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L, L * H * B, int(tri), dp.ptr, softmax_out.ptr,
                   scale_inv, dlogits.ptr)
         dq = DeviceArray(q.shape, dt)
         _bmm_strided(False, False, E, L, S, bdims, k, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, dq, lq.st,

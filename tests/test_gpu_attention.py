@@ -173,3 +173,37 @@ def test_dropout_of_the_attention_weights(gpu, dtype):
     assert_close(dq.to_numpy(), want_dq, dtype, "dq", rel=rel, scale=0.05)
     assert_close(dk.to_numpy(), want_dk, dtype, "dk", rel=rel, scale=0.05)
     assert_close(dv.to_numpy(), want_dv, dtype, "dv", rel=rel)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_causal_mask_with_dropout_of_the_weights(gpu, dtype):
+    """is_causal together with an fdrop over several tiles (S = L = 512): the products of the pullback run in
+    full, so every element of the logits' cotangent must have been written.  The allocator's pool is filled
+    with NaN first, so that memory a kernel skipped shows up in dq / dk."""
+    E, H, L, B = 64, 2, 512, 2
+    rng = np.random.default_rng(stable_seed("attn-causal-fdrop", dtype))
+    q, k, v = host_inputs(dtype, *(rng.normal(size=(E, H, L, B)) for _ in range(3)))
+    (dout,) = host_inputs(dtype, rng.normal(size=(E, H, L, B)))
+    poison = [dev(gpu, np.full((L, L, H, B), np.nan, np.float32), dtype) for _ in range(4)]
+    del poison                                           # back to the pool: the next tensors of this size reuse it
+    p = 0.25
+    fdrop = gpu.attention_dropout(gpu.PhiloxRNG(5, 0), p)
+    (y, w), back = gpu.pullback(gpu.scaled_dot_product_attention, dev(gpu, q, dtype), dev(gpu, k, dtype), dev(gpu, v, dtype),
+                                1, 3, None, None, True, None, fdrop)
+    dq, dk, dv = back(dev(gpu, dout, dtype))
+    _, wp = O.scaled_dot_product_attention(f64(q), f64(k), f64(v), 3, None, None, True, None)
+    noise = O.rand_uniform(wp.size, 5, 0, bf16=(dtype == "bf16")).reshape(wp.shape, order="F")
+    keep = np.where(noise > np.float32(p), 1.0 / (1.0 - p), 0.0)      # p = 0.25 is exact in both storage types
+    wd = wp * keep
+    rel = None if dtype == "f32" else 4e-2
+    assert_close(w.to_numpy(), wd, dtype, "dropped causal weights", rel=rel)
+    assert_close(y.to_numpy(), np.einsum("ehsb,slhb->ehlb", f64(v), wd), dtype, "output", rel=rel)
+    do, inv = f64(dout), 1.0 / np.sqrt(float(E))
+    dw = np.einsum("ehsb,ehlb->slhb", f64(v), do) * keep
+    ds = wp * (dw - (dw * wp).sum(axis=0, keepdims=True)) * inv
+    rel = None if dtype == "f32" else 6e-2
+    for got, want, name in ((dq, np.einsum("dhsb,slhb->dhlb", f64(k), ds), "dq"), (dk, np.einsum("dhlb,slhb->dhsb", f64(q), ds), "dk"),
+                            (dv, np.einsum("ehlb,slhb->ehsb", do, wd), "dv")):
+        g = got.to_numpy()
+        assert np.isfinite(g.astype(np.float64)).all(), name + " holds values from memory that no kernel wrote"
+        assert_close(g, want, dtype, name, rel=rel)

@@ -124,3 +124,21 @@ def test_separate_running_statistics_call_matches_the_fused_forward(gpu):
     want = O.instancenorm(x.astype(np.float64), None, None, rm.astype(np.float64), rv.astype(np.float64), True, "identity", 0.2, 1e-5)
     np.testing.assert_allclose(rm2.to_numpy(), want[1], rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(rv2.to_numpy(), want[2], rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_running_variance_of_a_constant_channel(gpu, dtype):
+    """A channel whose slices are constant (variance 0, far below eps) and one with a variance of 1e-9: the
+    running variance moves towards that variance, never below (1 - momentum) * running_var."""
+    rng = np.random.default_rng(5)
+    shape = (16, 8, 3, 4)
+    x = rng.normal(size=shape).astype(np.float32)
+    x[:, :, 0, :] = 3.0
+    x[:, :, 1, :] = 2.0 + (3e-5 * rng.normal(size=(16, 8, 4))).astype(np.float32)
+    (x,) = host_inputs(dtype, x)
+    rm, rv = np.zeros(3, np.float32), np.ones(3, np.float32)
+    (_, stats) = gpu.instancenorm(dev(gpu, x, dtype), None, None, dev(gpu, rm, dtype), dev(gpu, rv, dtype), True, "identity", 0.1, 1e-5)
+    want = O.instancenorm(f64(x), None, None, f64(rm), f64(rv), True, "identity", 0.1, 1e-5)
+    got = stats["running_var"].to_numpy().astype(np.float64)
+    assert got[0] == pytest.approx(0.9, rel=1e-2 if dtype == "bf16" else 1e-6) and (got >= 0.9 * (1 - 4e-3)).all()
+    assert_close(got, want[2], dtype, "running_var")

@@ -182,3 +182,48 @@ def test_plain_c_client_of_the_abi(gpu):
     gpu.synchronize()
     res = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert res.returncode == 0 and res.stdout.strip() == "OK", res.stdout + res.stderr
+
+
+def test_workspace_growth_does_not_wait_for_the_stream(gpu):
+    """The stream's scratch memory grows while earlier work is still queued: the call that grows it
+    returns long before that work is done (the outgrown block is retired behind an event, nothing
+    synchronises), and the operators before and after the growth give the right results."""
+    import time
+    rng = np.random.default_rng(11)
+    stream = _new_stream(gpu)
+    main = gpu.current_stream()
+    gpu.set_stream(stream)
+    try:
+        n = 4096
+        a = dev(gpu, rng.normal(size=(n, n)).astype(np.float32), "f32")
+        b = dev(gpu, rng.normal(size=(n, n)).astype(np.float32), "f32")
+        c = gpu.DeviceArray((n, n), "f32")
+        shape = (1, 96, 4000)                      # dense layout: partial sums in the workspace
+        x = rng.normal(size=shape).astype(np.float32)
+        dd, dy = dev(gpu, x, "f32"), dev(gpu, np.maximum(x, 0), "f32")
+        gx, gb = gpu.DeviceArray(shape, "f32"), gpu.DeviceArray((96,), "f32")
+        call = lambda: gpu._lib.call("luxhip_bias_activation_bwd", stream, 0, 1, 1, 96, 4000, dd.ptr, dy.ptr, None, gx.ptr, gb.ptr)
+        gpu._lib.call("luxhip_reserve", stream, 1 << 20)      # first block
+        call()
+        gpu._lib.call("luxhip_stream_synchronize", stream)
+        want_gb = gb.to_numpy().copy()
+        # about 80 ms of fp32 products (137 GFLOP each) queued on the stream
+        for _ in range(60):
+            gpu._lib.call("luxhip_matmul", stream, 0, 0, 0, n, n, n, a.ptr, n, b.ptr, n, None, c.ptr, n)
+        call()                                                 # uses the small block, queued behind the products
+        t0 = time.perf_counter()
+        gpu._lib.call("luxhip_reserve", stream, 96 << 20)     # outgrows it while that work is pending
+        call()                                                 # runs out of the new block
+        t_calls = time.perf_counter() - t0
+        gpu._lib.call("luxhip_stream_synchronize", stream)
+        t_drain = time.perf_counter() - t0 - t_calls
+        assert t_calls < 0.04 and t_drain > t_calls, (t_calls, t_drain)
+        np.testing.assert_array_equal(gb.to_numpy(), want_gb)
+        # a third growth after everything has finished recycles the retired blocks through the pool
+        gpu._lib.call("luxhip_reserve", stream, 200 << 20)
+        call()
+        gpu._lib.call("luxhip_stream_synchronize", stream)
+        np.testing.assert_array_equal(gb.to_numpy(), want_gb)
+    finally:
+        gpu.set_stream(main)
+        gpu._lib.call("luxhip_stream_destroy", stream)
