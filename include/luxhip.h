@@ -145,6 +145,20 @@ int luxhip_bias_activation_fwd(luxhip_stream_t s, int dtype, int act, int64_t I,
 int luxhip_bias_activation_bwd(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
                                const void* delta, const void* out, const void* pre, void* dx, void* dbias);
 
+/* luxhip_bias_activation_bwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and results; the partial sums and arrival counters of the bias
+ * gradient live in a fixed block of 2.25 MiB of device memory that the library holds per device from
+ * luxhip_init to the end of the process, instead of the stream's workspace, and the call makes no
+ * hipMalloc / hipFree and takes nothing from the library's pool (with luxhip_profile_enable off).
+ * Limit: the partial sums (4 C S bytes with at most 256 slices S per
+ * channel for I >= 64; 4 I C S bytes with S <= ceil(N / 8) batch slices otherwise) must fit 2 MiB:
+ * larger shapes return LUXHIP_INVALID.  All calls on a device share the block, which keeps the last
+ * call's contents (the counters are cleared on the stream by each call): calls that overlap in time
+ * on one device, i.e. on different streams, race. */
+int luxhip_bias_activation_bwd_noalloc(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                                       const void* delta, const void* out, const void* pre, void* dx, void* dbias);
+
 /* ---------------------------------------------------------------- batchnorm ----------
  * x, y, delta, dx: (I, C, N); gamma, beta, rmean, rvar, rmean_out, rvar_out, dgamma, dbeta:
  * length C in `dtype`; save_mean, save_invstd: length C, fp32. */

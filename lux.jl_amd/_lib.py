@@ -64,6 +64,7 @@ SIGNATURES = {
     "luxhip_fill_zero": [_vp, _sz, _vp],
     "luxhip_bias_activation_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp],
     "luxhip_bias_activation_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp],
+    "luxhip_bias_activation_bwd_noalloc": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp],
     "luxhip_batchnorm_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i, _d, _d, _vp, _vp, _vp, _fp, _fp],
     "luxhip_batchnorm_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _fp, _fp, _i, _vp, _vp, _vp],
     "luxhip_groupnorm_fwd": [_vp, _i, _i, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _d, _vp, _fp, _fp],

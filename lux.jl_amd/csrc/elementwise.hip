@@ -328,9 +328,33 @@ static int bias_act_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
     return LUXHIP_OK;
 }
 
+// Where the pullback's scratch memory (partial sums, arrival counters) comes from: the stream's
+// workspace, which may allocate, or a fixed block handed in by the entry point that allocates nothing.
+struct FixedScratch {
+    float* partial;
+    size_t partial_bytes;
+    uint32_t* counters;      // kWorkspaceCounters words, zero
+};
+static int bwd_scratch(hipStream_t s, const FixedScratch* fixed, size_t bytes, float** partial, uint32_t** counters) {
+    if (fixed != nullptr) {
+        LUX_INVALID_IF(bytes > fixed->partial_bytes,
+                       "bias_activation_bwd_noalloc: this shape needs %zu bytes of scratch memory, the fixed block has %zu", bytes,
+                       fixed->partial_bytes);
+        *partial = fixed->partial;
+        *counters = fixed->counters;
+        return LUXHIP_OK;
+    }
+    Workspace ws;
+    int rc = get_workspace(s, bytes, &ws);
+    if (rc != LUXHIP_OK) return rc;
+    *partial = reinterpret_cast<float*>(ws.data);
+    *counters = ws.counters;
+    return LUXHIP_OK;
+}
+
 template <typename T>
 static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, const T* delta, const T* out,
-                             const T* pre, T* dx, T* dbias) {
+                             const T* pre, T* dx, T* dbias, const FixedScratch* fixed = nullptr) {
     constexpr int V = Vec<T>::N;
     const int64_t total = I * C * N;
     const bool ptr_ok = aligned16(delta) && aligned16(dx) && (out == nullptr || aligned16(out)) &&
@@ -365,11 +389,10 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
         if (S < 1) S = 1;
         const uint32_t chunk = (uint32_t)ceil_div(nq, S);
         S = ceil_div(nq, chunk);
-        Workspace ws;
-        int rc = get_workspace(s, (size_t)C * S * sizeof(float), &ws);
+        float* partial = nullptr;
+        uint32_t* counters = nullptr;
+        int rc = bwd_scratch(s, fixed, (size_t)C * S * sizeof(float), &partial, &counters);
         if (rc != LUXHIP_OK) return rc;
-        float* partial = reinterpret_cast<float*>(ws.data);
-        uint32_t* counters = ws.counters;
         const FastDiv rowdiv((uint32_t)(I / vv));
         dim3 grid((unsigned)S, (unsigned)C);
 #define LAUNCH_CH(A)                                                                                               \
@@ -397,10 +420,10 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
     const uint32_t n_per_slice = (uint32_t)ceil_div(N, S);
     S = ceil_div(N, n_per_slice);
     LUX_UNSUPPORTED_IF(S > 65535, "bias_activation_bwd: batch split too large");
-    Workspace ws;
-    int rc = get_workspace(s, (size_t)P * S * sizeof(float), &ws);
+    float* partial = nullptr;
+    uint32_t* counters_unused = nullptr;
+    int rc = bwd_scratch(s, fixed, (size_t)P * S * sizeof(float), &partial, &counters_unused);
     if (rc != LUXHIP_OK) return rc;
-    float* partial = reinterpret_cast<float*>(ws.data);
     dim3 grid((unsigned)gx, (unsigned)S);
 #define LAUNCH_PL(A)                                                                                               \
     do {                                                                                                           \
@@ -459,6 +482,34 @@ __global__ __launch_bounds__(256) void convert_kernel(const TI* __restrict__ in,
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) st(out + i, ld(in + i));
 }
 
+// ------------------------------------------------------------------------------- scratch of the entry point that allocates nothing
+// luxhip_bias_activation_bwd_noalloc keeps its partial sums and arrival counters in this array instead
+// of the stream's workspace.  Every device the library runs on holds its own copy for the life of the
+// process.  In host code the array's name is only a handle for hipGetSymbolAddress: the device
+// address it returns (kept per device in g_noalloc_ptr) is what kernels and fills receive.
+constexpr size_t kNoAllocCounterBytes = kWorkspaceCounters * sizeof(uint32_t);    // 256 KiB
+constexpr size_t kNoAllocPartialBytes = size_t(2) << 20;                          // 2 MiB of partial sums
+constexpr int kNoAllocMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kNoAllocCounterBytes + kNoAllocPartialBytes];
+static unsigned char* g_noalloc_ptr[kNoAllocMaxDevices] = {};
+
+// Called by luxhip_init with `device` current.
+int noalloc_setup(int device) {
+    LUX_INVALID_IF(device < 0 || device >= kNoAllocMaxDevices, "device %d beyond the %d the library keeps scratch blocks for", device,
+                   kNoAllocMaxDevices);
+    if (g_noalloc_ptr[device] != nullptr) return LUXHIP_OK;
+    unsigned char* ptr = nullptr;
+    LUX_CHECK_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    LUX_INVALID_IF(ptr == nullptr, "hipGetSymbolAddress returned no address for the scratch block");
+    g_noalloc_ptr[device] = ptr;
+    return LUXHIP_OK;
+}
+
+__global__ void fill_zero_words_kernel(uint32_t* p, size_t nwords) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nwords) p[i] = 0u;
+}
+
 }  // namespace luxhip
 
 using namespace luxhip;
@@ -495,6 +546,41 @@ int luxhip_bias_activation_bwd(luxhip_stream_t s, int dtype, int act, int64_t I,
                                         (const float*)pre, (float*)dx, (float*)dbias);
     return bias_act_bwd_impl<bf16_t>((hipStream_t)s, act, I, C, N, (const bf16_t*)delta, (const bf16_t*)out,
                                      (const bf16_t*)pre, (bf16_t*)dx, (bf16_t*)dbias);
+}
+
+int luxhip_bias_activation_bwd_noalloc(luxhip_stream_t s, int dtype, int act, int64_t I, int64_t C, int64_t N,
+                                       const void* delta, const void* out, const void* pre, void* dx, void* dbias) {
+    LUX_REQUIRE_INIT();
+    int rc = check_common(dtype, act, I, C, N);
+    if (rc != LUXHIP_OK) return rc;
+    int device = -1;
+    LUX_CHECK_HIP(hipGetDevice(&device));
+    unsigned char* const block = (device >= 0 && device < kNoAllocMaxDevices) ? g_noalloc_ptr[device] : nullptr;
+    LUX_INVALID_IF(block == nullptr, "bias_activation_bwd_noalloc: no scratch block on device %d (luxhip_init sets it up)", device);
+    if (I * C * N == 0) {
+        if (dbias != nullptr && C > 0) return luxhip_fill_zero(dbias, (size_t)C * (dtype == LUXHIP_F32 ? 4 : 2), s);
+        return LUXHIP_OK;
+    }
+    LUX_INVALID_IF(delta == nullptr || dx == nullptr, "bias_activation_bwd_noalloc: delta and dx must not be NULL");
+    LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && !act_needs_pre(act) && out == nullptr,
+                   "bias_activation_bwd_noalloc: activation %d needs `out`", act);
+    LUX_INVALID_IF(act_needs_pre(act) && pre == nullptr, "bias_activation_bwd_noalloc: activation %d needs `pre`", act);
+    FixedScratch fx;
+    fx.counters = reinterpret_cast<uint32_t*>(block);
+    fx.partial = reinterpret_cast<float*>(block + kNoAllocCounterBytes);
+    fx.partial_bytes = kNoAllocPartialBytes;
+    if (dbias != nullptr) {
+        // the block keeps what the last call left: the arrival counters this call uses start at zero (a fill
+        // kernel, which a recording stream can hold, unlike a memset node)
+        const size_t words = std::min<size_t>((size_t)C * counter_stride(C), kWorkspaceCounters);
+        fill_zero_words_kernel<<<dim3((unsigned)ceil_div((int64_t)words, 256)), dim3(256), 0, (hipStream_t)s>>>(fx.counters, words);
+        LUX_CHECK_LAUNCH();
+    }
+    if (dtype == LUXHIP_F32)
+        return bias_act_bwd_impl<float>((hipStream_t)s, act, I, C, N, (const float*)delta, (const float*)out, (const float*)pre,
+                                        (float*)dx, (float*)dbias, &fx);
+    return bias_act_bwd_impl<bf16_t>((hipStream_t)s, act, I, C, N, (const bf16_t*)delta, (const bf16_t*)out, (const bf16_t*)pre,
+                                     (bf16_t*)dx, (bf16_t*)dbias, &fx);
 }
 
 int luxhip_convert(luxhip_stream_t s, int dtype_in, int dtype_out, int64_t n, const void* in, void* out) {

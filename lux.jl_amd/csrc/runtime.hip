@@ -119,6 +119,7 @@ int64_t option_gemm_tile() {
 }
 
 __global__ void fill_zero_kernel(uint32_t* p, size_t nwords);
+int noalloc_setup(int device);   // elementwise.hip: device address of the fixed scratch block
 
 bool stream_capturing(hipStream_t s) {
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
@@ -238,6 +239,10 @@ int luxhip_init(int device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(LUXHIP_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
                          prop.gcnArchName);
+    {
+        const int rc = noalloc_setup(device);
+        if (rc != LUXHIP_OK) return rc;
+    }
     g_cus = prop.multiProcessorCount;
     g_device = device;
     g_init = true;
