@@ -155,6 +155,20 @@ int launch_cfg(hipStream_t s, DenseArgs<T>& a) {
 
 int gemm_tile_override();   // gemm.hip: LUXHIP_GEMM_TILE=82|42|22|11 forces a tile (tuning aid), 0 = automatic
 
+// gemm_inst_bf16_kk.hip: the 256 x 256 kernel for two K-major bf16 operands (gemm_kk256.h); false if the
+// problem does not meet its conditions (then *rc is untouched)
+bool launch_kk256_if_applicable(hipStream_t s, DenseArgs<bf16_t>& a, int* rc);
+
+// whole 256 x 256 tiles of a large problem
+template <typename T, bool AK, bool BKM>
+int launch_big_tiles(hipStream_t s, DenseArgs<T>& a) {
+    if constexpr (sizeof(T) == 2 && AK && BKM) {
+        int rc = LUXHIP_OK;
+        if (gemm_tile_override() == 0 && launch_kk256_if_applicable(s, a, &rc)) return rc;
+    }
+    return launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, a);
+}
+
 template <typename T, bool AK, bool BKM>
 int launch_layout(hipStream_t s, DenseArgs<T>& a) {
     switch (gemm_tile_override()) {
@@ -169,6 +183,13 @@ int launch_layout(hipStream_t s, DenseArgs<T>& a) {
     // fastest on large problems; 64 x 64 for small ones.
     if constexpr (sizeof(T) == 2) {
         if (whole_tiles<T, 256, 256>(a) && (int64_t)(a.M / 256) * (a.N / 256) >= 128) {
+            if constexpr (AK && BKM) {
+                // two K-major operands: one launch of the 256 x 256 kernel of gemm_kk256.h.  A last round that
+                // is partly empty costs it less than the split below would (the small-tile kernel runs the rest
+                // at a quarter of its rate: 0.60 ms against 0.44 ms for 11008 x 8192 x 4096)
+                int rc = LUXHIP_OK;
+                if (gemm_tile_override() == 0 && launch_kk256_if_applicable(s, a, &rc)) return rc;
+            }
             // The 256 x 256 tiles are walked in rounds of one per compute unit.  When the last
             // round would be mostly empty, the matrix is cut along m or n: the part that makes
             // whole rounds keeps the big tiles, the rest (at most 10 % of the tiles) goes to
@@ -200,12 +221,12 @@ int launch_layout(hipStream_t s, DenseArgs<T>& a) {
                     big.A.rows = big.M; big.B.rows = big.N;
                     rest.tail = 1;
                     rest.A.rows = rest.M; rest.B.rows = rest.N;
-                    int rc = launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, big);
+                    int rc = launch_big_tiles<T, AK, BKM>(s, big);
                     if (rc != LUXHIP_OK) return rc;
                     return launch_cfg<T, 2, 2, AK, BKM>(s, rest);
                 }
             }
-            return launch_cfg_full<T, 4, 2, AK, BKM, true, 4>(s, a);
+            return launch_big_tiles<T, AK, BKM>(s, a);
         }
     }
     const int64_t t128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);

@@ -11,7 +11,8 @@
 #
 # There is no Julia toolchain where this repository is built and tested, so this file is
 # exercised nowhere yet; the Python mirror (lux.jl_amd/luxlib.py) drives the very same C ABI
-# with the very same argument order and is what the parity tests run.
+# with the very same argument order and is what the parity tests run.  A CPU test parses every
+# `ccall((:luxhip_...` below and checks symbol, argument count and C types against include/luxhip.h.
 module LuxHIP
 
 using LuxLib: LuxLib, Impl, Traits, Utils
@@ -89,6 +90,25 @@ end
 MLDataDevices.get_device_type(::HIPArray) = LuxHIPDevice          # feeds internal_operation_mode (traits.jl:191-197)
 MLDataDevices.get_device(::HIPArray) = LuxHIPDevice()
 
+# A HIPArray supports neither scalar indexing nor Base broadcasting (no kernel compiler sits behind
+# it): whatever libluxhip declines (status -1: an activation without a device kernel, an unsupported
+# shape) cannot fall back to LuxLib's generic broadcast path on this array type.  Those cases raise
+# this error, which names the way out: move the operands to the host (`Array(x)`) for that call.
+struct HIPFallbackError <: Exception
+    what::String
+end
+Base.showerror(io::IO, e::HIPFallbackError) = print(io, "LuxHIP: ", e.what, " is not handled by libluxhip (", last_error(),
+    ") and HIPArray has no generic broadcast/indexing path to fall back to; run this call on host arrays (`Array(x)`)")
+Base.getindex(::HIPArray, ::Int...) = throw(HIPFallbackError("scalar indexing"))
+Base.setindex!(::HIPArray, _, ::Int...) = throw(HIPFallbackError("scalar indexing"))
+Base.Broadcast.BroadcastStyle(::Type{<:HIPArray}) = throw(HIPFallbackError("broadcasting"))
+function Base.copyto!(dst::HIPArray{T}, src::HIPArray{T}) where {T}
+    length(dst) == length(src) || throw(DimensionMismatch("copyto!: lengths differ"))
+    check(ccall((:luxhip_memcpy_d2d, libluxhip), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), dst.ptr, src.ptr,
+        length(src) * sizeof(T), stream()))
+    return dst
+end
+
 const HIPOp = GPUBroadcastOp{LuxHIPDevice}
 optr(::Nothing) = C_NULL
 optr(a::HIPArray) = Ptr{Cvoid}(pointer(a))
@@ -124,11 +144,12 @@ function gemm!(C::HIPArray{T,2}, A, B, bias) where {T<:HIPFloat}
 end
 
 function Impl.matmul!(C::HIPArray{T,2}, ::HIPOp, A::AbstractMatrix, B::AbstractMatrix) where {T<:HIPFloat}
-    gemm!(C, A, B, nothing) || invoke(Impl.matmul!, Tuple{AbstractMatrix,Traits.AbstractInternalArrayOpMode,AbstractMatrix,AbstractMatrix}, C, HIPOp(), A, B)
+    gemm!(C, A, B, nothing) || throw(HIPFallbackError("matmul!"))
     return nothing
 end
+# C = A * B .+ bias in one kernel (the reference's fallback is `C .= bias; mul!(C, A, B, 1, 1)`, impl/matmul.jl:80-82)
 function Impl.matmuladd!(C::HIPArray{T,2}, ::HIPOp, A::AbstractMatrix, B::AbstractMatrix, bias::HIPArray{T,1}) where {T<:HIPFloat}
-    gemm!(C, A, B, bias) || (C .= bias; Impl.matmul!(C, HIPOp(), A, B))   # reference fallback is C .= bias; mul!(C, A, B, 1, 1)
+    gemm!(C, A, B, bias) || throw(HIPFallbackError("matmuladd!"))
     return nothing
 end
 
@@ -145,8 +166,10 @@ end
 
 function Impl.fused_dense!(y::HIPArray{T,2}, opmode::HIPOp, act::F, W::HIPArray{T,2}, x::HIPArray{T,2},
         b::Union{Nothing,HIPArray{T,1}}) where {F,T<:HIPFloat}
-    if !fused_dense_device!(y, nothing, act, W, x, b)            # -1: warn once, generic path (cublaslt.jl:359-402)
-        @warn "libluxhip cannot handle this fused dense call; using the generic path" maxlog = 1
+    if !fused_dense_device!(y, nothing, act, W, x, b)
+        # -1 (cublaslt.jl:359-402 warns and takes the unfused path): the product still runs on the device; an
+        # activation without a device kernel ends in HIPFallbackError inside bias_activation!
+        @warn "libluxhip cannot fuse this dense call; using matmul! followed by bias_activation!" maxlog = 1
         Impl.matmul!(y, opmode, W, x)
         Impl.bias_activation!(y, opmode, act, y, b)
     end
@@ -158,7 +181,7 @@ end
 function CRC.rrule(::typeof(Impl.fused_dense), opmode::HIPOp, act::F, W::HIPArray{T,2}, x::HIPArray{T,2},
         b::Union{Nothing,HIPArray{T,1}}) where {F,T<:HIPFloat}
     id = act_id(act)
-    id === nothing && return CRC.rrule_via_ad(CRC.NoForwardsMode(), Impl.fused_dense, Traits.GenericBroadcastOp(), act, W, x, b)
+    id === nothing && throw(HIPFallbackError("the pullback of fused_dense with activation $(act)"))
     M, K = size(W)
     N = size(x, 2)
     y = similar(W, T, (M, N))
@@ -190,7 +213,7 @@ function Impl.bias_activation!(y::HIPArray{T,N}, ::HIPOp, Ïƒ::F, x::HIPArray{T,N
     ok = id !== nothing && check(ccall((:luxhip_bias_activation_fwd, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
         stream(), dtype_code(T), id, I, C, Nb, optr(x), optr(bias), optr(y), C_NULL))
-    ok || broadcast!(Ïƒ âˆ˜ +, y, x, Impl.reshape_bias(x, bias))
+    ok || throw(HIPFallbackError("bias_activation! with activation $(Ïƒ)"))
     return nothing
 end
 Impl.activation!(y::HIPArray{T,N}, op::HIPOp, Ïƒ::F, x::HIPArray{T,N}) where {F,T<:HIPFloat,N} =
@@ -198,7 +221,7 @@ Impl.activation!(y::HIPArray{T,N}, op::HIPOp, Ïƒ::F, x::HIPArray{T,N}) where {F,
 
 function Impl.âˆ‡activation(::HIPOp, Î”::HIPArray{T,N}, out::HIPArray{T,N}, act::F, x) where {F,T<:HIPFloat,N}
     id = act_id(act)
-    id === nothing && return @. Î” * Utils.only_derivative(out, act, x)
+    id === nothing && throw(HIPFallbackError("âˆ‡activation of $(act)"))
     âˆ‚x = similar(out)
     pre = x isa HIPArray ? x : nothing
     check(ccall((:luxhip_bias_activation_bwd, libluxhip), Cint,
@@ -228,12 +251,13 @@ end
 
 function Impl.batchnorm(x::HIPArray{T,N}, Î³::Union{Nothing,HIPArray{T,1}}, Î²::Union{Nothing,HIPArray{T,1}},
         rÎ¼::Union{Nothing,HIPArray{T,1}}, rÏƒÂ²::Union{Nothing,HIPArray{T,1}}, training::StaticBool, act::F, m, Ïµ) where {F,T<:HIPFloat,N}
-    act_id(act) === nothing && return invoke(Impl.batchnorm, Tuple{AbstractArray,Any,Any,Any,Any,StaticBool,Any,Any,Any}, x, Î³, Î², rÎ¼, rÏƒÂ², training, act, m, Ïµ)
+    act_id(act) === nothing && throw(HIPFallbackError("batchnorm with activation $(act)"))
     y, rÎ¼â€², rÏƒÂ²â€², _, _ = batchnorm_device(x, Î³, Î², rÎ¼, rÏƒÂ², known(training), act, m, Ïµ, false)
     return y, rÎ¼â€², rÏƒÂ²â€²
 end
 
 function CRC.rrule(::typeof(Impl.batchnorm), x::HIPArray{T,N}, Î³, Î², rÎ¼, rÏƒÂ², training::StaticBool, act::F, m, Ïµ) where {F,T<:HIPFloat,N}
+    act_id(act) === nothing && throw(HIPFallbackError("the pullback of batchnorm with activation $(act)"))
     y, rÎ¼â€², rÏƒÂ²â€², Î¼s, is = batchnorm_device(x, Î³, Î², rÎ¼, rÏƒÂ², known(training), act, m, Ïµ, true)
     I, C, Nb = icn(x)
     from_batch = known(training) || rÎ¼ === nothing
@@ -253,10 +277,188 @@ function CRC.rrule(::typeof(Impl.batchnorm), x::HIPArray{T,N}, Î³, Î², rÎ¼, rÏƒÂ
     return (y, rÎ¼â€², rÏƒÂ²â€²), âˆ‡batchnorm_hip
 end
 
-# groupnorm and layernorm follow the same pattern on luxhip_groupnorm_{fwd,bwd} and
-# luxhip_layernorm_{fwd,bwd}: a whole-op method on Impl.groupnorm / Impl.layernorm for
-# HIPArray that returns y, and an rrule that keeps the saved statistics and makes one device
-# call for (âˆ‚x, âˆ‚Î³, âˆ‚Î²).  (lux.jl_amd/luxlib.py: rrule_groupnorm, rrule_layernorm.)
+# ---------------------------------------------------------------------------------------------
+# groupnorm: whole-op method + rrule  (impl/groupnorm.jl:5-22, 349-404; mean_var rrule impl/common_ops.jl:45-61)
+# ---------------------------------------------------------------------------------------------
+function groupnorm_device(x::HIPArray{T,N}, Î³, Î², groups::Int, act, Ïµ, save::Bool) where {T<:HIPFloat,N}
+    id = act_id(act)
+    id === nothing && throw(HIPFallbackError("groupnorm with activation $(act)"))
+    I, C, Nb = icn(x)
+    y = similar(x)
+    Î¼s = save ? HIPArray{Float32,1}(undef, (groups * Nb,)) : nothing
+    is = save ? HIPArray{Float32,1}(undef, (groups * Nb,)) : nothing
+    check(ccall((:luxhip_groupnorm_fwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), id, I, C, groups, Nb, optr(x), optr(Î³), optr(Î²), Float64(Ïµ), optr(y), optr(Î¼s), optr(is))) ||
+        throw(HIPFallbackError("groupnorm"))
+    return y, Î¼s, is
+end
+
+Impl.groupnorm(x::HIPArray{T,N}, Î³::Union{Nothing,HIPArray{T,1}}, Î²::Union{Nothing,HIPArray{T,1}}, groups::Int, act::F,
+    Ïµ) where {F,T<:HIPFloat,N} = first(groupnorm_device(x, Î³, Î², groups, act, Ïµ, false))
+
+function groupnorm_pullback(Î”::HIPArray{T,N}, x::HIPArray{T,N}, Î³, Î², groups::Int, id::Cint, Î¼s, is) where {T<:HIPFloat,N}
+    I, C, Nb = icn(x)
+    âˆ‚x = similar(x)
+    âˆ‚Î³ = Î³ === nothing ? nothing : similar(Î³)
+    âˆ‚Î² = Î² === nothing ? nothing : similar(Î²)
+    check(ccall((:luxhip_groupnorm_bwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
+            Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), id, I, C, groups, Nb, optr(Î”), optr(x), optr(Î³), optr(Î²), optr(Î¼s), optr(is), optr(âˆ‚x), optr(âˆ‚Î³),
+        optr(âˆ‚Î²))) || error(last_error())
+    return âˆ‚x, âˆ‚Î³, âˆ‚Î²
+end
+
+function CRC.rrule(::typeof(Impl.groupnorm), x::HIPArray{T,N}, Î³::Union{Nothing,HIPArray{T,1}}, Î²::Union{Nothing,HIPArray{T,1}},
+        groups::Int, act::F, Ïµ) where {F,T<:HIPFloat,N}
+    y, Î¼s, is = groupnorm_device(x, Î³, Î², groups, act, Ïµ, true)
+    id = act_id(act)
+    function âˆ‡groupnorm_hip(Î”â€²)
+        âˆ‚x, âˆ‚Î³, âˆ‚Î² = groupnorm_pullback(CRC.unthunk(Î”â€²), x, Î³, Î², groups, id, Î¼s, is)
+        nt = NoTangent()
+        return nt, âˆ‚x, something(âˆ‚Î³, nt), something(âˆ‚Î², nt), nt, nt, nt
+    end
+    return y, âˆ‡groupnorm_hip
+end
+
+# ---------------------------------------------------------------------------------------------
+# instancenorm (impl/normalization.jl:191-208): the groupnorm kernels with G = C; training with running
+# statistics updates them in the same launch; inference with running statistics is the inference batchnorm
+# ---------------------------------------------------------------------------------------------
+function instancenorm_device(x::HIPArray{T,N}, Î³, Î², rÎ¼, rÏƒÂ², training::Bool, act, m, Ïµ, save::Bool) where {T<:HIPFloat,N}
+    id = act_id(act)
+    id === nothing && throw(HIPFallbackError("instancenorm with activation $(act)"))
+    I, C, Nb = icn(x)
+    if !training && rÎ¼ !== nothing
+        y, _, _, Î¼s, is = batchnorm_device(x, Î³, Î², rÎ¼, rÏƒÂ², false, act, m, Ïµ, save)
+        return y, rÎ¼, rÏƒÂ², (:running, Î¼s, is)
+    end
+    if training && rÎ¼ !== nothing && length(x) > 0
+        y, rÎ¼â€², rÏƒÂ²â€² = similar(x), similar(rÎ¼), similar(rÏƒÂ²)
+        Î¼s, is = HIPArray{Float32,1}(undef, (C * Nb,)), HIPArray{Float32,1}(undef, (C * Nb,))
+        check(ccall((:luxhip_instancenorm_fwd, libluxhip), Cint,
+            (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
+                Cdouble, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+            stream(), dtype_code(T), id, I, C, Nb, optr(x), optr(Î³), optr(Î²), Float64(Ïµ), optr(y), optr(Î¼s), optr(is), Float64(m),
+            optr(rÎ¼), optr(rÏƒÂ²), optr(rÎ¼â€²), optr(rÏƒÂ²â€²))) || throw(HIPFallbackError("instancenorm"))
+        return y, rÎ¼â€², rÏƒÂ²â€², (:sample, Î¼s, is)
+    end
+    y, Î¼s, is = groupnorm_device(x, Î³, Î², C, act, Ïµ, save)
+    return y, rÎ¼, rÏƒÂ², (:sample, Î¼s, is)
+end
+
+function Impl.instancenorm(x::HIPArray{T,N}, Î³::Union{Nothing,HIPArray{T,1}}, Î²::Union{Nothing,HIPArray{T,1}},
+        rÎ¼::Union{Nothing,HIPArray{T,1}}, rÏƒÂ²::Union{Nothing,HIPArray{T,1}}, training::StaticBool, act::F, m, Ïµ) where {F,T<:HIPFloat,N}
+    y, rÎ¼â€², rÏƒÂ²â€², _ = instancenorm_device(x, Î³, Î², rÎ¼, rÏƒÂ², known(training), act, m, Ïµ, false)
+    return y, rÎ¼â€², rÏƒÂ²â€²
+end
+
+function CRC.rrule(::typeof(Impl.instancenorm), x::HIPArray{T,N}, Î³, Î², rÎ¼, rÏƒÂ², training::StaticBool, act::F, m, Ïµ) where {F,T<:HIPFloat,N}
+    y, rÎ¼â€², rÏƒÂ²â€², (kind, Î¼s, is) = instancenorm_device(x, Î³, Î², rÎ¼, rÏƒÂ², known(training), act, m, Ïµ, true)
+    id = act_id(act)
+    I, C, Nb = icn(x)
+    function âˆ‡instancenorm_hip(Î”â€²)
+        Î” = CRC.unthunk(first(CRC.unthunk(Î”â€²)))
+        nt = NoTangent()
+        if kind === :running      # statistics are constants: only âˆ‚x = âˆ‚y Î³â€² and the parameter gradients
+            âˆ‚x = similar(x)
+            âˆ‚Î³ = Î³ === nothing ? nothing : similar(Î³)
+            âˆ‚Î² = Î² === nothing ? nothing : similar(Î²)
+            check(ccall((:luxhip_batchnorm_bwd, libluxhip), Cint,
+                (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Cint,
+                    Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+                stream(), dtype_code(T), id, I, C, Nb, optr(Î”), optr(x), optr(Î³), optr(Î²), optr(Î¼s), optr(is), Cint(0), optr(âˆ‚x),
+                optr(âˆ‚Î³), optr(âˆ‚Î²))) || error(last_error())
+        else
+            âˆ‚x, âˆ‚Î³, âˆ‚Î² = groupnorm_pullback(Î”, x, Î³, Î², C, id, Î¼s, is)
+        end
+        return nt, âˆ‚x, something(âˆ‚Î³, nt), something(âˆ‚Î², nt), nt, nt, nt, nt, nt, nt
+    end
+    return (y, rÎ¼â€², rÏƒÂ²â€²), âˆ‡instancenorm_hip
+end
+
+# ---------------------------------------------------------------------------------------------
+# layernorm: the reference has no device hook (impl/layernorm.jl:3-14 is generic broadcasts), so the
+# whole op gets a method + rrule.  Statistics run over a prefix 1:k of the dims ((L, R) view).  Parameters
+# that span exactly those dims go into the same kernel; parameters that vary along one other run of dims
+# (e.g. (1, 1, C, 1) with dims = Colon()) are applied by a second per-channel pass: the inference batchnorm
+# kernel with mean 0, variance 1, Îµ = 0 on the (I, C, N) view, and its pullback yields their gradients.
+# ---------------------------------------------------------------------------------------------
+function layernorm_geometry(x::HIPArray{T,N}, Î³, Î², dims) where {T,N}
+    d = Impl.compute_layernorm_dims(x, Î³, Î², dims)                      # throws like the reference (impl/layernorm.jl:16-35)
+    d = d isa Colon ? (1:N) : d
+    dv = sort!(collect(Int, d))
+    dv == collect(1:length(dv)) || throw(HIPFallbackError("layernorm over the non-leading dims $(d)"))
+    k = length(dv)
+    L = prod(size(x)[1:k]; init=1)
+    R = L == 0 ? 0 : length(x) Ã· L
+    Î³ === nothing && return L, R, nothing
+    pshape = (size(Î³)..., ntuple(Returns(1), N - ndims(Î³))...)         # expand_layernorm_dims (impl/layernorm.jl:37-51)
+    pshape == (size(x)[1:k]..., ntuple(Returns(1), N - k)...) && return L, R, nothing
+    varying = findall(!=(1), collect(pshape))
+    a, b = isempty(varying) ? (N + 1, N) : (first(varying), last(varying))
+    all(i -> pshape[i] == size(x, i), a:b) || throw(HIPFallbackError("layernorm parameters of shape $(size(Î³)) with gaps between the dims they vary along"))
+    return L, R, (prod(size(x)[1:(a - 1)]; init=1), prod(size(x)[a:b]; init=1), prod(size(x)[(b + 1):N]; init=1))
+end
+
+function layernorm_device(x::HIPArray{T,N}, Î³, Î², act, dims, Ïµ, save::Bool) where {T<:HIPFloat,N}
+    id = act_id(act)
+    id === nothing && throw(HIPFallbackError("layernorm with activation $(act)"))
+    L, R, view = layernorm_geometry(x, Î³, Î², dims)
+    y = similar(x)
+    Î¼s = save ? HIPArray{Float32,1}(undef, (R,)) : nothing
+    is = save ? HIPArray{Float32,1}(undef, (R,)) : nothing
+    fused = view === nothing
+    check(ccall((:luxhip_layernorm_fwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), fused ? id : Cint(0), L, R, optr(x), fused ? optr(Î³) : C_NULL, fused ? optr(Î²) : C_NULL, Float64(Ïµ),
+        optr(y), optr(Î¼s), optr(is))) || throw(HIPFallbackError("layernorm"))
+    fused && return y, (Î¼s, is, L, R, nothing, nothing)
+    I, C, Nn = view
+    xÌ‚ = reshape(y, (I, C, Nn))
+    zeros_c, ones_c = fill_like(Î³, C, 0), fill_like(Î³, C, 1)
+    out, _, _, Î¼a, ia = batchnorm_device(xÌ‚, reshape(Î³, (C,)), reshape(Î², (C,)), zeros_c, ones_c, false, act, 0.1, 0.0, save)
+    return reshape(out, size(x)), (Î¼s, is, L, R, xÌ‚, (Î¼a, ia))
+end
+fill_like(a::HIPArray{T}, n::Integer, v) where {T} = HIPArray(fill(T(v), n))
+
+Impl.layernorm(x::HIPArray{T,N}, Î³::Union{Nothing,HIPArray{T}}, Î²::Union{Nothing,HIPArray{T}}, act::F, dims, Ïµ) where {F,T<:HIPFloat,N} =
+    first(layernorm_device(x, Î³, Î², act, dims, Ïµ, false))
+
+function CRC.rrule(::typeof(Impl.layernorm), x::HIPArray{T,N}, Î³::Union{Nothing,HIPArray{T}}, Î²::Union{Nothing,HIPArray{T}}, act::F, dims,
+        Ïµ) where {F,T<:HIPFloat,N}
+    y, (Î¼s, is, L, R, xÌ‚, affine) = layernorm_device(x, Î³, Î², act, dims, Ïµ, true)
+    id = act_id(act)
+    LnBwdSig = (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
+        Ptr{Cvoid}, Ptr{Cvoid})
+    function âˆ‡layernorm_hip(Î”â€²)
+        Î” = CRC.unthunk(Î”â€²)
+        nt = NoTangent()
+        âˆ‚x = similar(x)
+        âˆ‚Î³ = Î³ === nothing ? nothing : similar(Î³)
+        âˆ‚Î² = Î² === nothing ? nothing : similar(Î²)
+        if affine === nothing
+            check(ccall((:luxhip_layernorm_bwd, libluxhip), Cint, LnBwdSig,
+                stream(), dtype_code(T), id, L, R, optr(Î”), optr(x), optr(Î³), optr(Î²), optr(Î¼s), optr(is), optr(âˆ‚x), optr(âˆ‚Î³),
+                optr(âˆ‚Î²))) || error(last_error())
+        else
+            # second pass first: âˆ‚xÌ‚ and the parameter gradients from the per-channel pullback, then the normalisation's
+            I, C, Nn = size(xÌ‚)
+            âˆ‚xÌ‚ = similar(xÌ‚)
+            check(ccall((:luxhip_batchnorm_bwd, libluxhip), Cint,
+                (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Cint,
+                    Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+                stream(), dtype_code(T), id, I, C, Nn, optr(Î”), optr(xÌ‚), optr(Î³), optr(Î²), optr(affine[1]), optr(affine[2]), Cint(0),
+                optr(âˆ‚xÌ‚), optr(âˆ‚Î³), optr(âˆ‚Î²))) || error(last_error())
+            check(ccall((:luxhip_layernorm_bwd, libluxhip), Cint, LnBwdSig,
+                stream(), dtype_code(T), Cint(0), L, R, optr(âˆ‚xÌ‚), optr(x), C_NULL, C_NULL, optr(Î¼s), optr(is), optr(âˆ‚x), C_NULL,
+                C_NULL)) || error(last_error())
+        end
+        return nt, âˆ‚x, something(âˆ‚Î³, nt), something(âˆ‚Î², nt), nt, nt, nt
+    end
+    return y, âˆ‡layernorm_hip
+end
 
 # ---------------------------------------------------------------------------------------------
 # conv: Impl.conv!, Impl.âˆ‡conv_data, Impl.âˆ‡conv_filter, Impl.conv_bias_act  (impl/conv.jl:29-166)
@@ -280,29 +482,60 @@ function Impl.conv_bias_act(::Type{LuxHIPDevice}, x::HIPArray{T,4}, w::HIPArray{
     ok = id !== nothing && check(ccall((:luxhip_conv_fwd, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
         stream(), dtype_code(T), id, d, optr(x), optr(w), optr(bias), optr(y), C_NULL, C_NULL))
-    ok || return invoke(Impl.conv_bias_act, Tuple{Type,Any,Any,Any,Any,Any}, Nothing, x, w, cdims, bias, act)
+    ok || throw(HIPFallbackError("conv_bias_act with activation $(act)"))
     return y
 end
 function Impl.conv!(y::HIPArray{T,4}, ::Type{LuxHIPDevice}, x::HIPArray{T,4}, w::HIPArray{T,4}, cdims::DenseConvDims{2}) where {T<:HIPFloat}
     d = Ref(ConvDimsC(cdims, size(x, 4)))
     check(ccall((:luxhip_conv_fwd, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), Cint(0), d, optr(x), optr(w), C_NULL, optr(y), C_NULL, C_NULL)) || NNlib.conv!(y, x, w, cdims)
+        stream(), dtype_code(T), Cint(0), d, optr(x), optr(w), C_NULL, optr(y), C_NULL, C_NULL)) || throw(HIPFallbackError("conv!"))
     return nothing
 end
 function Impl.âˆ‡conv_data(dy::HIPArray{T,4}, w::HIPArray{T,4}, cdims::DenseConvDims{2}) where {T<:HIPFloat}
     dx = similar(dy, T, (NNlib.input_size(cdims)..., NNlib.channels_in(cdims), size(dy, 4)))
     d = Ref(ConvDimsC(cdims, size(dy, 4)))
     check(ccall((:luxhip_conv_bwd_data, libluxhip), Cint, (Ptr{Cvoid}, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), d, optr(dy), optr(w), optr(dx))) || return NNlib.âˆ‡conv_data(dy, w, cdims)
+        stream(), dtype_code(T), d, optr(dy), optr(w), optr(dx))) || throw(HIPFallbackError("âˆ‡conv_data"))
     return dx
 end
 function Impl.âˆ‡conv_filter(x::HIPArray{T,4}, dy::HIPArray{T,4}, cdims::DenseConvDims{2}) where {T<:HIPFloat}
     dw = similar(x, T, (NNlib.kernel_size(cdims)..., NNlib.channels_in(cdims) Ã· NNlib.groupcount(cdims), NNlib.channels_out(cdims)))
     d = Ref(ConvDimsC(cdims, size(x, 4)))
     check(ccall((:luxhip_conv_bwd_filter, libluxhip), Cint, (Ptr{Cvoid}, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), d, optr(x), optr(dy), optr(dw))) || return NNlib.âˆ‡conv_filter(x, dy, cdims)
+        stream(), dtype_code(T), d, optr(x), optr(dy), optr(dw))) || throw(HIPFallbackError("âˆ‡conv_filter"))
     return dw
+end
+
+# CRC.rrule(fused_conv) + âˆ‡fused_conv (impl/conv.jl:204-275) as one forward and one pullback call.  The forward
+# pass hands over the channel-contiguous copy of x that its kernels read (xt_keep); the pullback's filter
+# gradient reads it instead of transposing x again.
+function CRC.rrule(::CRC.RuleConfig{>:CRC.HasReverseMode}, ::typeof(Impl.fused_conv), ::HIPOp, act::F, w::HIPArray{T,4}, x::HIPArray{T,4},
+        bias::Union{Nothing,HIPArray{T,1}}, cdims::DenseConvDims{2}) where {F,T<:HIPFloat}
+    id = act_id(act)
+    id === nothing && throw(HIPFallbackError("the pullback of fused_conv with activation $(act)"))
+    y = similar(x, T, (NNlib.output_size(cdims)..., NNlib.channels_out(cdims), size(x, 4)))
+    pre = id in (4, 5, 6, 7, 8) ? similar(y) : nothing
+    xt = similar(x)
+    d = Ref(ConvDimsC(cdims, size(x, 4)))
+    check(ccall((:luxhip_conv_fwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), id, d, optr(x), optr(w), optr(bias), optr(y), optr(pre), optr(xt))) || throw(HIPFallbackError("fused_conv"))
+    ð’«w, ð’«x, ð’«b = ProjectTo(w), ProjectTo(x), ProjectTo(bias)
+    function âˆ‡fused_conv_hip(Î”â€²)
+        Î” = CRC.unthunk(Î”â€²)
+        âˆ‚w, âˆ‚x = similar(w), similar(x)
+        âˆ‚b = bias === nothing ? nothing : similar(bias)
+        dz = id == 0 ? nothing : similar(y)
+        check(ccall((:luxhip_fused_conv_bwd, libluxhip), Cint,
+            (Ptr{Cvoid}, Cint, Cint, Ptr{ConvDimsC}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
+                Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
+            stream(), dtype_code(T), id, d, optr(Î”), optr(y), optr(pre), optr(x), optr(w), optr(dz), optr(âˆ‚w), optr(âˆ‚x), optr(âˆ‚b),
+            optr(xt))) || error(last_error())
+        nt = NoTangent()
+        return nt, nt, nt, nt, ð’«w(âˆ‚w), ð’«x(âˆ‚x), bias === nothing ? nt : ð’«b(âˆ‚b), nt
+    end
+    return y, âˆ‡fused_conv_hip
 end
 
 # Three spatial dims (x (W, H, D, C, N), DenseConvDims{3}): the two-dimensional problem on the
@@ -368,6 +601,18 @@ function Impl.âˆ‡conv_filter(x::HIPArray{T,5}, dy::HIPArray{T,5}, cdims::DenseCo
         NNlib.channels_in(cdims) Ã· NNlib.groupcount(cdims), NNlib.channels_out(cdims))
 end
 
+function CRC.rrule(cfg::CRC.RuleConfig{>:CRC.HasReverseMode}, ::typeof(Impl.fused_conv), op::HIPOp, act::F, w::HIPArray{T,5},
+        x::HIPArray{T,5}, bias::Union{Nothing,HIPArray{T,1}}, cdims::DenseConvDims{3}) where {F,T<:HIPFloat}
+    xu, c2 = depth_unfold(x, cdims)
+    y2, back2 = CRC.rrule(cfg, Impl.fused_conv, op, act, w2d(w), xu, bias, c2)
+    N = size(x, 5)
+    function âˆ‡fused_conv3d_hip(Î”â€²)
+        _, _, _, _, âˆ‚w2, âˆ‚xu, âˆ‚b, _ = back2(to_inner(CRC.unthunk(Î”â€²), cdims))
+        return NoTangent(), NoTangent(), NoTangent(), NoTangent(), reshape(âˆ‚w2, size(w)), depth_fold(âˆ‚xu, cdims, N), âˆ‚b, NoTangent()
+    end
+    return from_inner(y2, cdims, N), âˆ‡fused_conv3d_hip
+end
+
 # ---------------------------------------------------------------------------------------------
 # batched_matmul: Impl.batched_matmul!(z, opmode, x, y)  (impl/batched_mul.jl:204-212) and the
 # products of the rrule (:320-334), which arrive as NNlib.BatchedAdjoint wrappers
@@ -384,7 +629,7 @@ function Impl.batched_matmul!(z::HIPArray{T,3}, ::HIPOp, x::AbstractArray{T,3}, 
         (Ptr{Cvoid}, Cint, Cint, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Int64, Int64, Ptr{Cvoid}, Int64, Int64,
          Ptr{Cvoid}, Int64, Int64),
         stream(), dtype_code(T), tx, ty, M, N, K, B, optr(xp), max(1, size(xp, 1)), bstride(xp), optr(yp), max(1, size(yp, 1)),
-        bstride(yp), optr(z), max(1, M), M * N)) || NNlib.batched_mul!(z, x, y)
+        bstride(yp), optr(z), max(1, M), M * N)) || throw(HIPFallbackError("batched_matmul!"))
     return nothing
 end
 
@@ -392,7 +637,7 @@ end
 function batch_sum(tmp::HIPArray{T,3}) where {T<:HIPFloat}
     out = similar(tmp, T, (size(tmp, 1), size(tmp, 2), 1))
     check(ccall((:luxhip_batch_sum, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), size(tmp, 1) * size(tmp, 2), size(tmp, 3), optr(tmp), optr(out))) || return sum(tmp; dims=3)
+        stream(), dtype_code(T), size(tmp, 1) * size(tmp, 2), size(tmp, 3), optr(tmp), optr(out))) || throw(HIPFallbackError("sum over the batch dim"))
     return out
 end
 
@@ -414,7 +659,7 @@ end
 
 function Impl.generate_dropout_mask!(y::HIPArray{T}, ::HIPOp, p, invp) where {T<:HIPFloat}
     check(ccall((:luxhip_dropout_mask, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, Cdouble, Cdouble, Ptr{Cvoid}),
-        stream(), dtype_code(T), length(y), Float64(p), Float64(invp), optr(y))) || (y .= (y .> T(p)) .* T(invp))
+        stream(), dtype_code(T), length(y), Float64(p), Float64(invp), optr(y))) || throw(HIPFallbackError("generate_dropout_mask!"))
     return nothing
 end
 
@@ -423,7 +668,7 @@ function Impl.dropout_dot_mul(x::HIPArray{T,N}, mask::HIPArray{T,N}) where {T<:H
     xs, ms = Int64[size(x)...], Int64[size(mask)...]
     check(ccall((:luxhip_dropout_mul, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), N, xs, ms, optr(x), optr(mask), optr(y))) || return x .* mask
+        stream(), dtype_code(T), N, xs, ms, optr(x), optr(mask), optr(y))) || throw(HIPFallbackError("dropout_dot_mul"))
     return y
 end
 
@@ -445,7 +690,7 @@ function Impl.alpha_dropout(::HIPOp, noise::HIPArray{T}, p, x::HIPArray{T}, Î±, 
     check(ccall((:luxhip_alpha_dropout_fwd, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Int64, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Cdouble, Cdouble, Cdouble, Ptr{Cvoid}),
         stream(), dtype_code(T), length(x), optr(noise), Float64(p), optr(x), Float64(Î±), Float64(A), Float64(B), optr(y))) ||
-        return @. muladd(ifelse(noise > p, x, T(Î±)), T(A), T(B))
+        throw(HIPFallbackError("alpha_dropout"))
     return y
 end
 function CRC.rrule(::typeof(Impl.alpha_dropout), op::HIPOp, noise::HIPArray{T}, p, x::HIPArray{T}, Î±, A, B) where {T<:HIPFloat}
@@ -456,30 +701,166 @@ function CRC.rrule(::typeof(Impl.alpha_dropout), op::HIPOp, noise::HIPArray{T}, 
         check(ccall((:luxhip_alpha_dropout_bwd, libluxhip), Cint,
             (Ptr{Cvoid}, Cint, Int64, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}),
             stream(), dtype_code(T), length(x), optr(noise), Float64(p), optr(Î”), Float64(A), optr(âˆ‚x))) ||
-            (âˆ‚x = Î” .* (noise .> p) .* T(A))
+            throw(HIPFallbackError("the pullback of alpha_dropout"))
         return (ntuple(Returns(NoTangent()), 4)..., âˆ‚x, ntuple(Returns(NoTangent()), 3)...)
     end
     return y, âˆ‡alpha_dropout_hip
 end
 
-# instancenorm (impl/normalization.jl:191-208) is Impl.groupnorm with G = C, followed in training
-# with running statistics by luxhip_instancenorm_running_stats on the saved (C, N) statistics;
-# scaled_dot_product_attention (impl/attention.jl:70-117) is two luxhip_batched_matmul_strided
-# calls around luxhip_attention_softmax_fwd, its rrule four products around
-# luxhip_attention_softmax_bwd.  (lux.jl_amd/luxlib.py: rrule_instancenorm,
-# rrule_scaled_dot_product_attention spell out the strides.)
-#
-# The same file holds the host side of what the hooks above do not cover one to one:
-#   * layernorm over 1:k with parameters that do not span exactly those dims (dims = Colon() with
-#     (1, 1, C, 1) parameters, dims = nothing): luxhip_layernorm_fwd without Î³, Î², then the per-channel
-#     affine transform and activation as luxhip_batchnorm_fwd in inference mode (mean 0, variance 1,
-#     Îµ = 0) on the (I, C, N) view; the pullback runs the two in reverse (_layernorm_fwd);
-#   * attention operands whose embedding dim is not the first: luxhip_permute_leading3 before, and on
-#     âˆ‚q, âˆ‚k, âˆ‚v after; `fdrop` between the softmax and the second product (attention_dropout);
-#   * batched_matmul with lhs_batching_dims / rhs_batching_dims anywhere and partly repeated operands:
-#     the arrays' own strides go to luxhip_batched_matmul_strided, no permutedims / repeat
-#     (_rrule_batched_matmul_general);
-#   * operands of mixed element types in fused_dense / fused_conv: luxhip_convert to the widest type
-#     first (the reference's own rule, ext/CUDAExt/cublaslt.jl:46-63), gradients converted back (_promote).
+# ---------------------------------------------------------------------------------------------
+# scaled_dot_product_attention (impl/attention.jl:5-117): two strided batched products around the fused
+# scale / mask / bias / softmax pass; grouped key/value heads are addressed with a stride of 0 along the
+# repeat (no repeat_inner_gqa copy); a causal mask is passed to the products as a triangular structure.
+# Covers head_dim = 1 (embedding dim first) with the token dim in position 2 or 3; other placements are
+# brought there with luxhip_permute_leading3 and the gradients taken back.
+# ---------------------------------------------------------------------------------------------
+struct AttnLayout
+    E::Int; tokens::Int; heads::Int; st::Int; sh::Int; sb::Int; batch::Int
+end
+function AttnLayout(a::HIPArray, token_dim::Int)
+    E, d2, d3 = size(a, 1), size(a, 2), size(a, 3)
+    tokens, heads = token_dim == 2 ? (d2, d3) : (d3, d2)
+    st, sh = token_dim == 2 ? (E, E * d2) : (E * d2, E)
+    sb = E * d2 * d3
+    return AttnLayout(E, tokens, heads, st, sh, sb, sb == 0 ? 0 : length(a) Ã· sb)
+end
+i64x3(t) = Int64[t[1], t[2], t[3]]
+
+function bmm_strided!(C::HIPArray{T}, tA::Bool, tB::Bool, M, N, K, bdims, A::HIPArray{T}, lda, sA, B::HIPArray{T}, ldb, sB, ldc, sC,
+        structure::Integer) where {T<:HIPFloat}
+    check(ccall((:luxhip_batched_matmul_strided, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Cint, Cint, Int64, Int64, Int64, Ptr{Int64}, Ptr{Cvoid}, Int64, Ptr{Int64}, Ptr{Cvoid}, Int64, Ptr{Int64},
+            Ptr{Cvoid}, Int64, Ptr{Int64}, Cint),
+        stream(), dtype_code(T), Cint(tA), Cint(tB), M, N, K, i64x3(bdims), optr(A), max(1, lda), i64x3(sA), optr(B), max(1, ldb),
+        i64x3(sB), optr(C), max(1, ldc), i64x3(sC), Cint(structure))) || throw(HIPFallbackError("batched_matmul"))
+    return C
+end
+
+function permute_leading3(a::HIPArray{T,N}, perm::NTuple{3,Int}) where {T<:HIPFloat,N}
+    out = similar(a, T, (size(a, perm[1]), size(a, perm[2]), size(a, perm[3]), size(a)[4:N]...))
+    check(ccall((:luxhip_permute_leading3, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Cint, Cint, Cint, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), size(a, 1), size(a, 2), size(a, 3), prod(size(a)[4:N]; init=1), Cint(perm[1]), Cint(perm[2]),
+        Cint(perm[3]), optr(a), optr(out))) || throw(HIPFallbackError("permutedims"))
+    return out
+end
+
+# mask: HIPArray{UInt8} or nothing; bias: HIPArray{T} or nothing; both [S, L, H or 1, B or 1]
+function side_strides(a, S, L, H, B)
+    a === nothing && return 0, 0
+    s3 = ndims(a) â‰¥ 3 ? size(a, 3) : 1
+    s4 = ndims(a) â‰¥ 4 ? prod(size(a)[4:end]) : 1
+    (size(a, 1) == S && size(a, 2) == L && s3 in (1, H) && s4 in (1, B)) ||
+        throw(DimensionMismatch("mask / bias of size $(size(a)) does not broadcast to the logits $((S, L, H, B))"))
+    return (s3 == H && H > 1 ? S * L : 0), (s4 == B && B > 1 ? S * L * s3 : 0)
+end
+
+function attention_device(q::HIPArray{T,N}, k::HIPArray{T,N}, v::HIPArray{T,N}, token_dim::Int, scale, mask, causal::Bool, bias,
+        fdrop::F) where {T<:HIPFloat,N,F}
+    lq, lk, lv = AttnLayout(q, token_dim), AttnLayout(k, token_dim), AttnLayout(v, token_dim)
+    E, Ev, H, G, L, S, B = lq.E, lv.E, lq.heads, lk.heads, lq.tokens, lk.tokens, lq.batch
+    r = G == 0 ? 1 : H Ã· G
+    bshape = size(q)[4:N]
+    scaleâ»Â¹ = 1 / (scale === nothing ? sqrt(Float64(E)) : Float64(scale))                  # impl/attention.jl:50-51
+    bdims = (r, G, B)
+    mask_sh, mask_sb = side_strides(mask, S, L, H, B)
+    bias_sh, bias_sb = side_strides(bias, S, L, H, B)
+    sC = (S * L, S * L * r, S * L * H)
+    sq = (lq.sh, lq.sh * r, lq.sb)
+    tri = causal && fdrop === identity        # an arbitrary fdrop need not keep the masked weights at zero
+    logits = similar(q, T, (S, L, H, bshape...))
+    bmm_strided!(logits, true, false, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, sq, S, sC, causal ? 1 : 0)
+    softmaxed = similar(logits)
+    check(ccall((:luxhip_attention_softmax_fwd, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Cdouble, Cint, Ptr{UInt8}, Int64, Int64, Ptr{Cvoid}, Int64, Int64,
+            Ptr{Cvoid}),
+        stream(), dtype_code(T), S, L, H, B, optr(logits), scaleâ»Â¹, Cint(causal), mask === nothing ? Ptr{UInt8}(C_NULL) : Ptr{UInt8}(pointer(mask)),
+        mask_sh, mask_sb, optr(bias), bias_sh, bias_sb, optr(softmaxed))) || throw(HIPFallbackError("softmax of the attention logits"))
+    probs, fdrop_back = fdrop === identity ? (softmaxed, nothing) : CRC.rrule_via_ad(ZygoteLikeConfig(), fdrop, softmaxed)
+    out = similar(q, T, (Ev, H, L, bshape...))
+    so = (Ev, Ev * r, Ev * H * L)
+    bmm_strided!(out, false, false, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, Ev * H, so, tri ? 2 : 0)
+    saved = (; lq, lk, lv, r, bdims, sC, sq, so, scaleâ»Â¹, tri, logits, softmaxed, probs, fdrop_back)
+    return out, probs, saved
+end
+# the rule configuration `fdrop`'s own pullback is taken with: whatever AD engine drives LuxLib supplies it
+struct ZygoteLikeConfig <: CRC.RuleConfig{Union{CRC.HasReverseMode,CRC.NoForwardsMode}} end
+
+function attention_canonical(f, q::HIPArray{T,N}, k, v, head_dim::Int, token_dim::Int) where {T,N}
+    head_dim == 1 && return f(q, k, v, token_dim, identity)
+    heads_dim = only(setdiff(1:3, (head_dim, token_dim)))
+    perm = (head_dim, heads_dim, token_dim)
+    inv = ntuple(d -> findfirst(==(d), perm), 3)
+    return f(permute_leading3(q, perm), permute_leading3(k, perm), permute_leading3(v, perm), 3, g -> permute_leading3(g, inv))
+end
+
+function attention_checks(q::HIPArray{T,N}, k, v, head_dim, token_dim, mask, is_causal) where {T,N}
+    # impl/attention.jl:16-43
+    @assert N â‰¥ 4 "N must be at least 4"
+    @assert 1 â‰¤ head_dim â‰¤ 3 && 1 â‰¤ token_dim â‰¤ 3 && head_dim â‰  token_dim "head_dim and token_dim must differ, in 1:3"
+    @assert size(q, head_dim) == size(k, head_dim) "`q` and `k` must have the same number of heads."
+    for i in 4:N
+        (size(q, i) == size(k, i) == size(v, i)) || throw(DimensionMismatch("All dimensions (except first 3) of q, k, v must be the same."))
+    end
+    @assert !(mask !== nothing && is_causal isa Bool) "`mask` and `is_causal` cannot both be specified"
+    return nothing
+end
+
+function Impl.scaled_dot_product_attention(q::HIPArray{T,N}, k::HIPArray{T,N}, v::HIPArray{T,N}; head_dim::Int=1, token_dim::Int=3,
+        scale=nothing, mask=nothing, is_causal::Union{Bool,Nothing}=nothing, bias=nothing, fdrop::F=identity) where {T<:HIPFloat,N,F}
+    attention_checks(q, k, v, head_dim, token_dim, mask, is_causal)
+    return attention_canonical(q, k, v, head_dim, token_dim) do qc, kc, vc, td, _
+        out, probs, _ = attention_device(qc, kc, vc, td, scale, mask, is_causal === true, bias, fdrop)
+        return out, probs
+    end
+end
+
+function CRC.rrule(::typeof(Impl.scaled_dot_product_attention), q::HIPArray{T,N}, k::HIPArray{T,N}, v::HIPArray{T,N}; head_dim::Int=1,
+        token_dim::Int=3, scale=nothing, mask=nothing, is_causal::Union{Bool,Nothing}=nothing, bias=nothing, fdrop::F=identity) where {T<:HIPFloat,N,F}
+    attention_checks(q, k, v, head_dim, token_dim, mask, is_causal)
+    return attention_canonical(q, k, v, head_dim, token_dim) do qc, kc, vc, td, back_perm
+        out, probs, s = attention_device(qc, kc, vc, td, scale, mask, is_causal === true, bias, fdrop)
+        (; lq, lk, lv, r, bdims, sC, sq, so, tri) = s
+        E, Ev, H, L, S = lq.E, lv.E, lq.heads, lq.tokens, lk.tokens
+        function âˆ‡attention_hip(Î”â€²)
+            Î” = CRC.unthunk(Î”â€²)
+            Î”out = CRC.unthunk(Î”[1])
+            Î”[2] isa CRC.AbstractZero || throw(HIPFallbackError("a cotangent for the returned attention weights"))
+            dp = similar(probs)
+            bmm_strided!(dp, true, false, S, L, Ev, bdims, vc, lv.st, (0, lv.sh, lv.sb), Î”out, Ev * H, so, S, sC, tri ? 1 : 0)
+            s.fdrop_back === nothing || (dp = CRC.unthunk(s.fdrop_back(dp)[2]))
+            dlogits = s.logits                                   # no longer needed
+            # tri, not is_causal: with an fdrop the products below run in full and read the whole cotangent
+            check(ccall((:luxhip_attention_softmax_bwd, libluxhip), Cint,
+                (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}),
+                stream(), dtype_code(T), S, L, L * H * lq.batch, Cint(tri), optr(dp), optr(s.softmaxed), s.scaleâ»Â¹, optr(dlogits))) ||
+                error(last_error())
+            âˆ‚q = similar(qc)
+            bmm_strided!(âˆ‚q, false, false, E, L, S, bdims, kc, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, lq.st, sq, tri ? 2 : 0)
+            function kv_grad(like, lay, A, lda, sA, Bm)
+                full = r > 1 ? similar(like, T, (r, size(like)...)) : similar(like)
+                bmm_strided!(full, false, true, lay.E, S, L, bdims, A, lda, sA, Bm, S, sC, lay.st,
+                    (r > 1 ? length(like) : 0, lay.sh, lay.sb), tri ? 3 : 0)
+                r == 1 && return full
+                red = similar(like)                               # pullback of repeat_inner_gqa: sum over the heads of a group
+                check(ccall((:luxhip_batch_sum, libluxhip), Cint, (Ptr{Cvoid}, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}),
+                    stream(), dtype_code(T), length(like), r, optr(full), optr(red))) || error(last_error())
+                return red
+            end
+            âˆ‚v = kv_grad(vc, lv, Î”out, Ev * H, so, probs)
+            âˆ‚k = kv_grad(kc, lk, qc, lq.st, sq, dlogits)
+            return NoTangent(), back_perm(âˆ‚q), back_perm(âˆ‚k), back_perm(âˆ‚v)
+        end
+        return (out, probs), âˆ‡attention_hip
+    end
+end
+
+# Host-side compositions that the Python mirror (lux.jl_amd/luxlib.py) has and this file does not repeat:
+#   * layernorm parameters with gaps between the dims they vary along ((3, 1, 3) against a 4-d x): repeated
+#     along the gaps first, gradients summed back (_expand_parameters); here they raise HIPFallbackError;
+#   * batched_matmul with lhs_batching_dims / rhs_batching_dims anywhere and partly repeated operands: the
+#     arrays' own strides go to luxhip_batched_matmul_strided (_rrule_batched_matmul_general);
+#   * operands of mixed element types in fused_dense / fused_conv: luxhip_convert to the widest type first
+#     (the reference's own rule, ext/CUDAExt/cublaslt.jl:46-63), gradients converted back (_promote).
 
 end # module
