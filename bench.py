@@ -152,15 +152,30 @@ class C2BatchnormBiasAct(Workload):
         self.step()
 
     def isolated_ops(self):
-        """kernel name -> call that launches exactly that kernel (default library options)."""
+        """kernel name -> call that launches exactly that kernel (default library options); successive calls go
+        through the sets of tensors in turn, like rotating_step()."""
         names = ["bn_fwd_resident_kernel", "bias_act_fwd_kernel", "bias_act_bwd_channel_kernel", "bn_bwd_resident_kernel"]
-        return {n: (lambda c=c: c[0](*c[1])) for n, c in zip(names, self.calls)}
+        turn = [0]
+
+        def one(i):
+            def call():
+                turn[0] = (turn[0] + 1) % len(self.sets)
+                fn, args = self.sets[turn[0]][1][i]
+                if fn(*args) != 0:
+                    raise RuntimeError(self.lux._lib.last_error())
+            return call
+        return {n: one(i) for i, n in enumerate(names)}
 
     def step_fused(self):
         for fn, args in self.fused_calls:
             rc = fn(*args)
             if rc != 0:
                 raise RuntimeError(self.lux._lib.last_error())
+
+    def rotating_step_fused(self):
+        self.turn = (self.turn + 1) % len(self.sets)
+        self.fused_calls = self.sets[self.turn][2]
+        self.step_fused()
 
     @property
     def E(self):
@@ -270,6 +285,24 @@ class C1Dense(_ApiWorkload):
     def kernel_work(self):
         return {"dense_gemm_kernel<f32>": 2.0 * 256 * 128 * 64}
 
+    def cpu_baseline(self, budget_s: float):
+        """The reference's CPU path for this op is `matmuladd` through BLAS + a fused bias/activation loop and, in
+        the pullback, two BLAS products with a transposed operand (impl/dense.jl:71-113): the same calls in numpy."""
+        rng = np.random.default_rng(1000)
+        lim = np.sqrt(6.0 / 384.0)
+        W = rng.uniform(-lim, lim, size=(256, 128)).astype(np.float32)
+        x = rng.standard_normal(size=(128, 64)).astype(np.float32)
+        b = (0.01 * rng.standard_normal(256)).astype(np.float32)
+        delta = rng.standard_normal(size=(256, 64)).astype(np.float32)
+
+        def cpu_step():
+            y = np.tanh(W @ x + b[:, None])
+            dz = delta * (1.0 - y * y)
+            return dz @ x.T, W.T @ dz, dz.sum(axis=1)
+
+        return _time_cpu(cpu_step, budget_s, self.work_per_step(), 1e12, "TFLOP/s", blas_threads(), "port",
+                         "full-size steps in numpy fp32 (BLAS products + elementwise loops, the structure of LuxLib's CPU path)")
+
 
 class C3Groupnorm(_ApiWorkload):
     """benchmark configuration 3: groupnorm(32 groups) + swish, x 64x64x256x16."""
@@ -301,6 +334,36 @@ class C3Groupnorm(_ApiWorkload):
 
     def kernel_work(self):
         return {"gn_fwd_kernel": 2 * self.E, "gn_bwd_kernel": 3 * self.E}
+
+    def cpu_baseline(self, budget_s: float):
+        path = os.path.join(ROOT, "oracle", "libluxcpu.so")
+        if not os.path.exists(path):
+            return None
+        cpu = C.CDLL(path)
+        rng = np.random.default_rng(1002)
+        fa = lambda a: np.asfortranarray(a, dtype=np.float32)
+        x = fa(rng.standard_normal(size=self.shape, dtype=np.float32))
+        g = rng.uniform(0.8, 1.2, 256).astype(np.float32)
+        b = (0.05 * rng.standard_normal(256)).astype(np.float32)
+        delta = fa(rng.standard_normal(size=self.shape, dtype=np.float32))
+        W, H, Cc, N = self.shape
+        G = self.groups
+        y, dx = np.empty(self.shape, np.float32, order="F"), np.empty(self.shape, np.float32, order="F")
+        mean, var = np.empty(G * N, np.float32), np.empty(G * N, np.float32)
+        dg, db = np.empty(Cc, np.float32), np.empty(Cc, np.float32)
+        ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+        i64 = C.c_int64
+
+        def cpu_step():
+            cpu.luxcpu_groupnorm_fwd(4, i64(W * H), i64(Cc // G), i64(G), i64(N), ptr(x), ptr(g), ptr(b), C.c_float(1e-5), ptr(y),
+                                     ptr(mean), ptr(var))
+            cpu.luxcpu_groupnorm_bwd(4, i64(W * H), i64(Cc // G), i64(G), i64(N), ptr(delta), ptr(x), ptr(g), ptr(b), ptr(mean),
+                                     ptr(var), C.c_float(1e-5), ptr(dx), ptr(dg), ptr(db))
+
+        E32 = int(np.prod(self.shape)) * 4
+        return _time_cpu(cpu_step, budget_s, 5 * E32, 1e9, "GB/s", 1, "port",
+                         "full-size fp32 steps of the C port of LuxLib's groupnorm CPU loops (serial @simd loops in the reference, "
+                         "one thread here; the bf16 workload has no CPU counterpart in LuxLib and is compared with the same fp32 figure)")
 
 
 class C4TransformerMLP(_ApiWorkload):
@@ -337,6 +400,43 @@ class C4TransformerMLP(_ApiWorkload):
 
     def kernel_work(self):
         return {"dense_gemm_kernel<bf16>": 2.0 * self.D * self.F * self.Ntok}
+
+    def cpu_baseline(self, budget_s: float):
+        """LuxLib's CPU path in fp32 (it has no bf16 code): layernorm as mean/var + broadcasts, dense layers as
+        BLAS products + bias/activation loops, the pullbacks as the rrules compose them, on 1/8 of the tokens."""
+        rng = np.random.default_rng(1003)
+        D, F, N = self.D, self.F, self.Ntok // 8
+        std = np.sqrt(2.0 / (D + F))
+        x = rng.standard_normal(size=(D, N), dtype=np.float32)
+        g = rng.uniform(0.5, 1.5, (D, 1)).astype(np.float32)
+        b = (0.1 * rng.standard_normal((D, 1))).astype(np.float32)
+        W1 = std * rng.standard_normal(size=(F, D), dtype=np.float32)
+        W2 = std * rng.standard_normal(size=(D, F), dtype=np.float32)
+        b1, b2 = np.zeros((F, 1), np.float32), np.zeros((D, 1), np.float32)
+        delta = 0.02 * rng.standard_normal(size=(D, N), dtype=np.float32)
+        c0, c1 = np.float32(0.7978845608028654), np.float32(0.044715)
+
+        def cpu_step():
+            mu = x.mean(axis=0, keepdims=True)
+            var = x.var(axis=0, keepdims=True)
+            inv = 1.0 / np.sqrt(var + np.float32(1e-5))
+            xh = (x - mu) * inv
+            h0 = xh * g + b
+            z1 = W1 @ h0 + b1
+            t = np.tanh(c0 * (z1 + c1 * z1 ** 3))
+            h1 = 0.5 * z1 * (1.0 + t)
+            h2 = W2 @ h1 + b2
+            dW2, dh1, db2 = delta @ h1.T, W2.T @ delta, delta.sum(axis=1)
+            dz1 = dh1 * (0.5 * (1.0 + t) + 0.5 * z1 * (1.0 - t * t) * c0 * (1.0 + 3.0 * c1 * z1 * z1))
+            dW1, dh0, db1 = dz1 @ h0.T, W1.T @ dz1, dz1.sum(axis=1)
+            dg, dbeta = (dh0 * xh).sum(axis=1), dh0.sum(axis=1)
+            gd = dh0 * g
+            dx = (gd - gd.mean(axis=0, keepdims=True) - xh * (gd * xh).mean(axis=0, keepdims=True)) * inv
+            return h2, dW2, db2, dW1, db1, dg, dbeta, dx
+
+        return _time_cpu(cpu_step, budget_s, self.work_per_step() / 8, 1e12, "TFLOP/s", blas_threads(), "port",
+                         f"steps of the same block on {N} of the {self.Ntok} tokens, numpy fp32 (BLAS products + elementwise "
+                         "passes, the structure of LuxLib's CPU path, which has no bf16 code); GEMM flops counted as on the GPU")
 
     def kernel_bytes(self):
         """HBM-bound kernels of this workload: name -> algorithmic bytes of one launch."""
@@ -375,6 +475,44 @@ class C5Conv(_ApiWorkload):
         f = 2.0 * (56 * 56 * 64) * 128 * 1152
         t = "bf16" if self.dtype == "bf16" else "f32"
         return {f"conv_fprop_kernel<{t}>": f, f"conv_dgrad_kernel<{t}>": f, f"conv_wgrad_kernel<{t}>": f}
+
+    def cpu_baseline(self, budget_s: float):
+        """NNlib's CPU convolution is im2col + GEMM per image (threaded over the batch); LuxLib adds the bias /
+        activation loop and, in the pullback, the activation gradient, the bias sum and the two NNlib gradients:
+        the same steps in numpy fp32 on 8 of the 64 images."""
+        rng = np.random.default_rng(1004)
+        N = 8
+        x = rng.standard_normal(size=(N, 128, 56, 56), dtype=np.float32)                  # image-major for the host loops
+        w = (np.sqrt(2.0 / 1152) * rng.standard_normal(size=(128, 128, 3, 3), dtype=np.float32))
+        b = (0.01 * rng.standard_normal(128)).astype(np.float32)
+        delta = rng.standard_normal(size=(N, 128, 56, 56), dtype=np.float32)
+        wm = np.ascontiguousarray(w[:, :, ::-1, ::-1].reshape(128, 1152))                  # true convolution: flipped taps
+        from numpy.lib.stride_tricks import sliding_window_view
+
+        def im2col(a):                                                                     # (C, 56, 56) -> (C*9, 3136), pad 1
+            p = np.pad(a, ((0, 0), (1, 1), (1, 1)))
+            return np.ascontiguousarray(sliding_window_view(p, (3, 3), axis=(1, 2)).transpose(0, 3, 4, 1, 2)).reshape(1152, 3136)
+
+        def cpu_step():
+            dw = np.zeros((128, 1152), np.float32)
+            db = np.zeros(128, np.float32)
+            for n in range(N):
+                col = im2col(x[n])
+                y = np.maximum(wm @ col + b[:, None], 0.0)
+                dz = delta[n].reshape(128, 3136) * (y > 0)
+                db += dz.sum(axis=1)
+                dw += dz @ col.T
+                dcol = wm.T @ dz                                                           # (1152, 3136): col2im
+                d = dcol.reshape(128, 3, 3, 56, 56)
+                dx = np.zeros((128, 58, 58), np.float32)
+                for p in range(3):
+                    for q in range(3):
+                        dx[:, p:p + 56, q:q + 56] += d[:, p, q]
+            return dw, db
+
+        return _time_cpu(cpu_step, budget_s, self.work_per_step() * N / 64, 1e12, "TFLOP/s", blas_threads(), "port",
+                         f"steps on {N} of the 64 images, numpy fp32: im2col + BLAS product per image (NNlib's CPU algorithm), "
+                         "bias/relu loop, pullback with col2im; the bf16 workload is compared with the same fp32 figure")
 
 
 class Conv3d(_ApiWorkload):
@@ -486,6 +624,30 @@ WORKLOADS = {"IN": InstanceNorm, "DROPOUT": Dropout, "SDPA": Attention, "C1": C1
              "CONV3D": lambda: Conv3d("bf16"), "CONV3Df32": lambda: Conv3d("f32")}
 
 
+# ----------------------------------------------------------------------------- CPU baselines
+def blas_threads() -> int:
+    try:
+        from threadpoolctl import threadpool_info
+        n = [p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"]
+        return int(max(n)) if n else 1
+    except Exception:
+        return int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+
+
+def _time_cpu(step, budget_s, work, scale, unit, cores, kind, sample):
+    step()                                  # warm-up / page-in
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        step()
+        n += 1
+        if time.perf_counter() - t0 > budget_s or n >= 2000:
+            break
+    dt = (time.perf_counter() - t0) / n
+    return {"value": work / dt / scale, "unit": unit, "cores": cores, "kind": kind, "ms_per_step": dt * 1e3,
+            "sample": f"{n} {sample}"}
+
+
 # ----------------------------------------------------------------------------- timing
 def timed(lux, fn, steps, warmup):
     for _ in range(warmup):
@@ -557,57 +719,53 @@ def kernel_profile(lux, fn, steps):
     return json.loads(buf.value.decode())
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None)
-    ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline (0 disables it)")
-    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
-                    help="library tuning switch (luxhip_set_option), e.g. bn_resident=0; may be repeated")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run three device-to-device copies of 256 MiB: a kernel of known traffic that "
-                         "scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
-    ap.add_argument("--rotate", type=int, default=1,
-                    help="number of separate sets of the large tensors that the timed steps use in turn "
-                         "(1 = every step on the same buffers)")
-    ap.add_argument("--cold-sets", type=int, default=8,
-                    help="HBM-bound workloads: also time the steps on this many sets of tensors used in turn (reported as cold_inputs; "
-                         "0 = skip, e.g. under a profiler, where its launches would enter the per-kernel averages)")
-    ap.add_argument("--graph", action="store_true",
-                    help="also record one step into a HIP graph and time its replays (reported as graph_replay; "
-                         "value stays the eager figure)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path is single-GPU; no collective is part of it); "
-              "run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+HEAVY = ("C4", "C5", "C5bf16", "SDPA", "CONV3D", "CONV3Df32")
+_CPU_DONE = {}
+DEFAULT_ORDER = ["C4", "C1", "C2", "C3", "C3bf16", "C5", "C5bf16"]      # the benchmark configurations; the largest one first (headline)
 
-    lux = load_package()
-    lux.init(0)
-    for opt in args.option:
-        name, _, val = opt.partition("=")
-        lux.set_option(name, int(val))
-    wl = WORKLOADS[args.workload]()
-    heavy = args.workload in ("C4", "C5", "C5bf16", "SDPA")
-    if args.steps is None:
-        args.steps = 20 if heavy else 200
-    if args.warmup is None:
-        args.warmup = 3 if heavy else 20
+
+def measure(lux, name, args):
+    """Times one workload and returns its entry: whole-step throughput, per-kernel table, roofline of the
+    dominant kernel, warm / cold figures for HBM-bound workloads, CPU baseline."""
+    wl = WORKLOADS[name]()
+    heavy = name in HEAVY
+    steps = args.steps if args.steps is not None else (30 if heavy else 200)
+    warmup = args.warmup if args.warmup is not None else (30 if heavy else 50)   # long enough for the clocks to settle
     wl.rotate = args.rotate
     wl.setup(lux)
-
-    ms_gpu, ms_wall = timed(lux, wl.rotating_step if args.rotate > 1 and hasattr(wl, "rotating_step") else wl.step, args.steps, args.warmup)
-    ms = max(ms_gpu, ms_wall)           # whole-job time: the slower of the device and host clocks
-    ms_graph = timed_graph(lux, wl.step, args.steps) if args.graph else None
+    peak = PEAK_HBM_GBS if wl.bound == "hbm" else PEAK_MFMA_TFLOPS[wl.dtype]
+    unit = "GB/s" if wl.bound == "hbm" else "TFLOP/s"
+    scale = 1e9 if wl.bound == "hbm" else 1e12
     work = wl.work_per_step()
-    if wl.bound == "hbm":
-        value, unit, peak = work / (ms * 1e-3) / 1e9, "GB/s", PEAK_HBM_GBS
-    else:
-        value, unit, peak = work / (ms * 1e-3) / 1e12, "TFLOP/s", PEAK_MFMA_TFLOPS[wl.dtype]
 
-    prof = kernel_profile(lux, wl.step, min(args.steps, 100))
+    step = wl.rotating_step if args.rotate > 1 and hasattr(wl, "rotating_step") else wl.step
+    ms_gpu, ms_wall = timed(lux, step, steps, warmup)
+    ms = max(ms_gpu, ms_wall)           # whole-job time: the slower of the device and host clocks
+    ms_graph = timed_graph(lux, wl.step, steps) if args.graph else None
+    warm = {"ms_per_step": round(ms, 5), "value": round(work / (ms * 1e-3) / scale, 2), "unit": unit,
+            "frac_of_peak": round(work / (ms * 1e-3) / scale / peak, 4),
+            "note": "every step on the same buffers (inputs may come from the 256 MB Infinity Cache)"}
+
+    # HBM-bound workloads: the headline figure is taken on several sets of tensors used in turn, so that no step
+    # finds its inputs in the Infinity Cache from the step before
+    cold_wl = None
+    cold = None
+    if wl.bound == "hbm" and args.rotate == 1 and not args.option and args.cold_sets > 1:
+        cold_wl = WORKLOADS[name]()
+        cold_wl.rotate = args.cold_sets
+        cold_wl.setup(lux)
+        cg, cw_ = timed(lux, cold_wl.rotating_step, steps, warmup)
+        cms = max(cg, cw_)
+        cold = {"sets_of_tensors": args.cold_sets, "ms_per_step": round(cms, 5), "value": round(work / (cms * 1e-3) / scale, 2),
+                "unit": unit, "frac_of_peak": round(work / (cms * 1e-3) / scale / peak, 4)}
+        ms_head, ms_gpu_head, ms_wall_head = cms, cg, cw_
+    else:
+        ms_head, ms_gpu_head, ms_wall_head = ms, ms_gpu, ms_wall
+    value = work / (ms_head * 1e-3) / scale
+
+    prof_wl = cold_wl if cold_wl is not None else wl
+    prof_step = prof_wl.rotating_step if cold_wl is not None else step
+    prof = kernel_profile(lux, prof_step, min(steps, 100))
     kw = wl.kernel_work()
     kernels = []
     # "<name>+tail" is a second launch that finishes the rows of <name>: one kernel's work, so its
@@ -624,7 +782,7 @@ def main():
         if "tail_launches" in k:
             ent["tail_launches"] = k["tail_launches"]
         if w:
-            ach = w / (avg_ms * 1e-3) / (1e9 if wl.bound == "hbm" else 1e12)
+            ach = w / (avg_ms * 1e-3) / scale
             ent.update({"algorithmic": w, "achieved": round(ach, 1), "frac": round(ach / peak, 4)})
         elif hasattr(wl, "kernel_bytes") and wl.kernel_bytes().get(k["kernel"]):
             # an HBM-bound kernel inside a contraction-bound workload: reported against the HBM peak
@@ -632,64 +790,127 @@ def main():
             gbs = b / (avg_ms * 1e-3) / 1e9
             ent.update({"algorithmic_bytes": b, "achieved_GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
         kernels.append(ent)
-    # Kernels that an API call launches alone are timed again back to back (two events around a
-    # run of identical launches): no per-launch event sits between the kernels, so the average is
-    # the kernel's duration plus the dispatch gap, which is what rocprofv3 --kernel-trace reports too.
-    iso = wl.isolated_ops() if hasattr(wl, "isolated_ops") and not args.option else {}
+    # Kernels that an API call launches alone are timed again back to back (two events around a run of
+    # identical launches, on the rotating sets when those are the headline): no per-launch event sits between
+    # the kernels, so the average is the kernel's duration plus the dispatch gap, which is what
+    # rocprofv3 --kernel-trace reports too.
+    iso = prof_wl.isolated_ops() if hasattr(prof_wl, "isolated_ops") and not args.option else {}
     seen = {e["kernel"] for e in kernels}
-    for name, call in iso.items():
-        if name not in seen:
+    for kname, call in iso.items():
+        if kname not in seen:
             continue
-        ms_iso, _ = timed(lux, call, 50, 5)
+        ms_iso, _ = timed(lux, call, 64, 8)
         for e in kernels:
-            if e["kernel"] == name:
+            if e["kernel"] == kname:
                 e["avg_us_per_launch_events"] = e["avg_us"]
                 e["avg_us"] = round(ms_iso * 1e3, 3)
                 if "algorithmic" in e:
-                    ach = e["algorithmic"] / (ms_iso * 1e-3) / (1e9 if wl.bound == "hbm" else 1e12)
+                    ach = e["algorithmic"] / (ms_iso * 1e-3) / scale
                     e.update({"achieved": round(ach, 1), "frac": round(ach / peak, 4)})
     kernels.sort(key=lambda e: -e["avg_us"])
     dom = next((e for e in kernels if "achieved" in e), None)
     roofline = None
     if dom is not None:
-        roofline = {"bound": wl.bound, "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": peak, "unit": unit,
-                    "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get((wl.name, dom["kernel"])), "avg_us": dom["avg_us"],
-                    "algorithmic_per_launch": dom["algorithmic"]}
+        roofline = {"bound": "hbm" if wl.bound == "hbm" else "mfma", "kernel": dom["kernel"], "achieved": dom["achieved"], "peak": peak,
+                    "unit": unit, "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get((wl.name, dom["kernel"])),
+                    "avg_us": dom["avg_us"], "algorithmic_per_launch": dom["algorithmic"]}
 
     out = {
-        "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype,
-        "data": "synthetic", "config": {"workload": f"{wl.name}: {wl.description}"},
-        "options": args.option + ([f"rotate={args.rotate}"] if args.rotate > 1 else []), "frac_of_peak": round(value / peak, 4), "ms_per_step_gpu_events": round(ms_gpu, 5),
-        "ms_per_step_host_clock": round(ms_wall, 5), "roofline": roofline, "kernels": kernels,
+        "workload": wl.name, "description": wl.description, "dtype": wl.dtype, "bound": wl.bound, "value": round(value, 2), "unit": unit,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_head, 5), "frac_of_peak": round(value / peak, 4),
+        "ms_per_step_gpu_events": round(ms_gpu_head, 5), "ms_per_step_host_clock": round(ms_wall_head, 5),
+        "roofline": roofline, "kernels": kernels,
     }
+    if cold is not None:
+        out["cold_inputs"] = cold
+        out["warm_inputs"] = warm
+        out["inputs"] = f"{args.cold_sets} sets of tensors used in turn (value, ms_per_step, kernels); warm_inputs: one set"
     if ms_graph is not None:
         out["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "speedup_over_eager": round(ms / ms_graph, 3),
                                "note": "one step recorded into a HIP graph, replayed; batchnorm/groupnorm record their two-pass kernels"}
-    if wl.bound == "hbm" and args.rotate == 1 and not args.option and args.cold_sets > 1:
-        # the same steps on several sets of input tensors used in turn: no step finds its inputs in the 256 MB
-        # Infinity Cache from the step before, as it does when every step runs on the same buffers
-        cold = WORKLOADS[args.workload]()
-        cold.rotate = args.cold_sets
-        cold.setup(lux)
-        cg, cw_ = timed(lux, cold.rotating_step, args.steps, args.warmup)
-        cms = max(cg, cw_)
-        out["cold_inputs"] = {"sets_of_tensors": args.cold_sets, "ms_per_step": round(cms, 5),
-                              "value": round(work / (cms * 1e-3) / 1e9, 2), "unit": "GB/s",
-                              "frac_of_peak": round(work / (cms * 1e-3) / 1e9 / peak, 4)}
-        del cold
     if hasattr(wl, "step_fused"):
-        fg, fw = timed(lux, wl.step_fused, args.steps, args.warmup)
+        fw_ = cold_wl if cold_wl is not None else wl
+        fstep = fw_.rotating_step_fused if cold_wl is not None and hasattr(fw_, "rotating_step_fused") else fw_.step_fused
+        fg, fw = timed(lux, fstep, steps, warmup)
         fms = max(fg, fw)
         out["fused_variant"] = {"workload": "batchnorm(..., relu) fwd+bwd (activation fused into batchnorm)",
                                 "ms_per_step": round(fms, 5), "value": round(wl.work_per_step_fused() / (fms * 1e-3) / 1e9, 2),
                                 "unit": "GB/s", "algorithmic_bytes": wl.work_per_step_fused()}
+    del cold_wl
     if args.cpu_seconds > 0:
-        cb = wl.cpu_baseline(args.cpu_seconds)
-        if cb is not None:
-            cb["value"] = round(cb["value"], 3)
-            cb["ms_per_step"] = round(cb["ms_per_step"], 3)
-            out["cpu_baseline"] = cb
+        key = type(wl).__name__         # the bf16 variant of a workload has the fp32 CPU figure beside it: timed once
+        if key not in _CPU_DONE:
+            cb = wl.cpu_baseline(args.cpu_seconds)
+            if cb is not None:
+                cb["value"] = round(cb["value"], 4)
+                cb["ms_per_step"] = round(cb["ms_per_step"], 3)
+            _CPU_DONE[key] = cb
+        if _CPU_DONE[key] is not None:
+            out["cpu_baseline"] = _CPU_DONE[key]
+    del wl
+    lux._lib.call("luxhip_trim")            # the next workload starts from an empty pool
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps per workload (default 200, heavy workloads 30)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps per workload (default 50, heavy workloads 30)")
+    ap.add_argument("--workload", default="ALL", choices=["ALL"] + sorted(WORKLOADS),
+                    help="ALL (default): the benchmark configurations C1, C2, C3, C3bf16, C4, C5, C5bf16 in one run; "
+                         "the headline (top-level fields) is C4, the largest one")
+    ap.add_argument("--cpu-seconds", type=float, default=8.0, help="budget of each CPU baseline (0 disables them)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library tuning switch (luxhip_set_option), e.g. bn_resident=0; may be repeated")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three device-to-device copies of 256 MiB: a kernel of known traffic that "
+                         "scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--rotate", type=int, default=1,
+                    help="number of separate sets of the large tensors that the timed steps use in turn "
+                         "(1 = every step on the same buffers)")
+    ap.add_argument("--cold-sets", type=int, default=8,
+                    help="HBM-bound workloads: the headline is timed on this many sets of tensors used in turn "
+                         "(0 = one set only, e.g. under a profiler)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also record one step into a HIP graph and time its replays (reported as graph_replay; "
+                         "value stays the eager figure)")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the measured copy / MFMA peaks")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path is single-GPU; no collective is part of it); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    lux = load_package()
+    lux.init(0)
+    for opt in args.option:
+        name, _, val = opt.partition("=")
+        lux.set_option(name, int(val))
+    names = DEFAULT_ORDER if args.workload == "ALL" else [args.workload]
+    entries = [measure(lux, n, args) for n in names]
+    head = entries[0]
+
+    out = {
+        "metric": METRIC, "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": head["steps"], "warmup": head["warmup"],
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic", "config": {"workload": f"{head['workload']}: {head['description']}"},
+        "options": args.option + ([f"rotate={args.rotate}"] if args.rotate > 1 else []), "frac_of_peak": head["frac_of_peak"],
+        "ms_per_step_gpu_events": head["ms_per_step_gpu_events"], "ms_per_step_host_clock": head["ms_per_step_host_clock"],
+        "roofline": head["roofline"], "kernels": head["kernels"],
+    }
+    for k in ("cold_inputs", "warm_inputs", "inputs", "graph_replay", "fused_variant", "cpu_baseline"):
+        if k in head:
+            out[k] = head[k]
+    out["configs"] = entries
+    if not args.no_peaks:
+        cp, mb, mf = C.c_double(), C.c_double(), C.c_double()
+        lux._lib.call("luxhip_measure_peaks", lux.current_stream(), C.byref(cp), C.byref(mb), C.byref(mf))
+        out["measured_peaks"] = {"copy_GBps": round(cp.value, 1), "mfma_bf16_TFLOPs": round(mb.value, 1), "mfma_f32_TFLOPs": round(mf.value, 1),
+                                 "published": {"hbm_GBps": PEAK_HBM_GBS, "mfma_bf16_TFLOPs": PEAK_MFMA_TFLOPS["bf16"],
+                                               "mfma_f32_TFLOPs": PEAK_MFMA_TFLOPS["f32"]},
+                                 "note": "streaming copy of 512 MiB (read + written bytes); register-only MFMA loops on pseudo-random "
+                                         "operands, 8 waves per compute unit, after the clocks have settled"}
     if args.calibrate_copy:
         nbytes = 256 << 20
         a, b = lux.DeviceArray((nbytes // 4,), "f32"), lux.DeviceArray((nbytes // 4,), "f32")

@@ -104,6 +104,14 @@ int luxhip_profile_enable(int on);
 int luxhip_set_option(const char* name, int64_t value);
 int luxhip_profile_report(char* buf, size_t len);
 
+/* Achievable peaks of the device (no counterpart in the reference; the benchmark reports them next to
+ * the published figures its roofline fractions divide by): a streaming copy of 512 MiB (GB/s of read +
+ * written bytes), and register-only loops of v_mfma_f32_16x16x32_bf16 / v_mfma_f32_32x32x2_f32 on
+ * pseudo-random operands, eight waves per compute unit, after a warm-up that lets the clocks settle
+ * (TFLOP/s).  Any pointer may be NULL to skip that measurement.  Synchronises the stream; allocates and
+ * frees 1 GiB of device memory. */
+int luxhip_measure_peaks(luxhip_stream_t s, double* copy_GBps, double* mfma_bf16_TFLOPs, double* mfma_f32_TFLOPs);
+
 /* Pooled device allocator, in place of the array package's pool that serves the reference's `similar`
  * calls (e.g. the outputs of src/impl/dense.jl:46-57, src/impl/conv.jl:62-72) (size-bucketed free lists; luxhip_free returns the block to the
  * pool, luxhip_trim releases the pool to the driver).  A freed block can be handed out again at

@@ -55,6 +55,7 @@ SIGNATURES = {
     "luxhip_profile_enable": [_i],
     "luxhip_profile_report": [C.c_char_p, _sz],
     "luxhip_set_option": [C.c_char_p, _i64],
+    "luxhip_measure_peaks": [_vp, C.POINTER(_d), C.POINTER(_d), C.POINTER(_d)],
     "luxhip_malloc": [C.POINTER(_vp), _sz],
     "luxhip_free": [_vp],
     "luxhip_trim": [],

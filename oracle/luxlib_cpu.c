@@ -201,3 +201,80 @@ void luxcpu_batchnorm_train_bwd(int64_t I, int64_t C, int64_t N, const float* dy
     if (dbeta) memcpy(dbeta, dbt, sizeof(float) * (size_t)C);
     free(dmu);
 }
+
+/* groupnorm (groupnorm.jl:5-22): x viewed as (I, Cg, G, N); statistics per (group, sample) as two
+ * serial passes (mean, then var about it, common_ops.jl:40-43); the affine-normalise loop
+ * (groupnorm_affine_normalize_act_cpu!, groupnorm.jl:131-205) is a serial @simd loop, as is its
+ * pullback (:477-533): nothing here is threaded, as in the reference.  mean/var: (G, N). */
+void luxcpu_groupnorm_fwd(int act, int64_t I, int64_t Cg, int64_t G, int64_t N, const float* x, const float* gamma,
+                          const float* beta, float eps, float* y, float* mean, float* var) {
+    const int64_t m = I * Cg;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t k = 0; k < G; ++k) {
+            const float* xs = x + (n * G + k) * m;
+            float s = 0.0f;
+            for (int64_t e = 0; e < m; ++e) s += xs[e];
+            const float mu = s / (float)m;
+            float d = 0.0f;
+            for (int64_t e = 0; e < m; ++e) d += (xs[e] - mu) * (xs[e] - mu);
+            mean[n * G + k] = mu;
+            var[n * G + k] = d / (float)m;
+        }
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t k = 0; k < G; ++k) {
+            const float idenom = 1.0f / sqrtf(var[n * G + k] + eps);
+            const float mu = mean[n * G + k];
+            for (int64_t j = 0; j < Cg; ++j) {
+                const int64_t c = k * Cg + j;
+                const float sc = (gamma ? gamma[c] : 1.0f) * idenom;
+                const float sh = (beta ? beta[c] : 0.0f) - mu * sc;
+                const float* xr = x + ((n * G + k) * Cg + j) * I;
+                float* yr = y + ((n * G + k) * Cg + j) * I;
+                for (int64_t i = 0; i < I; ++i) yr[i] = act_f(act, xr[i] * sc + sh);
+            }
+        }
+}
+
+/* Pullback of the same w.r.t. (x, gamma, beta): the activation's derivative from the recomputed
+ * pre-activation (the rrule keeps it, groupnorm.jl:349-404), the fused loop (:477-533) and the
+ * mean_var pullback broadcast (common_ops.jl:45-61). */
+void luxcpu_groupnorm_bwd(int act, int64_t I, int64_t Cg, int64_t G, int64_t N, const float* delta, const float* x,
+                          const float* gamma, const float* beta, const float* mean, const float* var, float eps,
+                          float* dx, float* dgamma, float* dbeta) {
+    const int64_t m = I * Cg, C = Cg * G;
+    if (dgamma) for (int64_t c = 0; c < C; ++c) dgamma[c] = 0.0f;
+    if (dbeta) for (int64_t c = 0; c < C; ++c) dbeta[c] = 0.0f;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t k = 0; k < G; ++k) {
+            const float mu = mean[n * G + k];
+            const float idenom = 1.0f / sqrtf(var[n * G + k] + eps);
+            const float idenom2 = idenom * idenom;
+            float dmu = 0.0f, dvar = 0.0f;
+            for (int64_t j = 0; j < Cg; ++j) {
+                const int64_t c = k * Cg + j;
+                const float g = gamma ? gamma[c] : 1.0f, b = beta ? beta[c] : 0.0f;
+                const float sc = g * idenom, sh = b - mu * sc;
+                const float* xr = x + ((n * G + k) * Cg + j) * I;
+                const float* dr = delta + ((n * G + k) * Cg + j) * I;
+                float* o = dx + ((n * G + k) * Cg + j) * I;
+                float ag = 0.0f, ab = 0.0f;
+                for (int64_t i = 0; i < I; ++i) {
+                    const float pre = xr[i] * sc + sh;
+                    const float dy = dr[i] * act_d(act, act_f(act, pre), pre);
+                    const float xmu = xr[i] - mu;
+                    o[i] = dy * sc;
+                    dmu -= o[i];
+                    dvar -= o[i] * xmu * 0.5f * idenom2;
+                    ag += dy * xmu * idenom;
+                    ab += dy;
+                }
+                if (dgamma) dgamma[c] += ag;
+                if (dbeta) dbeta[c] += ab;
+            }
+            const float a = dmu / (float)m, bb = (2.0f / (float)m) * dvar;
+            for (int64_t e = 0; e < m; ++e) {
+                float* o = dx + (n * G + k) * m;
+                o[e] += a + bb * (x[(n * G + k) * m + e] - mu);
+            }
+        }
+}

@@ -80,3 +80,31 @@ def test_batchnorm_known_answer_and_oracle(cpu):
     np.testing.assert_allclose(dx, wdx, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(dg, wdg, rtol=1e-4, atol=1e-4)
     np.testing.assert_allclose(db, wdb, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("act,aid", [("identity", 0), ("relu", 1), ("swish", 4)])
+def test_groupnorm_against_the_numpy_oracle(cpu, act, aid):
+    """The C port of groupnorm (benchmark baseline of the groupnorm workload) against the numpy oracle,
+    which torch's group_norm and finite differences pin."""
+    rng = np.random.default_rng(21)
+    shape = (5, 4, 6, 3)
+    I, Cc, G, N = 20, 6, 3, 3
+    x, delta = F(rng.normal(size=shape) * 1.5 + 0.2), F(rng.normal(size=shape))
+    g, b = rng.uniform(0.8, 1.2, Cc).astype(np.float32), (0.05 * rng.normal(size=Cc)).astype(np.float32)
+    y, dx = np.empty(shape, np.float32, order="F"), np.empty(shape, np.float32, order="F")
+    mean, var = np.empty(G * N, np.float32), np.empty(G * N, np.float32)
+    dg, db = np.empty(Cc, np.float32), np.empty(Cc, np.float32)
+    i64 = C.c_int64
+    cpu.luxcpu_groupnorm_fwd(aid, i64(I), i64(Cc // G), i64(G), i64(N), P(x), P(g), P(b), C.c_float(1e-5), P(y), P(mean), P(var))
+    f8 = lambda a: a.astype(np.float64)
+    wy = O.groupnorm(f8(x), f8(g), f8(b), G, act, 1e-5)
+    np.testing.assert_allclose(y, wy, rtol=2e-5, atol=2e-5)
+    if act == "relu":
+        pre = O.groupnorm(f8(x), f8(g), f8(b), G, "identity", 1e-5)
+        delta[np.abs(pre) < 1e-3] = 0
+    cpu.luxcpu_groupnorm_bwd(aid, i64(I), i64(Cc // G), i64(G), i64(N), P(delta), P(x), P(g), P(b), P(mean), P(var), C.c_float(1e-5),
+                             P(dx), P(dg), P(db))
+    wdx, wdg, wdb = O.groupnorm_pullback(f8(x), f8(g), f8(b), G, act, 1e-5, f8(delta))
+    np.testing.assert_allclose(dx, wdx, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(dg, wdg, rtol=2e-4, atol=2e-4)
+    np.testing.assert_allclose(db, wdb, rtol=2e-4, atol=2e-4)
