@@ -430,8 +430,6 @@ function CRC.rrule(::typeof(Impl.layernorm), x::HIPArray{T,N}, γ::Union{Nothing
         ϵ) where {F,T<:HIPFloat,N}
     y, (μs, is, L, R, x̂, affine) = layernorm_device(x, γ, β, act, dims, ϵ, true)
     id = act_id(act)
-    LnBwdSig = (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
-        Ptr{Cvoid}, Ptr{Cvoid})
     function ∇layernorm_hip(Δ′)
         Δ = CRC.unthunk(Δ′)
         nt = NoTangent()
@@ -439,7 +437,9 @@ function CRC.rrule(::typeof(Impl.layernorm), x::HIPArray{T,N}, γ::Union{Nothing
         ∂γ = γ === nothing ? nothing : similar(γ)
         ∂β = β === nothing ? nothing : similar(β)
         if affine === nothing
-            check(ccall((:luxhip_layernorm_bwd, libluxhip), Cint, LnBwdSig,
+            check(ccall((:luxhip_layernorm_bwd, libluxhip), Cint,
+                (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
+                    Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
                 stream(), dtype_code(T), id, L, R, optr(Δ), optr(x), optr(γ), optr(β), optr(μs), optr(is), optr(∂x), optr(∂γ),
                 optr(∂β))) || error(last_error())
         else
@@ -451,7 +451,9 @@ function CRC.rrule(::typeof(Impl.layernorm), x::HIPArray{T,N}, γ::Union{Nothing
                     Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
                 stream(), dtype_code(T), id, I, C, Nn, optr(Δ), optr(x̂), optr(γ), optr(β), optr(affine[1]), optr(affine[2]), Cint(0),
                 optr(∂x̂), optr(∂γ), optr(∂β))) || error(last_error())
-            check(ccall((:luxhip_layernorm_bwd, libluxhip), Cint, LnBwdSig,
+            check(ccall((:luxhip_layernorm_bwd, libluxhip), Cint,
+                (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid},
+                    Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
                 stream(), dtype_code(T), Cint(0), L, R, optr(∂x̂), optr(x), C_NULL, C_NULL, optr(μs), optr(is), optr(∂x), C_NULL,
                 C_NULL)) || error(last_error())
         end
@@ -552,18 +554,21 @@ end
 depth_args(c::DenseConvDims{3}, N::Integer) = (Int64(prod(NNlib.input_size(c)[1:2])), Int64(NNlib.input_size(c)[3]),
     Int64(NNlib.channels_in(c)), Int64(N), Int64(NNlib.kernel_size(c)[3]), Int64(NNlib.output_size(c)[3]),
     Int64(NNlib.stride(c)[3]), Int64(NNlib.padding(c)[5]), Int64(NNlib.dilation(c)[3]), Cint(NNlib.flipkernel(c)))
-const DepthSig = (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid})
 function depth_unfold(x::HIPArray{T,5}, c::DenseConvDims{3}) where {T<:HIPFloat}
     c2 = inner2d(c, size(x, 5))
     xu = similar(x, T, (NNlib.input_size(c2)..., NNlib.channels_in(c2), NNlib.output_size(c)[3] * size(x, 5)))
-    check(ccall((:luxhip_conv_depth_unfold, libluxhip), Cint, DepthSig, stream(), dtype_code(T), depth_args(c, size(x, 5))..., optr(x), optr(xu))) ||
-        error("luxhip_conv_depth_unfold")
+    I, D, Cin, N, kD, Dout, sD, pD, dD, flip = depth_args(c, size(x, 5))       # a ccall takes no splatted arguments
+    check(ccall((:luxhip_conv_depth_unfold, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), I, D, Cin, N, kD, Dout, sD, pD, dD, flip, optr(x), optr(xu))) || error("luxhip_conv_depth_unfold")
     return xu, c2
 end
 function depth_fold(dxu::HIPArray{T,4}, c::DenseConvDims{3}, N::Integer) where {T<:HIPFloat}
     dx = similar(dxu, T, (NNlib.input_size(c)..., NNlib.channels_in(c), N))
-    check(ccall((:luxhip_conv_depth_fold, libluxhip), Cint, DepthSig, stream(), dtype_code(T), depth_args(c, N)..., optr(dxu), optr(dx))) ||
-        error("luxhip_conv_depth_fold")
+    I, D, Cin, Nn, kD, Dout, sD, pD, dD, flip = depth_args(c, N)
+    check(ccall((:luxhip_conv_depth_fold, libluxhip), Cint,
+        (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid}),
+        stream(), dtype_code(T), I, D, Cin, Nn, kD, Dout, sD, pD, dD, flip, optr(dxu), optr(dx))) || error("luxhip_conv_depth_fold")
     return dx
 end
 function swap_middle(a::HIPArray{T}, inner, A, B, outer, shape) where {T<:HIPFloat}

@@ -171,3 +171,141 @@ def test_conv_dims_with_three_spatial_dims(lux):
     assert inner.y_shape == (6, 4, 6, 4 * 2)
     with pytest.raises(lux.Unsupported):
         lux.DenseConvDims((4, 4, 4, 4, 2, 1), (2, 2, 2, 2, 2, 3))
+
+
+# ----------------------------------------------------------------------------- the Julia glue file
+JULIA_GLUE = os.path.join(ROOT, "lux.jl_amd", "julia", "LuxHIP.jl")
+
+
+def header_prototypes():
+    """name -> (return type, [parameter types]) of include/luxhip.h, as C type strings without parameter names."""
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    protos = {}
+    for m in re.finditer(r"\b((?:const\s+)?[A-Za-z_0-9]+\s*\**)\s*\b(luxhip_[a-z0-9_]+)\s*\(([^;{}]*?)\)\s*;", text, flags=re.S):
+        params = []
+        for a in m.group(3).split(","):
+            a = " ".join(a.split())
+            if a in ("", "void"):
+                continue
+            t = re.sub(r"\b[A-Za-z_0-9]+$", "", a).strip()          # drop the parameter name
+            params.append(t.replace(" *", "*"))
+        protos[m.group(2)] = (" ".join(m.group(1).split()).replace(" *", "*"), params)
+    return protos
+
+
+def _matching_paren(text, i):
+    """Index of the parenthesis closing the one at text[i] (Julia strings and comments in the glue file hold no
+    unbalanced parentheses inside a ccall)."""
+    depth = 0
+    for j in range(i, len(text)):
+        if text[j] == "(":
+            depth += 1
+        elif text[j] == ")":
+            depth -= 1
+            if depth == 0:
+                return j
+    raise ValueError("unbalanced parentheses")
+
+
+def _split_top_level(s):
+    out, depth, cur = [], 0, ""
+    for ch in s:
+        if ch in "({[":
+            depth += 1
+        elif ch in ")}]":
+            depth -= 1
+        if ch == "," and depth == 0:
+            out.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        out.append(cur.strip())
+    return out
+
+
+def julia_ccalls():
+    """Every `ccall((:luxhip_x, libluxhip), Ret, (Types...,), args...)` of the glue file:
+    (symbol, return type, [argument types], number of values passed, line)."""
+    text = open(JULIA_GLUE).read()
+    text = "\n".join(line if not line.lstrip().startswith("#") else "" for line in text.split("\n"))
+    calls = []
+    for m in re.finditer(r"ccall\(\(:(luxhip_[a-z0-9_]+),\s*libluxhip\)", text):
+        start = text.index("(", m.start())
+        end = _matching_paren(text, start)
+        parts = _split_top_level(text[start + 1:end])
+        ret, types = parts[1], parts[2]
+        # Julia wants the type tuple spelled out in the call and takes no splatted values
+        assert types.startswith("(") and types.endswith(")"), f"{m.group(1)}: the argument types must be a literal tuple, got `{types}`"
+        assert not any(v.endswith("...") for v in parts[3:]), f"{m.group(1)}: a ccall cannot splat its arguments"
+        calls.append((m.group(1), ret, _split_top_level(types[1:-1]), len(parts) - 3, text.count("\n", 0, m.start()) + 1))
+    return calls
+
+
+# which Julia ccall types may stand for a C parameter type
+_JULIA_FOR_C = {
+    "int": {"Cint"}, "int64_t": {"Int64", "Clonglong"}, "uint64_t": {"UInt64", "Culonglong"}, "size_t": {"Csize_t"},
+    "double": {"Cdouble"}, "float": {"Cfloat"}, "const char*": {"Cstring", "Ptr{UInt8}", "Ptr{Cchar}"},
+    "char*": {"Ptr{UInt8}", "Ptr{Cchar}"}, "luxhip_stream_t": {"Ptr{Cvoid}"}, "luxhip_event_t": {"Ptr{Cvoid}"},
+    "luxhip_stream_t*": {"Ptr{Ptr{Cvoid}}"}, "luxhip_event_t*": {"Ptr{Ptr{Cvoid}}"}, "void**": {"Ptr{Ptr{Cvoid}}"},
+    "void*": {"Ptr{Cvoid}"}, "const void*": {"Ptr{Cvoid}"}, "int*": {"Ptr{Cint}", "Ref{Cint}"},
+    "int64_t*": {"Ptr{Int64}", "Ref{Int64}"}, "const int64_t*": {"Ptr{Int64}", "Ref{Int64}"},
+    "double*": {"Ptr{Cdouble}", "Ref{Cdouble}"}, "float*": {"Ptr{Cfloat}", "Ptr{Cvoid}"}, "const float*": {"Ptr{Cfloat}", "Ptr{Cvoid}"},
+    "const uint8_t*": {"Ptr{UInt8}", "Ptr{Cvoid}"}, "const luxhip_conv_dims_t*": {"Ptr{ConvDimsC}", "Ref{ConvDimsC}"},
+}
+
+
+def test_julia_glue_ccalls_match_the_header():
+    """There is no Julia toolchain to run the glue file with, so the one check that needs none: every ccall names a
+    symbol the header declares, passes as many values as it lists types, lists as many types as the C prototype has
+    parameters, and each type is one that has the C parameter's size and meaning."""
+    protos = header_prototypes()
+    assert set(protos) == set(declared_symbols())
+    calls = julia_ccalls()
+    assert len(calls) >= 40
+    for name, ret, types, nvalues, line in calls:
+        where = f"LuxHIP.jl:{line} {name}"
+        assert name in protos, f"{where}: not declared in include/luxhip.h"
+        cret, cparams = protos[name]
+        assert ret in _JULIA_FOR_C.get(cret, {cret}) or (cret == "int" and ret == "Cint"), f"{where}: returns {cret}, ccall says {ret}"
+        assert len(types) == len(cparams), f"{where}: {len(cparams)} C parameters, {len(types)} ccall types"
+        assert nvalues == len(types), f"{where}: {len(types)} ccall types but {nvalues} values passed"
+        for k, (jt, ct) in enumerate(zip(types, cparams)):
+            assert jt in _JULIA_FOR_C[ct], f"{where}: parameter {k + 1} is `{ct}`, ccall passes `{jt}`"
+
+
+def test_julia_struct_mirrors_the_conv_descriptor():
+    """ConvDimsC in the glue file lists the fields of luxhip_conv_dims_t in the same order with the same widths."""
+    htext = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    m = re.search(r"typedef\s+struct\s*(?:\w+\s*)?\{(.*?)\}\s*luxhip_conv_dims_t\s*;", htext, flags=re.S)
+    assert m
+    cfields = []
+    for decl in m.group(1).split(";"):
+        decl = " ".join(re.sub(r"//[^\n]*", "", decl).split())
+        if not decl:
+            continue
+        ctype, names = decl.split(" ", 1)
+        for nm in names.split(","):
+            nm = nm.strip()
+            arr = re.match(r"(\w+)\[(\d+)\]", nm)
+            cfields.append((arr.group(1), ctype, int(arr.group(2))) if arr else (nm, ctype, 1))
+    jtext = open(JULIA_GLUE).read()
+    m = re.search(r"struct ConvDimsC\n(.*?)\nend", jtext, flags=re.S)
+    assert m
+    jfields = []
+    for line in m.group(1).split("\n"):
+        line = line.split("#")[0].strip()
+        if not line:
+            continue
+        for part in line.split(";"):
+            nm, jt = (s.strip() for s in part.split("::"))
+            jfields.append((nm, jt))
+    width = {"int": "Cint", "int64_t": "Int64"}
+    flat = []
+    for nm, ct, n in cfields:
+        flat += [(nm, width[ct], n)]
+    assert len(flat) == len(jfields), (flat, jfields)
+    for (cn, jt_want, n), (jn, jt) in zip(flat, jfields):
+        want = jt_want if n == 1 else f"NTuple{{{n},{jt_want}}}"
+        assert jt.replace(" ", "") == want, f"field {cn}/{jn}: C {n} x {jt_want}, Julia {jt}"

@@ -36,19 +36,6 @@ def test_reference_known_answer(gpu):
 SHAPES = [(4, 4, 6, 2), (8, 2), (3, 5, 4), (16, 16, 8, 4), (64, 3, 5), (32, 32, 16, 8), (40, 40, 3, 7)]
 
 
-@pytest.fixture(params=["resident", "streaming", "no_wait"])
-def bn_path(gpu, request):
-    """The three ways the library can run a training-mode batchnorm: single-pass kernels that keep
-    the tensor in registers (default where it fits), the two-kernel streaming path, and the
-    single-pass kernels with the wait for peer workgroups cut to zero polls, which makes every
-    workgroup recompute its peers' partial results itself (the bounded-wait exit)."""
-    gpu.set_option("bn_resident", 0 if request.param == "streaming" else 1)
-    gpu.set_option("bn_spin_limit", 0 if request.param == "no_wait" else 1 << 22)
-    yield request.param
-    gpu.set_option("bn_resident", 1)
-    gpu.set_option("bn_spin_limit", 1 << 22)
-
-
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("act", ["identity", "relu", "sigmoid_fast", "swish", "gelu", "tanh"])
 @pytest.mark.parametrize("affine", [True, False])

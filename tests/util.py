@@ -10,30 +10,43 @@ from oracle import luxlib_oracle as O
 REL = {"f32": 1e-5, "bf16": 1e-2}
 
 
+# every comparison made by assert_close in this process: (what, dtype, rel, worst error as a multiple of |want| + rms,
+# worst error of the float32 oracle in the same unit or None, elements compared)
+ERROR_LOG = []
+
+
 def assert_close(got, want, dtype, what="", rel=None, scale=0.0, want32=None):
     """`scale`: magnitude of the terms the result is a sum of, for results that are small
     through cancellation (gradients of normalisations); the absolute floor is
     rel * max(rms(want), scale).
     `want32`: the same oracle evaluated in float32 arithmetic (what a CPU run of the reference
     produces); where the problem is so ill-conditioned that fp32 arithmetic itself misses the
-    exact answer by more than the bar, the allowance grows to 4x that fp32 error."""
+    exact answer by more than the bar, the allowance grows to 4x that fp32 error.
+    Returns the worst error found, as a multiple of |want| + max(rms(want), scale) (the unit `rel` is in)."""
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, f"{what}: shape {got.shape} != {want.shape}"
     if want.size == 0:
-        return
+        return 0.0
     rel = REL[dtype] if rel is None else rel
     rms = max(float(np.sqrt(np.mean(want * want))), float(scale))
-    bound = rel * (np.abs(want) + rms) + 1e-30
+    unit = np.abs(want) + rms + 1e-30
+    bound = rel * unit
+    err32 = None
     if want32 is not None:
-        bound = np.maximum(bound, 4.0 * np.abs(np.asarray(want32, dtype=np.float64) - want))
+        d32 = np.abs(np.asarray(want32, dtype=np.float64) - want)
+        bound = np.maximum(bound, 4.0 * d32)
+        err32 = float(np.max(d32 / unit))
     err = np.abs(got - want)
+    worst = float(np.max(err / unit)) if np.isfinite(err).all() else float("inf")
+    ERROR_LOG.append((what, dtype, rel, worst, err32, int(want.size)))
     bad = ~(err <= bound)
     if bad.any():
         i = np.unravel_index(np.argmax(err / bound), err.shape)
         raise AssertionError(
             f"{what}: {bad.sum()}/{bad.size} elements outside rel {rel:g}; worst at {i}: got {got[i]!r} want {want[i]!r} "
             f"(err {err[i]:.3e}, bound {bound[i]:.3e})")
+    return worst
 
 
 def host_inputs(dtype, *arrays):
