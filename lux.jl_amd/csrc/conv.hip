@@ -4,6 +4,7 @@
 
 #include "common.h"
 #include "conv_kernels.h"
+#include "conv_patch.h"
 
 namespace luxhip {
 
@@ -236,6 +237,23 @@ static int run_conv_gemm(hipStream_t s, const ConvGeom& g, bool dgrad, const T* 
         Wm.sr = K; Wm.sk = 1; Wm.rows = Ncols;
         Wm.vec_ok = aligned16(Wm.p) && ((size_t)K * sizeof(T)) % 16 == 0;
         int rc;
+        if constexpr (sizeof(T) == 2) {
+            // unit stride and dilation, output as large as the input: the kernel that keeps a tile's input window in LDS
+            if (option_conv_tile() == 0 && g.sw == 1 && g.sh == 1 && g.dw == 1 && g.dh == 1 && g.OW == g.W && g.OH == g.H) {
+                cpatch::Problem p;
+                p.src = reinterpret_cast<const bf16_t*>(src) + (size_t)grp * Cg;
+                p.wm = reinterpret_cast<const bf16_t*>(Wm.p);
+                p.bias = reinterpret_cast<const bf16_t*>(bias);
+                p.out = reinterpret_cast<bf16_t*>(out); p.pre = reinterpret_cast<bf16_t*>(pre); p.zero = zeros;
+                p.Ctot = dgrad ? g.Cout : g.Cin; p.Cg = Cg; p.P = g.W; p.Q = g.H; p.N = g.N;
+                p.kW = g.kW; p.kH = g.kH; p.pad_w = g.pw; p.pad_h = g.ph; p.dgrad = dgrad;
+                p.Ncols = Ncols; p.col_off = grp * Ncols; p.Ctot_out = dgrad ? g.Cin : g.Cout; p.act = act;
+                if (cpatch::applicable(p)) {
+                    if ((rc = cpatch::launch(s, p)) != LUXHIP_OK) return rc;
+                    continue;
+                }
+            }
+        }
         if (tap_path) {
             ConvTapArgs<T> a;
             TapGeom<T>& q = a.tap;

@@ -1,0 +1,36 @@
+// fprop / dgrad with the input window of a tile held in LDS (bf16): launch.
+#define LUXHIP_CONV_PATCH_KERNEL
+#include "conv_patch.h"
+namespace luxhip {
+namespace cpatch {
+int launch(hipStream_t s, const Problem& p) {
+    static ResidentOnce ro;   // here only the one-time raise of the dynamic LDS limit
+    ro.get([&](hipError_t& err) {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(conv_patch_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)LDS_BYTES);
+        return 1;
+    });
+    LUX_CHECK_HIP(ro.error);
+    Args a;
+    a.src = p.src; a.wm = p.wm; a.bias = p.bias; a.out = p.out; a.pre = p.pre; a.zero = p.zero;
+    a.Ctot = p.Ctot; a.Cg = p.Cg;
+    a.P = p.P; a.Q = p.Q; a.NQ = p.N * p.Q; a.PQ = p.P * p.Q; a.M = a.PQ * p.N;
+    a.kW = p.kW; a.kH = p.kH; a.H = p.Cg / 64;
+    a.rev = p.dgrad ? 1 : 0;
+    a.hlo = p.dgrad ? p.kW - 1 - p.pad_w : p.pad_w;
+    a.dq_min = p.dgrad ? p.pad_h - (p.kH - 1) : -p.pad_h;
+    a.pitch = p.P + p.kW - 1;
+    a.Ncols = p.Ncols; a.col_off = p.col_off; a.Ctot_out = p.Ctot_out; a.act = p.act;
+    a.tiles_m = (int)ceil_div(a.M, TILE_M);
+    a.tiles_n = (int)ceil_div(a.Ncols, TILE_N);
+    a.divP = FastDiv((uint32_t)a.P); a.divQ = FastDiv((uint32_t)a.Q); a.divPQ = FastDiv((uint32_t)a.PQ);
+    a.divPitch = FastDiv((uint32_t)a.pitch);
+    const int64_t cus = num_cus() > 0 ? num_cus() : 256;
+    const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, cus);   // the LDS holds one workgroup per compute unit
+    ProfScope ps(p.dgrad ? "conv_dgrad_kernel<bf16>" : "conv_fprop_kernel<bf16>", s);
+    conv_patch_kernel<<<dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, s>>>(a);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+}  // namespace cpatch
+}  // namespace luxhip

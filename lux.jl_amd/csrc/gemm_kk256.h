@@ -17,8 +17,8 @@
 // LDS layout of a block: row r at r * 128 bytes, its eight 16-byte chunks XORed with (r / 2) % 8:
 // the sixteen lanes that a ds_read_b128 serves together (lanes 0-3, 12-15, 20-23, 24-27 and so on)
 // then fall into sixteen different bank groups.  Rows of A are permuted inside each wave's 128 rows
-// (LDS row 32 i + j holds row 4 j + i) so that a lane of the accumulator owns four consecutive m and
-// stores them with one 8-byte instruction.
+// (LDS row 16 j + u holds row 8 u + j) so that a lane of the accumulator owns eight consecutive m and
+// stores them with one 16-byte instruction.
 #pragma once
 
 #include "common.h"
@@ -282,12 +282,12 @@ __global__ __launch_bounds__(THREADS) void dense_gemm_kk256_kernel(Args a) {
     }
 }
 
-// The kernel's conditions: whole tiles, K in whole steps and long enough to fill the ring, 8-byte
-// stores of four consecutive m.
+// The kernel's conditions: whole tiles, K in whole steps and long enough to fill the ring, 16-byte
+// loads of the bias and stores of eight consecutive m.
 inline bool applicable(const DenseArgs<bf16_t>& a) {
-    const auto al8 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; };
+    const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     return a.M % TILE == 0 && a.N % TILE == 0 && a.K % BK == 0 && a.K >= 2 * BK && a.A.sk == 1 && a.B.sk == 1 && a.A.vec_ok &&
-           a.B.vec_ok && al8(a.C) && al8(a.pre) && a.ldc % 4 == 0 &&
+           a.B.vec_ok && al16(a.C) && al16(a.pre) && al16(a.bias) && a.ldc % 8 == 0 &&
            256 * a.A.sr * 2 < (int64_t(1) << 31) && 256 * a.B.sr * 2 < (int64_t(1) << 31);
 }
 
