@@ -21,12 +21,14 @@ int launch(hipStream_t s, const Problem& p) {
     a.dq_min = p.dgrad ? p.pad_h - (p.kH - 1) : -p.pad_h;
     a.pitch = p.P + p.kW - 1;
     a.Ncols = p.Ncols; a.col_off = p.col_off; a.Ctot_out = p.Ctot_out; a.act = p.act;
-    a.tiles_m = (int)ceil_div(a.M, TILE_M);
     a.tiles_n = (int)ceil_div(a.Ncols, TILE_N);
+    a.frags = (int)ceil_div(a.M, 16);
     a.divP = FastDiv((uint32_t)a.P); a.divQ = FastDiv((uint32_t)a.Q); a.divPQ = FastDiv((uint32_t)a.PQ);
     a.divPitch = FastDiv((uint32_t)a.pitch);
+    // the LDS holds one workgroup per compute unit: as many workgroups as compute units share the fragments evenly
     const int64_t cus = num_cus() > 0 ? num_cus() : 256;
-    const int grid = (int)std::min<int64_t>((int64_t)a.tiles_m * a.tiles_n, cus);   // the LDS holds one workgroup per compute unit
+    a.groups_m = (int)std::max<int64_t>(1, std::min<int64_t>(cus / a.tiles_n, ceil_div(a.frags, 16)));
+    const int grid = a.groups_m * a.tiles_n;
     ProfScope ps(p.dgrad ? "conv_dgrad_kernel<bf16>" : "conv_fprop_kernel<bf16>", s);
     conv_patch_kernel<<<dim3((unsigned)grid), dim3(THREADS), LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();

@@ -19,7 +19,8 @@ int launch_conv_wgrad_direct(hipStream_t s, ConvWgradDirectArgs& a, int slices) 
     });
     LUX_CHECK_HIP(ro.error);
     ProfScope ps("conv_wgrad_kernel<bf16>", s);
-    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n), (unsigned)slices), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
+    a.slices = slices;
+    kernel<<<dim3((unsigned)(a.tiles_m * a.tiles_n * slices)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

@@ -701,7 +701,7 @@ struct ConvWgradDirectArgs {
     WgradGeomB B;
     int Ktotal, kslice;
     float* partial;            // [slice][Mrows][Ncols]
-    int tiles_m, tiles_n;
+    int tiles_m, tiles_n, slices;
 };
 
 template <int WM, int WN, int NWN, int NST, int NWM>
@@ -709,7 +709,23 @@ __global__ __launch_bounds__(NWM * NWN * 64) void conv_wgrad_direct_kernel(ConvW
     using ML = GemmMainloop<bf16_t, WM, WN, false, true, true, NWN, NST, NWM>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
-    const int tile = blockIdx.x, slice = blockIdx.y;
+    // Workgroups are handed to the eight XCDs in turn (workgroup i to XCD i % 8), each with an L2 of its own.
+    // All tiles of a slice read the same positions of x and dy, so they go to the same XCD, one after the
+    // other: XCD c takes the slices c, c + 8, ... and runs through the tiles of one before the next.
+    const int tiles = a.tiles_m * a.tiles_n;
+    int tile, slice;
+    {
+        const int id = blockIdx.x, xcd = id & 7, j = id >> 3;
+        const int whole = (a.slices >> 3) << 3;              // slices that fill whole groups of eight
+        if (id < whole * tiles) {
+            tile = j % tiles;
+            slice = xcd + 8 * (j / tiles);
+        } else {                                             // the rest: slice-major
+            const int r = id - whole * tiles;
+            tile = r % tiles;
+            slice = whole + r / tiles;
+        }
+    }
     const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
     const int m0 = tm * ML::TILE_M, n0 = tn * ML::TILE_N;
     const int kbeg = slice * a.kslice, kend = min(kbeg + a.kslice, a.Ktotal);

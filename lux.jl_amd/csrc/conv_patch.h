@@ -1,5 +1,5 @@
 // bf16 3 x 3 convolution (fprop and dgrad) for unit stride, unit dilation and "same" output size, with the
-// input window of a tile held in LDS: 256 output positions x 128 output channels per tile on eight waves.
+// input window of a tile held in LDS: 256 or 272 output positions x 128 output channels per tile on eight waves.
 //
 // An implicit GEMM that gathers its A operand per filter tap reads every input element nine times from
 // L2; here a tile first brings the rows of the image that it needs ("patch": the rows of its output
@@ -25,6 +25,12 @@
 // outside the image is read at position 464.  Per tile a lane keeps the position of each of its four output
 // positions under each of the three tap rows (or 464); a tap's address is three instructions from there.
 //
+// Work split: the output positions are cut into runs of 16 ("fragments"), every workgroup takes the same number
+// of consecutive fragments (one more for the first few) and cuts its share into tiles of at most 17: 12544
+// fragments on 256 compute units are 49 each, three tiles of 17 + 16 + 16, where tiles of 16 dealt out in turn
+// would leave 240 compute units idle for a quarter of the time.  The seventeenth fragment of a tile is
+// multiplied by two waves on different SIMDs on top of their own four.
+//
 // One step: 32 MFMAs 16x16x32 per wave (wave tile 64 positions x 64 channels, two k groups of 32); the
 // fragments of a k group are read while the MFMAs of the one before run; the step's barrier sits before its
 // last eight MFMAs; a load instruction in front of every eight MFMAs.  The nine taps of a half are unrolled.
@@ -36,7 +42,8 @@
 namespace luxhip {
 namespace cpatch {
 
-constexpr int THREADS = 512, TILE_M = 256, TILE_N = 128, TAPS = 9;
+constexpr int THREADS = 512, TILE_N = 128, TAPS = 9;
+constexpr int MAX_FRAGS = 17, TILE_M_MAX = 16 * MAX_FRAGS;           // fragments of 16 output positions per tile
 constexpr int PATCH_PIX = 464, PATCH_BYTES = PATCH_PIX * 128;          // 59392: 29 groups of 16 positions
 constexpr int ZERO_REL = PATCH_BYTES, ZERO_BYTES = 2048;               // behind each patch buffer
 constexpr int BUF_STRIDE = PATCH_BYTES + ZERO_BYTES;                   // 61440
@@ -60,7 +67,7 @@ struct Args {
     int rev, hlo, dq_min;    // dgrad walks the taps backwards; halo columns on the left; first source row relative to the output row
     int pitch;               // P + kW - 1
     int Ncols, col_off, Ctot_out, act;
-    int tiles_m, tiles_n;
+    int frags, groups_m, tiles_n;   // fragments of 16 positions in all; workgroups that share them; tiles along the output channels
     FastDiv divP, divQ, divPQ, divPitch;
 };
 
@@ -77,7 +84,14 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
     const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds);   // LDS byte address
     const int tid = threadIdx.x, l = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = (w & 3) * 64, wave_n = (w >> 2) * 64;
-    const int total = a.tiles_m * a.tiles_n;
+    // this workgroup's fragments [frag0, frag0 + nfrag) and its tiles
+    const int bm = blockIdx.x % a.groups_m, tn = blockIdx.x / a.groups_m;
+    const int fbase = a.frags / a.groups_m, frem = a.frags % a.groups_m;
+    const int frag0 = bm * fbase + min(bm, frem), nfrag = fbase + (bm < frem ? 1 : 0);
+    const int ntile = (nfrag + MAX_FRAGS - 1) / MAX_FRAGS, tbase = nfrag / ntile, trem = nfrag % ntile;
+    // tile i: first output position and number of fragments
+    auto tile_first = [&](int i) { return 16 * (frag0 + i * tbase + min(i, trem)); };
+    auto tile_frags = [&](int i) { return tbase + (i < trem ? 1 : 0); };
     const int Cg2 = a.Cg * 2;                                        // bytes of a tap's channels in a filter row
     const int K2 = TAPS * Cg2;                                       // bytes of a filter row
     const int64_t row_bytes = (int64_t)a.P * a.Ctot * 2;             // bytes of an image row of the source
@@ -108,8 +122,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
         __builtin_amdgcn_global_load_lds((glb_vp)p, (lds_vp)(lds + buf * BUF_STRIDE + g * 1024), 16, 0, 0);
     };
     auto patch_base = [&](int tile, int h, int& rbase) -> const char* {
-        const int tm = tile % a.tiles_m;
-        rbase = (int)a.divP.div((uint32_t)(tm * TILE_M)) + a.dq_min;
+        rbase = (int)a.divP.div((uint32_t)tile_first(tile)) + a.dq_min;
         return reinterpret_cast<const char*>(a.src) + (int64_t)rbase * row_bytes + h * 128;
     };
 
@@ -125,20 +138,17 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                                          0);
         ring_b = ring_b + 1 == RING ? 0 : ring_b + 1;
     };
-    // filter bytes of a tile's columns, first channel of half h, tap 0, k group 0
-    auto filter_base = [&](int tile, int h) -> const char* {
-        const int tn = tile / a.tiles_m;
-        return reinterpret_cast<const char*>(a.wm) + (int64_t)tn * TILE_N * K2 + h * 128;
-    };
+    // filter bytes of this workgroup's columns, first channel, tap 0
+    const char* const gp_first = reinterpret_cast<const char*>(a.wm) + (int64_t)tn * TILE_N * K2;
 
     // ---- fragment reads
     const uint32_t lane15 = l & 15, laneq = l >> 4;
     // B: row 16 j + l % 16 of the wave's half-block, chunk 4 g + l / 16 for k group g (g = 1: XOR 64)
     const uint32_t offB = (uint32_t)(lane15 * 128 + ((laneq ^ ((lane15 >> 1) & 7)) << 4));
 
-    int tile = blockIdx.x;
+    int tile = 0;
     int hc = 0;                              // halves consumed so far by this workgroup: patch buffer hc & 1
-    const char* gp_cur = filter_base(tile, 0);
+    const char* gp_cur = gp_first;
     // prologue: the first patch, three filter half-blocks (step 0 both, step 1 the first)
     {
         int rbase;
@@ -150,15 +160,23 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
         filter_issue(gp_cur + Cg2, 0);
     }
     const bool upper = wave_n != 0;          // this wave's columns are in the second half-block of a step
+    // the two waves (on different SIMDs) that take the seventeenth fragment of a tile, one per half of the columns
+    const bool extra_wave = w == 3 || w == 6;
     int slot0 = 0, slot1 = 1;                // ring slots of the two half-blocks of the current step
 
-    f32x4_v acc[4][4];
-    bf16x8_v fa[2][4], fb[2][4];
+    f32x4_v acc[4][4], accE[4];
+    bf16x8_v fa[2][4], fb[2][4], faE[2];
     for (;;) {
-        const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
-        const int m0 = tm * TILE_M, n0 = tn * TILE_N;
+        const int m0 = tile_first(tile), n0 = tn * TILE_N;
+        const int m_end = min(a.M, m0 + 16 * tile_frags(tile));
+        const bool extra = extra_wave && tile_frags(tile) > 16;
         const int r_first = (int)a.divP.div((uint32_t)m0);
-        const int tnext = tile + gridDim.x;
+        const int tnext = tile + 1;
+        const int total = ntile;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) accE[j][r] = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -167,10 +185,10 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
         // this lane's patch positions: fragment f (output position m0 + wave_m + 16 f + l % 16) under tap row jb, first
         // tap column; 464 (the zeros) where that row lies outside the image
-        uint32_t xrow[4][3];
+        uint32_t xrow[5][3];
 #pragma unroll
-        for (int f = 0; f < 4; ++f) {
-            const int m = m0 + wave_m + 16 * f + (int)lane15;
+        for (int f = 0; f < 5; ++f) {
+            const int m = m0 + (f < 4 ? wave_m + 16 * f : 256) + (int)lane15;
             const int mc = min(m, a.M - 1);
             const int R = (int)a.divP.div((uint32_t)mc), p = mc - R * a.P;
             const int q = R - (int)a.divQ.div((uint32_t)R) * a.Q;
@@ -203,6 +221,14 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                      : "+v"(fa[set][0]), "+v"(fa[set][1]), "+v"(fa[set][2]), "+v"(fa[set][3]), "+v"(fb[set][0]),   \
                        "+v"(fb[set][1]), "+v"(fb[set][2]), "+v"(fb[set][3]))
 #define CP_FENCE() __builtin_amdgcn_sched_barrier(0)
+        // the seventeenth fragment: one more read behind the eight of a set (so the waits above cover it), four more MFMAs
+#define CP_READ_E(set, ae, OFF) asm volatile("ds_read_b128 %0, %1 offset:" #OFF : "=&v"(faE[set]) : "v"(ae))
+#define CP_MFMA_E(set)                                                                                               \
+        do {                                                                                                        \
+            asm volatile("" : "+v"(faE[set]));                                                                      \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                           \
+                accE[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(faE[set], fb[set][j], accE[j], 0, 0, 0);          \
+        } while (0)
         auto mfmas = [&](int set, int i0) {      // two rows of accumulator tiles: eight MFMAs
 #pragma unroll
             for (int i = i0; i < i0 + 2; ++i)
@@ -216,14 +242,15 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
         __builtin_amdgcn_s_waitcnt(1 | (0x7 << 4));          // vmcnt(1) lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
 
-        uint32_t aA[4], aN[4];
+        uint32_t aA[5], aN[5];
         {
             const uint32_t bufbase = lds_addr + (uint32_t)(hc & 1) * BUF_STRIDE;
 #pragma unroll
-            for (int f = 0; f < 4; ++f) aA[f] = a_addr(f, 0, bufbase);
+            for (int f = 0; f < 5; ++f) aA[f] = a_addr(f, 0, bufbase);
         }
         CP_READ_A(0, aA[0], aA[1], aA[2], aA[3], 0);
         CP_READ_B(0, lds_addr + RING_OFF + (uint32_t)(upper ? slot1 : slot0) * HB_BYTES + at_use(offB));
+        if (extra) CP_READ_E(0, aA[4], 0);
 
         for (int h = 0; h < a.H; ++h) {
             // the half after this one: where its patch and its filter blocks come from
@@ -235,13 +262,14 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
             const char* gp_next = gp_cur;                    // past the last tile: the same blocks again, never read
             if (have_p) {
                 pb_p = patch_base(tile_p, h_p, rbase_p);
-                gp_next = h_p != 0 ? gp_cur + 128 : (a.tiles_n > 1 ? filter_base(tile_p, 0) : gp_cur - h * 128);
+                gp_next = h_p != 0 ? gp_cur + 128 : gp_first;
             }
             const uint32_t buf_cur = lds_addr + (uint32_t)(hc & 1) * BUF_STRIDE, buf_next = lds_addr + (uint32_t)((hc + 1) & 1) * BUF_STRIDE;
             static_for<TAPS>([&](auto TT) {
                 constexpr int t = decltype(TT)::value;
                 CP_READ_A(1, aA[0], aA[1], aA[2], aA[3], 1024);
                 CP_READ_B(1, lds_addr + RING_OFF + (uint32_t)(upper ? slot1 : slot0) * HB_BYTES + (at_use(offB) ^ 64u));
+                if (extra) CP_READ_E(1, aA[4], 1024);
                 if constexpr (t < PATCH_INSTR) {
                     if (have_p) patch_issue(t, pb_p, rbase_p, (hc + 1) & 1);
                 }
@@ -252,9 +280,11 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 {
                     const uint32_t nb = t + 1 < TAPS ? buf_cur : buf_next;
 #pragma unroll
-                    for (int f = 0; f < 4; ++f) aN[f] = a_addr(f, (t + 1) % TAPS, nb);
+                    for (int f = 0; f < 5; ++f) aN[f] = a_addr(f, (t + 1) % TAPS, nb);
                 }
                 CP_FENCE(); mfmas(0, 2); CP_FENCE();
+                if (extra) CP_MFMA_E(0);
+                CP_FENCE();
                 // first half-block of the step after the next
                 filter_issue(t + 2 < TAPS ? gp_cur + (t + 2) * Cg2 : gp_next + (t + 2 - TAPS) * Cg2, 0);
                 CP_READY(1, 0);
@@ -268,8 +298,14 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 CP_READ_A(0, aN[0], aN[1], aN[2], aN[3], 0);
                 CP_READ_B(0, lds_addr + RING_OFF + (uint32_t)(upper ? slot1 : slot0) * HB_BYTES + at_use(offB));
                 CP_FENCE(); mfmas(1, 2); CP_FENCE();
+                if (extra) {
+                    // the set's reads were complete at the boundary; its registers are not among those just requested
+                    CP_MFMA_E(1);
+                    CP_READ_E(0, aN[4], 0);
+                }
+                CP_FENCE();
 #pragma unroll
-                for (int f = 0; f < 4; ++f) aA[f] = aN[f];
+                for (int f = 0; f < 5; ++f) aA[f] = aN[f];
             });
             ++hc;
             gp_cur = gp_next;
@@ -285,7 +321,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int m = mrow + 16 * i;
-                mok[i] = m < a.M;                                      // M and PQ are multiples of 4: all four or none
+                mok[i] = m < m_end;                                    // m_end and PQ are multiples of 4: all four or none
                 const int img = (int)a.divPQ.div((uint32_t)(mok[i] ? m : 0));
                 rowoff[i] = (uint32_t)(m - img * a.PQ) + (uint32_t)a.PQ * (uint32_t)a.Ctot_out * (uint32_t)img;
             }
@@ -319,9 +355,43 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 }
             }
         }
+        if (extra) {            // the seventeenth fragment: positions m0 + 256 + 4 (l / 16) + r
+            const int m = m0 + 256 + 4 * (int)laneq;
+            if (m < m_end) {
+                const int img = (int)a.divPQ.div((uint32_t)m);
+                const uint32_t rowoffE = (uint32_t)(m - img * a.PQ) + (uint32_t)a.PQ * (uint32_t)a.Ctot_out * (uint32_t)img;
+                const int ncol = n0 + (upper ? 64 : 0) + (int)lane15;
+                const int act = a.act;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int col = ncol + 16 * j;
+                    if (col < a.Ncols) {
+                        const float b = a.bias ? ld(a.bias + a.col_off + col) : 0.0f;
+                        const uint32_t off = (uint32_t)a.PQ * (uint32_t)(a.col_off + col) + rowoffE;
+                        float v[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) v[r] = accE[j][r] + b;
+                        if (a.pre != nullptr) {
+                            uint2 pv;
+                            pv.x = f32x2_to_bf16x2(v[0], v[1]);
+                            pv.y = f32x2_to_bf16x2(v[2], v[3]);
+                            *reinterpret_cast<uint2*>(a.pre + off) = pv;
+                        }
+                        if (act == LUXHIP_ACT_RELU) act_vec_as<LUXHIP_ACT_RELU>(v);
+                        else if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v);
+                        uint2 ov;
+                        ov.x = f32x2_to_bf16x2(v[0], v[1]);
+                        ov.y = f32x2_to_bf16x2(v[2], v[3]);
+                        *reinterpret_cast<uint2*>(a.out + off) = ov;
+                    }
+                }
+            }
+        }
         if (tnext >= total) break;
         tile = tnext;
     }
+#undef CP_READ_E
+#undef CP_MFMA_E
 #undef CP_READ_A
 #undef CP_READ_B
 #undef CP_READY
@@ -347,7 +417,7 @@ inline bool applicable(const Problem& p) {
     const int64_t PQ = (int64_t)p.P * p.Q;
     if (p.kW != 3 || p.kH != 3 || p.Cg % 64 != 0 || p.Ctot % 8 != 0 || PQ % 4 != 0 || p.N < 1) return false;
     if (p.Ncols > TILE_N && p.Ncols % TILE_N != 0) return false;         // the filter loader clamps rows against Ncols only
-    const int rows = (p.P - 1 + TILE_M - 1) / p.P + 1 + (p.kH - 1);      // image rows under a tile that starts at the end of a row, plus halo
+    const int rows = (p.P - 1 + TILE_M_MAX - 1) / p.P + 1 + (p.kH - 1);      // image rows under a tile that starts at the end of a row, plus halo
     if ((int64_t)rows * pitch > PATCH_PIX) return false;
     if ((int64_t)(rows + 1) * p.P * p.Ctot * 2 >= (int64_t(1) << 31) || (int64_t)TILE_N * T * p.Cg * 2 >= (int64_t(1) << 31)) return false;
     return al(p.src, 16) && al(p.wm, 16) && al(p.out, 8) && al(p.pre, 8);
