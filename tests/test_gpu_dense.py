@@ -159,7 +159,7 @@ def test_config4_dense_full_size(gpu):
     dz_cols = f64(O.round_to_bf16((f64(delta[:, cols]) * O.act_derivative("gelu", O.act_value("gelu", pre_cq), pre_cq)).astype(np.float32)))
     assert_close(gx.to_numpy()[:, cols], f64(W).T @ dz_cols, "bf16", "config4 dx cols")
     assert_close(gb.to_numpy()[rows], (f64(delta[rows]) * O.act_derivative("gelu", O.act_value("gelu", pre_q), pre_q)).sum(axis=1),
-                 "bf16", "config4 db rows", rel=3e-2, scale=rms(delta) * 90)
+                 "bf16", "config4 db rows", scale=rms(delta) * 90)
     # linearity: pullback(2 * delta) == 2 * pullback(delta) (exact: scaling by 2 commutes with rounding)
     gW2, gx2, _ = back(dev(gpu, 2 * delta, "bf16"))
     np.testing.assert_array_equal(gW2.to_numpy()[rows], 2 * gW.to_numpy()[rows])

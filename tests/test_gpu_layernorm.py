@@ -91,14 +91,14 @@ def test_config4_layernorm_full_size(gpu):
     sub = slice(0, R, 257)
     assert_close(yh[:, sub], O.layernorm(f64(x[:, sub]), f64(g), f64(b), "identity", (0,), eps), "bf16", "config4 LN y")
     wdx, _, _ = O.layernorm_pullback(f64(x[:, sub]), f64(g), f64(b), "identity", (0,), eps, f64(delta[:, sub]))
-    assert_close(gxh[:, sub], wdx, "bf16", "config4 LN dx", rel=3e-2)
+    assert_close(gxh[:, sub], wdx, "bf16", "config4 LN dx")
     xh = (yh.astype(np.float64) - f64(b)) / f64(g)
     assert np.abs(xh.mean(axis=0)).max() < 2e-2
     assert np.abs(xh.var(axis=0) - 1).max() < 3e-2
     assert np.abs(gxh.sum(axis=0)).max() < 0.5            # 4096 bf16-rounded terms of size ~0.02
     _, wdg, wdb = O.layernorm_pullback(f64(x), f64(g), f64(b), "identity", (0,), eps, f64(delta))
-    assert_close(gg.to_numpy(), wdg, "bf16", "config4 LN dgamma", rel=3e-2, scale=rms(delta) * 90)
-    assert_close(gb.to_numpy(), wdb, "bf16", "config4 LN dbeta", rel=3e-2, scale=rms(delta) * 90)
+    assert_close(gg.to_numpy(), wdg, "bf16", "config4 LN dgamma", scale=rms(delta) * 90)
+    assert_close(gb.to_numpy(), wdb, "bf16", "config4 LN dbeta", scale=rms(delta) * 90)
 
 
 REFERENCE_CONFIGS = [(xs, aff, act) for xs in ((3, 3, 2, 1), (2, 2, 2, 1)) for aff in (None, "channel")
