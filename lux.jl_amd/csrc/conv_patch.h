@@ -128,7 +128,8 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
 
     // ---- filter loader: one instruction per thread and half-block (64 rows: row tid / 8, 16-byte chunk tid % 8);
     // rows past the last output channel read the last one's (their products go to columns that are never stored)
-    const int brow0 = min(tid >> 3, a.Ncols - 1), brow1 = min(64 + (tid >> 3), a.Ncols - 1);   // tiles_n > 1 only with Ncols % 128 == 0
+    const int last_row = a.Ncols - 1 - tn * TILE_N;                  // of this workgroup's (up to 128) output channels
+    const int brow0 = min(tid >> 3, last_row), brow1 = min(64 + (tid >> 3), last_row);
     const uint32_t bchunk = (uint32_t)(((tid & 7) ^ (((tid >> 3) >> 1) & 7)) << 4);
     const uint32_t boff0 = (uint32_t)(brow0 * K2) + bchunk, boff1 = (uint32_t)(brow1 * K2) + bchunk;
     int ring_b = 0;
@@ -416,7 +417,6 @@ inline bool applicable(const Problem& p) {
     const int T = p.kW * p.kH, pitch = p.P + p.kW - 1;
     const int64_t PQ = (int64_t)p.P * p.Q;
     if (p.kW != 3 || p.kH != 3 || p.Cg % 64 != 0 || p.Ctot % 8 != 0 || PQ % 4 != 0 || p.N < 1) return false;
-    if (p.Ncols > TILE_N && p.Ncols % TILE_N != 0) return false;         // the filter loader clamps rows against Ncols only
     const int rows = (p.P - 1 + TILE_M_MAX - 1) / p.P + 1 + (p.kH - 1);      // image rows under a tile that starts at the end of a row, plus halo
     if ((int64_t)rows * pitch > PATCH_PIX) return false;
     if ((int64_t)(rows + 1) * p.P * p.Ctot * 2 >= (int64_t(1) << 31) || (int64_t)TILE_N * T * p.Cg * 2 >= (int64_t(1) << 31)) return false;
