@@ -74,7 +74,9 @@ struct BlockLoader {
     }
     // instruction i of the block at `g` (uniform: tile base + k) -> LDS block `dst`
     __device__ __forceinline__ void issue(int i, const char* g, char* dst) const {
-        __builtin_amdgcn_global_load_lds((glb_vp)(g + step[i] + at_use(voff)), (lds_vp)(dst + lds_off + i * 8192), 16, 0, 0);
+        // cache policy sc0 sc1 (the data is used once per compute unit: nothing is gained by keeping it in the
+        // vector L1); measured 2.5-3.7 % faster than the default policy, the non-temporal policies 20 % slower
+        __builtin_amdgcn_global_load_lds((glb_vp)(g + step[i] + at_use(voff)), (lds_vp)(dst + lds_off + i * 8192), 16, 0, 17);
     }
 };
 
