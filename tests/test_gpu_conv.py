@@ -186,3 +186,48 @@ def test_config5_full_size(gpu, dtype):
     dzq = dz[..., sub].astype(np.float32)
     gw2 = gpu.conv_filter_grad(dev(gpu, x[..., sub], dtype), dev(gpu, dzq, dtype), gd2)
     assert_close(gw2.to_numpy(), O.conv_filter_grad(f64(x[..., sub]), f64(dzq), od2), dtype, "config5 dw (2 images)")
+
+
+# Shapes that the bf16 kernel with the tile's input window in LDS takes (3 x 3, unit stride and dilation, output as
+# large as the input, channels per group in multiples of 64), chosen for its special cases:
+WINDOW_CASES = [
+    # x shape, w shape, pad, groups, flip
+    ((20, 12, 128, 5), (3, 3, 128, 192), 1, 1, True),              # two 64-channel parts; two column tiles, the second half empty
+    ((12, 10, 128, 3), (3, 3, 64, 128), 1, 2, False),              # groups: 64 channels in, 64 columns out per group
+    ((14, 14, 64, 3), (3, 3, 64, 80), (0, 2, 2, 0), 1, False),     # asymmetric padding, 80 columns (a partial fragment row of channels)
+    ((56, 56, 64, 1), (3, 3, 64, 64), 1, 1, False),                # one image: 196 fragments on 13 workgroups (15 or 16 each)
+    ((6, 6, 64, 2), (3, 3, 64, 16), 1, 1, False),                  # 72 positions: one partial tile, rows past the last position
+    ((32, 34, 64, 64), (3, 3, 64, 64), 1, 1, True),                # 4352 fragments = 17 per compute unit: tiles with a seventeenth fragment
+]
+
+
+@pytest.mark.parametrize("case", range(len(WINDOW_CASES)))
+def test_window_kernel_shapes(gpu, case):
+    """fprop and dgrad on those shapes against the fp64 oracle (the larger problems on a few images, whose results
+    do not depend on the other images) and against the gather-per-tap kernels that the `conv_tile` switch selects."""
+    xs, ws, pad, groups, flip = WINDOW_CASES[case]
+    rng = np.random.default_rng(300 + case)
+    gd, od = cdims(gpu, xs, ws, padding=pad, groups=groups, flipkernel=flip)
+    assert od.y_shape()[:2] == xs[:2]
+    fan_in = 9 * ws[2]
+    x, w, b, dy = host_inputs("bf16", rng.normal(size=xs), rng.normal(size=ws) * np.sqrt(2.0 / fan_in), rng.normal(size=ws[3]) * 0.1,
+                              rng.normal(size=od.y_shape()))
+    dx_, dw_, db_, ddy_ = (dev(gpu, a, "bf16") for a in (x, w, b, dy))
+    y = gpu.fused_conv_bias_activation("relu", dw_, dx_, db_, gd).to_numpy()
+    gx = gpu.conv_data_grad(ddy_, dw_, gd).to_numpy()
+    gpu.set_option("conv_tile", 84)
+    try:
+        y_tap = gpu.fused_conv_bias_activation("relu", dw_, dx_, db_, gd).to_numpy()
+        gx_tap = gpu.conv_data_grad(ddy_, dw_, gd).to_numpy()
+    finally:
+        gpu.set_option("conv_tile", 0)
+    imgs = sorted({0, xs[3] // 2, xs[3] - 1})
+    sub = O.ConvDims(xs[:3] + (len(imgs),), ws, padding=pad, groups=groups, flipkernel=flip)
+    want_y = O.fused_conv_bias_activation("relu", f64(w), f64(x[..., imgs]), f64(b), sub)
+    want_gx = O.conv_data_grad(f64(dy[..., imgs]), f64(w), sub)
+    tag = f"window case {case} "
+    assert_close(y[..., imgs], want_y, "bf16", tag + "y")
+    assert_close(gx[..., imgs], want_gx, "bf16", tag + "dgrad")
+    # the two kernels add the same products in a different order: equal up to the bf16 rounding of the result
+    assert_close(y, f64(y_tap), "bf16", tag + "y vs gather kernel")
+    assert_close(gx, f64(gx_tap), "bf16", tag + "dgrad vs gather kernel")
