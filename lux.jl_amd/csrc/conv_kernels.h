@@ -617,40 +617,65 @@ struct WgradDirectLoaderA {
     static constexpr int INSTR = ROWS * BK / 8 / THREADS, STEP = THREADS / CPR;   // STEP: k rows per instruction
     static_assert(INSTR >= 1 && (ROWS * BK / 8) % THREADS == 0 && STEP % 4 == 0, "stage must split evenly over the workgroup");
     const WgradGeomA& g;
-    int kbeg, krow;            // first k' of the slice, this thread's k row inside an instruction's block
-    int dpx, dqy, coff;        // tap shift of the source position, channel offset
+    int dpx, dqy;              // tap shift of the source position
     bool valid_m;
     uint32_t lds_off;
-    __device__ __forceinline__ WgradDirectLoaderA(const WgradGeomA& gg, int m0, int kb_) : g(gg), kbeg(kb_) {
+    // The stages of a slice are issued in order (k0 = 0, BK, 2 BK, ...): the output position of each load is
+    // kept as (ow, oh) and the element offset of its source position at tap shift 0, and moved on by BK
+    // positions per stage with two compares (one row wrap at most for rows of at least BK positions).
+    mutable int ow[INSTR], oh[INSTR];
+    mutable int64_t pos[INSTR];        // ((n * SQ + oh * sh) * SP + ow * sw) * Ctot + the tap's shift and channel
+    int64_t d_step, d_row, d_img;      // what BK positions, a row wrap and an image wrap add to pos
+    __device__ __forceinline__ WgradDirectLoaderA(const WgradGeomA& gg, int m0, int kb_) : g(gg) {
         const int q = threadIdx.x, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-        krow = q / CPR;
+        const int krow = q / CPR;
         const int slot = q % CPR;
         const int r = (slot * 8) ^ ((krow & 3) << mn_swizzle_shift(ROWS));   // (krow + i*STEP) & 3 == krow & 3
         const int m = m0 + r;
         valid_m = m < g.Mrows;
         const int t = (int)g.divCg.div((uint32_t)(valid_m ? m : 0));
-        coff = (valid_m ? m : 0) - t * g.Cg;
+        const int coff = (valid_m ? m : 0) - t * g.Cg;
         const int kb = (int)g.divkW.div((uint32_t)t), ka = t - kb * g.kW;
         dpx = ka * g.dw - g.pw;
         dqy = kb * g.dh - g.ph;
         lds_off = (uint32_t)w * 1024u;
+        const int64_t shift = ((int64_t)dqy * g.SP + dpx) * g.Ctot + coff;
+#pragma unroll
+        for (int i = 0; i < INSTR; ++i) {
+            const int kp = kb_ + krow + i * STEP;
+            const int n = (int)g.divOWOH.div((uint32_t)kp);
+            const int rem = kp - n * g.OWOH;
+            oh[i] = (int)g.divOW.div((uint32_t)rem);
+            ow[i] = rem - oh[i] * g.OW;
+            pos[i] = (((int64_t)n * g.SQ + oh[i] * g.sh) * g.SP + ow[i] * g.sw) * g.Ctot + shift;
+        }
+        const int OH = g.OWOH / g.OW;
+        d_step = (int64_t)BK * g.sw * g.Ctot;
+        d_row = ((int64_t)g.sh * g.SP - (int64_t)g.OW * g.sw) * g.Ctot;
+        d_img = ((int64_t)g.SQ - (int64_t)OH * g.sh) * g.SP * g.Ctot;
     }
-    __device__ __forceinline__ void issue(int k0, T* lds_tile) const {
+    __device__ __forceinline__ void issue(int /*k0: the next stage in order*/, T* lds_tile) const {
         typedef __attribute__((address_space(3))) void* lds_vp;
         typedef const __attribute__((address_space(1))) void* glb_vp;
         char* l = reinterpret_cast<char*>(lds_tile) + lds_off;
+        const int OH = g.OWOH / g.OW;
 #pragma unroll
         for (int i = 0; i < INSTR; ++i) {
-            const int kp = kbeg + k0 + krow + i * STEP;
-            const int n = (int)g.divOWOH.div((uint32_t)kp);
-            const int rem = kp - n * g.OWOH;
-            const int oh = (int)g.divOW.div((uint32_t)rem);
-            const int ow = rem - oh * g.OW;
-            const int sp = ow * g.sw + dpx, sq = oh * g.sh + dqy;
+            const int sp = ow[i] * g.sw + dpx, sq = oh[i] * g.sh + dqy;
             const bool valid = valid_m && (unsigned)sp < (unsigned)g.SP && (unsigned)sq < (unsigned)g.SQ;
-            const T* src = g.src + ((((int64_t)n * g.SQ + sq) * g.SP + sp) * g.Ctot + coff);
-            const void* p = valid ? static_cast<const void*>(src) : g.zero;
+            const void* p = valid ? static_cast<const void*>(g.src + pos[i]) : g.zero;
             __builtin_amdgcn_global_load_lds((glb_vp)p, (lds_vp)(l + i * (THREADS * 16)), 16, 0, 0);
+            // on to the next stage's position
+            ow[i] += BK;
+            pos[i] += d_step;
+            while (ow[i] >= g.OW) {             // once for rows of at least BK positions
+                ow[i] -= g.OW;
+                pos[i] += d_row;
+                if (++oh[i] == OH) {
+                    oh[i] = 0;
+                    pos[i] += d_img;
+                }
+            }
         }
     }
 };

@@ -445,34 +445,71 @@ struct GemmMainloop {
         __builtin_amdgcn_s_waitcnt(0xF | (0x7 << 4) | (0x3 << 14));   // lgkmcnt(0): own LDS reads returned
         __builtin_amdgcn_s_barrier();
     }
+    // The barrier of a stage sits between its k groups (16 k each), not in front of it: behind the barrier the
+    // fragments of the next stage's first group are requested, then the MFMAs of this stage's last group run
+    // while those reads are in flight; the matrix pipe does not drain at the stage boundary.
     template <class LA, class LB>
     __device__ __forceinline__ static void pipeline_loop(const LA& la, const LB& lb, int K, T* lds, f32x16_v (&acc)[WM][WN]) {
         const int w = threadIdx.x >> 6;
         const int wave_m = (w % NWM) * (WM * 32), wave_n = (w / NWM) * (WN * 32);
         zero(acc);
+        constexpr int KK = Tr::BK / 16;
+        static_assert(KK >= 2, "a stage has at least two k groups");
         constexpr int IPS = LA::INSTR + LB::INSTR;               // load instructions per thread and stage
         constexpr int PENDING = (NST - 2) * IPS;                 // loads of later stages that may stay in flight
         static_assert(PENDING < 64, "vmcnt range");
         // s_waitcnt vmcnt(PENDING) lgkmcnt(0): expcnt left at its maximum; lgkmcnt(0) retires this wave's
-        // LDS reads of the previous stage before the barrier lets other waves refill that buffer
+        // LDS reads of the stage before the barrier lets other waves refill its buffer
         constexpr int WAIT_IMM = (PENDING & 0xF) | (0x7 << 4) | ((PENDING >> 4) << 14);
         const int KT = K / Tr::BK;
+        bf16x8_v fa[KK][WM], fb[KK][WN];
+        auto read = [&](int kk, const T* stage) {
+            const bf16_t* As = reinterpret_cast<const bf16_t*>(stage);
+            const bf16_t* Bs = reinterpret_cast<const bf16_t*>(stage + A_ELEMS);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) fb[kk][j] = load_frag_bf16<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kk);
+#pragma unroll
+            for (int i = 0; i < WM; ++i) fa[kk][i] = load_frag_bf16<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kk);
+        };
+        auto mma = [&](int kk) {
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+        };
         int cur = 0, fill = NST - 1;                             // buffer of stage kt, buffer to refill
+        // stage 0 has landed (every wave's share: barrier); its first fragments
+        if (NST - 2 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+        else __builtin_amdgcn_s_waitcnt(0);                      // fewer stages than the pipeline holds
+        __builtin_amdgcn_s_barrier();
+        read(0, lds);
         for (int kt = 0; kt < KT; ++kt) {
-            if (kt + NST - 2 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
-            else __builtin_amdgcn_s_waitcnt(0);                  // tail: fewer stages are in flight
-            // bare barrier: __syncthreads() would add a fence that drains every load in flight.
-            // This wave's share of stage kt has landed and its LDS reads of stage kt-1 have
-            // returned (wait above), so nothing else has to be waited for.
-            __builtin_amdgcn_s_barrier();
+            const T* cb = lds + cur * STAGE_ELEMS;
+            // the buffer of stage kt - 1 was released at that stage's barrier
             if (kt + NST - 1 < KT) {
                 la.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS);
                 lb.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS + A_ELEMS);
             }
-            const T* cb = lds + cur * STAGE_ELEMS;
-            compute_bf16(reinterpret_cast<const bf16_t*>(cb), reinterpret_cast<const bf16_t*>(cb + A_ELEMS), wave_m, wave_n, acc);
+#pragma unroll
+            for (int kk = 1; kk < KK; ++kk) read(kk, cb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < KK - 1; ++kk) mma(kk);
+            __builtin_amdgcn_sched_barrier(0);
             cur = cur + 1 == NST ? 0 : cur + 1;
             fill = fill + 1 == NST ? 0 : fill + 1;
+            if (kt + 1 < KT) {
+                // stage kt + 1 has landed, this wave's reads of stage kt have returned
+                if (kt + NST - 1 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+                else __builtin_amdgcn_s_waitcnt(0);              // tail: fewer stages are in flight
+                // bare barrier: __syncthreads() would add a fence that drains every load in flight
+                __builtin_amdgcn_s_barrier();
+                read(0, lds + cur * STAGE_ELEMS);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mma(KK - 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
     template <class LA, class LB>
