@@ -5,6 +5,7 @@
 #include "common.h"
 #include "conv_kernels.h"
 #include "conv_patch.h"
+#include "conv_wgrad_patch.h"
 
 namespace luxhip {
 
@@ -311,11 +312,24 @@ static int wgrad_plan(const ConvGeom& g, int* slices, int* kslice, bool* small) 
     return LUXHIP_OK;
 }
 
+// The filter gradient with the tile's input window in LDS (bf16, 3 x 3, unit stride and dilation, output as large
+// as the input): one partial sum per image.  Pointer alignment is checked again at the launch.
+template <typename T>
+static bool wgrad_window_shape(const ConvGeom& g) {
+    if (sizeof(T) != 2 || option_conv_tile() != 0) return false;
+    if (g.kW != 3 || g.kH != 3 || g.sw != 1 || g.sh != 1 || g.dw != 1 || g.dh != 1 || g.OW != g.W || g.OH != g.H) return false;
+    wpatch::Problem p;
+    p.src = nullptr; p.dz = nullptr; p.partial = nullptr; p.zero = nullptr;
+    p.Ctot = g.Cin; p.Cg = g.Cin_g; p.Cout = g.Cout; p.Ncols = g.Cout_g; p.P = g.W; p.Q = g.H; p.N = g.N; p.pad_w = g.pw; p.pad_h = g.ph;
+    return wpatch::applicable(p, num_cus() > 0 ? num_cus() : 256);
+}
+
 template <typename T>
 static size_t wgrad_partial_bytes(const ConvGeom& g) {
     int slices = 1, kslice = 0;
     bool small = false;
     if (wgrad_plan<T>(g, &slices, &kslice, &small) != LUXHIP_OK) return 0;
+    if (wgrad_window_shape<T>(g)) slices = std::max(slices, g.N);
     return align256((size_t)slices * g.kW * g.kH * g.Cin_g * g.Cout_g * sizeof(float));
 }
 
@@ -339,9 +353,21 @@ static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy,
     int rc = wgrad_plan<T>(g, &slices, &kslice, &small);
     if (rc != LUXHIP_OK) return rc;
     const bool direct = wgrad_direct_ok<T>(g, xT, dy);
+    const bool window = wgrad_window_shape<T>(g) && aligned16(xT) && aligned16(dy) && aligned16(partial);
     for (int grp = 0; grp < g.groups; ++grp) {
         const int Mrows = g.kW * g.kH * g.Cin_g;
-        if (direct) {
+        if (window) {
+            if constexpr (sizeof(T) == 2) {
+                wpatch::Problem p;
+                p.src = reinterpret_cast<const bf16_t*>(xT) + (size_t)grp * g.Cin_g;
+                p.dz = reinterpret_cast<const bf16_t*>(dy) + (size_t)grp * g.Cout_g * g.OW * g.OH;
+                p.partial = partial; p.zero = zeros;
+                p.Ctot = g.Cin; p.Cg = g.Cin_g; p.Cout = g.Cout; p.Ncols = g.Cout_g;
+                p.P = g.W; p.Q = g.H; p.N = g.N; p.pad_w = g.pw; p.pad_h = g.ph;
+                rc = wpatch::launch(s, p);
+                slices = g.N;
+            }
+        } else if (direct) {
             if constexpr (sizeof(T) == 2) {
                 ConvWgradDirectArgs a;
                 WgradGeomA& q = a.A;

@@ -152,8 +152,8 @@ def test_dimension_mismatch(gpu):
 def test_config5_full_size(gpu, dtype):
     """benchmark configuration 5 at full size: x 56x56x128x64, w 3x3x128x128 Kaiming-normal, stride 1,
     pad 1, relu.  Forward and input gradient: fp64 oracle on two images.  Filter gradient: the
-    adjoint identity <dw, w'> == <dz, conv(x, w')> against the (checked) forward kernel plus an
-    fp64 oracle on a two-image batch.  Bias gradient: fp64 channel sums."""
+    adjoint identity <dw, w'> == <dz, conv(x, w')> against the (checked) forward kernel, an
+    fp64 oracle on a two-image batch and the fp64 oracle on the whole batch.  Bias gradient: fp64 channel sums."""
     rng = np.random.default_rng(1004)
     xs, ws = (56, 56, 128, 64), (3, 3, 128, 128)
     gd, od = cdims(gpu, xs, ws, padding=1)
@@ -186,6 +186,8 @@ def test_config5_full_size(gpu, dtype):
     dzq = dz[..., sub].astype(np.float32)
     gw2 = gpu.conv_filter_grad(dev(gpu, x[..., sub], dtype), dev(gpu, dzq, dtype), gd2)
     assert_close(gw2.to_numpy(), O.conv_filter_grad(f64(x[..., sub]), f64(dzq), od2), dtype, "config5 dw (2 images)")
+    # the full-size filter gradient itself (in bf16 a kernel of its own: one partial sum per image): every element
+    assert_close(gw.to_numpy(), O.conv_filter_grad(f64(x), dz, od), dtype, "config5 dw (all images)")
 
 
 # Shapes that the bf16 kernel with the tile's input window in LDS takes (3 x 3, unit stride and dilation, output as
