@@ -60,6 +60,7 @@ __device__ __forceinline__ uint32_t at_use(uint32_t v) {
 __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
     extern __shared__ __align__(128) unsigned char lds_raw[];
     char* lds = reinterpret_cast<char*>(lds_raw);
+    const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds);   // LDS byte address
     const int tid = threadIdx.x, l = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wa = w & 3, ks = w >> 2;                 // channel block, which steps
     const int cb = blockIdx.x % a.CB, h = (blockIdx.x / a.CB) % a.H, n = blockIdx.x / (a.CB * a.H);
@@ -122,7 +123,6 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
     dz_issue(w >> 2);
     dz_issue(2 + (w >> 2));
 
-    typedef __attribute__((address_space(3))) s16x4_v* lds_tr;
     for (int ti = 0; ti < tiles; ++ti) {
         const int buf = ti & 1;
         const int q_first = (int)a.divP.div((uint32_t)(ti * TILE_PX));
@@ -158,29 +158,47 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
                     patch_issue(6, ti + 1, buf ^ 1); patch_issue(7, ti + 1, buf ^ 1);
                 }
             }
-            const char* patch = lds + buf * BUF_BYTES;
+            const uint32_t patch = lds_addr + (uint32_t)buf * BUF_BYTES;
+            const uint32_t row_step = (uint32_t)a.pitch * 32u;                // one tap row further down the patch
 #pragma unroll
             for (int v = 0; v < 2; ++v) {                                // this wave's two steps of the group
                 const int sl = 2 * v + ks;                               // step inside the group
                 const int u = S * 2 + v;                                 // index of the step among this wave's four of the tile
-                const char* blk = lds + RING_OFF + ((step0 + sl) & (RING - 1)) * BLK_BYTES;
-                bf16x8_v fb[4];
+                const uint32_t blk = lds_addr + RING_OFF + (uint32_t)((step0 + sl) & (RING - 1)) * BLK_BYTES + b_lane;
+                const uint32_t x0 = patch + (u == 0 ? xb[0][0] : u == 1 ? xb[1][0] : u == 2 ? xb[2][0] : xb[3][0]);
+                const uint32_t x1 = patch + (u == 0 ? xb[0][1] : u == 1 ? xb[1][1] : u == 2 ? xb[2][1] : xb[3][1]);
+                // The reads are written as assembly: left to the compiler, the first of them would wait for every
+                // global -> LDS load just requested (it must assume that they overwrite what is read; the ring and
+                // the two patch buffers rule that out).  22 reads per step, in the order B0-B3, then per tap the
+                // two halves of its A fragment; LDS reads return in order.
+                u32x4_v fb[4];
+                s16x4_v lo[TAPS], hi[TAPS];
+                asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\tds_read_b128 %2, %4 offset:2048\n\t"
+                             "ds_read_b128 %3, %4 offset:3072"
+                             : "=&v"(fb[0]), "=&v"(fb[1]), "=&v"(fb[2]), "=&v"(fb[3]) : "v"(blk));
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    fb[j] = __builtin_bit_cast(bf16x8_v, *reinterpret_cast<const u32x4_v*>(blk + j * 1024 + b_lane));
-                const uint32_t x0 = u == 0 ? xb[0][0] : u == 1 ? xb[1][0] : u == 2 ? xb[2][0] : xb[3][0];
-                const uint32_t x1 = u == 0 ? xb[0][1] : u == 1 ? xb[1][1] : u == 2 ? xb[2][1] : xb[3][1];
-#pragma unroll
-                for (int t = 0; t < TAPS; ++t) {
-                    const int kb = t / 3, ka = t - 3 * kb;
-                    const uint32_t shift = (uint32_t)((kb * a.pitch + ka) * 32);
-                    const s16x4_v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(patch + x0 + shift));
-                    const s16x4_v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(patch + x1 + shift));
-                    const s16x8_v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    const bf16x8_v fa = __builtin_bit_cast(bf16x8_v, both);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb[j], acc[t][j], 0, 0, 0);
+                for (int kb = 0; kb < 3; ++kb) {
+                    const uint32_t r0 = x0 + (uint32_t)kb * row_step, r1 = x1 + (uint32_t)kb * row_step;
+                    asm volatile("ds_read_b64_tr_b16 %0, %6\n\tds_read_b64_tr_b16 %1, %7\n\t"
+                                 "ds_read_b64_tr_b16 %2, %6 offset:32\n\tds_read_b64_tr_b16 %3, %7 offset:32\n\t"
+                                 "ds_read_b64_tr_b16 %4, %6 offset:64\n\tds_read_b64_tr_b16 %5, %7 offset:64"
+                                 : "=&v"(lo[3 * kb]), "=&v"(hi[3 * kb]), "=&v"(lo[3 * kb + 1]), "=&v"(hi[3 * kb + 1]), "=&v"(lo[3 * kb + 2]),
+                                   "=&v"(hi[3 * kb + 2])
+                                 : "v"(r0), "v"(r1));
                 }
+                // tap t may start when at most 16 - 2 t of the reads behind its own are outstanding
+#define WP_TAP(t, younger)                                                                                          \
+                do {                                                                                                \
+                    asm volatile("s_waitcnt lgkmcnt(" #younger ")"                                                  \
+                                 : "+v"(lo[t]), "+v"(hi[t]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));   \
+                    const s16x8_v both = {lo[t][0], lo[t][1], lo[t][2], lo[t][3], hi[t][0], hi[t][1], hi[t][2], hi[t][3]}; \
+                    const bf16x8_v fa = __builtin_bit_cast(bf16x8_v, both);                                         \
+                    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                   \
+                        acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, __builtin_bit_cast(bf16x8_v, fb[j]), acc[t][j], 0, 0, 0); \
+                } while (0)
+                WP_TAP(0, 15); WP_TAP(1, 14); WP_TAP(2, 12); WP_TAP(3, 10); WP_TAP(4, 8);
+                WP_TAP(5, 6); WP_TAP(6, 4); WP_TAP(7, 2); WP_TAP(8, 0);
+#undef WP_TAP
             }
         }
     }
