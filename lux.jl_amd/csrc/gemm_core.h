@@ -300,6 +300,51 @@ __device__ __forceinline__ bf16x8_v load_frag_bf16(const bf16_t* lds, int rbase,
     }
 }
 
+// The same fragment read written as assembly, for loops that keep global -> LDS loads in flight: a read the
+// compiler can see is made to wait for every such load already requested (the compiler must assume that the
+// load overwrites what is read; the stage ring rules that out), which would expose a full memory latency per
+// stage.  issue() requests the fragment, ready() is called once the caller's own s_waitcnt lgkmcnt has covered
+// it and ties the registers to that point, get() hands the fragment to the MFMA.
+template <bool KMAJOR, int ROWS>
+__device__ __forceinline__ uint32_t frag_offset_bf16(int rbase, int kk) {   // bytes from the operand tile's start
+    const int l = threadIdx.x & 63;
+    if constexpr (KMAJOR) {
+        const int r = rbase + (l & 31);
+        const int chunk = 2 * kk + (l >> 5);
+        return 2u * (uint32_t)(r * 32 + ((chunk ^ ((r >> 2) & 3)) << 3));
+    } else {
+        const int b = l >> 4, s = l & 15;
+        const int r = rbase + ((b & 1) << 4) + ((s & 3) << 2);
+        const int k = kk * 16 + ((b >> 1) << 3) + (s >> 2);
+        return 2u * (uint32_t)(k * ROWS + (r ^ ((k & 3) << mn_swizzle_shift(ROWS))));
+    }
+}
+template <bool KMAJOR, int ROWS> struct FragRegsBf16;
+template <int ROWS> struct FragRegsBf16<true, ROWS> {
+    static constexpr int READS = 1;
+    u32x4_v v;
+    __device__ __forceinline__ void issue(uint32_t addr) { asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr)); }
+    __device__ __forceinline__ void ready() { asm volatile("" : "+v"(v)); }
+    __device__ __forceinline__ bf16x8_v get() const { return __builtin_bit_cast(bf16x8_v, v); }
+};
+template <int ROWS> struct FragRegsBf16<false, ROWS> {
+    static constexpr int READS = 2;
+    s16x4_v lo, hi;
+    __device__ __forceinline__ void issue(uint32_t addr) {   // k and k + 4 share the swizzle
+        asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:%3"
+                     : "=&v"(lo), "=&v"(hi) : "v"(addr), "n"(4 * ROWS * 2));
+    }
+    __device__ __forceinline__ void ready() { asm volatile("" : "+v"(lo), "+v"(hi)); }
+    __device__ __forceinline__ bf16x8_v get() const {
+        const s16x8_v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(bf16x8_v, both);
+    }
+};
+template <int N> __device__ __forceinline__ void wait_lds_reads() {   // at most N of this wave's LDS reads outstanding
+    static_assert(N >= 0 && N <= 15, "lgkmcnt range");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
+}
+
 // fp32: 4 floats per lane covering one 8-k window `kw`: slot s <-> k = kw*8 + 4*(lane/32) + s
 template <bool KMAJOR, int ROWS>
 __device__ __forceinline__ void load_frag_f32(const float* lds, int rbase, int kw, float (&f)[4]) {
@@ -454,7 +499,7 @@ struct GemmMainloop {
         const int wave_m = (w % NWM) * (WM * 32), wave_n = (w / NWM) * (WN * 32);
         zero(acc);
         constexpr int KK = Tr::BK / 16;
-        static_assert(KK >= 2, "a stage has at least two k groups");
+        static_assert(KK == 2, "a stage has two k groups");
         constexpr int IPS = LA::INSTR + LB::INSTR;               // load instructions per thread and stage
         constexpr int PENDING = (NST - 2) * IPS;                 // loads of later stages that may stay in flight
         static_assert(PENDING < 64, "vmcnt range");
@@ -462,40 +507,55 @@ struct GemmMainloop {
         // LDS reads of the stage before the barrier lets other waves refill its buffer
         constexpr int WAIT_IMM = (PENDING & 0xF) | (0x7 << 4) | ((PENDING >> 4) << 14);
         const int KT = K / Tr::BK;
-        bf16x8_v fa[KK][WM], fb[KK][WN];
-        auto read = [&](int kk, const T* stage) {
-            const bf16_t* As = reinterpret_cast<const bf16_t*>(stage);
-            const bf16_t* Bs = reinterpret_cast<const bf16_t*>(stage + A_ELEMS);
+        using FA = FragRegsBf16<A_KMAJOR, TILE_M>;
+        using FB = FragRegsBf16<B_KMAJOR, TILE_N>;
+        constexpr int GROUP_READS = WM * FA::READS + WN * FB::READS;   // LDS read instructions of one k group
+        static_assert(GROUP_READS <= 15, "lgkmcnt range");
+        FA fa[KK][WM];
+        FB fb[KK][WN];
+        const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds);
+        uint32_t off_a[KK][WM], off_b[KK][WN];
 #pragma unroll
-            for (int j = 0; j < WN; ++j) fb[kk][j] = load_frag_bf16<B_KMAJOR, TILE_N>(Bs, wave_n + j * 32, kk);
+        for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
-            for (int i = 0; i < WM; ++i) fa[kk][i] = load_frag_bf16<A_KMAJOR, TILE_M>(As, wave_m + i * 32, kk);
+            for (int i = 0; i < WM; ++i) off_a[kk][i] = lds_addr + frag_offset_bf16<A_KMAJOR, TILE_M>(wave_m + i * 32, kk);
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+                off_b[kk][j] = lds_addr + (uint32_t)A_ELEMS * 2u + frag_offset_bf16<B_KMAJOR, TILE_N>(wave_n + j * 32, kk);
+        }
+        auto read = [&](int kk, int stage) {
+            const uint32_t sb = (uint32_t)stage * (uint32_t)(STAGE_ELEMS * 2);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) fb[kk][j].issue(off_b[kk][j] + sb);
+#pragma unroll
+            for (int i = 0; i < WM; ++i) fa[kk][i].issue(off_a[kk][i] + sb);
         };
-        auto mma = [&](int kk) {
+        auto mma = [&](int kk) {                                 // the caller's wait has covered group kk
+#pragma unroll
+            for (int j = 0; j < WN; ++j) fb[kk][j].ready();
+#pragma unroll
+            for (int i = 0; i < WM; ++i) fa[kk][i].ready();
 #pragma unroll
             for (int i = 0; i < WM; ++i)
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk][j].get(), fa[kk][i].get(), acc[i][j], 0, 0, 0);
         };
         int cur = 0, fill = NST - 1;                             // buffer of stage kt, buffer to refill
         // stage 0 has landed (every wave's share: barrier); its first fragments
         if (NST - 2 < KT) __builtin_amdgcn_s_waitcnt(WAIT_IMM);
         else __builtin_amdgcn_s_waitcnt(0);                      // fewer stages than the pipeline holds
         __builtin_amdgcn_s_barrier();
-        read(0, lds);
+        read(0, 0);
         for (int kt = 0; kt < KT; ++kt) {
-            const T* cb = lds + cur * STAGE_ELEMS;
             // the buffer of stage kt - 1 was released at that stage's barrier
             if (kt + NST - 1 < KT) {
                 la.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS);
                 lb.issue((kt + NST - 1) * Tr::BK, lds + fill * STAGE_ELEMS + A_ELEMS);
             }
-#pragma unroll
-            for (int kk = 1; kk < KK; ++kk) read(kk, cb);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kk = 0; kk < KK - 1; ++kk) mma(kk);
+            read(1, cur);
+            wait_lds_reads<GROUP_READS>();                       // the first group is in, the second may be on its way
+            mma(0);
             __builtin_amdgcn_sched_barrier(0);
             cur = cur + 1 == NST ? 0 : cur + 1;
             fill = fill + 1 == NST ? 0 : fill + 1;
@@ -505,10 +565,11 @@ struct GemmMainloop {
                 else __builtin_amdgcn_s_waitcnt(0);              // tail: fewer stages are in flight
                 // bare barrier: __syncthreads() would add a fence that drains every load in flight
                 __builtin_amdgcn_s_barrier();
-                read(0, lds + cur * STAGE_ELEMS);
+                read(0, cur);
+            } else {
+                wait_lds_reads<0>();
             }
-            __builtin_amdgcn_sched_barrier(0);
-            mma(KK - 1);
+            mma(1);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
