@@ -100,7 +100,8 @@ int luxhip_profile_enable(int on);
  *   "workspace_epoch" (tests) the epoch from which the per-stream exchange words continue; the 32-bit
  *                   epoch wraps after 2^32 calls, at which point the library clears those words
  *   "conv_tile"     0 automatic (default); bf16 whole-tap convolution kernels: 82 = 256x256 tile on
- *                   8 waves, 84 / 83 = 512x128 on 8 waves with 4 / 3 LDS stages, 42 = 256x128 on 4 waves */
+ *                   8 waves, 84 / 83 = 512x128 on 8 waves with 4 / 3 LDS stages, 42 = 256x128 on 4 waves;
+ *                   1 / 2: the 3x3 window kernel in tiles of 64 / 128 output channels whatever their number */
 int luxhip_set_option(const char* name, int64_t value);
 int luxhip_profile_report(char* buf, size_t len);
 

@@ -240,7 +240,7 @@ static int run_conv_gemm(hipStream_t s, const ConvGeom& g, bool dgrad, const T* 
         int rc;
         if constexpr (sizeof(T) == 2) {
             // unit stride and dilation, output as large as the input: the kernel that keeps a tile's input window in LDS
-            if (option_conv_tile() == 0 && g.sw == 1 && g.sh == 1 && g.dw == 1 && g.dh == 1 && g.OW == g.W && g.OH == g.H) {
+            if (option_conv_tile() <= 2 && g.sw == 1 && g.sh == 1 && g.dw == 1 && g.dh == 1 && g.OW == g.W && g.OH == g.H) {
                 cpatch::Problem p;
                 p.src = reinterpret_cast<const bf16_t*>(src) + (size_t)grp * Cg;
                 p.wm = reinterpret_cast<const bf16_t*>(Wm.p);
@@ -316,7 +316,7 @@ static int wgrad_plan(const ConvGeom& g, int* slices, int* kslice, bool* small) 
 // as the input): one partial sum per image.  Pointer alignment is checked again at the launch.
 template <typename T>
 static bool wgrad_window_shape(const ConvGeom& g) {
-    if (sizeof(T) != 2 || option_conv_tile() != 0) return false;
+    if (sizeof(T) != 2 || option_conv_tile() > 2) return false;
     if (g.kW != 3 || g.kH != 3 || g.sw != 1 || g.sh != 1 || g.dw != 1 || g.dh != 1 || g.OW != g.W || g.OH != g.H) return false;
     wpatch::Problem p;
     p.src = nullptr; p.dz = nullptr; p.partial = nullptr; p.zero = nullptr;

@@ -68,6 +68,7 @@ struct Args {
     int pitch;               // P + kW - 1
     int Ncols, col_off, Ctot_out, act;
     int frags, groups_m, tiles_n;   // fragments of 16 positions in all; workgroups that share them; tiles along the output channels
+    int staged;                     // the epilogue may go through LDS: PQ % 8 == 0, no pre-activation output, out 16-byte aligned
     FastDiv divP, divQ, divPQ, divPitch;
 };
 
@@ -78,6 +79,10 @@ __device__ __forceinline__ uint32_t at_use(uint32_t v) {
     return v;
 }
 
+// ANY_ACT false: identity or relu only.  The epilogue is unrolled over the accumulator tiles, and with every activation
+// inlined into each copy the kernel grows to several times the instruction cache, which the workgroup then refills
+// from L2 after every tile.
+template <bool ANY_ACT>
 __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
     extern __shared__ __align__(128) unsigned char lds_raw[];
     char* lds = reinterpret_cast<char*>(lds_raw);
@@ -147,6 +152,16 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
     // B: row 16 j + l % 16 of the wave's half-block, chunk 4 g + l / 16 for k group g (g = 1: XOR 64)
     const uint32_t offB = (uint32_t)(lane15 * 128 + ((laneq ^ ((lane15 >> 1) & 7)) << 4));
 
+    // the bias of this lane's four columns (channel n0 + wave_n + 16 j + l % 16), read once: a load inside the epilogue
+    // would have to wait for the stores issued before it
+    float bias_v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int col = tn * TILE_N + wave_n + 16 * j + (int)lane15;
+        bias_v[j] = a.bias != nullptr && col < a.Ncols ? ld(a.bias + a.col_off + col) : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(bias_v[j]));       // the wait for these loads belongs here, before the tile loop
     int tile = 0;
     int hc = 0;                              // halves consumed so far by this workgroup: patch buffer hc & 1
     const char* gp_cur = gp_first;
@@ -313,7 +328,44 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
         }
 
         // ---- epilogue: lane l owns positions m0 + wave_m + 16 i + 4 (l / 16) + r and channel n0 + wave_n + 16 j + l % 16
-        {
+        if (a.staged) {
+            // Through LDS, sixteen channels at a time, so that a store instruction writes whole 128-byte lines (64
+            // positions of a channel) instead of sixteen pieces of 32 bytes: the wave's 2304 bytes lie in the patch
+            // buffer of the half just finished, which nobody reads after that half's last boundary and which the
+            // loads of the half after the next only enter behind the next tile's first barrier.  Rows of 144 bytes
+            // (64 positions + 16 bytes) keep the writes (lane l: channel l % 16) and the reads (lane l: channel l / 8
+            // and l / 8 + 8, positions 8 (l % 8) .. + 7) free of bank conflicts.
+            char* st = lds + ((hc - 1) & 1) * BUF_STRIDE + w * 2304;
+            const int mq = m0 + wave_m + 8 * (l & 7);
+            const bool qok = mq < m_end;                                // m_end and PQ are multiples of 8 here
+            const int img = (int)a.divPQ.div((uint32_t)(qok ? mq : 0));
+            const uint32_t rowoffq = (uint32_t)(mq - img * a.PQ) + (uint32_t)a.PQ * (uint32_t)a.Ctot_out * (uint32_t)img;
+            const int act = a.act;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float b = bias_v[j];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = acc[i][j][r] + b;
+                    if (act == LUXHIP_ACT_RELU) act_vec_as<LUXHIP_ACT_RELU>(v);
+                    else if constexpr (ANY_ACT) { if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v); }
+                    uint2 ov;
+                    ov.x = f32x2_to_bf16x2(v[0], v[1]);
+                    ov.y = f32x2_to_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<uint2*>(st + lane15 * 144 + (16 * i + 4 * laneq) * 2) = ov;
+                }
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    const int c = (l >> 3) + 8 * hh;
+                    const uint4 val = *reinterpret_cast<const uint4*>(st + c * 144 + (l & 7) * 16);
+                    const int col = n0 + wave_n + 16 * j + c;
+                    if (qok && col < a.Ncols)
+                        *reinterpret_cast<uint4*>(a.out + ((uint32_t)a.PQ * (uint32_t)(a.col_off + col) + rowoffq)) = val;
+                }
+            }
+        } else {
             const int mrow = m0 + wave_m + 4 * (int)laneq;
             const int ncol = n0 + (upper ? 64 : 0) + (int)lane15;
             // element offsets inside one image's block of the output fit 32 bits (the tensor has fewer than 2^31 elements)
@@ -332,7 +384,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
             for (int j = 0; j < 4; ++j) {
                 const int col = ncol + 16 * j;
                 if (col < a.Ncols) {
-                    const float b = a.bias ? ld(a.bias + a.col_off + col) : 0.0f;
+                    const float b = bias_v[j];
                     const uint32_t coloff = (uint32_t)a.PQ * (uint32_t)(a.col_off + col);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
@@ -347,7 +399,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                             *reinterpret_cast<uint2*>(a.pre + (coloff + rowoff[i])) = pv;
                         }
                         if (act == LUXHIP_ACT_RELU) act_vec_as<LUXHIP_ACT_RELU>(v);
-                        else if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v);
+                        else if constexpr (ANY_ACT) { if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v); }
                         uint2 ov;
                         ov.x = f32x2_to_bf16x2(v[0], v[1]);
                         ov.y = f32x2_to_bf16x2(v[2], v[3]);
@@ -367,7 +419,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 for (int j = 0; j < 4; ++j) {
                     const int col = ncol + 16 * j;
                     if (col < a.Ncols) {
-                        const float b = a.bias ? ld(a.bias + a.col_off + col) : 0.0f;
+                        const float b = bias_v[j];
                         const uint32_t off = (uint32_t)a.PQ * (uint32_t)(a.col_off + col) + rowoffE;
                         float v[4];
 #pragma unroll
@@ -379,7 +431,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                             *reinterpret_cast<uint2*>(a.pre + off) = pv;
                         }
                         if (act == LUXHIP_ACT_RELU) act_vec_as<LUXHIP_ACT_RELU>(v);
-                        else if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v);
+                        else if constexpr (ANY_ACT) { if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v); }
                         uint2 ov;
                         ov.x = f32x2_to_bf16x2(v[0], v[1]);
                         ov.y = f32x2_to_bf16x2(v[2], v[3]);

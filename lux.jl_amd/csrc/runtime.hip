@@ -282,8 +282,8 @@ int luxhip_set_option(const char* name, int64_t value) {
                        "set_option: gemm_tile must be 0, 82, 42, 22 or 11");
         g_opt_gemm_tile.store(value);
     } else if (strcmp(name, "conv_tile") == 0) {
-        LUX_INVALID_IF(value != 0 && value != 82 && value != 83 && value != 84 && value != 42,
-                       "set_option: conv_tile must be 0, 82, 83, 84 or 42");
+        LUX_INVALID_IF(value != 0 && value != 1 && value != 2 && value != 82 && value != 83 && value != 84 && value != 42,
+                       "set_option: conv_tile must be 0, 1, 2, 82, 83, 84 or 42");
         g_opt_conv_tile.store(value);
     } else if (strcmp(name, "gemm_pretranspose") == 0) {
         LUX_INVALID_IF(value != 0 && value != 1, "set_option: gemm_pretranspose must be 0 or 1");

@@ -200,6 +200,7 @@ WINDOW_CASES = [
     ((56, 56, 64, 1), (3, 3, 64, 64), 1, 1, False),                # one image: 196 fragments on 13 workgroups (15 or 16 each)
     ((6, 6, 64, 2), (3, 3, 64, 16), 1, 1, False),                  # 72 positions: one partial tile, rows past the last position
     ((32, 34, 64, 64), (3, 3, 64, 64), 1, 1, True),                # 4352 fragments = 17 per compute unit: tiles with a seventeenth fragment
+    ((12, 10, 128, 3), (3, 3, 128, 48), 1, 1, False),              # two 64-channel parts into 48 columns (the kernel for at most 64)
 ]
 
 
@@ -233,3 +234,13 @@ def test_window_kernel_shapes(gpu, case):
     # the two kernels add the same products in a different order: equal up to the bf16 rounding of the result
     assert_close(y, f64(y_tap), "bf16", tag + "y vs gather kernel")
     assert_close(gx, f64(gx_tap), "bf16", tag + "dgrad vs gather kernel")
+    # both window kernels on every shape, whichever the library would pick: tiles of 64 (1) and of 128 (2) output channels
+    for forced in (1, 2):
+        gpu.set_option("conv_tile", forced)
+        try:
+            y_f = gpu.fused_conv_bias_activation("relu", dw_, dx_, db_, gd).to_numpy()
+            gx_f = gpu.conv_data_grad(ddy_, dw_, gd).to_numpy()
+        finally:
+            gpu.set_option("conv_tile", 0)
+        assert_close(y_f[..., imgs], want_y, "bf16", tag + f"y, column tiles {64 * forced}")
+        assert_close(gx_f[..., imgs], want_gx, "bf16", tag + f"dgrad, column tiles {64 * forced}")
