@@ -32,7 +32,7 @@ int launch(hipStream_t s, const Problem& p) {
     const bool narrow = forced == 1 || (forced != 2 && a.Ncols <= 64);
     a.tiles_n = (int)ceil_div(a.Ncols, narrow ? 64 : TILE_N);
     a.frags = (int)ceil_div(a.M, 16);
-    a.staged = !narrow && a.PQ % 8 == 0 && a.pre == nullptr && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0;
+    a.staged = a.PQ % 8 == 0 && a.pre == nullptr && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0;
     a.divP = FastDiv((uint32_t)a.P); a.divQ = FastDiv((uint32_t)a.Q); a.divPQ = FastDiv((uint32_t)a.PQ);
     a.divPitch = FastDiv((uint32_t)a.pitch);
     // the LDS holds one workgroup per compute unit: as many workgroups as compute units share the fragments evenly

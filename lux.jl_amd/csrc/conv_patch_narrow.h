@@ -185,13 +185,13 @@ __global__ __launch_bounds__(THREADS) void conv_patch_narrow_kernel(Args a) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
         };
 
-        if (tile == 0) {
-            // the first patch and the half-block of the first step have landed: of the loads issued so far at most the
-            // three youngest (half-blocks further ahead) are outstanding.  Later tiles start behind the boundary
-            // of the step before, which has covered their patch and first half-block.
-            __builtin_amdgcn_s_waitcnt(3 | (0x7 << 4));      // vmcnt(3) lgkmcnt(0)
-            __builtin_amdgcn_s_barrier();
-        }
+        // the first patch and the half-block of the first step have landed: of the loads issued so far at most the
+        // three youngest (half-blocks further ahead) are outstanding.  Later tiles start behind the boundary of the
+        // step before, which has covered their patch and first half-block; their barrier keeps the next patch loads
+        // out of the buffer in which slower waves still turn their results around.
+        if (tile == 0) __builtin_amdgcn_s_waitcnt(3 | (0x7 << 4));      // vmcnt(3) lgkmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0xF | (0x7 << 4) | (0x3 << 14));   // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
 
         uint32_t aA[3], aN[3];
         {
@@ -277,7 +277,40 @@ __global__ __launch_bounds__(THREADS) void conv_patch_narrow_kernel(Args a) {
         }
 
         // ---- epilogue: lane l owns positions m0 + wave_m + 16 i + 4 (l / 16) + r and channel 16 j + l % 16
-        {
+        if (a.staged) {
+            // Through LDS, sixteen channels at a time, so that a store instruction writes 64 contiguous bytes per channel
+            // (the wave's 32 positions) instead of sixteen pieces of 32 bytes: the wave's 1280 bytes lie in the patch
+            // buffer of the half just finished, which nobody reads after that half's last boundary and which the
+            // loads of the half after the next only enter behind the next tile's first barrier.  Rows of 80 bytes
+            // keep the writes (lane l: channel l % 16) and the reads (lane l: channel l / 4, positions 8 (l % 4) .. + 7)
+            // free of bank conflicts.
+            char* st = lds + ((hc - 1) & 1) * BUF_STRIDE + w * 1280;
+            const int mq = m0 + wave_m + 8 * (l & 3);
+            const bool qok = mq < m_end;                                // m_end and PQ are multiples of 8 here
+            const int img = (int)a.divPQ.div((uint32_t)(qok ? mq : 0));
+            const uint32_t rowoffq = (uint32_t)(mq - img * a.PQ) + (uint32_t)a.PQ * (uint32_t)a.Ctot_out * (uint32_t)img;
+            const int act = a.act;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float b = bias_v[j];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    float v[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = acc[i][j][r] + b;
+                    if (act == LUXHIP_ACT_RELU) act_vec_as<LUXHIP_ACT_RELU>(v);
+                    else if constexpr (ANY_ACT) { if (act != LUXHIP_ACT_IDENTITY) act_vec(act, v); }
+                    uint2 ov;
+                    ov.x = f32x2_to_bf16x2(v[0], v[1]);
+                    ov.y = f32x2_to_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<uint2*>(st + lane15 * 80 + (16 * i + 4 * laneq) * 2) = ov;
+                }
+                const int c = l >> 2;
+                const uint4 val = *reinterpret_cast<const uint4*>(st + c * 80 + (l & 3) * 16);
+                const int col = tn * 64 + 16 * j + c;
+                if (qok && col < a.Ncols) *reinterpret_cast<uint4*>(a.out + ((uint32_t)a.PQ * (uint32_t)(a.col_off + col) + rowoffq)) = val;
+            }
+        } else {
             const int mrow = m0 + wave_m + 4 * (int)laneq;
             // element offsets inside one image's block of the output fit 32 bits (the tensor has fewer than 2^31 elements)
             uint32_t rowoff[2];
