@@ -19,7 +19,7 @@ int launch(hipStream_t s, const Problem& p) {
     a.H = p.Cg / 64; a.CB = (p.Ncols + 63) / 64;
     a.divP = FastDiv((uint32_t)a.P); a.divPitch = FastDiv((uint32_t)a.pitch);
     ProfScope ps("conv_wgrad_kernel<bf16>", s);
-    conv_wgrad_patch_kernel<<<dim3((unsigned)(p.N * a.H * a.CB)), dim3(THREADS), LDS_BYTES, s>>>(a);
+    conv_wgrad_patch_kernel<<<dim3((unsigned)(((p.N + 7) / 8) * 8 * a.H * a.CB)), dim3(THREADS), LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

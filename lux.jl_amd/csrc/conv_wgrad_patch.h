@@ -63,7 +63,13 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
     const uint32_t lds_addr = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds);   // LDS byte address
     const int tid = threadIdx.x, l = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wa = w & 3, ks = w >> 2;                 // channel block, which steps
-    const int cb = blockIdx.x % a.CB, h = (blockIdx.x / a.CB) % a.H, n = blockIdx.x / (a.CB * a.H);
+    // The parts of an image (64 input x 64 output channels each) read the same input and the same dz: they go to one
+    // XCD (workgroup i runs on XCD i % 8), next to each other in its order of dispatch, so that its L2 serves the repeats.
+    const int parts = a.CB * a.H;
+    const int slot = blockIdx.x >> 3;
+    const int n = (slot / parts) * 8 + (blockIdx.x & 7), part = slot % parts;
+    if (n >= a.N) return;                                   // the last group of eight images may be incomplete
+    const int cb = part % a.CB, h = part / a.CB;
     const int steps = a.PQ / STEP_PX;                  // of the image
     const int tiles = (a.PQ + TILE_PX - 1) / TILE_PX;
     const int64_t row_bytes = (int64_t)a.P * a.Ctot * 2;

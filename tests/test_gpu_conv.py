@@ -244,3 +244,23 @@ def test_window_kernel_shapes(gpu, case):
             gpu.set_option("conv_tile", 0)
         assert_close(y_f[..., imgs], want_y, "bf16", tag + f"y, column tiles {64 * forced}")
         assert_close(gx_f[..., imgs], want_gx, "bf16", tag + f"dgrad, column tiles {64 * forced}")
+
+
+@pytest.mark.parametrize("xs,ws", [((16, 16, 128, 36), (3, 3, 128, 128)),      # 36 images: the last group of eight is incomplete
+                                   ((16, 8, 64, 136), (3, 3, 64, 64))])        # one 64 x 64 channel part per image, 17 groups of eight
+def test_filter_gradient_window_kernel_batches(gpu, xs, ws):
+    """bf16 filter gradient with the input window of an image in LDS (one workgroup per image and 64 x 64 channel
+    part, the parts of eight images dealt to the eight XCDs) against the fp64 oracle and against the gather kernel."""
+    rng = np.random.default_rng(777 + xs[3])
+    gd, od = cdims(gpu, xs, ws, padding=1)
+    x, dy = host_inputs("bf16", rng.normal(size=xs), rng.normal(size=od.y_shape()))
+    dx_, ddy_ = dev(gpu, x, "bf16"), dev(gpu, dy, "bf16")
+    dw = gpu.conv_filter_grad(dx_, ddy_, gd).to_numpy()
+    gpu.set_option("conv_tile", 84)
+    try:
+        dw_gather = gpu.conv_filter_grad(dx_, ddy_, gd).to_numpy()
+    finally:
+        gpu.set_option("conv_tile", 0)
+    want = O.conv_filter_grad(f64(x), f64(dy), od)
+    assert_close(dw, want, "bf16", f"window wgrad N={xs[3]}")
+    assert_close(dw_gather, want, "bf16", f"gather wgrad N={xs[3]}")
