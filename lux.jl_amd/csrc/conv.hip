@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void whcn_to_cwhn_kernel(const T* __restrict__
 // (66 two-byte or 65 four-byte elements) spreads the strided reads of the second phase over
 // the banks.
 template <typename T>
-__global__ __launch_bounds__(256) void whcn_to_cwhn_vec_kernel(const T* __restrict__ in, T* __restrict__ out, int P, int C) {
+__device__ __forceinline__ void whcn_to_cwhn_vec_tile(const T* __restrict__ in, T* __restrict__ out, int P, int C) {
     constexpr int V = 16 / sizeof(T), TP = 64, TC = 64;
     constexpr int PITCH = TP + 4 / sizeof(T);   // 66 (bf16) / 65 (fp32) elements: rows stay 4-byte aligned
     __shared__ __align__(16) T tile[TC * PITCH];
@@ -78,13 +78,17 @@ __global__ __launch_bounds__(256) void whcn_to_cwhn_vec_kernel(const T* __restri
     }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void whcn_to_cwhn_vec_kernel(const T* __restrict__ in, T* __restrict__ out, int P, int C) {
+    whcn_to_cwhn_vec_tile<T>(in, out, P, C);
+}
+
 // wF[(co*T + t)*Cin_g + ci] (fprop, K = T*Cin_g) or wD[((g*Cin_g + ci)*T + t)*Cout_g + col]
 // (dgrad, K = T*Cout_g) from w[a + kW*(b + kH*(ci + Cin_g*co))]; tap t = ka + kW*kb with
 // a = flip ? ka : kW-1-ka (same for b).
 template <typename T>
-__global__ void pack_filter_kernel(const T* __restrict__ w, T* __restrict__ out, ConvGeom g, int for_dgrad) {
+__device__ __forceinline__ void pack_filter_element(const T* __restrict__ w, T* __restrict__ out, const ConvGeom& g, int for_dgrad, int idx) {
     const int total = g.kW * g.kH * g.Cin_g * g.Cout;
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int Tt = g.kW * g.kH;
     int co, t, ci;
@@ -103,6 +107,23 @@ __global__ void pack_filter_kernel(const T* __restrict__ w, T* __restrict__ out,
     const int ka = t % g.kW, kb = t / g.kW;
     const int a = g.flip ? ka : g.kW - 1 - ka, b = g.flip ? kb : g.kH - 1 - kb;
     out[idx] = w[a + g.kW * (b + g.kH * (ci + g.Cin_g * co))];
+}
+template <typename T>
+__global__ void pack_filter_kernel(const T* __restrict__ w, T* __restrict__ out, ConvGeom g, int for_dgrad) {
+    pack_filter_element<T>(w, out, g, for_dgrad, (int)(blockIdx.x * blockDim.x + threadIdx.x));
+}
+// The layout transform of a tensor and the repacking of the filter in one launch (the filter is a few hundred
+// KiB: a launch of its own costs more than the work): the z slices 0 .. N - 1 of the grid transform image n, the
+// slices behind them repack 256 filter elements per workgroup.
+template <typename T>
+__global__ __launch_bounds__(256) void whcn_to_cwhn_pack_kernel(const T* __restrict__ in, T* __restrict__ out, int P, int C, int N,
+                                                                const T* __restrict__ w, T* __restrict__ wout, ConvGeom g, int for_dgrad) {
+    if ((int)blockIdx.z < N) {
+        whcn_to_cwhn_vec_tile<T>(in, out, P, C);
+    } else {
+        const int block = ((int)(blockIdx.z - N) * (int)gridDim.y + (int)blockIdx.y) * (int)gridDim.x + (int)blockIdx.x;
+        pack_filter_element<T>(w, wout, g, for_dgrad, block * 256 + (int)threadIdx.x);
+    }
 }
 
 // dw[a, b, ci, g*Cout_g + col] = sum over slices of partial[slice][m' = t*Cin_g + ci][col].
@@ -198,6 +219,25 @@ static int pack_filter(hipStream_t s, const T* w, T* out, const ConvGeom& g, int
     ProfScope ps("pack_filter_kernel", s);
     const int total = g.kW * g.kH * g.Cin_g * g.Cout;
     pack_filter_kernel<T><<<(unsigned)ceil_div(total, 256), 256, 0, s>>>(w, out, g, for_dgrad);
+    LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+// transpose_to_cwhn(in -> out) and pack_filter(w -> wout) in one launch where the 16-byte transform applies
+template <typename T>
+static int transpose_and_pack(hipStream_t s, const T* in, T* out, int P, int C, int N, const T* w, T* wout, const ConvGeom& g, int for_dgrad) {
+    constexpr int V = 16 / (int)sizeof(T);
+    const bool vec = P % V == 0 && C % V == 0 && aligned16(in) && aligned16(out);
+    const int64_t gx = ceil_div(P, 64), gy = ceil_div(C, 64);
+    const int64_t pack_blocks = ceil_div((int64_t)g.kW * g.kH * g.Cin_g * g.Cout, 256);
+    const int64_t gz = N + ceil_div(pack_blocks, gx * gy);
+    if (!vec || N < 1 || gy > 65535 || gz > 65535) {
+        int rc = transpose_to_cwhn<T>(s, in, out, P, C, N);
+        if (rc != LUXHIP_OK) return rc;
+        return pack_filter<T>(s, w, wout, g, for_dgrad);
+    }
+    ProfScope ps("whcn_to_cwhn_kernel", s);
+    whcn_to_cwhn_pack_kernel<T><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), 256, 0, s>>>(in, out, P, C, N, w, wout, g, for_dgrad);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }
@@ -421,8 +461,7 @@ static int conv_fwd_t(hipStream_t s, int act, const ConvGeom& g, const T* x, con
     if (rc != LUXHIP_OK) return rc;
     T* xT = xt_keep ? xt_keep : reinterpret_cast<T*>(ws.data);
     T* wF = reinterpret_cast<T*>(ws.data + xb);
-    if ((rc = transpose_to_cwhn<T>(s, x, xT, g.W * g.H, g.Cin, g.N)) != LUXHIP_OK) return rc;
-    if ((rc = pack_filter<T>(s, w, wF, g, 0)) != LUXHIP_OK) return rc;
+    if ((rc = transpose_and_pack<T>(s, x, xT, g.W * g.H, g.Cin, g.N, w, wF, g, 0)) != LUXHIP_OK) return rc;
     return run_conv_gemm<T>(s, g, false, xT, wF, bias, y, pre, act, ws.zeros);
 }
 
@@ -435,8 +474,7 @@ static int conv_bwd_data_t(hipStream_t s, const ConvGeom& g, const T* dy, const 
     if (rc != LUXHIP_OK) return rc;
     T* dyT = reinterpret_cast<T*>(ws.data);
     T* wD = reinterpret_cast<T*>(ws.data + yb);
-    if ((rc = transpose_to_cwhn<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
-    if ((rc = pack_filter<T>(s, w, wD, g, 1)) != LUXHIP_OK) return rc;
+    if ((rc = transpose_and_pack<T>(s, dy, dyT, g.OW * g.OH, g.Cout, g.N, w, wD, g, 1)) != LUXHIP_OK) return rc;
     return run_conv_gemm<T>(s, g, true, dyT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY, ws.zeros);
 }
 
@@ -482,9 +520,10 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
     T* dzT = reinterpret_cast<T*>(ws.data + xb);
     T* wD = reinterpret_cast<T*>(ws.data + xb + yb);
     float* partial = reinterpret_cast<float*>(ws.data + xb + yb + wb);
-    if ((rc = transpose_to_cwhn<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N)) != LUXHIP_OK) return rc;
+    if (dx != nullptr) rc = transpose_and_pack<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N, w, wD, g, 1);
+    else rc = transpose_to_cwhn<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N);
+    if (rc != LUXHIP_OK) return rc;
     if (dx != nullptr) {
-        if ((rc = pack_filter<T>(s, w, wD, g, 1)) != LUXHIP_OK) return rc;
         if ((rc = run_conv_gemm<T>(s, g, true, dzT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY, ws.zeros)) != LUXHIP_OK) return rc;
     }
     if (dw != nullptr) {
