@@ -154,7 +154,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_narrow_kernel(Args a) {
         auto a_addr = [&](int f, int t, uint32_t bufbase) -> uint32_t {
             const int kb = t / 3, ka = t - 3 * kb;                               // kW = kH = 3
             const uint32_t x = at_use(xrow[f][a.rev ? 2 - kb : kb]) + (uint32_t)(a.rev ? 2 - ka : ka);
-            return bufbase + (x << 4) + ((x >> 4) * 1792u + lq8);
+            return bufbase + (x << 4) + (__umul24(x >> 4, 1792u) + lq8);   // 24-bit multiply: full rate (the 32-bit one takes four times as long)
         };
 #define CPN_READ_A(set, a0, a1, OFF)                                                                                \
         asm volatile("ds_read_b128 %0, %2 offset:" #OFF "\n\tds_read_b128 %1, %3 offset:" #OFF                      \
