@@ -14,7 +14,8 @@
 //   in place of a patch row above or below the image;
 //   a ring of five filter half-blocks (64 output channels x 64 k = 8 KiB each, rows of 128 bytes with their
 //   16-byte chunks XORed with (row / 2) % 8); a step (one tap of one half, 64 k) consumes two, one per half
-//   of the waves, and the loads run three to four half-blocks ahead.
+//   of the waves, and the loads run three to four half-blocks ahead: a step requests the first half-block of
+//   the step after the next between its MFMAs and the second one right behind its barrier.
 //
 // Patch layout: position x = pr * pitch + pc (row pr, column pc of the patch, pitch = P + 2 with zero-filled halo
 // columns) belongs to the group x / 16 of 2 KiB, which holds its sixteen positions chunk by chunk: 16-byte chunk
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
     int tile = 0;
     int hc = 0;                              // halves consumed so far by this workgroup: patch buffer hc & 1
     const char* gp_cur = gp_first;
-    // prologue: the first patch, three filter half-blocks (step 0 both, step 1 the first)
+    // prologue: the first patch, four filter half-blocks (steps 0 and 1)
     {
         int rbase;
         const char* pb = patch_base(tile, 0, rbase);
@@ -174,6 +175,7 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
         filter_issue(gp_cur, 0);
         filter_issue(gp_cur, 1);
         filter_issue(gp_cur + Cg2, 0);
+        filter_issue(gp_cur + Cg2, 1);
     }
     const bool upper = wave_n != 0;          // this wave's columns are in the second half-block of a step
     // the two waves (on different SIMDs) that take the seventeenth fragment of a tile, one per half of the columns
@@ -254,8 +256,8 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
         };
 
         // the patch of the first half and the two half-blocks of the first step have landed: of the loads
-        // issued so far at most the youngest (a filter half-block further ahead) is outstanding
-        __builtin_amdgcn_s_waitcnt(1 | (0x7 << 4));          // vmcnt(1) lgkmcnt(0)
+        // issued so far at most the two youngest (the half-blocks of the second step) are outstanding
+        __builtin_amdgcn_s_waitcnt(2 | (0x7 << 4));          // vmcnt(2) lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
 
         uint32_t aA[5], aN[5];
@@ -286,11 +288,6 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 CP_READ_A(1, aA[0], aA[1], aA[2], aA[3], 1024);
                 CP_READ_B(1, lds_addr + RING_OFF + (uint32_t)(upper ? slot1 : slot0) * HB_BYTES + (at_use(offB) ^ 64u));
                 if (extra) CP_READ_E(1, aA[4], 1024);
-                if constexpr (t < PATCH_INSTR) {
-                    if (have_p) patch_issue(t, pb_p, rbase_p, (hc + 1) & 1);
-                }
-                // second half-block of the next step
-                filter_issue(t + 1 < TAPS ? gp_cur + (t + 1) * Cg2 : gp_next, 1);
                 CP_READY(0, 8);
                 CP_FENCE(); mfmas(0, 0); CP_FENCE();
                 {
@@ -309,6 +306,13 @@ __global__ __launch_bounds__(THREADS) void conv_patch_kernel(Args a) {
                 // has landed (loads return in order: only the half-block requested last may be outstanding)
                 __builtin_amdgcn_s_waitcnt(1 | (0x7 << 4));      // vmcnt(1) lgkmcnt(0)
                 __builtin_amdgcn_s_barrier();
+                // Requested first thing behind the barrier, so that they have a whole step to arrive (the boundary of the
+                // next step waits for them): the second half-block of the step after the next, into the slot this
+                // barrier has released, and a block of the next half's patch.
+                filter_issue(t + 2 < TAPS ? gp_cur + (t + 2) * Cg2 : gp_next + (t + 2 - TAPS) * Cg2, 1);
+                if constexpr (t < PATCH_INSTR) {
+                    if (have_p) patch_issue(t, pb_p, rbase_p, (hc + 1) & 1);
+                }
                 slot0 = slot0 + 2 >= RING ? slot0 + 2 - RING : slot0 + 2;
                 slot1 = slot1 + 2 >= RING ? slot1 + 2 - RING : slot1 + 2;
                 CP_READ_A(0, aN[0], aN[1], aN[2], aN[3], 0);
