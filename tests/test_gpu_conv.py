@@ -264,3 +264,45 @@ def test_filter_gradient_window_kernel_batches(gpu, xs, ws):
     want = O.conv_filter_grad(f64(x), f64(dy), od)
     assert_close(dw, want, "bf16", f"window wgrad N={xs[3]}")
     assert_close(dw_gather, want, "bf16", f"gather wgrad N={xs[3]}")
+
+
+def _random_window_shapes(count, seed):
+    """Shapes that the 3 x 3 window kernels accept (unit stride, output as large as the input, channels per group in
+    multiples of 64, W * H a multiple of 4), drawn with a fixed seed."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        W, H = int(rng.integers(3, 61)), int(rng.integers(3, 41))
+        if (W * H) % 4 != 0:
+            continue
+        groups = int(rng.choice([1, 1, 2]))
+        cin = 64 * groups * int(rng.integers(1, 3))
+        cout = groups * int(rng.choice([8, 16, 48, 64, 72, 128, 136]))
+        N = int(rng.integers(1, 8))
+        pad = [(1, 1, 1, 1), (0, 2, 2, 0), (2, 0, 1, 1), (1, 1, 0, 2)][int(rng.integers(0, 4))]
+        shapes.append(((W, H, cin, N), (3, 3, cin // groups, cout), pad, groups, bool(rng.integers(0, 2))))
+    return shapes
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_window_kernels_random_shapes(gpu, case):
+    """fprop (with bias and relu) and dgrad of both window kernels against the gather-per-tap kernels, which the other
+    tests pin against the oracle: the same products in another order, so equal up to the bf16 rounding of the result."""
+    xs, ws, pad, groups, flip = _random_window_shapes(16, 4242)[case]
+    rng = np.random.default_rng(900 + case)
+    gd, od = cdims(gpu, xs, ws, padding=pad, groups=groups, flipkernel=flip)
+    assert od.y_shape()[:2] == xs[:2]
+    x, w, b, dy = host_inputs("bf16", rng.normal(size=xs), rng.normal(size=ws) * np.sqrt(2.0 / (9 * ws[2])), rng.normal(size=ws[3]) * 0.1,
+                              rng.normal(size=od.y_shape()))
+    dx_, dw_, db_, ddy_ = (dev(gpu, a, "bf16") for a in (x, w, b, dy))
+    out = {}
+    for tile in (84, 1, 2, 0):
+        gpu.set_option("conv_tile", tile)
+        try:
+            out[tile] = (gpu.fused_conv_bias_activation("relu", dw_, dx_, db_, gd).to_numpy(), gpu.conv_data_grad(ddy_, dw_, gd).to_numpy())
+        finally:
+            gpu.set_option("conv_tile", 0)
+    tag = f"random window shape {xs} {ws} pad {pad} groups {groups} flip {flip}: "
+    for tile in (1, 2, 0):
+        assert_close(out[tile][0], f64(out[84][0]), "bf16", tag + f"y, conv_tile {tile}")
+        assert_close(out[tile][1], f64(out[84][1]), "bf16", tag + f"dgrad, conv_tile {tile}")
