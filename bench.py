@@ -42,6 +42,12 @@ MEASURED_TRAFFIC = {
     ("IN", "gn_bwd_kernel"): 202833217,
     ("DROPOUT", "dropout_fwd_kernel"): 100695712,      # dropout_rng_kernel<float, 4, 2> in the trace
     ("DROPOUT", "dropout_mul_kernel"): 100691762,
+    # contractions (profiles/c4_gemm_mfma_lds_pmc.md, profiles/c5_conv_bf16_mfma_lds_pmc.md): reads + writes that
+    # left the per-XCD L2s, mean per launch; much of the GEMM's comes from the Infinity Cache rather than HBM
+    ("C4", "dense_gemm_kernel<bf16>"): 1557583872,
+    ("C5bf16", "conv_wgrad_kernel<bf16>"): 140685312,
+    ("C5bf16", "conv_fprop_kernel<bf16>"): 137945088,
+    ("C5bf16", "conv_dgrad_kernel<bf16>"): 137945088,
 }
 METRIC = "fwd+bwd TFLOP/s & HBM GB/s (% MI355X roofline) per LuxLib fused op, 1 GPU"
 
