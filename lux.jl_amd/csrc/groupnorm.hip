@@ -216,10 +216,34 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     using K = Kept<T, VEC>;
     typename K::type kd[CACHED ? kGnCache : 1], kv[CACHED ? kGnCache : 1];
     float d[1][VEC], v[1][VEC];
-    // fp32 storage: after the first pass kd holds dy * gamma, so the second pass needs no
-    // activation derivative; bf16 storage keeps delta (packing dy * gamma would round it) and
-    // recomputes
-    constexpr bool KEEP_G = sizeof(T) == 4;
+    // After the first pass kd holds g = dy * act'(y) * gamma, so the second pass needs neither the activation
+    // derivative nor the parameters (whose loads, between the dx stores, would each wait for the stores before
+    // them).  fp32 storage keeps g as it is; bf16 storage keeps it as eight fp16 values in the vector's four
+    // registers (11 bits against the 8 that dx is rounded to anyway; |g| stays far inside the fp16 range for
+    // cotangents and parameters that bf16 training produces, and saturates instead of overflowing).
+    constexpr bool KEEP_G = sizeof(T) == 4 || VEC == 8;
+    constexpr bool HALF_G = sizeof(T) == 2 && VEC == 8;
+    auto keep_half = [](const float (&gv)[VEC]) {
+        raw16_t r;
+        if constexpr (VEC == 8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const _Float16 lo = (_Float16)fminf(fmaxf(gv[2 * i], -65504.0f), 65504.0f);
+                const _Float16 hi = (_Float16)fminf(fmaxf(gv[2 * i + 1], -65504.0f), 65504.0f);
+                r[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+            }
+        }
+        return r;
+    };
+    auto get_half = [](const raw16_t& r, float (&gv)[VEC]) {
+        if constexpr (VEC == 8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                gv[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r[i] & 0xffffu));
+                gv[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r[i] >> 16));
+            }
+        }
+    };
     float s1 = 0.0f, s2 = 0.0f;
 
     // dy and g = dy * gamma for one vector; also returns the channel's parameters
@@ -270,7 +294,8 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                         s1 += gv[e];
                         s2 = fmaf(gv[e], xh, s2);
                     }
-                    if constexpr (KEEP_G) kd[u] = keep<T, VEC>(gv);
+                    if constexpr (HALF_G) kd[u] = keep_half(gv);
+                    else if constexpr (KEEP_G) kd[u] = keep<T, VEC>(gv);
                 }
                 if constexpr (AFFINE) {
                     // the first lane of the wave decides whether the wave has work in this pass
@@ -389,9 +414,10 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = qbeg + u * T_ + threadIdx.x;
             if (q < qend) {
-                K::get(kd[u], d[0]);
+                if constexpr (HALF_G) get_half(kd[u], d[0]);
+                else K::get(kd[u], d[0]);
                 K::get(kv[u], v[0]);
-                if constexpr (KEEP_G) {             // kd[u] holds dy * gamma
+                if constexpr (KEEP_G) {             // kd[u] holds dy * act' * gamma
                     float o[VEC];
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
