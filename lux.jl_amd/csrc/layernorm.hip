@@ -149,6 +149,21 @@ __device__ __forceinline__ void ln_dy(const T* gamma, const T* beta, uint32_t q,
     }
 }
 
+// the same with the parameters already in registers
+template <int ACT, int VEC>
+__device__ __forceinline__ void ln_dy_regs(const float (&gm)[VEC], const float (&bt)[VEC], float mean, float invstd,
+                                           const float (&dv)[VEC], const float (&xv)[VEC], float (&dy)[VEC]) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        dy[e] = dv[e];
+        if constexpr (ACT != LUXHIP_ACT_IDENTITY) {
+            const float sc = gm[e] * invstd;
+            const float pre = fmaf(xv[e], sc, fmaf(-mean, sc, bt[e]));
+            dy[e] *= Act<ACT>::d(Act<ACT>::f(pre), pre);
+        }
+    }
+}
+
 template <typename T, int ACT, int VEC, bool WAVE, bool CACHED>
 __global__ __launch_bounds__(WAVE ? 256 : 1024) void ln_bwd_dx_kernel(const T* __restrict__ delta, const T* __restrict__ x, const T* __restrict__ gamma,
                                  const T* __restrict__ beta, const float* __restrict__ save_mean,
@@ -254,6 +269,28 @@ __global__ __launch_bounds__(256) void ln_bwd_fused_kernel(const T* __restrict__
     for (int u = 0; u < kLnFusedCache; ++u)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) { ag[u][e] = 0.0f; ab[u][e] = 0.0f; }
+    // The affine parameters at this thread's positions are the same for every column: read once and kept as they lie
+    // in memory.  (Read inside the second pass they would sit between the dx stores, and a wave's memory operations
+    // complete in the order of their issue: every such load would wait for the store before it.)
+    typename K::type kgm[kLnFusedCache], kbt[kLnFusedCache];
+    const bool affine = gamma != nullptr;
+    if (affine) {
+#pragma unroll
+        for (int u = 0; u < kLnFusedCache; ++u) {
+            const size_t off = (size_t)min(u * 128u + t, nvec - 1) * VEC;
+            kgm[u] = K::load(gamma, off);
+            if constexpr (ACT != LUXHIP_ACT_IDENTITY) kbt[u] = K::load(beta, off);
+        }
+    }
+    auto params = [&](int u, float (&gm)[VEC], float (&bt)[VEC]) {
+        if (affine) {
+            K::get(kgm[u], gm);
+            if constexpr (ACT != LUXHIP_ACT_IDENTITY) K::get(kbt[u], bt);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) { gm[e] = 1.0f; bt[e] = 0.0f; }
+        }
+    };
     const uint32_t rounds = (R + pairs - 1) / pairs;              // the same for every wavefront: barriers inside
     for (uint32_t it = 0; it < rounds; ++it) {
         const uint32_t r = it * pairs + blockIdx.x * 2u + pair;
@@ -273,10 +310,11 @@ __global__ __launch_bounds__(256) void ln_bwd_fused_kernel(const T* __restrict__
         for (int u = 0; u < kLnFusedCache; ++u) {
             const uint32_t q = u * 128u + t;
             if (q < nvec && live) {
-                float d[VEC], v[VEC], dy[VEC], gm[VEC];
+                float d[VEC], v[VEC], dy[VEC], gm[VEC], bt[VEC];
                 K::get(kd[u], d);
                 K::get(kv[u], v);
-                ln_dy<T, ACT, VEC>(gamma, beta, q, mean, invstd, d, v, dy, gm);
+                params(u, gm, bt);
+                ln_dy_regs<ACT, VEC>(gm, bt, mean, invstd, d, v, dy);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     const float xh = (v[e] - mean) * invstd;
@@ -299,10 +337,11 @@ __global__ __launch_bounds__(256) void ln_bwd_fused_kernel(const T* __restrict__
         for (int u = 0; u < kLnFusedCache; ++u) {
             const uint32_t q = u * 128u + t;
             if (q < nvec && live) {
-                float d[VEC], v[VEC], dy[VEC], gm[VEC], o[VEC];
+                float d[VEC], v[VEC], dy[VEC], gm[VEC], bt[VEC], o[VEC];
                 K::get(kd[u], d);
                 K::get(kv[u], v);
-                ln_dy<T, ACT, VEC>(gamma, beta, q, mean, invstd, d, v, dy, gm);
+                params(u, gm, bt);
+                ln_dy_regs<ACT, VEC>(gm, bt, mean, invstd, d, v, dy);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     const float xh = (v[e] - mean) * invstd;
