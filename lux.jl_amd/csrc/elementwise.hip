@@ -221,7 +221,22 @@ __global__ __launch_bounds__(kThreads) void bias_act_bwd_plane_kernel(const T* _
     float acc[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-    for (uint32_t n = n0; n < n1; ++n) {
+    // Four n at a time, their loads before the first store: a load behind a store waits for it (a wave's memory
+    // operations complete in the order of their issue), so one n per trip pays a store and a load latency per n.
+    constexpr uint32_t U = 4;
+    uint32_t n = n0;
+    for (; n + U <= n1; n += U) {
+        float r[U][VEC];
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) dx_vec<T, ACT, VEC>(delta, out, pre, (size_t)(n + u) * P + p, r[u]);
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            if (dx) store_vec<T, VEC>(dx, (size_t)(n + u) * P + p, r[u]);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] += r[u][k];
+        }
+    }
+    for (; n < n1; ++n) {
         const size_t off = (size_t)n * P + p;
         float r[VEC];
         dx_vec<T, ACT, VEC>(delta, out, pre, off, r);
