@@ -143,11 +143,24 @@ __global__ void gn_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gam
         if (save_mean) save_mean[slice] = mean;
         if (save_invstd) save_invstd[slice] = invstd;
     }
-    // pass 3: normalise
+    // pass 3: normalise.  Scale and shift of the group's channels go through LDS (groups of up to 64 channels): read
+    // from global memory per vector, the loads would sit between the stores of this pass, and a load waits for the
+    // store before it (a wave's memory operations complete in the order of their issue).
+    __shared__ float chan[2 * 64];
+    const bool tabled = g.Cg <= 64;
+    if (tabled) {
+        if (threadIdx.x < g.Cg) {
+            const uint32_t c = k * g.Cg + threadIdx.x;
+            const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
+            chan[2 * threadIdx.x] = sc;
+            chan[2 * threadIdx.x + 1] = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+        }
+        __syncthreads();
+    }
     auto emit = [&](uint32_t q, const float (&xv)[VEC]) {
-        const uint32_t c = k * g.Cg + g.chdiv.div(q);
-        const float sc = (gamma ? ld(gamma + c) : 1.0f) * invstd;
-        const float sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+        const uint32_t j = g.chdiv.div(q), c = k * g.Cg + j;
+        const float sc = tabled ? chan[2 * j] : (gamma ? ld(gamma + c) : 1.0f) * invstd;
+        const float sh = tabled ? chan[2 * j + 1] : fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
         float o[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o[e] = Act<ACT>::f(fmaf(xv[e], sc, sh));
