@@ -259,12 +259,26 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     };
     float s1 = 0.0f, s2 = 0.0f;
 
+    // gamma, scale and shift of the group's channels through LDS (groups of up to 64 channels): one global load per
+    // workgroup and channel instead of two per vector, each with its own wait
+    __shared__ float chan[3 * 64];
+    const bool tabled = g.Cg <= 64;
+    if (tabled) {
+        if (threadIdx.x < g.Cg) {
+            const uint32_t c = k * g.Cg + threadIdx.x;
+            const float gm = gamma ? ld(gamma + c) : 1.0f;
+            chan[3 * threadIdx.x] = gm;
+            chan[3 * threadIdx.x + 1] = gm * invstd;
+            chan[3 * threadIdx.x + 2] = fmaf(-mean, gm * invstd, beta ? ld(beta + c) : 0.0f);
+        }
+        __syncthreads();
+    }
     // dy and g = dy * gamma for one vector; also returns the channel's parameters
     auto grad_terms = [&](uint32_t q, const float (&dv)[VEC], const float (&xv)[VEC], float (&gv)[VEC], float& a, float& b) {
-        const uint32_t c = k * g.Cg + g.chdiv.div(q);
-        const float gm = gamma ? ld(gamma + c) : 1.0f;
-        const float sc = gm * invstd;
-        const float sh = fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
+        const uint32_t j = g.chdiv.div(q), c = k * g.Cg + j;
+        const float gm = tabled ? chan[3 * j] : (gamma ? ld(gamma + c) : 1.0f);
+        const float sc = tabled ? chan[3 * j + 1] : gm * invstd;
+        const float sh = tabled ? chan[3 * j + 2] : fmaf(-mean, sc, beta ? ld(beta + c) : 0.0f);
         a = 0.0f;
         b = 0.0f;
 #pragma unroll
