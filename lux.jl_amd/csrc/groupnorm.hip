@@ -232,10 +232,13 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     // After the first pass kd holds g = dy * act'(y) * gamma, so the second pass needs neither the activation
     // derivative nor the parameters (whose loads, between the dx stores, would each wait for the stores before
     // them).  fp32 storage keeps g as it is; bf16 storage keeps it as eight fp16 values in the vector's four
-    // registers (11 bits against the 8 that dx is rounded to anyway; |g| stays far inside the fp16 range for
-    // cotangents and parameters that bf16 training produces, and saturates instead of overflowing).
-    constexpr bool KEEP_G = sizeof(T) == 4 || VEC == 8;
-    constexpr bool HALF_G = sizeof(T) == 2 && VEC == 8;
+    // registers (11 bits against the 8 that dx is rounded to anyway), scaled by a power of two that the thread
+    // takes from its first vector (its largest |g| lands in [256, 512): cotangents of any magnitude keep their
+    // bits, and later vectors may be 128 times larger).  A workgroup in which a value still leaves the fp16
+    // range reads the cotangent and x from memory again and recomputes (the check below).
+    // (identity and relu recompute their derivative in the second pass instead: cheaper than the packing)
+    constexpr bool HALF_G = sizeof(T) == 2 && VEC == 8 && ACT != LUXHIP_ACT_IDENTITY && ACT != LUXHIP_ACT_RELU;
+    constexpr bool KEEP_G = sizeof(T) == 4 || HALF_G;
     auto keep_half = [](const float (&gv)[VEC]) {
         raw16_t r;
         if constexpr (VEC == 8) {
@@ -258,6 +261,8 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         }
     };
     float s1 = 0.0f, s2 = 0.0f;
+    float gmax = 0.0f;                              // largest scaled |g| this thread has packed as fp16
+    float gscale = 0.0f, gunscale = 0.0f;           // the thread's power of two and its inverse; 0: not chosen yet
 
     // gamma, scale and shift of the group's channels through LDS (groups of up to 64 channels): one global load per
     // workgroup and channel instead of two per vector, each with its own wait
@@ -321,8 +326,27 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                         s1 += gv[e];
                         s2 = fmaf(gv[e], xh, s2);
                     }
-                    if constexpr (HALF_G) kd[u] = keep_half(gv);
-                    else if constexpr (KEEP_G) kd[u] = keep<T, VEC>(gv);
+                    if constexpr (HALF_G) {
+                        float m = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) m = fmaxf(m, fabsf(gv[e]));
+                        if (gscale == 0.0f && m > 0.0f) {
+                            if (m < 3.0e38f) {
+                                const int ex = __builtin_amdgcn_frexp_expf(m);   // m = f * 2^ex, 0.5 <= f < 1
+                                gscale = __builtin_ldexpf(1.0f, 9 - ex);
+                                gunscale = __builtin_ldexpf(1.0f, ex - 9);
+                            } else {
+                                gmax = m;                                        // infinite: recompute from memory
+                            }
+                        }
+                        float hv[VEC];
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) hv[e] = gv[e] * gscale;
+                        gmax = fmaxf(gmax, m * gscale);
+                        kd[u] = keep_half(hv);
+                    } else if constexpr (KEEP_G) {
+                        kd[u] = keep<T, VEC>(gv);
+                    }
                 }
                 if constexpr (AFFINE) {
                     // the first lane of the wave decides whether the wave has work in this pass
@@ -426,6 +450,9 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         }
     }
 
+    // a scaled |g| beyond the fp16 range (a vector far larger than the thread's first one, or an infinite value) was
+    // saturated in the registers: such a workgroup takes the cotangent and x from memory again and recomputes
+    const bool refetch = HALF_G && __syncthreads_or(gmax > 65504.0f);
     auto emit = [&](uint32_t q, const float (&dv)[VEC], const float (&xv)[VEC]) {
         float gv[VEC], a, b, o[VEC];
         grad_terms(q, dv, xv, gv, a, b);
@@ -441,8 +468,19 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         for (int u = 0; u < kGnCache; ++u) {
             const uint32_t q = qbeg + u * T_ + threadIdx.x;
             if (q < qend) {
-                if constexpr (HALF_G) get_half(kd[u], d[0]);
-                else K::get(kd[u], d[0]);
+                if (refetch) {
+                    gn_load<T, VEC>(delta, base + (size_t)q * VEC, d[0]);
+                    gn_load<T, VEC>(x, base + (size_t)q * VEC, v[0]);
+                    emit(q, d[0], v[0]);
+                    continue;
+                }
+                if constexpr (HALF_G) {
+                    get_half(kd[u], d[0]);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) d[0][e] *= gunscale;
+                } else {
+                    K::get(kd[u], d[0]);
+                }
                 K::get(kv[u], v[0]);
                 if constexpr (KEEP_G) {             // kd[u] holds dy * act' * gamma
                     float o[VEC];

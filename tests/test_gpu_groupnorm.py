@@ -104,3 +104,26 @@ def test_config3_full_size(gpu, gn_path, dtype):
     _, wdg, wdb = O.groupnorm_pullback(f64(x), f64(g), f64(b), G, "swish", eps, f64(delta))
     assert_close(gg.to_numpy(), wdg, dtype, "config3 dgamma", scale=rms(delta) * 10)
     assert_close(gb.to_numpy(), wdb, dtype, "config3 dbeta", scale=rms(delta) * 10)
+
+
+@pytest.mark.parametrize("scale", [1e6, 3e-6, 1e-20, "uneven"])
+@pytest.mark.parametrize("act", ["identity", "swish"])
+def test_pullback_with_scaled_cotangents_bf16(gpu, act, scale):
+    """bf16 cotangents far outside and far below the fp16 range, and cotangents whose magnitude differs by 1e4 between
+    the halves of a slice: the pullback keeps an intermediate as scaled fp16 in registers where it can, and must neither
+    saturate large values nor lose small ones (the result scales with the cotangent)."""
+    rng = np.random.default_rng(99)
+    shape, groups, eps = (16, 16, 8, 3), 2, 1e-3
+    if scale == "uneven":
+        factor = np.where(np.arange(8) % 4 >= 2, 1e4, 1.0).reshape(1, 1, 8, 1)
+    else:
+        factor = scale
+    x, g, b, delta = host_inputs("bf16", rng.normal(size=shape), rng.uniform(0.8, 1.2, 8), rng.normal(size=8) * 0.05,
+                                 rng.normal(size=shape) * factor)
+    y, back = gpu.pullback(gpu.groupnorm, dev(gpu, x, "bf16"), dev(gpu, g, "bf16"), dev(gpu, b, "bf16"), groups, act, eps)
+    gx, gg, gb = back(dev(gpu, delta, "bf16"))
+    wdx, wdg, wdb = O.groupnorm_pullback(f64(x), f64(g), f64(b), groups, act, eps, f64(delta))
+    tag = f"bf16 {act} cotangent x {scale}"
+    assert_close(gx.to_numpy(), wdx, "bf16", tag + " dx", rel=3e-2, scale=dx_scale(x, g, groups, eps, delta))
+    assert_close(gg.to_numpy(), wdg, "bf16", tag + " dgamma", rel=3e-2, scale=rms(delta))
+    assert_close(gb.to_numpy(), wdb, "bf16", tag + " dbeta", rel=3e-2, scale=rms(delta))
