@@ -244,8 +244,8 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         if constexpr (VEC == 8) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const _Float16 lo = (_Float16)fminf(fmaxf(gv[2 * i], -65504.0f), 65504.0f);
-                const _Float16 hi = (_Float16)fminf(fmaxf(gv[2 * i + 1], -65504.0f), 65504.0f);
+                const _Float16 lo = (_Float16)gv[2 * i];         // beyond the fp16 range: infinite, and the workgroup
+                const _Float16 hi = (_Float16)gv[2 * i + 1];     // recomputes from memory (gmax below), never reading it
                 r[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
             }
         }
@@ -300,6 +300,23 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         }
     };
 
+    // Parameter-gradient terms of a lane stay in its registers while its vectors lie in one channel (rows are
+    // usually many vectors long); the wave adds them up across lanes (DPP chain, LDS accumulators) only when a lane
+    // moves on to another channel, and once at the end.  j = jc for a lane without a vector in this trip.
+    constexpr uint32_t kNoChannel = 0xffffffffu;
+    uint32_t jc = kNoChannel;
+    float ac = 0.0f, bc = 0.0f;
+    auto gather = [&](uint32_t j, float a, float b) {
+        if (__any((int)(j != jc && jc != kNoChannel))) {       // uniform over the wave
+            wave_channel_accumulate(accg, accb, jc, ac, bc, jc != kNoChannel);
+            ac = 0.0f;
+            bc = 0.0f;
+        }
+        jc = j;
+        ac += a;
+        bc += b;
+    };
+
     const uint32_t iters = (qend - qbeg + T_ - 1) / T_;
     if constexpr (CACHED) {
 #pragma unroll
@@ -348,11 +365,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                         kd[u] = keep<T, VEC>(gv);
                     }
                 }
-                if constexpr (AFFINE) {
-                    // the first lane of the wave decides whether the wave has work in this pass
-                    if (qbeg + u * T_ + (w << 6) < qend)
-                        wave_channel_accumulate(accg, accb, active ? g.chdiv.div(q) : 0u, a, b, active);
-                }
+                if constexpr (AFFINE) gather(active ? g.chdiv.div(q) : jc, a, b);
             }
         }
     } else {
@@ -371,12 +384,10 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                     s2 = fmaf(gv[e], xh, s2);
                 }
             }
-            if constexpr (AFFINE) {
-                if (u * T_ + (w << 6) < g.nvec)
-                    wave_channel_accumulate(accg, accb, active ? g.chdiv.div(q) : 0u, a, b, active);
-            }
+            if constexpr (AFFINE) gather(active ? g.chdiv.div(q) : jc, a, b);
         }
     }
+    if constexpr (AFFINE) wave_channel_accumulate(accg, accb, jc, ac, bc, jc != kNoChannel);
     s1 = block_sum(s1, sm);
     s2 = block_sum(s2, sm);
     if (parts > 1) {
@@ -474,20 +485,17 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                     emit(q, d[0], v[0]);
                     continue;
                 }
-                if constexpr (HALF_G) {
-                    get_half(kd[u], d[0]);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) d[0][e] *= gunscale;
-                } else {
-                    K::get(kd[u], d[0]);
-                }
+                if constexpr (HALF_G) get_half(kd[u], d[0]);
+                else K::get(kd[u], d[0]);
                 K::get(kv[u], v[0]);
-                if constexpr (KEEP_G) {             // kd[u] holds dy * act' * gamma
+                if constexpr (KEEP_G) {             // kd[u] holds dy * act' * gamma (HALF_G: times gscale)
+                    // invstd * (g - s1 - xh * s2) as two fused multiply-adds per element
+                    const float kg = HALF_G ? invstd * gunscale : invstd, k1 = -s1 * invstd, k2 = -s2 * invstd;
                     float o[VEC];
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         const float xh = (v[0][e] - mean) * invstd;
-                        o[e] = invstd * (d[0][e] - s1 - xh * s2);
+                        o[e] = fmaf(xh, k2, fmaf(d[0][e], kg, k1));
                     }
                     gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
                 } else {
