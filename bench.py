@@ -30,18 +30,18 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a copy of known
 # size (profiles/*_hbm_traffic_pmc.md hold the commands and the raw counter values).
 MEASURED_TRAFFIC = {
-    ("C2", "bn_fwd_resident_kernel"): 67758714,
-    ("C2", "bias_act_fwd_kernel"): 67137042,
-    ("C2", "bias_act_bwd_channel_kernel"): 100892887,
-    ("C2", "bn_bwd_resident_kernel"): 100993602,
-    ("C3", "gn_fwd_kernel"): 134327510,
-    ("C3", "gn_bwd_kernel"): 202204269,
-    ("C3bf16", "gn_fwd_kernel"): 67290712,
-    ("C3bf16", "gn_bwd_kernel"): 101301450,
-    ("IN", "gn_fwd_kernel"): 135315416,
-    ("IN", "gn_bwd_kernel"): 202833217,
-    ("DROPOUT", "dropout_fwd_kernel"): 100695712,      # dropout_rng_kernel<float, 4, 2> in the trace
-    ("DROPOUT", "dropout_mul_kernel"): 100691762,
+    ("C2", "bn_fwd_resident_kernel"): 67769957,
+    ("C2", "bias_act_fwd_kernel"): 67141018,
+    ("C2", "bias_act_bwd_channel_kernel"): 100903236,
+    ("C2", "bn_bwd_resident_kernel"): 100990363,
+    ("C3", "gn_fwd_kernel"): 134388357,
+    ("C3", "gn_bwd_kernel"): 202241307,
+    ("C3bf16", "gn_fwd_kernel"): 67319219,
+    ("C3bf16", "gn_bwd_kernel"): 101392385,
+    ("IN", "gn_fwd_kernel"): 135504475,
+    ("IN", "gn_bwd_kernel"): 202878042,
+    ("DROPOUT", "dropout_fwd_kernel"): 100695641,      # dropout_rng_kernel<float, 4, 2> in the trace
+    ("DROPOUT", "dropout_mul_kernel"): 100691812,
     # contractions (profiles/c4_gemm_mfma_lds_pmc.md, profiles/c5_conv_bf16_mfma_lds_pmc.md): reads + writes that
     # left the per-XCD L2s, mean per launch; much of the GEMM's comes from the Infinity Cache rather than HBM
     ("C4", "dense_gemm_kernel<bf16>"): 1557583872,
