@@ -11,7 +11,9 @@ pytestmark = pytest.mark.gpu
 CASES = [((6, 2), 2), ((4, 4, 6, 2), 3), ((2, 2, 6, 2), 2), ((5, 12, 3), 4), ((16, 16, 8, 3), 2), ((64, 6, 2), 3),
          ((32, 32, 12, 2), 1), ((8, 8, 16, 2), 16), ((96, 96, 4, 2), 1),
          # slices that two workgroups share (fp32: 19200 elements per slice, bf16: 65536)
-         ((40, 40, 24, 2), 2), ((64, 64, 32, 2), 2)]
+         ((40, 40, 24, 2), 2), ((64, 64, 32, 2), 2),
+         # 72 channels per group: more than the kernels' LDS tables of channel parameters hold
+         ((4, 4, 144, 2), 2)]
 
 
 @pytest.fixture(params=["wait", "no_wait"])
