@@ -671,6 +671,35 @@ def timed(lux, fn, steps, warmup):
     return ms_gpu / steps, ms_wall / steps
 
 
+REGIONS = 3
+
+
+def timed_regions(lux, fn, steps, warmup):
+    """The warm-up, then REGIONS timed regions of `steps` steps each, back to back.  Returns the region with the
+    median time (device events, host clock) and the per-step times of all regions: one sample cannot tell a slow
+    box from a clock that has not settled."""
+    for _ in range(warmup):
+        fn()
+    lux.synchronize()
+    samples = []
+    for _ in range(REGIONS):
+        e0, e1 = lux.Event(), lux.Event()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        ms_gpu = e0.elapsed_ms(e1)          # waits for e1
+        lux.synchronize()
+        ms_wall = (time.perf_counter() - t0) * 1e3
+        samples.append((max(ms_gpu, ms_wall) / steps, ms_gpu / steps, ms_wall / steps))
+    order = sorted(samples)
+    med = order[len(order) // 2]
+    spread = {"regions": REGIONS, "ms_per_step_median": round(med[0], 5), "ms_per_step_min": round(order[0][0], 5),
+              "ms_per_step_max": round(order[-1][0], 5), "ms_per_step_in_order": [round(x[0], 5) for x in samples]}
+    return med[1], med[2], spread
+
+
 def timed_graph(lux, fn, steps):
     """One step recorded into a HIP graph on the library's stream (after the eager warm-up has sized the
     workspace and filled the allocator's pool) and replayed `steps` times: the step without the host's
@@ -745,7 +774,7 @@ def measure(lux, name, args):
     work = wl.work_per_step()
 
     step = wl.rotating_step if args.rotate > 1 and hasattr(wl, "rotating_step") else wl.step
-    ms_gpu, ms_wall = timed(lux, step, steps, warmup)
+    ms_gpu, ms_wall, spread = timed_regions(lux, step, steps, warmup)
     ms = max(ms_gpu, ms_wall)           # whole-job time: the slower of the device and host clocks
     ms_graph = timed_graph(lux, wl.step, steps) if args.graph else None
     warm = {"ms_per_step": round(ms, 5), "value": round(work / (ms * 1e-3) / scale, 2), "unit": unit,
@@ -760,7 +789,7 @@ def measure(lux, name, args):
         cold_wl = WORKLOADS[name]()
         cold_wl.rotate = args.cold_sets
         cold_wl.setup(lux)
-        cg, cw_ = timed(lux, cold_wl.rotating_step, steps, warmup)
+        cg, cw_, spread = timed_regions(lux, cold_wl.rotating_step, steps, warmup)
         cms = max(cg, cw_)
         cold = {"sets_of_tensors": args.cold_sets, "ms_per_step": round(cms, 5), "value": round(work / (cms * 1e-3) / scale, 2),
                 "unit": unit, "frac_of_peak": round(work / (cms * 1e-3) / scale / peak, 4)}
@@ -825,6 +854,7 @@ def measure(lux, name, args):
         "workload": wl.name, "description": wl.description, "dtype": wl.dtype, "bound": wl.bound, "value": round(value, 2), "unit": unit,
         "steps": steps, "warmup": warmup, "ms_per_step": round(ms_head, 5), "frac_of_peak": round(value / peak, 4),
         "ms_per_step_gpu_events": round(ms_gpu_head, 5), "ms_per_step_host_clock": round(ms_wall_head, 5),
+        "timing": f"median of {REGIONS} timed regions of {steps} steps each, after {warmup} warm-up steps", "spread": spread,
         "roofline": roofline, "kernels": kernels,
     }
     if cold is not None:
@@ -893,6 +923,12 @@ def main():
     for opt in args.option:
         name, _, val = opt.partition("=")
         lux.set_option(name, int(val))
+    def peaks():
+        cp, mb, mf = C.c_double(), C.c_double(), C.c_double()
+        lux._lib.call("luxhip_measure_peaks", lux.current_stream(), C.byref(cp), C.byref(mb), C.byref(mf))
+        return {"copy_GBps": round(cp.value, 1), "mfma_bf16_TFLOPs": round(mb.value, 1), "mfma_f32_TFLOPs": round(mf.value, 1)}
+
+    peaks_before = None if args.no_peaks else peaks()
     names = DEFAULT_ORDER if args.workload == "ALL" else [args.workload]
     entries = [measure(lux, n, args) for n in names]
     head = entries[0]
@@ -903,6 +939,7 @@ def main():
         "data": "synthetic", "config": {"workload": f"{head['workload']}: {head['description']}"},
         "options": args.option + ([f"rotate={args.rotate}"] if args.rotate > 1 else []), "frac_of_peak": head["frac_of_peak"],
         "ms_per_step_gpu_events": head["ms_per_step_gpu_events"], "ms_per_step_host_clock": head["ms_per_step_host_clock"],
+        "timing": head["timing"], "spread": head["spread"],
         "roofline": head["roofline"], "kernels": head["kernels"],
     }
     for k in ("cold_inputs", "warm_inputs", "inputs", "graph_replay", "fused_variant", "cpu_baseline"):
@@ -910,13 +947,13 @@ def main():
             out[k] = head[k]
     out["configs"] = entries
     if not args.no_peaks:
-        cp, mb, mf = C.c_double(), C.c_double(), C.c_double()
-        lux._lib.call("luxhip_measure_peaks", lux.current_stream(), C.byref(cp), C.byref(mb), C.byref(mf))
-        out["measured_peaks"] = {"copy_GBps": round(cp.value, 1), "mfma_bf16_TFLOPs": round(mb.value, 1), "mfma_f32_TFLOPs": round(mf.value, 1),
-                                 "published": {"hbm_GBps": PEAK_HBM_GBS, "mfma_bf16_TFLOPs": PEAK_MFMA_TFLOPS["bf16"],
-                                               "mfma_f32_TFLOPs": PEAK_MFMA_TFLOPS["f32"]},
-                                 "note": "streaming copy of 512 MiB (read + written bytes); register-only MFMA loops on pseudo-random "
-                                         "operands, 8 waves per compute unit, after the clocks have settled"}
+        after = peaks()
+        out["measured_peaks"] = dict(after, before_the_workloads=peaks_before, after_the_workloads=after,
+                                     published={"hbm_GBps": PEAK_HBM_GBS, "mfma_bf16_TFLOPs": PEAK_MFMA_TFLOPS["bf16"],
+                                                "mfma_f32_TFLOPs": PEAK_MFMA_TFLOPS["f32"]},
+                                     note="streaming copy of 512 MiB (read + written bytes); register-only MFMA loops on pseudo-random "
+                                          "operands, 8 waves per compute unit, after the clocks have settled; measured once before and "
+                                          "once after the workloads (the top-level figures are the later ones)")
     if args.calibrate_copy:
         nbytes = 256 << 20
         a, b = lux.DeviceArray((nbytes // 4,), "f32"), lux.DeviceArray((nbytes // 4,), "f32")

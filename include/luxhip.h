@@ -41,6 +41,9 @@ extern "C" {
 /* storage types */
 #define LUXHIP_F32 0
 #define LUXHIP_BF16 1
+/* bf16 storage with one tensor of the call kept in fp32: accepted only where a function's comment
+ * says which tensor that is (the products and the softmax passes of attention) */
+#define LUXHIP_BF16_WIDE 2
 
 /* activation ids.  tanh_fast / sigmoid_fast (NNlib.fast_act, src/layers/basic.jl:366-371 of
  * the reference) map to TANH / SIGMOID on the host side. */
@@ -61,7 +64,10 @@ typedef void* luxhip_event_t;  /* a hipEvent_t */
 /* ---------------------------------------------------------------- runtime ------------
  * The reference leaves device buffers and streams to CUDA.jl / AMDGPU.jl (task-local
  * handles, ext/CUDAExt/cublaslt.jl:80-82,156-178; CUDA.stream() :287).  This library owns
- * them instead. */
+ * them instead.
+ * One device per process: luxhip_init(device) binds the library to that device until
+ * luxhip_shutdown; a second call with the same device is a no-op, with another device it returns
+ * LUXHIP_INVALID ("already initialised on device N").  More than one GPU means one process per GPU. */
 int luxhip_init(int device);
 int luxhip_shutdown(void);
 const char* luxhip_last_error(void);
@@ -75,7 +81,11 @@ int luxhip_stream_destroy(luxhip_stream_t s);
  * least `bytes` ahead of time.  Operators grow it on demand without making the host wait for the
  * device (the outgrown block is retired behind an event on the stream), but not while the stream
  * records a HIP graph: there a call that finds it too small returns LUXHIP_INVALID.  A caller that
- * records graphs runs each operator once eagerly before, or reserves here.  No counterpart in the
+ * records graphs runs each operator once eagerly before, or reserves here.  A recorded graph keeps
+ * the address of the block that the stream had while it was recorded: if a later eager call on that
+ * stream outgrows the block, the library keeps the old block allocated (it is never reused until
+ * luxhip_shutdown, also when the stream is destroyed), so replays stay valid; they then use their
+ * own scratch memory and must not overlap with each other, as before.  No counterpart in the
  * reference, whose vendor wrappers allocate their scratch arrays per call
  * (ext/cuDNNExt/batchnorm.jl:17-18). */
 int luxhip_reserve(luxhip_stream_t s, size_t bytes);
@@ -238,7 +248,11 @@ int luxhip_instancenorm_running_stats(luxhip_stream_t s, int dtype, int64_t I, i
  * scaled_dot_product_attention (src/impl/attention.jl:5-117) = batched_matmul(k, q .* scale) ->
  * apply_attention_mask_bias -> softmax over the key positions -> batched_matmul(v, probs).  The two
  * products are luxhip_batched_matmul_strided calls; these are the passes between them.
- * logits, probs, dprobs, dlogits: (S, L, H, B) column-major, S = key positions. */
+ * logits, probs, dprobs, dlogits: (S, L, H, B) column-major, S = key positions.
+ * dtype LUXHIP_BF16_WIDE: bf16 storage, but the logits (forward) and dprobs (pullback) are fp32 as
+ * luxhip_batched_matmul_strided writes them under the same dtype: a logit rounded to bf16 carries
+ * an error of 2^-9 |logit|, which the exponential turns into a relative error of that size in the
+ * weight; with the two tensors in fp32 the weights and gradients stay within the bf16 parity bar. */
 
 /* probs[:, l, h, b] = softmax_s(scale * logits[s, l, h, b] + bias[s, l, h, b], -inf where masked)
  * (apply_attention_mask_bias, src/impl/attention.jl:119-128; NNlib.softmax(...; dims=1), :94-104).
@@ -338,7 +352,9 @@ int luxhip_batched_matmul(luxhip_stream_t s, int dtype, int transA, int transB, 
  *   2: op(B)[k, n] is zero for k > n (weights and their cotangent as the right operand, contracted
  *      over s): the contraction of a tile stops at its last column;
  *   3: op(B)[k, n] is zero for k < n (the same matrices transposed, contracted over l): it starts
- *      at the tile's first column. */
+ *      at the tile's first column.
+ * dtype LUXHIP_BF16_WIDE: A and B bf16, C fp32 (the accumulators unrounded; ldc and stridesC in
+ * elements as before). */
 int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int transB, int64_t M, int64_t N,
                                   int64_t K, const int64_t* batch_dims, const void* A, int64_t lda,
                                   const int64_t* stridesA, const void* B, int64_t ldb, const int64_t* stridesB,

@@ -25,9 +25,10 @@ __device__ __forceinline__ float wave_add(float v) {
     return v;
 }
 
-template <typename T>
+// TL: type of the logits (T, or float under LUXHIP_BF16_WIDE)
+template <typename T, typename TL>
 struct SoftmaxCol {
-    const T* x;
+    const TL* x;
     const T* bias;
     const uint8_t* mask;
     float scale;
@@ -41,8 +42,8 @@ struct SoftmaxCol {
 };
 
 // NV > 0: the column (S <= 64 NV) is held in registers; NV == 0: any S, re-read per pass
-template <typename T, int NV>
-__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_kernel(const T* __restrict__ logits, T* __restrict__ probs,
+template <typename T, typename TL, int NV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_kernel(const TL* __restrict__ logits, T* __restrict__ probs,
                                                                            int S, int L, int H, int64_t cols, float scale,
                                                                            int causal, const uint8_t* __restrict__ mask,
                                                                            int64_t mask_sh, int64_t mask_sb,
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_kernel(const
     const int64_t hb = col / L;
     const int h = (int)(hb % H);
     const int64_t b = hb / H;
-    SoftmaxCol<T> c;
+    SoftmaxCol<T, TL> c;
     c.x = logits + col * S;
     c.bias = bias ? bias + (int64_t)l * S + h * bias_sh + b * bias_sb : nullptr;
     c.mask = mask ? mask + (int64_t)l * S + h * mask_sh + b * mask_sb : nullptr;
@@ -96,14 +97,14 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_kernel(const
 }
 
 // dlogits = scale * probs .* (dprobs - sum_s dprobs .* probs)
-template <typename T, int NV>
-__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_kernel(const T* __restrict__ dprobs,
+template <typename T, typename TL, int NV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_kernel(const TL* __restrict__ dprobs,
                                                                            const T* __restrict__ probs, T* __restrict__ dlogits,
                                                                            int S, int L, int causal, int64_t cols, float scale) {
     const int lane = threadIdx.x & 63;
     const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
     if (col >= cols) return;
-    const T* dy = dprobs + col * S;
+    const TL* dy = dprobs + col * S;
     const T* y = probs + col * S;
     T* dx = dlogits + col * S;
     const int limit = causal ? (int)(col % L) : S - 1;      // positions past it: weight 0, cotangent not read
@@ -137,9 +138,21 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_kernel(const
 
 // The same with 16-byte accesses: lane j owns the vectors j, j + 64, ... of the column
 // (S a multiple of the vector width, S <= 64 VEC NVV, every pointer 16-byte aligned).
-template <typename T, int NVV>
+// A wide tensor is read as VEC values of TL per lane and vector (two 16-byte loads for fp32 beside bf16).
+template <typename T, typename TL>
+__device__ __forceinline__ void load_wide(const TL* p, float (&v)[Vec<T>::N]) {
+    if constexpr (sizeof(TL) == sizeof(T)) {
+        Vec<T>::load(reinterpret_cast<const T*>(p), v);
+    } else {
+        static_assert(Vec<T>::N == 8 && sizeof(TL) == 4, "bf16 storage beside fp32");
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+}
+
+template <typename T, typename TL, int NVV>
 __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_vec_kernel(
-    const T* __restrict__ logits, T* __restrict__ probs, int S, int L, int H, int64_t cols, float scale, int causal,
+    const TL* __restrict__ logits, T* __restrict__ probs, int S, int L, int H, int64_t cols, float scale, int causal,
     const uint8_t* __restrict__ mask, int64_t mask_sh, int64_t mask_sb, const T* __restrict__ bias, int64_t bias_sh,
     int64_t bias_sb) {
     constexpr int VEC = Vec<T>::N;
@@ -150,7 +163,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_vec_kernel(
     const int64_t hb = col / L;
     const int h = (int)(hb % H);
     const int64_t b = hb / H;
-    const T* x = logits + col * S;
+    const TL* x = logits + col * S;
     const T* bp = bias ? bias + (int64_t)l * S + h * bias_sh + b * bias_sb : nullptr;
     const uint8_t* mp = mask ? mask + (int64_t)l * S + h * mask_sh + b * mask_sb : nullptr;
     const int limit = causal ? l : S - 1;
@@ -160,7 +173,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_vec_kernel(
     for (int i = 0; i < NVV; ++i) {
         const int s0 = (lane + 64 * i) * VEC;
         if (s0 < S && s0 <= limit) {            // vectors past the causal limit are never read
-            Vec<T>::load(x + s0, z[i]);
+            load_wide<T, TL>(x + s0, z[i]);
             float bv[VEC];
             if (bp) Vec<T>::load(bp + s0, bv);
 #pragma unroll
@@ -198,8 +211,8 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_fwd_vec_kernel(
     }
 }
 
-template <typename T, int NVV>
-__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(const T* __restrict__ dprobs,
+template <typename T, typename TL, int NVV>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(const TL* __restrict__ dprobs,
                                                                                const T* __restrict__ probs,
                                                                                T* __restrict__ dlogits, int S, int L, int causal,
                                                                                int64_t cols, float scale) {
@@ -207,7 +220,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(c
     const int lane = threadIdx.x & 63;
     const int64_t col = (int64_t)blockIdx.x * kAttnWaves + (threadIdx.x >> 6);
     if (col >= cols) return;
-    const T* dy = dprobs + col * S;
+    const TL* dy = dprobs + col * S;
     const T* y = probs + col * S;
     const int limit = causal ? (int)(col % L) : S - 1;
     const int wend = causal ? min(S, ((limit >> 7) + 1) << 7) : S;       // see attn_softmax_bwd_kernel
@@ -218,7 +231,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_softmax_bwd_vec_kernel(c
         const int s0 = (lane + 64 * i) * VEC;
         if (s0 < S && s0 <= limit) {            // vectors wholly past the limit: weights are 0, nothing is read
             Vec<T>::load(y + s0, yv[i]);
-            Vec<T>::load(dy + s0, dv[i]);
+            load_wide<T, TL>(dy + s0, dv[i]);
 #pragma unroll
             for (int k = 0; k < VEC; ++k) dot += yv[i][k] * dv[i][k];
         } else {
@@ -255,8 +268,8 @@ static inline int cached_vectors(int64_t S) {
     return 0;
 }
 
-template <typename T>
-static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int64_t B, const T* logits, float scale, int causal,
+template <typename T, typename TL>
+static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int64_t B, const TL* logits, float scale, int causal,
                             const uint8_t* mask, int64_t mask_sh, int64_t mask_sb, const T* bias, int64_t bias_sh,
                             int64_t bias_sb, T* probs) {
     const int64_t cols = L * H * B;
@@ -265,7 +278,7 @@ static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int6
     const bool aligned = aligned16(logits) && aligned16(probs) && (bias == nullptr || aligned16(bias)) &&
                          (mask == nullptr || (reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
 #define LUX_SOFTMAX_FWD_VEC(NVV)                                                                                                \
-    attn_softmax_fwd_vec_kernel<T, NVV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
+    attn_softmax_fwd_vec_kernel<T, TL, NVV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
                                                                          mask, mask_sh, mask_sb, bias, bias_sh, bias_sb)
     switch (lane_vectors<T>(S, aligned)) {
         case 1: LUX_SOFTMAX_FWD_VEC(1); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
@@ -276,7 +289,7 @@ static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int6
     }
 #undef LUX_SOFTMAX_FWD_VEC
 #define LUX_SOFTMAX_FWD(NV)                                                                                                   \
-    attn_softmax_fwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
+    attn_softmax_fwd_kernel<T, TL, NV><<<grid, kAttnWaves * 64, 0, s>>>(logits, probs, (int)S, (int)L, (int)H, cols, scale, causal, \
                                                                     mask, mask_sh, mask_sb, bias, bias_sh, bias_sb)
     switch (cached_vectors(S)) {
         case 1: LUX_SOFTMAX_FWD(1); break;
@@ -291,13 +304,13 @@ static int softmax_fwd_impl(hipStream_t s, int64_t S, int64_t L, int64_t H, int6
     return LUXHIP_OK;
 }
 
-template <typename T>
-static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t L, int causal, int64_t cols, const T* dprobs, const T* probs,
+template <typename T, typename TL>
+static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t L, int causal, int64_t cols, const TL* dprobs, const T* probs,
                             float scale, T* dlogits) {
     const unsigned grid = (unsigned)ceil_div(cols, kAttnWaves);
     ProfScope ps("attn_softmax_bwd_kernel", s);
 #define LUX_SOFTMAX_BWD_VEC(NVV) \
-    attn_softmax_bwd_vec_kernel<T, NVV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, (int)L, causal, cols, scale)
+    attn_softmax_bwd_vec_kernel<T, TL, NVV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, (int)L, causal, cols, scale)
     switch (lane_vectors<T>(S, aligned16(dprobs) && aligned16(probs) && aligned16(dlogits))) {
         case 1: LUX_SOFTMAX_BWD_VEC(1); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
         case 2: LUX_SOFTMAX_BWD_VEC(2); LUX_CHECK_LAUNCH(); return LUXHIP_OK;
@@ -306,7 +319,7 @@ static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t L, int causal, int
         default: break;
     }
 #undef LUX_SOFTMAX_BWD_VEC
-#define LUX_SOFTMAX_BWD(NV) attn_softmax_bwd_kernel<T, NV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, (int)L, causal, cols, scale)
+#define LUX_SOFTMAX_BWD(NV) attn_softmax_bwd_kernel<T, TL, NV><<<grid, kAttnWaves * 64, 0, s>>>(dprobs, probs, dlogits, (int)S, (int)L, causal, cols, scale)
     switch (cached_vectors(S)) {
         case 1: LUX_SOFTMAX_BWD(1); break;
         case 2: LUX_SOFTMAX_BWD(2); break;
@@ -321,7 +334,7 @@ static int softmax_bwd_impl(hipStream_t s, int64_t S, int64_t L, int causal, int
 }
 
 static int softmax_check(int dtype, int64_t S, int64_t cols) {
-    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
+    LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16 && dtype != LUXHIP_BF16_WIDE, "unsupported dtype %d", dtype);
     LUX_INVALID_IF(S < 0 || cols < 0, "invalid dimension");
     LUX_UNSUPPORTED_IF(S >= (1ll << 31) || cols >= (1ll << 33), "attention softmax: dimension too large");
     return LUXHIP_OK;
@@ -360,9 +373,13 @@ int luxhip_attention_softmax_fwd(luxhip_stream_t s, int dtype, int64_t S, int64_
     LUX_INVALID_IF(mask_stride_h < 0 || mask_stride_b < 0 || bias_stride_h < 0 || bias_stride_b < 0, "negative stride");
     LUX_INVALID_IF(causal != 0 && mask != nullptr, "`mask` and `is_causal` cannot both be specified");
     if (dtype == LUXHIP_F32)
-        return softmax_fwd_impl<float>((hipStream_t)s, S, L, H, B, (const float*)logits, (float)scale, causal, mask, mask_stride_h,
-                                       mask_stride_b, (const float*)bias, bias_stride_h, bias_stride_b, (float*)probs);
-    return softmax_fwd_impl<bf16_t>((hipStream_t)s, S, L, H, B, (const bf16_t*)logits, (float)scale, causal, mask, mask_stride_h,
+        return softmax_fwd_impl<float, float>((hipStream_t)s, S, L, H, B, (const float*)logits, (float)scale, causal, mask, mask_stride_h,
+                                              mask_stride_b, (const float*)bias, bias_stride_h, bias_stride_b, (float*)probs);
+    if (dtype == LUXHIP_BF16_WIDE)
+        return softmax_fwd_impl<bf16_t, float>((hipStream_t)s, S, L, H, B, (const float*)logits, (float)scale, causal, mask,
+                                               mask_stride_h, mask_stride_b, (const bf16_t*)bias, bias_stride_h, bias_stride_b,
+                                               (bf16_t*)probs);
+    return softmax_fwd_impl<bf16_t, bf16_t>((hipStream_t)s, S, L, H, B, (const bf16_t*)logits, (float)scale, causal, mask, mask_stride_h,
                                     mask_stride_b, (const bf16_t*)bias, bias_stride_h, bias_stride_b, (bf16_t*)probs);
 }
 
@@ -376,9 +393,12 @@ int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_
     LUX_INVALID_IF(dprobs == nullptr || probs == nullptr || dlogits == nullptr,
                    "attention_softmax_bwd: dprobs, probs and dlogits must not be NULL");
     if (dtype == LUXHIP_F32)
-        return softmax_bwd_impl<float>((hipStream_t)s, S, L, causal, cols, (const float*)dprobs, (const float*)probs, (float)scale,
-                                       (float*)dlogits);
-    return softmax_bwd_impl<bf16_t>((hipStream_t)s, S, L, causal, cols, (const bf16_t*)dprobs, (const bf16_t*)probs, (float)scale,
+        return softmax_bwd_impl<float, float>((hipStream_t)s, S, L, causal, cols, (const float*)dprobs, (const float*)probs,
+                                              (float)scale, (float*)dlogits);
+    if (dtype == LUXHIP_BF16_WIDE)
+        return softmax_bwd_impl<bf16_t, float>((hipStream_t)s, S, L, causal, cols, (const float*)dprobs, (const bf16_t*)probs,
+                                               (float)scale, (bf16_t*)dlogits);
+    return softmax_bwd_impl<bf16_t, bf16_t>((hipStream_t)s, S, L, causal, cols, (const bf16_t*)dprobs, (const bf16_t*)probs, (float)scale,
                                     (bf16_t*)dlogits);
 }
 

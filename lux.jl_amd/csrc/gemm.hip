@@ -15,7 +15,6 @@ int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t 
 int transpose_matrix_bf16(hipStream_t s, const bf16_t* in, bf16_t* out, int64_t P, int64_t C);   // conv.hip
 
 int gemm_tile_override() { return (int)option_gemm_tile(); }
-
 // The 256 x 256 bf16 kernel reads K-major operands from LDS at twice the rate of M/N-major ones
 // (plain 16-byte reads against transposing reads): 1090-1190 TFLOP/s against 800-950 measured on
 // 4096..11008-sized problems.  A large M/N-major operand is therefore copied into the K-major
@@ -80,9 +79,10 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
 template <typename T>
 static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const int64_t* bdim, const T* A,
                         int64_t lda, const int64_t* sA, const T* B, int64_t ldb, const int64_t* sB, T* C, int64_t ldc,
-                        const int64_t* sC, int structure) {
+                        const int64_t* sC, int structure, int c_f32 = 0) {
     DenseArgs<T> a;
     a.structure = structure;
+    a.c_f32 = c_f32;
     const bool a_kmajor = transA != 0, b_kmajor = transB == 0;
     a.A.p = A;
     a.A.sr = a_kmajor ? lda : 1;
@@ -129,7 +129,7 @@ static int batched_dispatch(hipStream_t s, int dtype, int transA, int transB, in
         return batched_impl<float>(s, transA, transB, M, N, K, bdim, (const float*)A, lda, sA, (const float*)B, ldb, sB, (float*)C,
                                    ldc, sC, structure);
     return batched_impl<bf16_t>(s, transA, transB, M, N, K, bdim, (const bf16_t*)A, lda, sA, (const bf16_t*)B, ldb, sB,
-                                (bf16_t*)C, ldc, sC, structure);
+                                (bf16_t*)C, ldc, sC, structure, dtype == LUXHIP_BF16_WIDE ? 1 : 0);
 }
 
 // out[i] = sum_b in[i + b n]: `sum(tmp; dims=3)` of a stack of matrices, accumulated in fp32 in batch order
@@ -223,7 +223,7 @@ int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int 
                                   int64_t ldb, const int64_t* stridesB, void* C, int64_t ldc, const int64_t* stridesC,
                                   int structure) {
     LUX_REQUIRE_INIT();
-    int rc = gemm_check(dtype, 0, M, N, K);
+    int rc = gemm_check(dtype == LUXHIP_BF16_WIDE ? LUXHIP_BF16 : dtype, 0, M, N, K);
     if (rc != LUXHIP_OK) return rc;
     LUX_INVALID_IF(batch_dims == nullptr || stridesA == nullptr || stridesB == nullptr || stridesC == nullptr,
                    "batched_matmul_strided: batch extents and strides must not be NULL");

@@ -241,6 +241,7 @@ template <typename T>
 struct BatchTile {
     Operand<T> A, B;
     T* C;
+    int64_t coff;   // elements between a.C and this product's C
     int m0, n0;
     int K;          // extent of the contraction for this tile (a.structure may shorten it)
     bool store;     // false: the tile is not computed (a.structure == 1, every m > n)
@@ -262,7 +263,8 @@ __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t,
     bt.B = a.B;
     bt.A.p = a.A.p + i0 * a.bsA[0] + i1 * a.bsA[1] + i2 * a.bsA[2];
     bt.B.p = a.B.p + i0 * a.bsB[0] + i1 * a.bsB[1] + i2 * a.bsB[2];
-    bt.C = a.C + i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
+    bt.coff = i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
+    bt.C = a.C + bt.coff;
     bt.m0 = tm * TILE_M;
     bt.n0 = tn * TILE_N;
     bt.K = a.K;
@@ -278,6 +280,17 @@ __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t,
         bt.K = a.K - k_lo;
     }
     return bt;
+}
+
+// The tile as fp32 (a.c_f32): the accumulators go to memory unrounded, for results that feed a
+// softmax or its pullback, where an error of one bf16 unit in the last place of a logit is a
+// relative error of the same size times the logit in the weight.
+template <class ML, typename T, int WM, int WN, bool FULL>
+__device__ __forceinline__ void store_tile_f32(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int64_t coff, int m0, int n0) {
+    float* C = reinterpret_cast<float*>(a.C) + coff;
+    ML::for_each(acc, m0, n0, [&](int m, int n, float v) {
+        if (FULL || (m < a.M && n < a.N)) C[(int64_t)n * a.ldc + m] = v;
+    });
 }
 
 template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
@@ -300,6 +313,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
             DenseArgs<T> out = a;
             out.C = cur.C;
             const int m0 = cur.m0, n0 = cur.n0;
+            const int64_t coff = cur.coff;
             const bool store = cur.store;
             if (tnext < total) {
                 cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, tnext, tiles);
@@ -308,7 +322,10 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
                 ML::pipeline_drain();
                 ML::pipeline_fill(la, lb, cur.K, lds);
             }
-            if (store) dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
+            if (store) {
+                if (a.c_f32) store_tile_f32<ML, T, WM, WN, FULL>(acc, a, coff, m0, n0);
+                else dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
+            }
             if (tnext >= total) break;
             t = tnext;
         }
@@ -319,7 +336,8 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
             ML::run(cur.A, cur.B, cur.K, cur.m0, cur.n0, lds, acc);
             DenseArgs<T> out = a;
             out.C = cur.C;
-            dense_epilogue<ML, T, WM, WN, FULL>(acc, out, cur.m0, cur.n0);
+            if (a.c_f32) store_tile_f32<ML, T, WM, WN, FULL>(acc, a, cur.coff, cur.m0, cur.n0);
+            else dense_epilogue<ML, T, WM, WN, FULL>(acc, out, cur.m0, cur.n0);
             __syncthreads();   // every wave is done with the LDS stages before the next tile refills them
         }
     }

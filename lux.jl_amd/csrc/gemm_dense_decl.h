@@ -18,6 +18,7 @@ struct DenseArgs {
     int tiles_m, tiles_n;
     int c_vec = 0;   // C and pre allow 8-byte stores at every (m multiple of 4, n): aligned base, ldc a multiple of 4
     int tail = 0;    // this launch finishes the rows or columns of another one (profile name "...+tail")
+    int c_f32 = 0;   // batched products of bf16 operands only: C points to fp32 values (same ldc and strides, in elements)
     // batched products: the batch index runs over up to three nested dims (bdim[0] innermost); along
     // dim d the matrices of an operand lie stride[d] elements apart (0: one matrix shared by all)
     int batch = 1;

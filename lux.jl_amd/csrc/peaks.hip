@@ -76,19 +76,24 @@ __global__ __launch_bounds__(512) void peak_mfma_f32_kernel(float* out, int iter
 
 template <typename Launch>
 int time_ms(hipStream_t s, int warm, int reps, Launch&& launch, float* ms) {
-    hipEvent_t e0, e1;
-    LUX_CHECK_HIP(hipEventCreate(&e0));
-    LUX_CHECK_HIP(hipEventCreate(&e1));
-    for (int i = 0; i < warm; ++i) launch();
-    LUX_CHECK_HIP(hipEventRecord(e0, s));
-    for (int i = 0; i < reps; ++i) launch();
-    LUX_CHECK_HIP(hipEventRecord(e1, s));
-    LUX_CHECK_HIP(hipEventSynchronize(e1));
-    LUX_CHECK_HIP(hipEventElapsedTime(ms, e0, e1));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t err = hipEventCreate(&e0);
+    if (err == hipSuccess) err = hipEventCreate(&e1);
+    if (err == hipSuccess) {
+        for (int i = 0; i < warm; ++i) launch();
+        err = hipEventRecord(e0, s);
+    }
+    if (err == hipSuccess) {
+        for (int i = 0; i < reps; ++i) launch();
+        err = hipEventRecord(e1, s);
+    }
+    if (err == hipSuccess) err = hipEventSynchronize(e1);
+    if (err == hipSuccess) err = hipEventElapsedTime(ms, e0, e1);
+    if (err == hipSuccess) err = hipGetLastError();
+    if (e0) (void)hipEventDestroy(e0);       // on every path
+    if (e1) (void)hipEventDestroy(e1);
+    LUX_CHECK_HIP(err);
     *ms /= (float)reps;
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }
 
@@ -106,15 +111,16 @@ extern "C" int luxhip_measure_peaks(luxhip_stream_t stream, double* copy_GBps, d
     if (copy_GBps) {
         // 1 GiB moved per launch (512 MiB read + 512 MiB written): twice the size of the Infinity Cache
         const size_t bytes = size_t(512) << 20, n = bytes / 16;
+        // through the pooled allocator: it gives its free blocks back to the driver and retries when memory is short
         void *a = nullptr, *b = nullptr;
-        LUX_CHECK_HIP(hipMalloc(&a, bytes));
-        if (hipMalloc(&b, bytes) != hipSuccess) { (void)hipFree(a); return set_error(LUXHIP_HIP_ERROR, "measure_peaks: out of memory"); }
+        if ((rc = luxhip_malloc(&a, bytes)) != LUXHIP_OK) return rc;
+        if ((rc = luxhip_malloc(&b, bytes)) != LUXHIP_OK) { (void)luxhip_free(a); return rc; }
         (void)hipMemsetAsync(a, 0x11, bytes, s);
         rc = time_ms(s, 3, 10, [&] {
             peak_copy_kernel<<<dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s>>>((const float4*)a, (float4*)b, n);
         }, &ms);
-        (void)hipFree(a);
-        (void)hipFree(b);
+        (void)luxhip_free(a);
+        (void)luxhip_free(b);
         if (rc != LUXHIP_OK) return rc;
         *copy_GBps = 2.0 * (double)bytes / (ms * 1e-3) / 1e9;
     }

@@ -41,8 +41,11 @@ struct WsEntry {
     uint32_t* counters = nullptr;   // kWorkspaceCounters words, zero between kernels, then kWorkspaceFlags words
     uint32_t epoch = 0;
     std::vector<RetiredBlock> retired;
+    bool recorded = false;          // a graph recorded on this stream holds the address of `base`
+    std::vector<void*> pinned;      // outgrown blocks that recorded graphs still write to: kept until luxhip_shutdown
 };
 std::map<hipStream_t, WsEntry> g_ws;
+std::vector<void*> g_pinned;        // pinned blocks of destroyed streams (a graph outlives the stream it was recorded on)
 
 // One event is recorded after every profiled launch; a launch that directly follows another
 // profiled launch on the same stream takes that event as its start, so a launch costs one event
@@ -158,7 +161,9 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
     WsEntry& e = g_ws[s];
     if (!e.retired.empty()) collect_retired(e, false);
     const bool grow = e.base == nullptr || e.data_bytes < bytes;
-    if ((grow || e.counters == nullptr) && stream_capturing(s))
+    const bool capturing = stream_capturing(s);
+    if (capturing) e.recorded = true;
+    if ((grow || e.counters == nullptr) && capturing)
         return set_error(LUXHIP_INVALID,
                          "the stream is recording a graph and its workspace (%zu bytes) is smaller than the %zu bytes this call "
                          "needs: call luxhip_reserve(stream, bytes) or run the operator once eagerly before recording",
@@ -171,9 +176,22 @@ int get_workspace(hipStream_t s, size_t bytes, Workspace* out) {
             p = it->second;
             g_pool.free_blocks.erase(it);
         } else {
-            LUX_CHECK_HIP(hipMalloc(&p, want));
+            hipError_t rc = hipMalloc(&p, want);
+            if (rc != hipSuccess) {
+                // out of memory: give the pooled blocks back to the driver and try once more, as luxhip_malloc does
+                (void)hipGetLastError();
+                for (auto& kv : g_pool.free_blocks) (void)hipFree(kv.second);
+                g_pool.free_blocks.clear();
+                rc = hipMalloc(&p, want);
+            }
+            LUX_CHECK_HIP(rc);
         }
-        if (e.base != nullptr) {
+        if (e.base != nullptr && e.recorded) {
+            // a graph recorded on this stream has the old block's address in its kernels: the block is
+            // never handed out again, so a replay still writes to memory that nobody else owns
+            e.pinned.push_back(e.base);
+            e.recorded = false;
+        } else if (e.base != nullptr) {
             // the old block may still be in use by kernels queued on this stream
             hipEvent_t done;
             hipError_t rc = hipEventCreateWithFlags(&done, hipEventDisableTiming);
@@ -257,8 +275,11 @@ int luxhip_shutdown(void) {
         collect_retired(kv.second, true);       // into the pool, which is released below
         if (kv.second.base) (void)hipFree(kv.second.base);
         if (kv.second.counters) (void)hipFree(kv.second.counters);
+        for (void* p : kv.second.pinned) (void)hipFree(p);
     }
     g_ws.clear();
+    for (void* p : g_pinned) (void)hipFree(p);
+    g_pinned.clear();
     for (auto& kv : g_pool.free_blocks) (void)hipFree(kv.second);
     g_pool.free_blocks.clear();
     for (auto& kv : g_pool.live) (void)hipFree(kv.first);
@@ -331,8 +352,16 @@ int luxhip_stream_destroy(luxhip_stream_t s) {
         auto it = g_ws.find((hipStream_t)s);
         if (it != g_ws.end()) {
             collect_retired(it->second, true);  // the stream has been synchronised: into the pool
-            if (it->second.base) (void)hipFree(it->second.base);
-            if (it->second.counters) (void)hipFree(it->second.counters);
+            WsEntry& e = it->second;
+            g_pinned.insert(g_pinned.end(), e.pinned.begin(), e.pinned.end());
+            if (e.recorded) {
+                // graphs recorded on this stream can still be launched (on any stream): their scratch memory stays
+                if (e.base) g_pinned.push_back(e.base);
+                if (e.counters) g_pinned.push_back(e.counters);
+            } else {
+                if (e.base) (void)hipFree(e.base);
+                if (e.counters) (void)hipFree(e.counters);
+            }
             g_ws.erase(it);
         }
     }

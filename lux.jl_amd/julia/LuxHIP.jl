@@ -164,16 +164,43 @@ function fused_dense_device!(y::HIPArray{T,2}, pre, act, W::HIPArray{T,2}, x::HI
         max(1, stride(y, 2)), optr(pre)))
 end
 
+# Activations without a device kernel (arbitrary closures, e.g. the `x -> x^3` of LuxLib's dense tests): the
+# contraction and the bias run on the device with the identity, the closure is applied to a staged host copy.
+# Slow (two PCIe transfers) and correct; rule branch 3 of the reference (impl/dense.jl:103-112) does the same with
+# its generic broadcast.
+function host_activation!(y::HIPArray{T,N}, σ::F) where {F,T<:HIPFloat,N}
+    h = Array(y)
+    h .= σ.(h)
+    copyto!(y, HIPArray(h))
+    return y
+end
+# (σ.(z), Δ -> Δ .* σ'.(z)) through the caller's AD on host arrays
+function host_activation_rule(cfg, σ::F, z::HIPArray{T,N}) where {F,T<:HIPFloat,N}
+    yh, back = CRC.rrule_via_ad(cfg, Base.Fix1(broadcast, σ), Array(z))
+    return HIPArray(yh), Δ -> HIPArray(convert(Array{T,N}, CRC.unthunk(back(Array(CRC.unthunk(Δ)))[2])))
+end
+
 function Impl.fused_dense!(y::HIPArray{T,2}, opmode::HIPOp, act::F, W::HIPArray{T,2}, x::HIPArray{T,2},
         b::Union{Nothing,HIPArray{T,1}}) where {F,T<:HIPFloat}
-    if !fused_dense_device!(y, nothing, act, W, x, b)
-        # -1 (cublaslt.jl:359-402 warns and takes the unfused path): the product still runs on the device; an
-        # activation without a device kernel ends in HIPFallbackError inside bias_activation!
+    if act_id(act) === nothing
+        fused_dense_device!(y, nothing, identity, W, x, b) || error(last_error())
+        host_activation!(y, act)
+    elseif !fused_dense_device!(y, nothing, act, W, x, b)
+        # -1 (cublaslt.jl:359-402 warns and takes the unfused path): the product still runs on the device
         @warn "libluxhip cannot fuse this dense call; using matmul! followed by bias_activation!" maxlog = 1
         Impl.matmul!(y, opmode, W, x)
         Impl.bias_activation!(y, opmode, act, y, b)
     end
     return nothing
+end
+
+# rule branch 3 (impl/dense.jl:103-112) for closures: z = W x .+ b and its pullback on the device, σ on the host
+function CRC.rrule(cfg::CRC.RuleConfig{>:CRC.HasReverseMode}, ::typeof(Impl.fused_dense), opmode::HIPOp, act::F, W::HIPArray{T,2},
+        x::HIPArray{T,2}, b::Union{Nothing,HIPArray{T,1}}) where {F,T<:HIPFloat}
+    act_id(act) === nothing || return CRC.rrule(Impl.fused_dense, opmode, act, W, x, b)
+    z, ∇z = CRC.rrule(Impl.fused_dense, opmode, identity, W, x, b)
+    y, ∇act = host_activation_rule(cfg, act, z)
+    return y, Δ -> ∇z(∇act(Δ))
 end
 
 # rrule with the saved pre-activation for activations that need it (precedent: the cuBLASLt AUX
@@ -210,10 +237,11 @@ end
 function Impl.bias_activation!(y::HIPArray{T,N}, ::HIPOp, σ::F, x::HIPArray{T,N}, bias::Union{Nothing,HIPArray{T,1}}) where {F,T<:HIPFloat,N}
     id = act_id(σ)
     I, C, Nb = icn(x)
-    ok = id !== nothing && check(ccall((:luxhip_bias_activation_fwd, libluxhip), Cint,
+    ok = check(ccall((:luxhip_bias_activation_fwd, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Cint, Int64, Int64, Int64, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}),
-        stream(), dtype_code(T), id, I, C, Nb, optr(x), optr(bias), optr(y), C_NULL))
+        stream(), dtype_code(T), something(id, Cint(0)), I, C, Nb, optr(x), optr(bias), optr(y), C_NULL))
     ok || throw(HIPFallbackError("bias_activation! with activation $(σ)"))
+    id === nothing && host_activation!(y, σ)        # a closure: the bias on the device, σ on a staged host copy
     return nothing
 end
 Impl.activation!(y::HIPArray{T,N}, op::HIPOp, σ::F, x::HIPArray{T,N}) where {F,T<:HIPFloat,N} =
@@ -731,12 +759,17 @@ function AttnLayout(a::HIPArray, token_dim::Int)
 end
 i64x3(t) = Int64[t[1], t[2], t[3]]
 
-function bmm_strided!(C::HIPArray{T}, tA::Bool, tB::Bool, M, N, K, bdims, A::HIPArray{T}, lda, sA, B::HIPArray{T}, ldb, sB, ldc, sC,
-        structure::Integer) where {T<:HIPFloat}
+# LUXHIP_BF16_WIDE: bf16 operands with the attention logits and the cotangent of the weights in fp32
+const BF16_WIDE = Cint(2)
+wide_type(::Type{T}) where {T} = T === Core.BFloat16 ? Float32 : T
+wide_code(::Type{T}, ::Type{TW}) where {T,TW} = (T === Core.BFloat16 && TW === Float32) ? BF16_WIDE : dtype_code(T)
+
+function bmm_strided!(C::HIPArray{TC}, tA::Bool, tB::Bool, M, N, K, bdims, A::HIPArray{T}, lda, sA, B::HIPArray{T}, ldb, sB, ldc, sC,
+        structure::Integer) where {T<:HIPFloat,TC<:HIPFloat}
     check(ccall((:luxhip_batched_matmul_strided, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Cint, Cint, Int64, Int64, Int64, Ptr{Int64}, Ptr{Cvoid}, Int64, Ptr{Int64}, Ptr{Cvoid}, Int64, Ptr{Int64},
             Ptr{Cvoid}, Int64, Ptr{Int64}, Cint),
-        stream(), dtype_code(T), Cint(tA), Cint(tB), M, N, K, i64x3(bdims), optr(A), max(1, lda), i64x3(sA), optr(B), max(1, ldb),
+        stream(), wide_code(T, TC), Cint(tA), Cint(tB), M, N, K, i64x3(bdims), optr(A), max(1, lda), i64x3(sA), optr(B), max(1, ldb),
         i64x3(sB), optr(C), max(1, ldc), i64x3(sC), Cint(structure))) || throw(HIPFallbackError("batched_matmul"))
     return C
 end
@@ -773,13 +806,14 @@ function attention_device(q::HIPArray{T,N}, k::HIPArray{T,N}, v::HIPArray{T,N}, 
     sC = (S * L, S * L * r, S * L * H)
     sq = (lq.sh, lq.sh * r, lq.sb)
     tri = causal && fdrop === identity        # an arbitrary fdrop need not keep the masked weights at zero
-    logits = similar(q, T, (S, L, H, bshape...))
+    TW = wide_type(T)                         # bf16: logits in fp32 (see luxhip.h, attention)
+    logits = similar(q, TW, (S, L, H, bshape...))
     bmm_strided!(logits, true, false, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, sq, S, sC, causal ? 1 : 0)
-    softmaxed = similar(logits)
+    softmaxed = similar(q, T, (S, L, H, bshape...))
     check(ccall((:luxhip_attention_softmax_fwd, libluxhip), Cint,
         (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Int64, Ptr{Cvoid}, Cdouble, Cint, Ptr{UInt8}, Int64, Int64, Ptr{Cvoid}, Int64, Int64,
             Ptr{Cvoid}),
-        stream(), dtype_code(T), S, L, H, B, optr(logits), scale⁻¹, Cint(causal), mask === nothing ? Ptr{UInt8}(C_NULL) : Ptr{UInt8}(pointer(mask)),
+        stream(), wide_code(T, TW), S, L, H, B, optr(logits), scale⁻¹, Cint(causal), mask === nothing ? Ptr{UInt8}(C_NULL) : Ptr{UInt8}(pointer(mask)),
         mask_sh, mask_sb, optr(bias), bias_sh, bias_sb, optr(softmaxed))) || throw(HIPFallbackError("softmax of the attention logits"))
     probs, fdrop_back = fdrop === identity ? (softmaxed, nothing) : CRC.rrule_via_ad(ZygoteLikeConfig(), fdrop, softmaxed)
     out = similar(q, T, (Ev, H, L, bshape...))
@@ -831,14 +865,16 @@ function CRC.rrule(::typeof(Impl.scaled_dot_product_attention), q::HIPArray{T,N}
             Δ = CRC.unthunk(Δ′)
             Δout = CRC.unthunk(Δ[1])
             Δ[2] isa CRC.AbstractZero || throw(HIPFallbackError("a cotangent for the returned attention weights"))
-            dp = similar(probs)
+            # the cotangent of the weights in fp32 too, unless it has to pass through fdrop's pullback first
+            TD = s.fdrop_back === nothing ? wide_type(T) : T
+            dp = similar(probs, TD)
             bmm_strided!(dp, true, false, S, L, Ev, bdims, vc, lv.st, (0, lv.sh, lv.sb), Δout, Ev * H, so, S, sC, tri ? 1 : 0)
             s.fdrop_back === nothing || (dp = CRC.unthunk(s.fdrop_back(dp)[2]))
-            dlogits = s.logits                                   # no longer needed
+            dlogits = eltype(s.logits) === T ? s.logits : similar(probs)   # the logits are no longer needed
             # tri, not is_causal: with an fdrop the products below run in full and read the whole cotangent
             check(ccall((:luxhip_attention_softmax_bwd, libluxhip), Cint,
                 (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}),
-                stream(), dtype_code(T), S, L, L * H * lq.batch, Cint(tri), optr(dp), optr(s.softmaxed), s.scale⁻¹, optr(dlogits))) ||
+                stream(), wide_code(T, eltype(dp)), S, L, L * H * lq.batch, Cint(tri), optr(dp), optr(s.softmaxed), s.scale⁻¹, optr(dlogits))) ||
                 error(last_error())
             ∂q = similar(qc)
             bmm_strided!(∂q, false, false, E, L, S, bdims, kc, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, lq.st, sq, tri ? 2 : 0)

@@ -32,13 +32,40 @@ class ArgumentError(ValueError):
     """Julia's ArgumentError (api/groupnorm.jl:40-64 of the reference)."""
 
 
-def _act_id(act: str) -> int:
+def _act_id(act) -> int:
     try:
         return _lib.ACT_IDS[act]
-    except KeyError:
-        # arbitrary closures are differentiated by host-side AD in the reference
-        # (impl/dense.jl:104-112); the device backend reports "unsupported" for them.
+    except (KeyError, TypeError):
         raise _lib.Unsupported(_lib.UNSUPPORTED, f"activation {act!r} has no device kernel") from None
+
+
+# Activations without a device kernel (arbitrary closures: branch 3 of the reference's rules, impl/dense.jl:103-112,
+# impl/conv.jl:271-275, impl/bias_activation.jl:96-104; its dense tests use `x -> x^3`).  The contraction and the bias
+# run on the device with the identity; σ is applied, and differentiated, on a staged host copy: slow, correct.
+# A closure is any Python callable that maps a float64 numpy array to one of the same shape, elementwise; its derivative
+# is `act.derivative` (same calling convention) if it has one, central differences in float64 otherwise.
+def _is_closure(act) -> bool:
+    return callable(act) and not isinstance(act, str)
+
+
+def _closure_derivative(act, z: np.ndarray) -> np.ndarray:
+    d = getattr(act, "derivative", None)
+    if d is not None:
+        return np.asarray(d(z), np.float64)
+    h = 1e-6 * np.maximum(1.0, np.abs(z))
+    return (np.asarray(act(z + h), np.float64) - np.asarray(act(z - h), np.float64)) / (2.0 * h)
+
+
+def _closure_rule(act, z: DeviceArray):
+    """(σ.(z), Δ -> Δ .* σ'.(z)) through a host copy of z (what `rrule_via_ad(cfg, broadcast, σ, z)` gives the reference)."""
+    zh = z.to_numpy().astype(np.float64)
+    y = DeviceArray.from_numpy(np.asarray(act(zh), np.float64).astype(np.float32), z.dtype)
+
+    def back(delta: DeviceArray) -> DeviceArray:
+        dz = delta.to_numpy().astype(np.float64) * _closure_derivative(act, zh)
+        return DeviceArray.from_numpy(dz.astype(np.float32), z.dtype)
+
+    return y, back
 
 
 _NEEDS_PRE = {4, 5, 6, 7, 8}   # swish, gelu, softplus, logsigmoid, lisht (rrule branch 2)
@@ -120,6 +147,8 @@ def _check_bias(x: DeviceArray, bias: Optional[DeviceArray]):
 def bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray]) -> DeviceArray:
     """`bias_activation(σ, x, bias)` (api/bias_activation.jl:16-21)."""
     _check_bias(x, bias)
+    if _is_closure(act):
+        return _closure_rule(act, bias_activation("identity", x, bias))[0]
     aid = _act_id(act)
     y = DeviceArray(x.shape, _same_dtype(x, bias))
     I, Cc, N = _icn(x)
@@ -131,6 +160,10 @@ def bias_activation_inplace(act: str, x: DeviceArray, bias: Optional[DeviceArray
     """`bias_activation!!(σ, x, bias)` (api/bias_activation.jl:31-36): overwrites and returns x."""
     _check_bias(x, bias)
     _same_dtype(x, bias)
+    if _is_closure(act):
+        y = _closure_rule(act, bias_activation_inplace("identity", x, bias))[0]
+        _lib.call("luxhip_memcpy_d2d", x.ptr, y.ptr, x.nbytes, current_stream())
+        return x
     I, Cc, N = _icn(x)
     _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, _act_id(act), I, Cc, N, x.ptr, _p(bias), x.ptr, None)
     return x
@@ -139,6 +172,10 @@ def bias_activation_inplace(act: str, x: DeviceArray, bias: Optional[DeviceArray
 def rrule_bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray]):
     """CRC.rrule(bias_activation) (impl/bias_activation.jl:64-104): (y, Δ -> (∂x, ∂b))."""
     _check_bias(x, bias)
+    if _is_closure(act):
+        z, back_z = rrule_bias_activation("identity", x, bias)
+        y, back_act = _closure_rule(act, z)
+        return y, (lambda delta: back_z(back_act(delta)))
     aid = _act_id(act)
     dt = _same_dtype(x, bias)
     I, Cc, N = _icn(x)
@@ -159,6 +196,8 @@ def rrule_bias_activation(act: str, x: DeviceArray, bias: Optional[DeviceArray])
 # ------------------------------------------------------------------------------- fast_activation
 def fast_activation(act: str, x: DeviceArray) -> DeviceArray:
     """`fast_activation(σ, x)` (api/activation.jl:55-57): σ.(x) into a new array."""
+    if _is_closure(act):
+        return _closure_rule(act, x)[0]
     aid = _act_id(act)
     y = DeviceArray(x.shape, x.dtype)
     _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, aid, 1, 1, x.size, x.ptr, None, y.ptr, None)
@@ -167,6 +206,10 @@ def fast_activation(act: str, x: DeviceArray) -> DeviceArray:
 
 def fast_activation_inplace(act: str, x: DeviceArray) -> DeviceArray:
     """`fast_activation!!(σ, x)` (api/activation.jl:27-29): overwrites and returns x."""
+    if _is_closure(act):
+        y = _closure_rule(act, x)[0]
+        _lib.call("luxhip_memcpy_d2d", x.ptr, y.ptr, x.nbytes, current_stream())
+        return x
     _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, _act_id(act), 1, 1, x.size, x.ptr, None, x.ptr, None)
     return x
 
@@ -174,6 +217,9 @@ def fast_activation_inplace(act: str, x: DeviceArray) -> DeviceArray:
 def rrule_fast_activation(act: str, x: DeviceArray):
     """CRC.rrule(activation!!) (impl/activation.jl:20-49): (y, Δ -> (∂x,)); ∂x = Δ·dσ(y, x)
     (∇activation, impl/activation.jl:135-154).  x itself is the saved pre-activation."""
+    if _is_closure(act):
+        y, back_act = _closure_rule(act, x)
+        return y, (lambda delta: (back_act(delta),))
     aid = _act_id(act)
     y = DeviceArray(x.shape, x.dtype)
     _lib.call("luxhip_bias_activation_fwd", current_stream(), x.code, aid, 1, 1, x.size, x.ptr, None, y.ptr, None)
@@ -315,6 +361,8 @@ def _check_dense(weight, x, b):
 def fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b: Optional[DeviceArray]) -> DeviceArray:
     """`fused_dense_bias_activation(σ, weight, x, b)` (api/dense.jl:33-37): σ.(weight * x .+ b)."""
     _check_dense(weight, x, b)
+    if _is_closure(act):
+        return _closure_rule(act, fused_dense_bias_activation("identity", weight, x, b))[0]
     (weight, x, b), _ = _promote(weight, x, b)
     dt = _same_dtype(weight, x, b)
     M, K = weight.shape
@@ -328,6 +376,10 @@ def fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b
 def rrule_fused_dense_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b: Optional[DeviceArray]):
     """CRC.rrule(fused_dense) (impl/dense.jl:71-134): (y, Δ -> (∂W, ∂x, ∂b))."""
     _check_dense(weight, x, b)
+    if _is_closure(act):                      # impl/dense.jl:103-112: matmuladd on the device, σ and its pullback around it
+        z, back_z = rrule_fused_dense_bias_activation("identity", weight, x, b)
+        y, back_act = _closure_rule(act, z)
+        return y, (lambda delta: back_z(back_act(delta)))
     (pw, px, pb), orig = _promote(weight, x, b)
     if orig is not None:
         return _promoted_rule(lambda *a: rrule_fused_dense_bias_activation(act, *a), orig, pw, px, pb)
@@ -585,8 +637,12 @@ def _i64x3(v):
     return (C.c_int64 * 3)(*v)
 
 
+_BF16_WIDE = 2      # LUXHIP_BF16_WIDE: bf16 storage with the logits / their cotangent in fp32
+
+
 def _bmm_strided(tA, tB, M, N, K, bdims, A, lda, sA, B, ldb, sB, Cm, ldc, sC, structure=0):
-    _lib.call("luxhip_batched_matmul_strided", current_stream(), Cm.code, int(tA), int(tB), M, N, K, _i64x3(bdims),
+    code = _BF16_WIDE if (A.dtype == "bf16" and Cm.dtype == "f32") else Cm.code
+    _lib.call("luxhip_batched_matmul_strided", current_stream(), code, int(tA), int(tB), M, N, K, _i64x3(bdims),
               A.ptr, max(lda, 1), _i64x3(sA), B.ptr, max(ldb, 1), _i64x3(sB), Cm.ptr, max(ldc, 1), _i64x3(sC), int(structure))
 
 
@@ -677,7 +733,11 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
 
     mask_a, mask_sh, mask_sb = side(mask, "mask", "mask")
     bias_a, bias_sh, bias_sb = side(bias, "bias", "bias")
-    logits = DeviceArray((S, L, H) + bshape, dt)
+    # bf16: the logits and the cotangent of the weights stay in fp32 between the products and the softmax passes
+    # (a logit rounded to bf16 is off by 2^-9 |logit|, the weight then by that relative amount)
+    wide = "f32" if dt == "bf16" else dt
+    sm_code = _BF16_WIDE if dt == "bf16" else None
+    logits = DeviceArray((S, L, H) + bshape, wide)
     sC = (S * L, S * L * r, S * L * H)
     # a causal mask (keep s <= l) leaves whole tiles of the logits unused and makes the weights and every
     # cotangent of the same shape triangular: the products skip what is known to be zero or unused
@@ -686,7 +746,7 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
     _bmm_strided(True, False, S, L, E, bdims, k, lk.st, (0, lk.sh, lk.sb), q, lq.st, (lq.sh, lq.sh * r, lq.sb), logits, S, sC,
                  1 if causal else 0)
     probs = DeviceArray((S, L, H) + bshape, dt)
-    _lib.call("luxhip_attention_softmax_fwd", current_stream(), probs.code, S, L, H, B, logits.ptr, scale_inv,
+    _lib.call("luxhip_attention_softmax_fwd", current_stream(), probs.code if sm_code is None else sm_code, S, L, H, B, logits.ptr, scale_inv,
               int(causal), _p(mask_a), mask_sh, mask_sb, _p(bias_a), bias_sh, bias_sb, probs.ptr)
     softmax_out, fdrop_back = probs, None
     if fdrop is not None:
@@ -696,18 +756,21 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
     _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so, 2 if tri else 0)
 
     def back(d_out: DeviceArray, d_probs: Optional[DeviceArray] = None):
-        dp = DeviceArray(probs.shape, dt)
+        # with an fdrop the cotangent passes through its pullback in the storage type first
+        dp_wide = wide if fdrop_back is None else dt
+        dp = DeviceArray(probs.shape, dp_wide)
         _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC, 1 if tri else 0)
         if d_probs is not None:
             raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: a cotangent for the returned weights")
         if fdrop_back is not None:
             dp = fdrop_back(dp)
-        dlogits = logits                                              # the logits are no longer needed
+        dlogits = logits if logits.dtype == dt else DeviceArray(logits.shape, dt)   # the logits are no longer needed
         # the causal shortcut of the softmax pullback leaves dlogits beyond the diagonal block untouched, which
         # only the triangular products that follow tolerate: with an fdrop those run in full, so the whole
         # column is computed (masked weights are zero, hence so is their dlogits)
-        _lib.call("luxhip_attention_softmax_bwd", current_stream(), dp.code, S, L, L * H * B, int(tri), dp.ptr, softmax_out.ptr,
-                  scale_inv, dlogits.ptr)
+        _lib.call("luxhip_attention_softmax_bwd", current_stream(),
+                  _BF16_WIDE if (dt == "bf16" and dp.dtype == "f32") else softmax_out.code, S, L, L * H * B, int(tri), dp.ptr,
+                  softmax_out.ptr, scale_inv, dlogits.ptr)
         dq = DeviceArray(q.shape, dt)
         _bmm_strided(False, False, E, L, S, bdims, k, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, dq, lq.st,
                      (lq.sh, lq.sh * r, lq.sb), 2 if tri else 0)
@@ -1120,6 +1183,8 @@ def _check_conv(weight, x, b, cdims):
 def fused_conv_bias_activation(act: str, weight: DeviceArray, x: DeviceArray, b, cdims: DenseConvDims) -> DeviceArray:
     """`fused_conv_bias_activation(σ, weight, x, b, cdims)` (api/conv.jl:30-38)."""
     _check_conv(weight, x, b, cdims)
+    if _is_closure(act):
+        return _closure_rule(act, fused_conv_bias_activation("identity", weight, x, b, cdims))[0]
     (weight, x, b), _ = _promote(weight, x, b)
     dt = _same_dtype(weight, x, b)
     if cdims.inner is not None:
@@ -1175,6 +1240,10 @@ def _to_inner_output(cdims, dy):
 def rrule_fused_conv_bias_activation(act: str, weight, x, b, cdims: DenseConvDims):
     """CRC.rrule(fused_conv) + ∇fused_conv (impl/conv.jl:204-275): (y, Δ -> (∂w, ∂x, ∂b))."""
     _check_conv(weight, x, b, cdims)
+    if _is_closure(act):                      # impl/conv.jl:271-275
+        z, back_z = rrule_fused_conv_bias_activation("identity", weight, x, b, cdims)
+        y, back_act = _closure_rule(act, z)
+        return y, (lambda delta: back_z(back_act(delta)))
     (pw, px, pb), orig = _promote(weight, x, b)
     if orig is not None:
         return _promoted_rule(lambda *a: rrule_fused_conv_bias_activation(act, *a, cdims), orig, pw, px, pb)

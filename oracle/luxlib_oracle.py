@@ -611,8 +611,11 @@ def _attn_canonical(a, token_dim):
     return a4 if token_dim == 3 else np.swapaxes(a4, 1, 2)
 
 
-def scaled_dot_product_attention(q, k, v, token_dim=3, scale=None, mask=None, is_causal=None, bias=None):
+def scaled_dot_product_attention(q, k, v, token_dim=3, scale=None, mask=None, is_causal=None, bias=None, weights=None):
     """Returns (output [Ev, H, L, B...], weights [S, L, H, B...]).
+    `weights` (optional): the weights as an earlier call stored them (bf16 storage: rounded); the output is then
+    the product of v with these, which is what the reference's second batched product computes from its stored
+    softmax result (impl/attention.jl:107-117).
     logits[s,l,h,b] = (1/scale) Σ_d k[d,h,s,b] q[d,h,l,b] (+ bias), -inf where the mask is false
     (impl/attention.jl:90-104, 119-128); weights = softmax over s; output[e,h,l,b] =
     Σ_s v[e,h,s,b] weights[s,l,h,b] (:107-117).  Fewer key/value heads than query heads: each is
@@ -639,14 +642,23 @@ def scaled_dot_product_attention(q, k, v, token_dim=3, scale=None, mask=None, is
     z = logits - logits.max(axis=0, keepdims=True)
     w = np.exp(z)
     w = w / w.sum(axis=0, keepdims=True)
+    if weights is not None:
+        w = np.asarray(weights, dtype=q4.dtype).reshape(w.shape)
     out = np.einsum("ehsb,slhb->ehlb", v4, w)
     return out.reshape(out.shape[:3] + tail), w.reshape(w.shape[:3] + tail)
 
 
-def scaled_dot_product_attention_pullback(q, k, v, d_out, token_dim=3, scale=None, mask=None, is_causal=None, bias=None):
+def scaled_dot_product_attention_pullback(q, k, v, d_out, token_dim=3, scale=None, mask=None, is_causal=None, bias=None,
+                                          weights=None, stored=None):
     """(∂q, ∂k, ∂v) for a cotangent of the output only: the chain of the batched_matmul rrules
     (impl/batched_mul.jl:320-334), the softmax rule dS = W ∘ (dW - Σ_s dW ∘ W), the scale, and the
-    sum over the query heads that share a key/value head."""
+    sum over the query heads that share a key/value head.
+    The reference's pullbacks work on the arrays that the forward pass stored: `weights` (optional)
+    are the attention weights as the forward pass returned them (in bf16 storage: rounded), used in
+    place of the exact ones; `stored` (optional) is applied to the arrays of the storage type that the
+    pullback itself passes from one rule to the next: the cotangent of the logits (softmax rule ->
+    the two products) and the per-query-head gradients of k and v (products -> the sum over the heads
+    of a key/value group, the pullback of repeat_inner_gqa), e.g. `round_to_bf16`."""
     q0, k0, v0 = np.asarray(q), np.asarray(k), np.asarray(v)
     q4, k4, v4 = (_attn_canonical(a, token_dim) for a in (q0, k0, v0))
     E, H, L, B = q4.shape
@@ -655,14 +667,21 @@ def scaled_dot_product_attention_pullback(q, k, v, d_out, token_dim=3, scale=Non
     kr, vr = np.repeat(k4, r, axis=1), np.repeat(v4, r, axis=1)
     T = q4.dtype.type
     inv = T(1) / (np.sqrt(T(E)) if scale is None else T(scale))
-    _, w = scaled_dot_product_attention(q, k, v, token_dim, scale, mask, is_causal, bias)
+    if weights is None:
+        _, w = scaled_dot_product_attention(q, k, v, token_dim, scale, mask, is_causal, bias)
+    else:
+        w = np.asarray(weights, dtype=q4.dtype)
     w = w.reshape(w.shape[:3] + (-1,))
     do = np.asarray(d_out).reshape(np.asarray(d_out).shape[:3] + (-1,))       # [Ev, H, L, B]
     dw = np.einsum("ehsb,ehlb->slhb", vr, do)
     dvr = np.einsum("ehlb,slhb->ehsb", do, w)
     ds = w * (dw - (dw * w).sum(axis=0, keepdims=True)) * inv
+    if stored is not None:
+        ds = np.asarray(stored(ds), dtype=q4.dtype)
     dq4 = np.einsum("dhsb,slhb->dhlb", kr, ds)
     dkr = np.einsum("dhlb,slhb->dhsb", q4, ds)
+    if stored is not None:
+        dkr, dvr = np.asarray(stored(dkr), dtype=q4.dtype), np.asarray(stored(dvr), dtype=q4.dtype)
     dk4 = dkr.reshape(E, G, r, S, B).sum(axis=2)
     dv4 = dvr.reshape(v4.shape[0], G, r, S, B).sum(axis=2)
     back = (lambda a, like: (a if token_dim == 3 else np.swapaxes(a, 1, 2)).reshape(like.shape))

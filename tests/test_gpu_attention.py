@@ -9,6 +9,14 @@ from tests.util import stable_seed, assert_close, dev, f64, host_inputs
 
 pytestmark = pytest.mark.gpu
 
+
+def stored_as(dtype):
+    """What storing an array of the pullback does to its values: the reference's rules pass arrays of the storage
+    type from one rule to the next (bf16: rounded), and they read the forward pass's stored weights."""
+    if dtype == "bf16":
+        return lambda a: f64(O.round_to_bf16(np.asarray(a, np.float32)))
+    return lambda a: a
+
 CASES = [
     # E, Ev, H, G, L, S, batch dims, token_dim, kind
     (8, 8, 4, 4, 5, 5, (2,), 3, "plain"), (8, 6, 4, 2, 5, 7, (2,), 3, "plain"), (4, 4, 2, 2, 6, 6, (3,), 3, "causal"),
@@ -42,14 +50,18 @@ def test_forward_and_pullback(gpu, dtype, case):
     assert out.shape == wout.shape and w.shape == ww.shape
     # bf16: logits and weights are stored (rounded to 8 bits) between the three passes, as they are in the
     # reference's chain of array operations; sums of a few hundred such terms stray up to ~5 sigma somewhere
-    rel = None if dtype == "f32" else 4e-2
+    rel = None
     assert_close(w.to_numpy(), ww, dtype, tag + " weights", rel=rel)
+    if dtype == "bf16":     # the output is the product of v with the weights as stored (rounded to bf16), as in the reference
+        wout, _ = O.scaled_dot_product_attention(f64(q), f64(k), f64(v), token_dim, None, mask, causal, f64(bias), weights=f64(w.to_numpy()))
     assert_close(out.to_numpy(), wout, dtype, tag + " out", rel=rel)
     (d_out,) = host_inputs(dtype, rng.normal(size=wout.shape))
     dq, dk, dv = back(dev(gpu, d_out, dtype))
+    # the pullback starts from the weights as the forward pass stored them (checked above) and stores the logits' cotangent
     wdq, wdk, wdv = O.scaled_dot_product_attention_pullback(f64(q), f64(k), f64(v), f64(d_out), token_dim, None, mask, causal,
-                                                            f64(bias))
-    rel = None if dtype == "f32" else 6e-2
+                                                            f64(bias), weights=f64(w.to_numpy()) if dtype == "bf16" else None,
+                                                            stored=stored_as(dtype))
+    rel = None
     assert_close(dq.to_numpy(), wdq, dtype, tag + " dq", rel=rel)
     assert_close(dk.to_numpy(), wdk, dtype, tag + " dk", rel=rel)
     assert_close(dv.to_numpy(), wdv, dtype, tag + " dv", rel=rel)
@@ -98,11 +110,10 @@ def test_reference_batch_sizes_and_token_first_layout(gpu, dtype, bdims, nheads)
     q, k, v, dout = host_inputs(dtype, rng.normal(size=(e, nheads, lenq) + bdims), rng.normal(size=(e, nheads, lenkv) + bdims),
                                 rng.normal(size=(e, nheads, lenkv) + bdims), rng.normal(size=(e, nheads, lenq) + bdims))
     wy, ww = O.scaled_dot_product_attention(f64(q), f64(k), f64(v))
-    wdq, wdk, wdv = O.scaled_dot_product_attention_pullback(f64(q), f64(k), f64(v), f64(dout))
-    rel = None if dtype == "f32" else 4e-2
+    rel = None
     (y1, w1), back1 = gpu.pullback(gpu.scaled_dot_product_attention, dev(gpu, q, dtype), dev(gpu, k, dtype), dev(gpu, v, dtype))
     assert y1.shape == (e, nheads, lenq) + bdims and w1.shape == (lenkv, lenq, nheads) + bdims
-    np.testing.assert_allclose(w1.to_numpy().sum(axis=0), 1.0, rtol=2e-2 if dtype == "bf16" else 1e-5)
+    np.testing.assert_allclose(w1.to_numpy().sum(axis=0), 1.0, rtol=1e-2 if dtype == "bf16" else 1e-5)
     assert_close(y1.to_numpy(), wy, dtype, "y", rel=rel)
     perm = (2, 1, 0) + tuple(range(3, 3 + len(bdims)))
     q2, k2, v2 = (np.ascontiguousarray(np.transpose(a, perm)) for a in (q, k, v))
@@ -112,11 +123,14 @@ def test_reference_batch_sizes_and_token_first_layout(gpu, dtype, bdims, nheads)
     np.testing.assert_array_equal(y2.to_numpy(), y1.to_numpy())        # the same kernels on the same canonical operands
     np.testing.assert_array_equal(w2.to_numpy(), w1.to_numpy())
     assert_close(w2.to_numpy(), ww, dtype, "weights", rel=rel)
+    wdq, wdk, wdv = O.scaled_dot_product_attention_pullback(f64(q), f64(k), f64(v), f64(dout),
+                                                            weights=f64(w1.to_numpy()) if dtype == "bf16" else None,
+                                                            stored=stored_as(dtype))
     g1 = back1(dev(gpu, dout, dtype))
     g2 = back2(dev(gpu, dout, dtype))
     for got1, got2, want, like, name in zip(g1, g2, (wdq, wdk, wdv), (q, k, v), "qkv"):
         assert got1.shape == like.shape and got2.shape == np.transpose(like, perm).shape
-        assert_close(got1.to_numpy(), want, dtype, "d" + name, rel=None if dtype == "f32" else 6e-2)
+        assert_close(got1.to_numpy(), want, dtype, "d" + name, rel=None)
         np.testing.assert_array_equal(got2.to_numpy(), np.transpose(got1.to_numpy(), perm))
 
 
@@ -158,18 +172,19 @@ def test_dropout_of_the_attention_weights(gpu, dtype):
     noise = O.rand_uniform(wp.size, 77, 0, bf16=(dtype == "bf16")).reshape(wp.shape, order="F")
     keep = noise > 0.5
     assert_close(wn, np.where(keep, 2.0 * wp, 0.0), dtype, "dropped weights")
-    assert_close(y.to_numpy(), np.einsum("ehsb,slhb->ehlb", f64(q), wn), dtype, "output", rel=None if dtype == "f32" else 4e-2)
+    assert_close(y.to_numpy(), np.einsum("ehsb,slhb->ehlb", f64(q), wn), dtype, "output", rel=None)
     # pullback against the oracle's chain with the mask applied to the weights' cotangent
     (dout,) = host_inputs(dtype, rng.normal(size=q.shape))
     dq, dk, dv = back(dev(gpu, dout, dtype))
     qf, do = f64(q), f64(dout)
     inv = 1.0 / np.sqrt(5.0)
-    dw = np.einsum("ehsb,ehlb->slhb", qf, do) * np.where(keep, 2.0, 0.0)
-    ds = wp * (dw - (dw * wp).sum(axis=0, keepdims=True)) * inv
+    st = stored_as(dtype)
+    dw = st(st(np.einsum("ehsb,ehlb->slhb", qf, do)) * np.where(keep, 2.0, 0.0))     # product, then fdrop's pullback: two stored arrays
+    ds = st(wp * (dw - (dw * wp).sum(axis=0, keepdims=True)) * inv)
     want_dq = np.einsum("dhsb,slhb->dhlb", qf, ds)
     want_dk = np.einsum("dhlb,slhb->dhsb", qf, ds)
     want_dv = np.einsum("ehlb,slhb->ehsb", do, wn)
-    rel = None if dtype == "f32" else 6e-2
+    rel = None
     assert_close(dq.to_numpy(), want_dq, dtype, "dq", rel=rel, scale=0.05)
     assert_close(dk.to_numpy(), want_dk, dtype, "dk", rel=rel, scale=0.05)
     assert_close(dv.to_numpy(), want_dv, dtype, "dv", rel=rel)
@@ -193,15 +208,21 @@ def test_causal_mask_with_dropout_of_the_weights(gpu, dtype):
     dq, dk, dv = back(dev(gpu, dout, dtype))
     _, wp = O.scaled_dot_product_attention(f64(q), f64(k), f64(v), 3, None, None, True, None)
     noise = O.rand_uniform(wp.size, 5, 0, bf16=(dtype == "bf16")).reshape(wp.shape, order="F")
-    keep = np.where(noise > np.float32(p), 1.0 / (1.0 - p), 0.0)      # p = 0.25 is exact in both storage types
+    # p = 0.25 is exact in both storage types; the mask holds 1 / (1 - p) in the storage type (bf16: 1.3359375)
+    keep = np.where(noise > np.float32(p), float(stored_as(dtype)(np.array(1.0 / (1.0 - p)))), 0.0)
     wd = wp * keep
-    rel = None if dtype == "f32" else 4e-2
+    rel = None
     assert_close(w.to_numpy(), wd, dtype, "dropped causal weights", rel=rel)
+    if dtype == "bf16":                                   # the products read the weights as the forward pass stored them
+        wd = f64(w.to_numpy())
     assert_close(y.to_numpy(), np.einsum("ehsb,slhb->ehlb", f64(v), wd), dtype, "output", rel=rel)
     do, inv = f64(dout), 1.0 / np.sqrt(float(E))
-    dw = np.einsum("ehsb,ehlb->slhb", f64(v), do) * keep
-    ds = wp * (dw - (dw * wp).sum(axis=0, keepdims=True)) * inv
-    rel = None if dtype == "f32" else 6e-2
+    st = stored_as(dtype)
+    if dtype == "bf16":                                   # the pullback reads the softmax result as stored
+        wp = st(wp)
+    dw = st(st(np.einsum("ehsb,ehlb->slhb", f64(v), do)) * keep)
+    ds = st(wp * (dw - (dw * wp).sum(axis=0, keepdims=True)) * inv)
+    rel = None
     for got, want, name in ((dq, np.einsum("dhsb,slhb->dhlb", f64(k), ds), "dq"), (dk, np.einsum("dhlb,slhb->dhsb", f64(q), ds), "dk"),
                             (dv, np.einsum("ehlb,slhb->ehsb", do, wd), "dv")):
         g = got.to_numpy()

@@ -42,7 +42,7 @@ def test_forward_and_pullback(gpu, dtype, case):
     shared_x = int(np.prod(xs[2:])) == 1 and batch > 1
     shared_y = int(np.prod(ys[2:])) == 1 and batch > 1
     # a shared operand's gradient is a sum of per-product results that are stored (bf16: rounded) first
-    rel = None if dtype == "f32" else 2e-2
+    rel = None
     assert_close(dx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=np.sqrt(wz.shape[1] * (batch if shared_x else 1)))
     assert_close(dy.to_numpy(), wdy, dtype, tag + " dy", rel=rel, scale=np.sqrt(wz.shape[0] * (batch if shared_y else 1)))
 
@@ -103,7 +103,7 @@ def test_general_batching_dims(gpu, dtype, case):
     dx, dy = back(dev(gpu, delta, dtype))
     wdx, wdy = O.batched_matmul_general_pullback(f64(x), f64(y), f64(delta), cx, cy, bx, by)
     assert dx.shape == tuple(xs) and dy.shape == tuple(ys)
-    rel = None if dtype == "f32" else 3e-2
+    rel = None
     assert_close(dx.to_numpy(), wdx, dtype, f"case {case} dx", rel=rel)
     assert_close(dy.to_numpy(), wdy, dtype, f"case {case} dy", rel=rel)
 

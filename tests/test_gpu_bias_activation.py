@@ -37,7 +37,7 @@ def test_forward_and_pullback(gpu, act, dtype):
         # the bias gradient is a long sum of rounded terms in bf16 storage: compare at the
         # same relative bar against the magnitude of the summed terms
         assert_close(gb.to_numpy(), wdb, dtype, f"{act} {shape} db",
-                     rel=None if dtype == "f32" else 2e-2)
+                     rel=None)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])

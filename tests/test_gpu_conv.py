@@ -104,7 +104,7 @@ def test_fused_conv_pullback(gpu, dtype, act):
             assert_close(gw.to_numpy(), wdw, dtype, tag + " dw", scale=np.sqrt(np.prod(od.y_shape()) / ws[3]) * dzr * rms(x) * 0.5)
             assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", scale=np.sqrt(ws[0] * ws[1] * ws[3] / groups) * dzr * rms(w) * 0.5)
             if with_bias:
-                assert_close(gb.to_numpy(), wdb, dtype, tag + " db", rel=None if dtype == "f32" else 2e-2)
+                assert_close(gb.to_numpy(), wdb, dtype, tag + " db", rel=None)
             else:
                 assert gb is None
 
@@ -134,7 +134,7 @@ def test_one_spatial_dim(gpu, dtype, xs, ws, stride, pad, dil, groups, flip):
     assert gw.shape == tuple(ws) and gx.shape == tuple(xs)
     assert_close(gw.to_numpy(), wdw.reshape(ws), dtype, "1-d dw", scale=np.sqrt(np.prod(gd.y_shape) / ws[2]) * rms(delta) * rms(x) * 0.5)
     assert_close(gx.to_numpy(), wdx.reshape(xs), dtype, "1-d dx", scale=np.sqrt(ws[0] * ws[2] / groups) * rms(delta) * rms(w) * 0.5)
-    assert_close(gb.to_numpy(), wdb, dtype, "1-d db", rel=None if dtype == "f32" else 2e-2)
+    assert_close(gb.to_numpy(), wdb, dtype, "1-d db", rel=None)
     with pytest.raises(gpu.Unsupported):
         gpu.DenseConvDims((4, 4, 4, 4, 2, 1), (2, 2, 2, 2, 2, 3))       # four spatial dims
 
@@ -180,7 +180,7 @@ def test_config5_full_size(gpu, dtype):
     cwp = gpu.conv(dx_, dev(gpu, wp, dtype), gd).to_numpy().astype(np.float64)
     lhs = float((gw.to_numpy().astype(np.float64) * f64(wp)).sum())
     rhs = float((dz * cwp).sum())
-    assert abs(lhs - rhs) <= (2e-4 if dtype == "f32" else 2e-2) * max(abs(rhs), np.sqrt(dz.size)), (lhs, rhs)
+    assert abs(lhs - rhs) <= (2e-4 if dtype == "f32" else 1e-2) * max(abs(rhs), np.sqrt(dz.size)), (lhs, rhs)
     # and an oracle check of the same kernel on a two-image batch
     gd2 = gpu.DenseConvDims(xs[:3] + (2,), ws, padding=1)
     dzq = dz[..., sub].astype(np.float32)

@@ -86,7 +86,7 @@ def test_fused_conv_pullback(gpu, dtype, act):
             assert_close(gw.to_numpy(), wdw, dtype, tag + " dw", scale=np.sqrt(np.prod(gd.y_shape) / ws[4]) * dzr * rms(x) * 0.5)
             assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", scale=np.sqrt(ws[0] * ws[1] * ws[2] * ws[4] / groups) * dzr * rms(w) * 0.5)
             if with_bias:
-                assert_close(gb.to_numpy(), wdb, dtype, tag + " db", rel=None if dtype == "f32" else 2e-2)
+                assert_close(gb.to_numpy(), wdb, dtype, tag + " db", rel=None)
             else:
                 assert gb is None
 

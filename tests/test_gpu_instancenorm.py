@@ -58,7 +58,7 @@ def test_forward_and_pullback(gpu, dtype, act, affine, mode):
         wdx, wdg, wdb = O.instancenorm_pullback(f64(x), f64(g), f64(b), act, eps, f64(delta), **kw)
         w32 = O.instancenorm_pullback(x, g, b, act, np.float32(eps), delta, training=training, rmean=rm, rvar=rv)
         var = f64(rv) if (running and not training) else f64(x).var(axis=tuple(range(len(shape) - 2)))
-        rel = None if dtype == "f32" else 3e-2
+        rel = None
         assert_close(gx.to_numpy(), wdx, dtype, tag + " dx", rel=rel, scale=dx_scale(x, g, eps, delta, var), want32=w32[0])
         if affine:
             sc = rms(delta) * max(1.0, float(np.abs(pre).max()))
@@ -98,7 +98,7 @@ def test_fast_activation(gpu, dtype, act):
         (dx,) = back(dev(gpu, delta, dtype))
         yq = f64(O.round_to_bf16(want.astype(np.float32))) if dtype == "bf16" else want
         assert_close(dx.to_numpy(), O.grad_activation(f64(delta), yq, act, f64(x)), dtype, f"{act} {shape} dx",
-                     rel=None if dtype == "f32" else 2e-2)
+                     rel=None)
 
 
 def test_separate_running_statistics_call_matches_the_fused_forward(gpu):

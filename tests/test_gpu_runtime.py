@@ -186,10 +186,12 @@ def test_plain_c_client_of_the_abi(gpu):
 
 def test_workspace_growth_does_not_wait_for_the_stream(gpu):
     """The stream's scratch memory grows while earlier work is still queued: the call that grows it
-    returns long before that work is done (the outgrown block is retired behind an event, nothing
+    returns while that work is still pending (the outgrown block is retired behind an event, nothing
     synchronises), and the operators before and after the growth give the right results."""
-    import time
     rng = np.random.default_rng(11)
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipEventQuery.argtypes = [C.c_void_p]
+    HIP_ERROR_NOT_READY = 600
     stream = _new_stream(gpu)
     main = gpu.current_stream()
     gpu.set_stream(stream)
@@ -207,17 +209,20 @@ def test_workspace_growth_does_not_wait_for_the_stream(gpu):
         call()
         gpu._lib.call("luxhip_stream_synchronize", stream)
         want_gb = gb.to_numpy().copy()
-        # about 80 ms of fp32 products (137 GFLOP each) queued on the stream
+        queued = C.c_void_p()
+        gpu._lib.call("luxhip_event_create", C.byref(queued))
+        # about 80 ms of fp32 products (137 GFLOP each) queued on the stream, an event behind them
         for _ in range(60):
             gpu._lib.call("luxhip_matmul", stream, 0, 0, 0, n, n, n, a.ptr, n, b.ptr, n, None, c.ptr, n)
+        gpu._lib.call("luxhip_event_record", queued, stream)
         call()                                                 # uses the small block, queued behind the products
-        t0 = time.perf_counter()
         gpu._lib.call("luxhip_reserve", stream, 96 << 20)     # outgrows it while that work is pending
         call()                                                 # runs out of the new block
-        t_calls = time.perf_counter() - t0
+        # the products queued before the growth have not finished: nothing above waited for the stream
+        assert hip.hipEventQuery(queued) == HIP_ERROR_NOT_READY
         gpu._lib.call("luxhip_stream_synchronize", stream)
-        t_drain = time.perf_counter() - t0 - t_calls
-        assert t_calls < 0.04 and t_drain > t_calls, (t_calls, t_drain)
+        assert hip.hipEventQuery(queued) == 0
+        gpu._lib.call("luxhip_event_destroy", queued)
         np.testing.assert_array_equal(gb.to_numpy(), want_gb)
         # a third growth after everything has finished recycles the retired blocks through the pool
         gpu._lib.call("luxhip_reserve", stream, 200 << 20)
@@ -225,5 +230,61 @@ def test_workspace_growth_does_not_wait_for_the_stream(gpu):
         gpu._lib.call("luxhip_stream_synchronize", stream)
         np.testing.assert_array_equal(gb.to_numpy(), want_gb)
     finally:
+        gpu.set_stream(main)
+        gpu._lib.call("luxhip_stream_destroy", stream)
+
+
+def test_a_recorded_graph_keeps_its_workspace_block_after_growth(gpu):
+    """A graph recorded on a stream has the address of that stream's scratch block in its kernels.  When a
+    later eager call outgrows the block, the block must not go back to the allocator: a replay would write
+    partial sums into whatever tensor received it."""
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    rng = np.random.default_rng(12)
+    stream = _new_stream(gpu)
+    main = gpu.current_stream()
+    gpu.set_stream(stream)
+    graph, graph_exec = C.c_void_p(), C.c_void_p()
+    try:
+        shape = (1, 96, 4000)                      # dense layout: partial sums in the workspace
+        x = rng.normal(size=shape).astype(np.float32)
+        dd, dy = dev(gpu, x, "f32"), dev(gpu, np.maximum(x, 0), "f32")
+        gx, gb = gpu.DeviceArray(shape, "f32"), gpu.DeviceArray((96,), "f32")
+        call = lambda: gpu._lib.call("luxhip_bias_activation_bwd", stream, 0, 1, 1, 96, 4000, dd.ptr, dy.ptr, None, gx.ptr, gb.ptr)
+        first = 8 << 20                            # the smallest block the workspace takes
+        gpu._lib.call("luxhip_reserve", stream, first)
+        call()
+        gpu._lib.call("luxhip_stream_synchronize", stream)
+        want_gb = gb.to_numpy().copy()
+        assert hip.hipStreamBeginCapture(stream, 1) == 0
+        try:
+            call()
+        finally:
+            rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0 and graph.value
+        assert hip.hipGraphInstantiate(C.byref(graph_exec), graph, None, None, 0) == 0
+        gpu._lib.call("luxhip_reserve", stream, 64 << 20)     # eager growth after the recording
+        call()
+        gpu._lib.call("luxhip_stream_synchronize", stream)
+        # tensors of the outgrown block's size: had the block been pooled, one of them would be it
+        sentinels = [gpu.DeviceArray.from_numpy(np.full(first // 4, 7.0, np.float32)) for _ in range(4)]
+        gb2 = gpu.DeviceArray.from_numpy(np.zeros(96, np.float32))
+        gpu._lib.call("luxhip_memcpy_d2d", gb.ptr, gb2.ptr, 96 * 4, stream)       # clear the result
+        for _ in range(2):
+            assert hip.hipGraphLaunch(graph_exec, stream) == 0
+            gpu._lib.call("luxhip_stream_synchronize", stream)
+            np.testing.assert_array_equal(gb.to_numpy(), want_gb)
+            for t in sentinels:
+                assert (t.to_numpy() == 7.0).all()
+    finally:
+        if graph_exec.value:
+            hip.hipGraphExecDestroy(graph_exec)
+        if graph.value:
+            hip.hipGraphDestroy(graph)
         gpu.set_stream(main)
         gpu._lib.call("luxhip_stream_destroy", stream)

@@ -48,7 +48,7 @@ def run_both(gpu, dtype, fn, arrays, delta_shape_of=None, rel=None):
 def test_bias_activation_and_norms(gpu, dtype):
     rng = np.random.default_rng(1)
     x, g, b = host_inputs(dtype, rng.normal(size=(16, 8, 16, 4)), rng.uniform(0.5, 1.5, 16), rng.normal(size=16))
-    rel = None if dtype == "f32" else 3e-2
+    rel = None
     run_both(gpu, dtype, lambda x_, b_: gpu.pullback(gpu.bias_activation, "gelu", x_, b_), [x, b], rel=rel)
     run_both(gpu, dtype, lambda x_, g_, b_: (lambda r: (r[0][0], r[1]))(
         gpu.pullback(gpu.batchnorm, x_, g_, b_, None, None, True, "relu", 0.1, 1e-3)), [x, g, b], rel=rel)
@@ -64,7 +64,7 @@ def test_bias_activation_and_norms(gpu, dtype):
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_dense_conv_and_products(gpu, dtype):
     rng = np.random.default_rng(2)
-    rel = None if dtype == "f32" else 3e-2
+    rel = None
     w, x, b = host_inputs(dtype, rng.normal(size=(128, 64)) / 8, rng.normal(size=(64, 96)), rng.normal(size=128))
     run_both(gpu, dtype, lambda w_, x_, b_: gpu.pullback(gpu.fused_dense_bias_activation, "gelu", w_, x_, b_), [w, x, b], rel=rel)
     w, x, b = host_inputs(dtype, rng.normal(size=(256, 256)) / 16, rng.normal(size=(256, 256)), rng.normal(size=256))
@@ -75,7 +75,7 @@ def test_dense_conv_and_products(gpu, dtype):
     a, bm = host_inputs(dtype, rng.normal(size=(64, 32, 6)), rng.normal(size=(32, 48, 6)))
     run_both(gpu, dtype, lambda a_, b_: gpu.pullback(gpu.batched_matmul, a_, b_), [a, bm], rel=rel)
     q, k, v = host_inputs(dtype, rng.normal(size=(32, 4, 64, 2)), rng.normal(size=(32, 2, 128, 2)), rng.normal(size=(32, 2, 128, 2)))
-    rel_a = None if dtype == "f32" else 6e-2
+    rel_a = None
     run_both(gpu, dtype, lambda q_, k_, v_: (lambda r: (r[0][0], r[1]))(
         gpu.pullback(gpu.scaled_dot_product_attention, q_, k_, v_, 1, 3, None, None, True)), [q, k, v], rel=rel_a)
 
