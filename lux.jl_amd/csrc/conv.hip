@@ -369,7 +369,8 @@ static size_t wgrad_partial_bytes(const ConvGeom& g) {
     int slices = 1, kslice = 0;
     bool small = false;
     if (wgrad_plan<T>(g, &slices, &kslice, &small) != LUXHIP_OK) return 0;
-    if (wgrad_window_shape<T>(g)) slices = std::max(slices, g.N);
+    if (wgrad_window_shape<T>(g))
+        slices = std::max(slices, wpatch::image_lanes(g.N, (g.Cin_g / 64) * ((g.Cout_g + 63) / 64), num_cus() > 0 ? num_cus() : 256));
     return align256((size_t)slices * g.kW * g.kH * g.Cin_g * g.Cout_g * sizeof(float));
 }
 
@@ -405,7 +406,7 @@ static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy,
                 p.Ctot = g.Cin; p.Cg = g.Cin_g; p.Cout = g.Cout; p.Ncols = g.Cout_g;
                 p.P = g.W; p.Q = g.H; p.N = g.N; p.pad_w = g.pw; p.pad_h = g.ph;
                 rc = wpatch::launch(s, p);
-                slices = g.N;
+                slices = wpatch::image_lanes(g.N, (g.Cin_g / 64) * ((g.Cout_g + 63) / 64), num_cus() > 0 ? num_cus() : 256);
             }
         } else if (direct) {
             if constexpr (sizeof(T) == 2) {

@@ -17,9 +17,10 @@ int launch(hipStream_t s, const Problem& p) {
     a.P = p.P; a.Q = p.Q; a.PQ = p.P * p.Q; a.N = p.N;
     a.pad_w = p.pad_w; a.pad_h = p.pad_h; a.pitch = p.P + 2;
     a.H = p.Cg / 64; a.CB = (p.Ncols + 63) / 64;
+    a.lanes = image_lanes(p.N, a.H * a.CB, num_cus() > 0 ? num_cus() : 256);
     a.divP = FastDiv((uint32_t)a.P); a.divPitch = FastDiv((uint32_t)a.pitch);
     ProfScope ps("conv_wgrad_kernel<bf16>", s);
-    conv_wgrad_patch_kernel<<<dim3((unsigned)(((p.N + 7) / 8) * 8 * a.H * a.CB)), dim3(THREADS), LDS_BYTES, s>>>(a);
+    conv_wgrad_patch_kernel<<<dim3((unsigned)(((a.lanes + 7) / 8) * 8 * a.H * a.CB)), dim3(THREADS), LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
 }

@@ -8,8 +8,10 @@
 // image, 64 input channels and 64 output channels and walks over the image in tiles of 256 positions; the
 // rows of the image under a tile (plus the halo) are brought into LDS once, and all nine taps read them at
 // shifted addresses.  The accumulators of a workgroup are the whole 9 x 64 x 64 block of dw for its
-// channels (144 registers per lane), written once per image as a partial sum; wgrad_reduce_kernel adds the
-// images in order.
+// channels (144 registers per lane).  Workgroup "lane" i of a part takes the images i, i + lanes, ... and writes one
+// partial sum at the end; wgrad_reduce_kernel adds the lanes in order.  There are as many lanes as images while
+// that keeps the workgroups within two per compute unit, otherwise fewer (a multiple of eight): the partial sums
+// then stay a small multiple of the filter's size however large the batch is.
 //
 // Waves: wave w owns the 16 input channels 16 (w % 4) .. + 15 and every second 32-position step of the
 // contraction (w / 4 selects which); the two waves of a channel block add their accumulators through LDS at
@@ -42,10 +44,10 @@ typedef const __attribute__((address_space(1))) void* glb_vp;
 struct Args {
     const bf16_t* src;       // channel-contiguous x (C, P, Q, N), first channel of the group
     const bf16_t* dz;        // (P, Q, Cout, N), first output channel of the group
-    float* partial;          // [image][column][9 * Cg]
+    float* partial;          // [lane][column][9 * Cg]
     const void* zero;        // 16 zero bytes in device memory
     int Ctot, Cg, Cout, Ncols;   // channels of x (all groups), of the group; output channels in all, of the group
-    int P, Q, PQ, N;
+    int P, Q, PQ, N, lanes;  // lanes: workgroups per part, each walks the images lane, lane + lanes, ...
     int pad_w, pad_h, pitch;     // pitch = P + 2
     int H, CB;                   // 64-channel parts of Cg, of Ncols
     FastDiv divP, divPitch;
@@ -67,8 +69,8 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
     // XCD (workgroup i runs on XCD i % 8), next to each other in its order of dispatch, so that its L2 serves the repeats.
     const int parts = a.CB * a.H;
     const int slot = blockIdx.x >> 3;
-    const int n = (slot / parts) * 8 + (blockIdx.x & 7), part = slot % parts;
-    if (n >= a.N) return;                                   // the last group of eight images may be incomplete
+    const int lane = (slot / parts) * 8 + (blockIdx.x & 7), part = slot % parts;
+    if (lane >= a.N) return;                                // the last group of eight may be incomplete
     const int cb = part % a.CB, h = part / a.CB;
     const int steps = a.PQ / STEP_PX;                  // of the image
     const int tiles = (a.PQ + TILE_PX - 1) / TILE_PX;
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
         poff[i] = ((pr * a.P + ps) * a.Ctot + 16 * plane + 8 * (l & 1)) * 2;
         prv[i] = ((unsigned)ps < (unsigned)a.P && x < PATCH_PIX) ? pr : -(1 << 28);   // halo columns and the tail never pass the row test
     }
-    const char* const src_img = reinterpret_cast<const char*>(a.src) + ((int64_t)n * a.Q * row_bytes) + h * 128;
+    const char* src_img = reinterpret_cast<const char*>(a.src) + ((int64_t)lane * a.Q * row_bytes) + h * 128;
     // patch of tile `ti` of the image into buffer `buf`: rows q_first - pad_h .. of the image
     auto patch_issue = [&](int i, int ti, int buf) {
         const int q0 = (int)a.divP.div((uint32_t)(ti * TILE_PX)) - a.pad_h;
@@ -101,8 +103,8 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
     // w / 4 and 2 + w / 4 of the group; lane: row l % 16, 16-byte chunk (8 positions) l / 16
     const int zrow = 16 * (w & 3) + (l & 15);
     const bool zrow_ok = cb * 64 + zrow < a.Ncols;
-    const char* const dz_row = reinterpret_cast<const char*>(a.dz) +
-                               (((int64_t)n * a.Cout + cb * 64 + (zrow_ok ? zrow : 0)) * a.PQ + 8 * (l >> 4)) * 2;
+    const char* dz_row = reinterpret_cast<const char*>(a.dz) +
+                         (((int64_t)lane * a.Cout + cb * 64 + (zrow_ok ? zrow : 0)) * a.PQ + 8 * (l >> 4)) * 2;
     auto dz_issue = [&](int step) {              // step of the image (uniform); past the image: zeros
         const void* p = (step < steps && zrow_ok) ? static_cast<const void*>(dz_row + (int64_t)step * (STEP_PX * 2)) : a.zero;
         __builtin_amdgcn_global_load_lds((glb_vp)p, (lds_vp)(lds + RING_OFF + (step & (RING - 1)) * BLK_BYTES + (w & 3) * 1024), 16, 0, 0);
@@ -123,7 +125,8 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[t][j][r] = 0.0f;
 
-    // prologue: the first tile's patch, the dz blocks of the first four steps
+    for (int n = lane;;) {
+    // prologue of an image: the first tile's patch, the dz blocks of the first four steps
 #pragma unroll
     for (int i = 0; i < PATCH_INSTR; ++i) patch_issue(i, 0, 0);
     dz_issue(w >> 2);
@@ -209,6 +212,15 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
         }
     }
 
+    // the next image of this lane: every wave has read the last fragments of this one before the buffers are refilled
+    n += a.lanes;
+    if (n >= a.N) break;
+    src_img += (int64_t)a.lanes * a.Q * row_bytes;
+    dz_row += (int64_t)a.lanes * a.Cout * a.PQ * 2;
+    __builtin_amdgcn_s_waitcnt(0 | (0x7 << 4));
+    __builtin_amdgcn_s_barrier();
+    }
+
     // ---- the two waves of a channel block add their halves through LDS; the first stores
     __builtin_amdgcn_s_waitcnt(0 | (0x7 << 4));
     __builtin_amdgcn_s_barrier();
@@ -224,7 +236,7 @@ __global__ __launch_bounds__(THREADS) void conv_wgrad_patch_kernel(Args a) {
     if (ks == 0) {
         const int Mrows = TAPS * a.Cg;
         // acc[t][j][r]: input channel 64 h + 16 wa + 4 g + r, output channel 64 cb + 16 j + s
-        float* out = a.partial + (size_t)n * a.Ncols * Mrows + 64 * h + 16 * wa + 4 * g;
+        float* out = a.partial + (size_t)lane * a.Ncols * Mrows + 64 * h + 16 * wa + 4 * g;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int col = cb * 64 + 16 * j + s;
@@ -249,7 +261,14 @@ struct Problem {
     int Ctot, Cg, Cout, Ncols, P, Q, N, pad_w, pad_h;
 };
 
-// 3 x 3, unit stride and dilation, output as large as the input are the caller's to check; one partial sum per image.
+// Workgroups per part (= partial sums that wgrad_reduce_kernel adds): one per image while the grid stays within two
+// workgroups per compute unit, otherwise as many groups of eight as fit that bound (at least one).
+inline int image_lanes(int N, int parts, int cus) {
+    if ((int64_t)N * parts <= 2 * (int64_t)cus) return N;
+    return std::min(N, std::max(8, (int)(2 * (int64_t)cus / parts) / 8 * 8));
+}
+
+// 3 x 3, unit stride and dilation, output as large as the input are the caller's to check.
 inline bool applicable(const Problem& p, int cus) {
     const auto al = [](const void* q, uintptr_t n) { return (reinterpret_cast<uintptr_t>(q) & (n - 1)) == 0; };
     const int pitch = p.P + 2;

@@ -266,6 +266,28 @@ def test_filter_gradient_window_kernel_batches(gpu, xs, ws):
     assert_close(dw_gather, want, "bf16", f"gather wgrad N={xs[3]}")
 
 
+@pytest.mark.parametrize("xs,ws", [((16, 16, 128, 300), (3, 3, 128, 128)),     # 4 parts x 300 images: 128 workgroups per part, 2-3 images each
+                                   ((8, 8, 256, 200), (3, 3, 256, 256))])       # 16 parts x 200 images: 32 per part, 6-7 images each
+def test_filter_gradient_window_kernel_large_batches(gpu, xs, ws):
+    """Batches so large that one workgroup per image and channel part would be more than two per compute unit: a workgroup
+    then walks several images and the number of fp32 partial sums (and the scratch memory for them) stays bounded.  Against
+    the gather kernel on the whole gradient and against the fp64 oracle on the first eight output channels."""
+    rng = np.random.default_rng(778 + xs[3])
+    gd, od = cdims(gpu, xs, ws, padding=1)
+    x, dy = host_inputs("bf16", rng.normal(size=xs), rng.normal(size=od.y_shape()))
+    dx_, ddy_ = dev(gpu, x, "bf16"), dev(gpu, dy, "bf16")
+    dw = gpu.conv_filter_grad(dx_, ddy_, gd).to_numpy()
+    gpu.set_option("conv_tile", 84)
+    try:
+        dw_gather = gpu.conv_filter_grad(dx_, ddy_, gd).to_numpy()
+    finally:
+        gpu.set_option("conv_tile", 0)
+    assert_close(dw, f64(dw_gather), "bf16", f"window against gather wgrad N={xs[3]}")
+    _, od8 = cdims(gpu, xs, ws[:3] + (8,), padding=1)
+    want = O.conv_filter_grad(f64(x), f64(dy[:, :, :8]), od8)
+    assert_close(dw[..., :8], want, "bf16", f"window wgrad N={xs[3]}, first output channels")
+
+
 def _random_window_shapes(count, seed):
     """Shapes that the 3 x 3 window kernels accept (unit stride, output as large as the input, channels per group in
     multiples of 64, W * H a multiple of 4), drawn with a fixed seed."""
