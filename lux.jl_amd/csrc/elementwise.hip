@@ -284,6 +284,54 @@ __global__ __launch_bounds__(1024) void plane_finalize_dense_kernel(const float*
     }
 }
 
+// Dense pullback, bf16, large matrices: dz = delta .* act'(y, pre) (M x N, m contiguous), its transpose dzT (n
+// contiguous: the layout in which the weight-gradient product reads it along its contraction index) and the bias
+// gradient's partial sums over the 64 columns of a tile, in one pass over delta.  A 64 x 64 tile goes through LDS
+// as fp32 (the sums add unrounded values): phase 1 reads 16-byte vectors along m, stores dz and fills the tile;
+// phase 2 reads eight n of one m per thread (rows of 65 words: the 64 lanes of a wave hit 64 banks in both phases),
+// stores 16 bytes of dzT and adds its eight values; the eight threads of an m add theirs in a fixed order.
+// M and N multiples of 64, every pointer 16-byte aligned.  dz may be null (identity: dz is delta), partial may be null.
+template <int ACT>
+__global__ __launch_bounds__(256) void dense_dz_transposed_kernel(const bf16_t* __restrict__ delta, const bf16_t* __restrict__ out,
+                                                                  const bf16_t* __restrict__ pre, bf16_t* dz, bf16_t* __restrict__ dzT,
+                                                                  float* __restrict__ partial, uint32_t M, uint32_t N) {
+    constexpr int PITCH = 65;
+    __shared__ float tile[64 * PITCH];
+    const uint32_t m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+    float r[2][8];
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {                 // loads first, then the stores
+        const uint32_t idx = threadIdx.x + it * 256, nl = idx >> 3, mv = idx & 7;
+        dx_vec<bf16_t, ACT, 8>(delta, out, pre, (size_t)(n0 + nl) * M + m0 + mv * 8, r[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const uint32_t idx = threadIdx.x + it * 256, nl = idx >> 3, mv = idx & 7;
+        if (dz != nullptr) store_vec<bf16_t, 8>(dz, (size_t)(n0 + nl) * M + m0 + mv * 8, r[it]);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) tile[nl * PITCH + mv * 8 + k] = r[it][k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const uint32_t idx = threadIdx.x + it * 256, ml = idx >> 3, nv = idx & 7;
+        float v[8], sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            v[k] = tile[(nv * 8 + k) * PITCH + ml];
+            sum += v[k];
+        }
+        store_vec<bf16_t, 8>(dzT, (size_t)(m0 + ml) * N + n0 + nv * 8, v);
+        if (partial != nullptr) {
+            // the eight threads of this m are neighbouring lanes: (((s0 + s1) + (s2 + s3)) + ((s4 + s5) + (s6 + s7)))
+            sum += __shfl_xor(sum, 1);
+            sum += __shfl_xor(sum, 2);
+            sum += __shfl_xor(sum, 4);
+            if (nv == 0) partial[(size_t)blockIdx.y * M + m0 + ml] = sum;
+        }
+    }
+}
+
 static inline unsigned grid_for(uint32_t total_vec) {
     return (unsigned)ceil_div(total_vec, kThreads * kUnroll);
 }
@@ -468,6 +516,28 @@ static int check_common(int dtype, int act, int64_t I, int64_t C, int64_t N) {
     if (I > 0 && C > 0 && N > 0) {
         const long double tot = (long double)I * (long double)C * (long double)N;
         LUX_UNSUPPORTED_IF(tot >= 2147483648.0L, "tensors of 2^31 or more elements are not supported");
+    }
+    return LUXHIP_OK;
+}
+
+// The dense pullback's first pass when the weight-gradient product wants dz transposed (gemm.hip decides): dz (may be
+// NULL for the identity), dzT and, if dbias != NULL, the bias gradient.  `partial`: N / 64 * M floats of scratch.
+int dense_dz_transposed(hipStream_t s, int act, int64_t M, int64_t N, const bf16_t* delta, const bf16_t* out, const bf16_t* pre,
+                        bf16_t* dz, bf16_t* dzT, float* partial, bf16_t* dbias) {
+    LUX_INVALID_IF(M % 64 != 0 || N % 64 != 0 || N / 64 > 65535, "dense_dz_transposed: whole 64 x 64 tiles only");
+    const dim3 grid((unsigned)(M / 64), (unsigned)(N / 64));
+    float* const part = dbias != nullptr ? partial : nullptr;
+#define LAUNCH_DZT(A) dense_dz_transposed_kernel<A><<<grid, 256, 0, s>>>(delta, out, pre, dz, dzT, part, (uint32_t)M, (uint32_t)N)
+    {
+        ProfScope ps("dense_dz_transposed_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_DZT);
+    }
+#undef LAUNCH_DZT
+    LUX_CHECK_LAUNCH();
+    if (dbias != nullptr) {
+        ProfScope ps2("plane_finalize_kernel", s);
+        plane_finalize_dense_kernel<bf16_t><<<(unsigned)ceil_div(M, 64), 1024, 0, s>>>(partial, dbias, (uint32_t)M, (uint32_t)(N / 64));
+        LUX_CHECK_LAUNCH();
     }
     return LUXHIP_OK;
 }

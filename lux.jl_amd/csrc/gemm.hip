@@ -13,8 +13,11 @@ int bias_act_bwd_dispatch(hipStream_t s, int dtype, int act, int64_t I, int64_t 
                           const void* out, const void* pre, void* dx, void* dbias);   // elementwise.hip
 
 int transpose_matrix_bf16(hipStream_t s, const bf16_t* in, bf16_t* out, int64_t P, int64_t C);   // conv.hip
+int dense_dz_transposed(hipStream_t s, int act, int64_t M, int64_t N, const bf16_t* delta, const bf16_t* out, const bf16_t* pre,
+                        bf16_t* dz, bf16_t* dzT, float* partial, bf16_t* dbias);                 // elementwise.hip
 
 int gemm_tile_override() { return (int)option_gemm_tile(); }
+static inline size_t align256(size_t b) { return (b + 255) & ~size_t(255); }
 // The 256 x 256 bf16 kernel reads K-major operands from LDS at twice the rate of M/N-major ones
 // (plain 16-byte reads against transposing reads): 1090-1190 TFLOP/s against 800-950 measured on
 // 4096..11008-sized problems.  A large M/N-major operand is therefore copied into the K-major
@@ -27,9 +30,10 @@ static bool pretranspose_pays(int64_t M, int64_t N, int64_t K, int64_t other, in
            (M / 256) * (N / 256) >= 128 && K >= 1024 && other >= 4096 && ld == rows && aligned16(p);
 }
 
+// ws_front: bytes at the start of the stream's workspace that the caller is using (operand copies go behind them)
 template <typename T>
 static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const T* A, int64_t lda,
-                     const T* B, int64_t ldb, const T* bias, T* C, int64_t ldc, T* pre, int act) {
+                     const T* B, int64_t ldb, const T* bias, T* C, int64_t ldc, T* pre, int act, size_t ws_front = 0) {
     DenseArgs<T> a;
     bool a_kmajor = transA != 0, b_kmajor = transB == 0;
     if constexpr (sizeof(T) == 2) {
@@ -42,8 +46,9 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
             const size_t ab = ta ? (((size_t)M * K * sizeof(T) + 255) & ~size_t(255)) : 0;
             const size_t bb = tb ? (size_t)N * K * sizeof(T) : 0;
             Workspace ws;
-            int rc = get_workspace(s, ab + bb, &ws);
+            int rc = get_workspace(s, ws_front + ab + bb, &ws);
             if (rc != LUXHIP_OK) return rc;
+            ws.data += ws_front;
             if (ta) {
                 T* At = reinterpret_cast<T*>(ws.data);
                 if ((rc = transpose_matrix_bf16(s, A, At, M, K)) != LUXHIP_OK) return rc;
@@ -180,7 +185,7 @@ static int gemm_check(int dtype, int act, int64_t M, int64_t N, int64_t K) {
 
 static int gemm_dispatch(hipStream_t s, int dtype, int transA, int transB, int64_t M, int64_t N, int64_t K, const void* A,
                          int64_t lda, const void* B, int64_t ldb, const void* bias, void* C, int64_t ldc, void* pre,
-                         int act) {
+                         int act, size_t ws_front = 0) {
     if (M == 0 || N == 0) return LUXHIP_OK;
     LUX_INVALID_IF(C == nullptr, "matmul: C must not be NULL");
     LUX_INVALID_IF(K > 0 && (A == nullptr || B == nullptr), "matmul: A and B must not be NULL");
@@ -189,7 +194,7 @@ static int gemm_dispatch(hipStream_t s, int dtype, int transA, int transB, int64
         return gemm_impl<float>(s, transA, transB, M, N, K, (const float*)A, lda, (const float*)B, ldb, (const float*)bias,
                                 (float*)C, ldc, (float*)pre, act);
     return gemm_impl<bf16_t>(s, transA, transB, M, N, K, (const bf16_t*)A, lda, (const bf16_t*)B, ldb, (const bf16_t*)bias,
-                             (bf16_t*)C, ldc, (bf16_t*)pre, act);
+                             (bf16_t*)C, ldc, (bf16_t*)pre, act, ws_front);
 }
 
 }  // namespace luxhip
@@ -261,6 +266,31 @@ int luxhip_fused_dense_bwd(luxhip_stream_t s, int dtype, int act, int64_t M, int
     LUX_INVALID_IF(act != LUXHIP_ACT_IDENTITY && !act_needs_pre(act) && y == nullptr, "fused_dense_bwd: activation %d needs y", act);
     LUX_INVALID_IF(act_needs_pre(act) && pre == nullptr, "fused_dense_bwd: activation %d needs the pre-activation", act);
     const void* dzp = delta;
+    // Large bf16 layers: the weight-gradient product reads dz along n, so it would copy dz into that layout first
+    // (pretranspose_pays); the pass that computes dz writes that copy as well, and the bias gradient's partial sums,
+    // instead of a pass for dz / dbias followed by a transposing copy.
+    const int64_t ldxe = std::max<int64_t>(ldx, 1);
+    const bool dz_both = dtype == LUXHIP_BF16 && dW != nullptr && M % 64 == 0 && N % 64 == 0 && N / 64 <= 65535 && N >= 2048 &&
+                         pretranspose_pays<bf16_t>(M, K, N, K, M, M, (const bf16_t*)delta) &&
+                         pretranspose_pays<bf16_t>(M, K, N, M, ldxe, K, (const bf16_t*)x) && aligned16(y) && aligned16(pre) &&
+                         aligned16(dz) && M * N < (int64_t(1) << 31);
+    if (dz_both) {
+        const size_t tb = align256((size_t)M * N * 2), pb = dbias != nullptr ? align256((size_t)(N / 64) * M * sizeof(float)) : 0;
+        const size_t xb = align256((size_t)K * N * 2);          // the product's own copy of x, behind ours
+        Workspace ws;
+        rc = get_workspace((hipStream_t)s, tb + pb + xb, &ws);
+        if (rc != LUXHIP_OK) return rc;
+        bf16_t* dzT = reinterpret_cast<bf16_t*>(ws.data);
+        void* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : dz;
+        rc = dense_dz_transposed((hipStream_t)s, act, M, N, (const bf16_t*)delta, (const bf16_t*)y, (const bf16_t*)pre, (bf16_t*)dz_out,
+                                 dzT, reinterpret_cast<float*>(ws.data + tb), (bf16_t*)dbias);
+        if (rc != LUXHIP_OK) return rc;
+        if (dz_out) dzp = dz_out;
+        // dW (M x K) = dz (M x N) * x' (N x K) with dz given as its transpose (N contiguous)
+        rc = gemm_dispatch((hipStream_t)s, dtype, 1, 1, M, K, N, dzT, N, x, ldx, nullptr, dW, std::max<int64_t>(M, 1), nullptr,
+                           LUXHIP_ACT_IDENTITY, tb + pb);
+        if (rc != LUXHIP_OK) return rc;
+    } else {
     if (act != LUXHIP_ACT_IDENTITY || dbias != nullptr) {
         // dz = delta .* act'(y, pre) and dbias = sum over the batch, one pass (dense layout: I = 1)
         void* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : dz;
@@ -272,6 +302,7 @@ int luxhip_fused_dense_bwd(luxhip_stream_t s, int dtype, int act, int64_t M, int
         rc = gemm_dispatch((hipStream_t)s, dtype, 0, 1, M, K, N, dzp, std::max<int64_t>(M, 1), x, ldx, nullptr, dW,
                            std::max<int64_t>(M, 1), nullptr, LUXHIP_ACT_IDENTITY);
         if (rc != LUXHIP_OK) return rc;
+    }
     }
     if (dx != nullptr) {   // dx (K x N) = W' (K x M) * dz (M x N);  W is stored M x K
         rc = gemm_dispatch((hipStream_t)s, dtype, 1, 0, K, N, M, W, ldw, dzp, std::max<int64_t>(M, 1), nullptr, dx,
