@@ -274,6 +274,25 @@ int luxhip_attention_softmax_fwd(luxhip_stream_t s, int dtype, int64_t S, int64_
 int luxhip_attention_softmax_bwd(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t cols, int causal,
                                  const void* dprobs, const void* probs, double scale, void* dlogits);
 
+/* The two steps above the pullback of the attention weights in one: the batched product
+ * dprobs = v' d_out (the pullback of batched_matmul(v, probs), src/impl/batched_mul.jl:320-334) with the
+ * softmax rule as its epilogue, dlogits = scale * probs .* (dprobs - sum_s dprobs .* probs).  The inner
+ * sum equals sum_e d_out[e, l] out[e, l] (out = v probs), so it is taken from the forward result and the
+ * cotangent of the weights never goes to memory (and stays fp32 in bf16 storage).  The identity holds for
+ * the unrounded out: with dtype LUXHIP_BF16_WIDE `out` is the fp32 result of the forward product
+ * (luxhip_batched_matmul_strided under the same dtype), which the caller keeps beside the bf16 array it
+ * returns; an out rounded to bf16 shifts whole columns of dlogits by probs times the rounding error.
+ * v: (Ev, S) per product with leading dimension ldv and batch strides strides_v; d_out, out: (Ev, L) with
+ * ldo and strides_o (the same array layout); probs, dlogits: (S, L) with ldc and strides_c; batch_dims as
+ * in luxhip_batched_matmul_strided.  structure 1: tiles with every s > l are left untouched (causal mask).
+ * Not for calls with an fdrop (the weights that multiply v are then not the softmax result): those take
+ * luxhip_batched_matmul_strided and luxhip_attention_softmax_bwd. */
+int luxhip_attention_weights_pullback(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t Ev,
+                                      const int64_t* batch_dims, const void* v, int64_t ldv,
+                                      const int64_t* strides_v, const void* d_out, const void* out, int64_t ldo,
+                                      const int64_t* strides_o, const void* probs, double scale, void* dlogits,
+                                      int64_t ldc, const int64_t* strides_c, int structure);
+
 /* ---------------------------------------------------------------- dropout ----------
  * The reference draws its noise with `rand!(rng, y)` from the array package's generator
  * (src/impl/dropout.jl:171-190); here a counter-based Philox4x32-10 stream stands in for it:

@@ -85,6 +85,8 @@ SIGNATURES = {
     "luxhip_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64],
     "luxhip_batched_matmul": [_vp, _i, _i, _i, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64],
     "luxhip_batched_matmul_strided": [_vp, _i, _i, _i, _i64, _i64, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64, _vp, _i64, _ip64, _i],
+    "luxhip_attention_weights_pullback": [_vp, _i, _i64, _i64, _i64, _ip64, _vp, _i64, _ip64, _vp, _vp, _i64, _ip64, _vp, _d, _vp, _i64,
+                                          _ip64, _i],
     "luxhip_batch_sum": [_vp, _i, _i64, _i64, _vp, _vp],
     "luxhip_fused_dense_fwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp],
     "luxhip_fused_dense_bwd": [_vp, _i, _i, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp],

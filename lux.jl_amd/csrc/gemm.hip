@@ -84,10 +84,14 @@ static int gemm_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N
 template <typename T>
 static int batched_impl(hipStream_t s, int transA, int transB, int64_t M, int64_t N, int64_t K, const int64_t* bdim, const T* A,
                         int64_t lda, const int64_t* sA, const T* B, int64_t ldb, const int64_t* sB, T* C, int64_t ldc,
-                        const int64_t* sC, int structure, int c_f32 = 0) {
+                        const int64_t* sC, int structure, int c_f32 = 0, const T* ep_probs = nullptr, const float* ep_d = nullptr,
+                        float ep_scale = 0.0f) {
     DenseArgs<T> a;
     a.structure = structure;
     a.c_f32 = c_f32;
+    a.ep_probs = ep_probs;
+    a.ep_d = ep_d;
+    a.ep_scale = ep_scale;
     const bool a_kmajor = transA != 0, b_kmajor = transB == 0;
     a.A.p = A;
     a.A.sr = a_kmajor ? lda : 1;
@@ -175,6 +179,30 @@ static int batch_sum_impl(hipStream_t s, int64_t n, int64_t batch, const T* in, 
     return LUXHIP_OK;
 }
 
+// d[b * N + n] = sum_e dO[e, n] O[e, n] of product b (both E x N with leading dimension ldo and the given batch strides):
+// one wavefront per column, fp32.  This is sum_s probs[s, n] dprobs[s, n], the inner product that the softmax rule needs,
+// without the cotangent of the weights -- exactly so only for the unrounded O = V probs, which is why bf16 storage
+// hands O over in fp32 (TO = float): an O rounded to bf16 shifts a whole column of the result by probs times the
+// rounding error.
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void attn_rowdot_kernel(const T* __restrict__ dO, const TO* __restrict__ O, float* __restrict__ d, int E,
+                                                          int N, int64_t ldo, int bd0, int bd1, int64_t s0, int64_t s1, int64_t s2,
+                                                          int64_t cols) {
+    const int64_t col = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (col >= cols) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t b = col / N;
+    const int n = (int)(col - b * N);
+    const int i0 = (int)(b % bd0), i1 = (int)((b / bd0) % bd1);
+    const int64_t i2 = b / ((int64_t)bd0 * bd1);
+    const int64_t off = i0 * s0 + i1 * s1 + i2 * s2 + (int64_t)n * ldo;
+    float acc = 0.0f;
+    for (int e = lane; e < E; e += 64) acc = fmaf(ld(dO + off + e), ld(O + off + e), acc);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) acc += __shfl_xor(acc, o);
+    if (lane == 0) d[col] = acc;
+}
+
 static int gemm_check(int dtype, int act, int64_t M, int64_t N, int64_t K) {
     LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
     LUX_UNSUPPORTED_IF(act < 0 || act >= LUXHIP_ACT_COUNT, "unsupported activation id %d", act);
@@ -234,6 +262,58 @@ int luxhip_batched_matmul_strided(luxhip_stream_t s, int dtype, int transA, int 
                    "batched_matmul_strided: batch extents and strides must not be NULL");
     return batched_dispatch((hipStream_t)s, dtype, transA, transB, M, N, K, batch_dims, A, lda, stridesA, B, ldb, stridesB, C, ldc,
                             stridesC, structure);
+}
+
+int luxhip_attention_weights_pullback(luxhip_stream_t s, int dtype, int64_t S, int64_t L, int64_t Ev, const int64_t* batch_dims,
+                                      const void* v, int64_t ldv, const int64_t* strides_v, const void* d_out, const void* out,
+                                      int64_t ldo, const int64_t* strides_o, const void* probs, double scale, void* dlogits,
+                                      int64_t ldc, const int64_t* strides_c, int structure) {
+    LUX_REQUIRE_INIT();
+    const bool wide = dtype == LUXHIP_BF16_WIDE;
+    if (wide) dtype = LUXHIP_BF16;
+    int rc = gemm_check(dtype, 0, S, L, Ev);
+    if (rc != LUXHIP_OK) return rc;
+    LUX_INVALID_IF(batch_dims == nullptr || strides_v == nullptr || strides_o == nullptr || strides_c == nullptr,
+                   "attention_weights_pullback: batch extents and strides must not be NULL");
+    LUX_INVALID_IF(structure != 0 && structure != 1, "attention_weights_pullback: structure must be 0 or 1");
+    int64_t batch = 1;
+    for (int d = 0; d < 3; ++d) {
+        LUX_INVALID_IF(batch_dims[d] < 0 || strides_v[d] < 0 || strides_o[d] < 0 || strides_c[d] < 0,
+                       "attention_weights_pullback: negative batch extent or stride");
+        batch *= batch_dims[d];
+        LUX_UNSUPPORTED_IF(batch >= (1ll << 31), "attention_weights_pullback: batch of 2^31 or more");
+    }
+    if (S == 0 || L == 0 || batch == 0) return LUXHIP_OK;
+    LUX_INVALID_IF(v == nullptr || d_out == nullptr || out == nullptr || probs == nullptr || dlogits == nullptr,
+                   "attention_weights_pullback: null operand");
+    LUX_INVALID_IF(ldv < Ev || ldo < Ev || ldc < S, "attention_weights_pullback: leading dimension too small");
+    const int64_t cols = batch * L;
+    Workspace ws;
+    rc = get_workspace((hipStream_t)s, (size_t)cols * sizeof(float), &ws);
+    if (rc != LUXHIP_OK) return rc;
+    float* d = reinterpret_cast<float*>(ws.data);
+    {
+        ProfScope ps("attn_rowdot_kernel", (hipStream_t)s);
+        const unsigned grid = (unsigned)ceil_div(cols, 4);
+        const int b0 = (int)batch_dims[0], b1 = (int)batch_dims[1];
+        const int64_t *so = strides_o;
+        if (dtype == LUXHIP_F32)
+            attn_rowdot_kernel<float, float><<<grid, 256, 0, (hipStream_t)s>>>((const float*)d_out, (const float*)out, d, (int)Ev, (int)L, ldo,
+                                                                               b0, b1, so[0], so[1], so[2], cols);
+        else if (wide)
+            attn_rowdot_kernel<bf16_t, float><<<grid, 256, 0, (hipStream_t)s>>>((const bf16_t*)d_out, (const float*)out, d, (int)Ev, (int)L,
+                                                                                ldo, b0, b1, so[0], so[1], so[2], cols);
+        else
+            attn_rowdot_kernel<bf16_t, bf16_t><<<grid, 256, 0, (hipStream_t)s>>>((const bf16_t*)d_out, (const bf16_t*)out, d, (int)Ev, (int)L,
+                                                                                 ldo, b0, b1, so[0], so[1], so[2], cols);
+        LUX_CHECK_LAUNCH();
+    }
+    // dprobs (S x L) = v' (S x Ev) * d_out (Ev x L), with the softmax rule as its epilogue
+    if (dtype == LUXHIP_F32)
+        return batched_impl<float>((hipStream_t)s, 1, 0, S, L, Ev, batch_dims, (const float*)v, ldv, strides_v, (const float*)d_out, ldo,
+                                   strides_o, (float*)dlogits, ldc, strides_c, structure, 0, (const float*)probs, d, (float)scale);
+    return batched_impl<bf16_t>((hipStream_t)s, 1, 0, S, L, Ev, batch_dims, (const bf16_t*)v, ldv, strides_v, (const bf16_t*)d_out, ldo,
+                                strides_o, (bf16_t*)dlogits, ldc, strides_c, structure, 0, (const bf16_t*)probs, d, (float)scale);
 }
 
 int luxhip_batch_sum(luxhip_stream_t s, int dtype, int64_t n, int64_t batch, const void* in, void* out) {

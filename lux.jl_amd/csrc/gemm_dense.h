@@ -242,6 +242,7 @@ struct BatchTile {
     Operand<T> A, B;
     T* C;
     int64_t coff;   // elements between a.C and this product's C
+    int product;    // index of the product
     int m0, n0;
     int K;          // extent of the contraction for this tile (a.structure may shorten it)
     bool store;     // false: the tile is not computed (a.structure == 1, every m > n)
@@ -264,13 +265,16 @@ __device__ __forceinline__ BatchTile<T> batch_tile(const DenseArgs<T>& a, int t,
     bt.A.p = a.A.p + i0 * a.bsA[0] + i1 * a.bsA[1] + i2 * a.bsA[2];
     bt.B.p = a.B.p + i0 * a.bsB[0] + i1 * a.bsB[1] + i2 * a.bsB[2];
     bt.coff = i0 * a.bsC[0] + i1 * a.bsC[1] + i2 * a.bsC[2];
+    bt.product = b;
     bt.C = a.C + bt.coff;
     bt.m0 = tm * TILE_M;
     bt.n0 = tn * TILE_N;
     bt.K = a.K;
     bt.store = true;
     if (a.structure == 1) {
-        if (bt.m0 >= bt.n0 + TILE_N) { bt.store = false; bt.K = 0; }
+        // computed: everything up to the end of the block of 128 rows that holds the diagonal of the tile's last column
+        // (what the products with structure 2 or 3 read, whatever their own tile size)
+        if (bt.m0 >= ((bt.n0 + TILE_N - 1) / 128 + 1) * 128) { bt.store = false; bt.K = 0; }
     } else if (a.structure == 2) {
         bt.K = min(a.K, bt.n0 + TILE_N);
     } else if (a.structure == 3) {
@@ -293,19 +297,131 @@ __device__ __forceinline__ void store_tile_f32(const f32x16_v (&acc)[WM][WN], co
     });
 }
 
-template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM>
-__global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<T> a) {
+// The softmax rule as the epilogue of the product that computes the cotangent of the attention weights
+// (a.ep_probs): C = scale * probs .* (acc - d[n]), d[n] = sum over the column of probs .* acc, which the caller
+// has computed as sum_e dO[e, n] O[e, n].  The cotangent itself never goes to memory, and stays fp32.
+// The weights and d of a tile do not depend on the product, so their loads are issued before the tile's main loop
+// and have arrived when it ends: the epilogue itself only stores.  The loaded words stay as they came from memory
+// until the epilogue (unpacking them at the load would put a wait behind every load), and the choice between the
+// packed and the element-wise access is made once per tile, not per column, for the same reason.
+template <class ML, typename T, int WM, int WN, bool FULL>
+struct SoftmaxRuleOperands {
+    static constexpr bool CHECK = !FULL;
+    static constexpr bool CAN_PACK = ML::M_STEP == 1 && sizeof(T) == 2 && !CHECK && (WM == 2 || WM == 4);
+    // packed: pairs of bf16 per word; else one element's bits per word.  A kernel that can pack holds registers for
+    // the packed words only; when the destination does not allow them (unaligned), its epilogue loads on the spot.
+    uint32_t w[WN * 16][CAN_PACK ? WM / 2 : WM];
+    float d[WN * 16];
+    bool packed;
+
+    template <bool PACKED>
+    __device__ __forceinline__ void load_as(const DenseArgs<T>& a, const T* P, const float* dvec, int mb, int nb) {
+        static_for<WN * 16>([&](auto JR) {
+            constexpr int c = decltype(JR)::value, j = c / 16, r = c % 16;
+            const int n = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
+            const int nc = CHECK ? min(n, a.N - 1) : n;       // out-of-range lanes read a valid element and store nothing
+            const T* col = P + (int64_t)nc * a.ldc;
+            if constexpr (PACKED) {
+                if constexpr (WM == 4) {
+                    const uint2 v = *reinterpret_cast<const uint2*>(col + mb);
+                    w[c][0] = v.x; w[c][1] = v.y;
+                } else {
+                    w[c][0] = *reinterpret_cast<const uint32_t*>(col + mb);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < WM; ++i) {
+                    const int m = CHECK ? min(mb + i * ML::M_STEP, a.M - 1) : mb + i * ML::M_STEP;
+                    if constexpr (sizeof(T) == 2) w[c][i] = col[m];
+                    else w[c][i] = __float_as_uint(col[m]);
+                }
+            }
+            d[c] = dvec[nc];
+        });
+    }
+    __device__ __forceinline__ void load_d(const float* dvec, int nb) {
+        static_for<WN * 16>([&](auto JR) {
+            constexpr int c = decltype(JR)::value, j = c / 16, r = c % 16;
+            d[c] = dvec[nb + j * 32 + ((r >> 2) << 3) + (r & 3)];
+        });
+    }
+    __device__ __forceinline__ void load(const DenseArgs<T>& a, int64_t coff, int product, int m0, int n0) {
+        const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
+        const T* P = a.ep_probs + coff;
+        const float* dvec = a.ep_d + (int64_t)product * a.N;
+        packed = CAN_PACK && a.c_vec != 0;
+        if constexpr (CAN_PACK) {
+            if (packed) load_as<true>(a, P, dvec, mb, nb);
+            else load_d(dvec, nb);
+        } else {
+            load_as<false>(a, P, dvec, mb, nb);
+        }
+    }
+    template <bool PACKED>
+    __device__ __forceinline__ void store_as(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, T* C, int mb, int nb) const {
+        const float scale = a.ep_scale;
+        static_for<WN * 16>([&](auto JR) {
+            constexpr int c = decltype(JR)::value, j = c / 16, r = c % 16;
+            const int n = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
+            if (!CHECK || n < a.N) {
+                float v[WM];
+#pragma unroll
+                for (int i = 0; i < WM; ++i) {
+                    float p;
+                    if constexpr (PACKED) p = __uint_as_float((i & 1) ? (w[c][i / 2] & 0xffff0000u) : (w[c][i / 2] << 16));
+                    else if constexpr (sizeof(T) == 2) p = __uint_as_float(w[c][i] << 16);
+                    else p = __uint_as_float(w[c][i]);
+                    v[i] = scale * p * (acc[i][j][r] - d[c]);
+                }
+                store_column<ML, T, WM, CHECK>(C + (int64_t)n * a.ldc + mb, v, mb, a.M, PACKED);
+            }
+        });
+    }
+    __device__ __forceinline__ void store(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, int64_t coff, int m0, int n0) const {
+        const int mb = ML::lane_m(m0), nb = ML::lane_n(n0);
+        T* C = a.C + coff;
+        if constexpr (CAN_PACK) {
+            if (packed) store_as<true>(acc, a, C, mb, nb);
+            else store_unprepared(acc, a, C, a.ep_probs + coff, mb, nb);
+        } else {
+            store_as<false>(acc, a, C, mb, nb);
+        }
+    }
+    // nothing was loaded ahead: element-wise loads, column by column (the rare destination that is not 8-byte aligned)
+    __device__ __forceinline__ void store_unprepared(const f32x16_v (&acc)[WM][WN], const DenseArgs<T>& a, T* C, const T* P, int mb,
+                                                     int nb) const {
+        const float scale = a.ep_scale;
+        static_for<WN * 16>([&](auto JR) {
+            constexpr int c = decltype(JR)::value, j = c / 16, r = c % 16;
+            const int n = nb + j * 32 + ((r >> 2) << 3) + (r & 3);
+            float v[WM];
+#pragma unroll
+            for (int i = 0; i < WM; ++i) v[i] = scale * ld(P + (int64_t)n * a.ldc + mb + i * ML::M_STEP) * (acc[i][j][r] - d[c]);
+            store_column<ML, T, WM, CHECK>(C + (int64_t)n * a.ldc + mb, v, mb, a.M, false);
+        });
+    }
+};
+struct NoOperands {};
+
+// EP: the variant with the softmax rule as its epilogue (a.ep_probs), a kernel of its own so that the plain products
+// keep their register budget (and with it two workgroups per compute unit)
+template <typename T, int WM, int WN, bool A_KMAJOR, bool B_KMAJOR, bool FULL, int NWN, int NWM, bool EP = false>
+__global__ __launch_bounds__(NWM * NWN * 64, (EP && FULL) ? 2 : 1) void batched_gemm_kernel(DenseArgs<T> a) {
     using ML = GemmMainloop<T, WM, WN, A_KMAJOR, B_KMAJOR, FULL, NWN, 0, NWM, true>;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* lds = reinterpret_cast<T*>(lds_raw);
     const int tiles = a.tiles_m * a.tiles_n;
     const int total = tiles * a.batch;
     f32x16_v acc[WM][WN];
+    std::conditional_t<EP, SoftmaxRuleOperands<ML, T, WM, WN, FULL>, NoOperands> ep;
     if constexpr (ML::DIRECT) {
         int t = blockIdx.x;
         BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
         typename ML::DirectLoaderA la(cur.A, cur.m0);
         typename ML::DirectLoaderB lb(cur.B, cur.n0);
+        if constexpr (EP) {
+            if (cur.store) ep.load(a, cur.coff, cur.product, cur.m0, cur.n0);
+        }
         ML::pipeline_fill(la, lb, cur.K, lds);
         for (;;) {
             ML::pipeline_loop(la, lb, cur.K, lds, acc);
@@ -315,49 +431,64 @@ __global__ __launch_bounds__(NWM * NWN * 64) void batched_gemm_kernel(DenseArgs<
             const int m0 = cur.m0, n0 = cur.n0;
             const int64_t coff = cur.coff;
             const bool store = cur.store;
-            if (tnext < total) {
+            if constexpr (EP) {
+                // the stores first: they free the registers that take the next tile's weights, whose loads go out
+                // ahead of the next tile's stages (the stage waits of the main loop count the youngest loads)
+                if (store) ep.store(acc, a, coff, m0, n0);
+                if (tnext >= total) break;
                 cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, tnext, tiles);
+                if (cur.store) ep.load(a, cur.coff, cur.product, cur.m0, cur.n0);
                 la.move_to(cur.A, cur.m0);
                 lb.move_to(cur.B, cur.n0);
                 ML::pipeline_drain();
                 ML::pipeline_fill(la, lb, cur.K, lds);
+            } else {
+                if (tnext < total) {
+                    cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, tnext, tiles);
+                    la.move_to(cur.A, cur.m0);
+                    lb.move_to(cur.B, cur.n0);
+                    ML::pipeline_drain();
+                    ML::pipeline_fill(la, lb, cur.K, lds);
+                }
+                if (store) {
+                    if (a.c_f32) store_tile_f32<ML, T, WM, WN, FULL>(acc, a, coff, m0, n0);
+                    else dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
+                }
+                if (tnext >= total) break;
             }
-            if (store) {
-                if (a.c_f32) store_tile_f32<ML, T, WM, WN, FULL>(acc, a, coff, m0, n0);
-                else dense_epilogue<ML, T, WM, WN, FULL>(acc, out, m0, n0);
-            }
-            if (tnext >= total) break;
             t = tnext;
         }
     } else {
         for (int t = blockIdx.x; t < total; t += gridDim.x) {
             const BatchTile<T> cur = batch_tile<T, ML::TILE_M, ML::TILE_N>(a, t, tiles);
             if (!cur.store) continue;          // uniform
+            if constexpr (EP) ep.load(a, cur.coff, cur.product, cur.m0, cur.n0);
             ML::run(cur.A, cur.B, cur.K, cur.m0, cur.n0, lds, acc);
             DenseArgs<T> out = a;
             out.C = cur.C;
-            if (a.c_f32) store_tile_f32<ML, T, WM, WN, FULL>(acc, a, cur.coff, cur.m0, cur.n0);
+            if constexpr (EP) ep.store(acc, a, cur.coff, cur.m0, cur.n0);
+            else if (a.c_f32) store_tile_f32<ML, T, WM, WN, FULL>(acc, a, cur.coff, cur.m0, cur.n0);
             else dense_epilogue<ML, T, WM, WN, FULL>(acc, out, cur.m0, cur.n0);
             __syncthreads();   // every wave is done with the LDS stages before the next tile refills them
         }
     }
 }
 
-template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL>
+template <typename T, int WM, int WN, bool AK, bool BKM, bool FULL, bool EP = false>
 int launch_batched_cfg(hipStream_t s, DenseArgs<T>& a) {
     using ML = GemmMainloop<T, WM, WN, AK, BKM, FULL, 2, 0, 2>;
     a.tiles_m = (int)ceil_div(a.M, ML::TILE_M);
     a.tiles_n = (int)ceil_div(a.N, ML::TILE_N);
     const int64_t total = (int64_t)a.tiles_m * a.tiles_n * a.batch;
     LUX_UNSUPPORTED_IF(total >= (1ll << 31), "batched_matmul: too many tiles");
-    auto kernel = batched_gemm_kernel<T, WM, WN, AK, BKM, FULL, 2, 2>;
+    auto kernel = batched_gemm_kernel<T, WM, WN, AK, BKM, FULL, 2, 2, EP>;
     static ResidentOnce ro;
     const int resident = ro.get([&](hipError_t& err) {
         err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ML::LDS_BYTES);
         return err == hipSuccess ? persistent_grid(kernel, ML::THREADS, ML::LDS_BYTES, int64_t(1) << 40) : 0;
     });
     LUX_CHECK_HIP(ro.error);
-    ProfScope ps(sizeof(T) == 2 ? "batched_gemm_kernel<bf16>" : "batched_gemm_kernel<f32>", s);
+    ProfScope ps(EP ? "batched_gemm_kernel+softmax_rule" : (sizeof(T) == 2 ? "batched_gemm_kernel<bf16>" : "batched_gemm_kernel<f32>"), s);
     kernel<<<dim3((unsigned)std::min<int64_t>(total, resident)), dim3(ML::THREADS), ML::LDS_BYTES, s>>>(a);
     LUX_CHECK_LAUNCH();
     return LUXHIP_OK;
@@ -367,6 +498,18 @@ template <typename T, bool AK, bool BKM>
 int launch_batched_layout(hipStream_t s, DenseArgs<T>& a) {
     // 128 x 128 tiles when a product has at least one whole tile of them, 64 x 64 otherwise;
     // the variant without bounds checks when every product is made of whole, aligned tiles
+    if (a.ep_probs != nullptr) {
+        // the product with the softmax rule as its epilogue has two K-major operands (v' and d_out)
+        if constexpr (AK && BKM) {
+            if (a.M >= 128 && a.N >= 128) {
+                if (whole_tiles<T, 128, 128>(a)) return launch_batched_cfg<T, 2, 2, AK, BKM, true, true>(s, a);
+                return launch_batched_cfg<T, 2, 2, AK, BKM, false, true>(s, a);
+            }
+            return launch_batched_cfg<T, 1, 1, AK, BKM, false, true>(s, a);
+        } else {
+            return set_error(LUXHIP_INVALID, "the softmax-rule epilogue exists for two K-major operands only");
+        }
+    }
     if (a.M >= 128 && a.N >= 128) {
         if (whole_tiles<T, 128, 128>(a)) return launch_batched_cfg<T, 2, 2, AK, BKM, true>(s, a);
         return launch_batched_cfg<T, 2, 2, AK, BKM, false>(s, a);

@@ -19,6 +19,12 @@ struct DenseArgs {
     int c_vec = 0;   // C and pre allow 8-byte stores at every (m multiple of 4, n): aligned base, ldc a multiple of 4
     int tail = 0;    // this launch finishes the rows or columns of another one (profile name "...+tail")
     int c_f32 = 0;   // batched products of bf16 operands only: C points to fp32 values (same ldc and strides, in elements)
+    // batched products only: the softmax rule as the epilogue (attention pullback).  ep_probs != null: with acc = the
+    // cotangent of the weights, C = ep_scale * probs .* (acc - ep_d[column]); probs lies as C does (same ldc and
+    // strides), ep_d holds one value per column of every product: product b's N values from ep_d + b * N on
+    const T* ep_probs = nullptr;
+    const float* ep_d = nullptr;
+    float ep_scale = 0.0f;
     // batched products: the batch index runs over up to three nested dims (bdim[0] innermost); along
     // dim d the matrices of an operand lie stride[d] elements apart (0: one matrix shared by all)
     int batch = 1;

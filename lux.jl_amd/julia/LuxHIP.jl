@@ -816,10 +816,18 @@ function attention_device(q::HIPArray{T,N}, k::HIPArray{T,N}, v::HIPArray{T,N}, 
         stream(), wide_code(T, TW), S, L, H, B, optr(logits), scale⁻¹, Cint(causal), mask === nothing ? Ptr{UInt8}(C_NULL) : Ptr{UInt8}(pointer(mask)),
         mask_sh, mask_sb, optr(bias), bias_sh, bias_sb, optr(softmaxed))) || throw(HIPFallbackError("softmax of the attention logits"))
     probs, fdrop_back = fdrop === identity ? (softmaxed, nothing) : CRC.rrule_via_ad(ZygoteLikeConfig(), fdrop, softmaxed)
-    out = similar(q, T, (Ev, H, L, bshape...))
     so = (Ev, Ev * r, Ev * H * L)
+    # bf16 without an fdrop: the product is written unrounded (fp32) and kept for the pullback, whose softmax rule takes
+    # its inner product from it; the array that is returned is its rounded copy
+    out_wide = (fdrop === identity && TW !== T) ? similar(q, TW, (Ev, H, L, bshape...)) : nothing
+    out = out_wide === nothing ? similar(q, T, (Ev, H, L, bshape...)) : out_wide
     bmm_strided!(out, false, false, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, Ev * H, so, tri ? 2 : 0)
-    saved = (; lq, lk, lv, r, bdims, sC, sq, so, scale⁻¹, tri, logits, softmaxed, probs, fdrop_back)
+    if out_wide !== nothing
+        out = similar(q, T, (Ev, H, L, bshape...))
+        check(ccall((:luxhip_convert, libluxhip), Cint, (Ptr{Cvoid}, Cint, Cint, Int64, Ptr{Cvoid}, Ptr{Cvoid}),
+            stream(), dtype_code(TW), dtype_code(T), length(out), optr(out_wide), optr(out))) || error(last_error())
+    end
+    saved = (; lq, lk, lv, r, bdims, sC, sq, so, scale⁻¹, tri, logits, softmaxed, probs, fdrop_back, out_wide)
     return out, probs, saved
 end
 # the rule configuration `fdrop`'s own pullback is taken with: whatever AD engine drives LuxLib supplies it
@@ -865,17 +873,27 @@ function CRC.rrule(::typeof(Impl.scaled_dot_product_attention), q::HIPArray{T,N}
             Δ = CRC.unthunk(Δ′)
             Δout = CRC.unthunk(Δ[1])
             Δ[2] isa CRC.AbstractZero || throw(HIPFallbackError("a cotangent for the returned attention weights"))
-            # the cotangent of the weights in fp32 too, unless it has to pass through fdrop's pullback first
-            TD = s.fdrop_back === nothing ? wide_type(T) : T
-            dp = similar(probs, TD)
-            bmm_strided!(dp, true, false, S, L, Ev, bdims, vc, lv.st, (0, lv.sh, lv.sb), Δout, Ev * H, so, S, sC, tri ? 1 : 0)
-            s.fdrop_back === nothing || (dp = CRC.unthunk(s.fdrop_back(dp)[2]))
             dlogits = eltype(s.logits) === T ? s.logits : similar(probs)   # the logits are no longer needed
-            # tri, not is_causal: with an fdrop the products below run in full and read the whole cotangent
-            check(ccall((:luxhip_attention_softmax_bwd, libluxhip), Cint,
-                (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}),
-                stream(), wide_code(T, eltype(dp)), S, L, L * H * lq.batch, Cint(tri), optr(dp), optr(s.softmaxed), s.scale⁻¹, optr(dlogits))) ||
-                error(last_error())
+            if s.fdrop_back === nothing
+                # the cotangent of the weights (v' Δout) and the softmax rule in one call: the cotangent stays in the
+                # product's fp32 accumulators, its inner product with the weights comes from Δout and out
+                check(ccall((:luxhip_attention_weights_pullback, libluxhip), Cint,
+                    (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Ptr{Int64}, Ptr{Cvoid}, Int64, Ptr{Int64}, Ptr{Cvoid}, Ptr{Cvoid}, Int64,
+                        Ptr{Int64}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}, Int64, Ptr{Int64}, Cint),
+                    stream(), s.out_wide === nothing ? dtype_code(T) : BF16_WIDE, S, L, Ev, i64x3(bdims), optr(vc), max(1, lv.st),
+                    i64x3((0, lv.sh, lv.sb)), optr(Δout), optr(something(s.out_wide, out)), max(1, Ev * H), i64x3(so), optr(s.softmaxed),
+                    s.scale⁻¹, optr(dlogits), max(1, S), i64x3(sC),
+                    Cint(tri ? 1 : 0))) || error(last_error())
+            else
+                dp = similar(probs)
+                bmm_strided!(dp, true, false, S, L, Ev, bdims, vc, lv.st, (0, lv.sh, lv.sb), Δout, Ev * H, so, S, sC, tri ? 1 : 0)
+                dp = CRC.unthunk(s.fdrop_back(dp)[2])
+                # tri, not is_causal: with an fdrop the products below run in full and read the whole cotangent
+                check(ccall((:luxhip_attention_softmax_bwd, libluxhip), Cint,
+                    (Ptr{Cvoid}, Cint, Int64, Int64, Int64, Cint, Ptr{Cvoid}, Ptr{Cvoid}, Cdouble, Ptr{Cvoid}),
+                    stream(), dtype_code(T), S, L, L * H * lq.batch, Cint(tri), optr(dp), optr(s.softmaxed), s.scale⁻¹, optr(dlogits))) ||
+                    error(last_error())
+            end
             ∂q = similar(qc)
             bmm_strided!(∂q, false, false, E, L, S, bdims, kc, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, lq.st, sq, tri ? 2 : 0)
             function kv_grad(like, lay, A, lda, sA, Bm)

@@ -751,26 +751,36 @@ def rrule_scaled_dot_product_attention(q, k, v, head_dim=1, token_dim=3, scale=N
     softmax_out, fdrop_back = probs, None
     if fdrop is not None:
         probs, fdrop_back = fdrop(softmax_out)         # impl/attention.jl:88-104: fdrop(softmax(...))
-    out = DeviceArray((Ev, H, L) + bshape, dt)
     so = (Ev, Ev * r, Ev * H * L)
+    # bf16 without an fdrop: the product is written unrounded (fp32) and kept for the pullback, whose softmax rule takes
+    # its inner product from it; the array that is returned is its rounded copy
+    out_wide = DeviceArray((Ev, H, L) + bshape, wide) if (fdrop is None and wide != dt) else None
+    out = out_wide if out_wide is not None else DeviceArray((Ev, H, L) + bshape, dt)
     _bmm_strided(False, False, Ev, L, S, bdims, v, lv.st, (0, lv.sh, lv.sb), probs, S, sC, out, Ev * H, so, 2 if tri else 0)
+    if out_wide is not None:
+        out = _convert(out_wide, dt)
 
     def back(d_out: DeviceArray, d_probs: Optional[DeviceArray] = None):
-        # with an fdrop the cotangent passes through its pullback in the storage type first
-        dp_wide = wide if fdrop_back is None else dt
-        dp = DeviceArray(probs.shape, dp_wide)
-        _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC, 1 if tri else 0)
         if d_probs is not None:
             raise _lib.Unsupported(_lib.UNSUPPORTED, "attention: a cotangent for the returned weights")
-        if fdrop_back is not None:
-            dp = fdrop_back(dp)
         dlogits = logits if logits.dtype == dt else DeviceArray(logits.shape, dt)   # the logits are no longer needed
-        # the causal shortcut of the softmax pullback leaves dlogits beyond the diagonal block untouched, which
-        # only the triangular products that follow tolerate: with an fdrop those run in full, so the whole
-        # column is computed (masked weights are zero, hence so is their dlogits)
-        _lib.call("luxhip_attention_softmax_bwd", current_stream(),
-                  _BF16_WIDE if (dt == "bf16" and dp.dtype == "f32") else softmax_out.code, S, L, L * H * B, int(tri), dp.ptr,
-                  softmax_out.ptr, scale_inv, dlogits.ptr)
+        if fdrop_back is None:
+            # the cotangent of the weights (v' d_out) and the softmax rule in one: the cotangent stays in the product's
+            # fp32 accumulators, its inner product with the weights comes from d_out and out
+            _lib.call("luxhip_attention_weights_pullback", current_stream(), softmax_out.code if out_wide is None else _BF16_WIDE, S, L,
+                      Ev, _i64x3(bdims), v.ptr, max(lv.st, 1), _i64x3((0, lv.sh, lv.sb)), d_out.ptr,
+                      (out if out_wide is None else out_wide).ptr, max(Ev * H, 1), _i64x3(so), softmax_out.ptr,
+                      scale_inv, dlogits.ptr, max(S, 1), _i64x3(sC), 1 if tri else 0)
+        else:
+            # with an fdrop the cotangent passes through its pullback in the storage type first
+            dp = DeviceArray(probs.shape, dt)
+            _bmm_strided(True, False, S, L, Ev, bdims, v, lv.st, (0, lv.sh, lv.sb), d_out, Ev * H, so, dp, S, sC, 1 if tri else 0)
+            dp = fdrop_back(dp)
+            # the causal shortcut of the softmax pullback leaves dlogits beyond the diagonal block untouched, which
+            # only the triangular products that follow tolerate: with an fdrop those run in full, so the whole
+            # column is computed (masked weights are zero, hence so is their dlogits)
+            _lib.call("luxhip_attention_softmax_bwd", current_stream(), softmax_out.code, S, L, L * H * B, int(tri), dp.ptr,
+                      softmax_out.ptr, scale_inv, dlogits.ptr)
         dq = DeviceArray(q.shape, dt)
         _bmm_strided(False, False, E, L, S, bdims, k, lk.st, (0, lk.sh, lk.sb), dlogits, S, sC, dq, lq.st,
                      (lq.sh, lq.sh * r, lq.sb), 2 if tri else 0)
