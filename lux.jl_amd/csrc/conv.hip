@@ -3,6 +3,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "act_vec.h"
 #include "conv_kernels.h"
 #include "conv_patch.h"
 #include "conv_wgrad_patch.h"
@@ -126,6 +127,99 @@ __global__ __launch_bounds__(256) void whcn_to_cwhn_pack_kernel(const T* __restr
     }
 }
 
+// First pass of the fused pullback (bf16; P and C multiples of 8, 16-byte aligned pointers): one pass over delta
+// writes dz = delta .* act'(y, pre) as it lies (p contiguous: what the window and the direct filter-gradient kernels
+// read), its channel-contiguous copy dzT (what the input-gradient kernels read) and the bias gradient's partial sums,
+// where a pass for dz and the bias gradient followed by a transposing copy reads dz once more.  A workgroup walks
+// `chunk` tiles of 64 positions x 64 channels of one image; a tile goes through LDS as fp32 (rows of 65 words: the
+// 64 lanes of a wave hit 64 banks in both phases).  Phase 1: 16-byte vectors along p, dz stored, per-channel sums
+// kept in registers; phase 2: eight channels of one position per thread, 16 bytes of dzT.  The eight threads of a
+// channel add their sums in a fixed order; partial[(n * gridDim.x + blockIdx.x) * C + c].  The z slices behind
+// the N images repack the filter for the input-gradient kernel (as in whcn_to_cwhn_pack_kernel).
+template <int ACT>
+__global__ __launch_bounds__(256) void conv_dz_cwhn_pack_kernel(const bf16_t* __restrict__ delta, const bf16_t* __restrict__ y,
+                                                                const bf16_t* __restrict__ pre, bf16_t* dz, bf16_t* __restrict__ dzT,
+                                                                float* __restrict__ partial, int P, int C, int N, int chunk,
+                                                                const bf16_t* __restrict__ w, bf16_t* __restrict__ wout, ConvGeom g) {
+    if ((int)blockIdx.z >= N) {
+        const int block = ((int)(blockIdx.z - N) * (int)gridDim.y + (int)blockIdx.y) * (int)gridDim.x + (int)blockIdx.x;
+        pack_filter_element<bf16_t>(w, wout, g, 1, block * 256 + (int)threadIdx.x);
+        return;
+    }
+    constexpr int PITCH = 65;
+    __shared__ float tile[64 * PITCH];
+    const int n = blockIdx.z, c0 = blockIdx.y * 64;
+    const size_t image = (size_t)n * C * P;
+    float bsum[2] = {0.0f, 0.0f};
+    const int tiles_p = (P + 63) / 64;
+    const int t_end = min(tiles_p, ((int)blockIdx.x + 1) * chunk);
+    for (int tp = blockIdx.x * chunk; tp < t_end; ++tp) {
+        const int p0 = tp * 64;
+        float r[2][8];
+        bool ok[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {                 // loads first, then the stores
+            const int idx = threadIdx.x + it * 256, cl = idx >> 3, pv = idx & 7;
+            ok[it] = c0 + cl < C && p0 + pv * 8 < P;
+            if (ok[it]) {
+                dx_vec<bf16_t, ACT, 8>(delta, y, pre, image + (size_t)(c0 + cl) * P + p0 + pv * 8, r[it]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) r[it][k] = 0.0f;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int idx = threadIdx.x + it * 256, cl = idx >> 3, pv = idx & 7;
+            if (ok[it] && dz != nullptr) store_vec<bf16_t, 8>(dz, image + (size_t)(c0 + cl) * P + p0 + pv * 8, r[it]);
+            float t = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                tile[cl * PITCH + pv * 8 + k] = r[it][k];
+                t += r[it][k];
+            }
+            bsum[it] += t;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int idx = threadIdx.x + it * 256, pl = idx >> 3, cv = idx & 7;
+            if (p0 + pl < P && c0 + cv * 8 < C) {
+                float v[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) v[k] = tile[(cv * 8 + k) * PITCH + pl];
+                store_vec<bf16_t, 8>(dzT, image + (size_t)(p0 + pl) * C + c0 + cv * 8, v);
+            }
+        }
+        __syncthreads();
+    }
+    if (partial != nullptr) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int idx = threadIdx.x + it * 256, cl = idx >> 3, pv = idx & 7;
+            // the eight threads of a channel are neighbouring lanes: (((s0 + s1) + (s2 + s3)) + ((s4 + s5) + (s6 + s7)))
+            float t = bsum[it];
+            t += __shfl_xor(t, 1);
+            t += __shfl_xor(t, 2);
+            t += __shfl_xor(t, 4);
+            if (pv == 0 && c0 + cl < C) partial[((size_t)n * gridDim.x + blockIdx.x) * C + c0 + cl] = t;
+        }
+    }
+}
+
+// dbias[c] = sum over slices of partial[slice][c]: one workgroup per channel, thread t adds slices t, t + 256, ...;
+// the threads' sums are added in a fixed order (within a wave, then the four waves in turn).
+__global__ __launch_bounds__(256) void conv_dbias_finalize_kernel(const float* __restrict__ partial, bf16_t* dbias, int C, int S) {
+    __shared__ float sw[4];
+    const int c = blockIdx.x;
+    float t = 0.0f;
+    for (int sl = threadIdx.x; sl < S; sl += 256) t += partial[(size_t)sl * C + c];
+    t = wave_sum(t);
+    if ((threadIdx.x & 63) == 0) sw[threadIdx.x >> 6] = t;
+    __syncthreads();
+    if (threadIdx.x == 0) st(dbias + c, ((sw[0] + sw[1]) + sw[2]) + sw[3]);
+}
+
 // dw[a, b, ci, g*Cout_g + col] = sum over slices of partial[slice][m' = t*Cin_g + ci][col].
 // A thread owns 4 consecutive m' (one 16-byte load per slice, eight slices in flight); slices are
 // added in order.
@@ -239,6 +333,47 @@ static int transpose_and_pack(hipStream_t s, const T* in, T* out, int P, int C, 
     ProfScope ps("whcn_to_cwhn_kernel", s);
     whcn_to_cwhn_pack_kernel<T><<<dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), 256, 0, s>>>(in, out, P, C, N, w, wout, g, for_dgrad);
     LUX_CHECK_LAUNCH();
+    return LUXHIP_OK;
+}
+
+// Tiles of 64 positions that one workgroup of conv_dz_cwhn_pack_kernel walks: as many as leave about four workgroups
+// per compute unit, eight at most (each workgroup contributes one slice of partial sums per channel)
+static int dz_cwhn_chunk(int P, int C, int N) {
+    const int64_t tiles = ceil_div(P, 64) * ceil_div(C, 64) * N;
+    return (int)std::min<int64_t>(8, std::max<int64_t>(1, tiles / (4 * (int64_t)std::max(1, num_cus()))));
+}
+static size_t dz_cwhn_partial_bytes(int P, int C, int N) {
+    const int64_t groups = ceil_div(ceil_div(P, 64), dz_cwhn_chunk(P, C, N));
+    return align256((size_t)groups * N * C * sizeof(float));
+}
+static bool dz_cwhn_ok(int P, int C, int N, const void* delta, const void* y, const void* pre, const void* dz, const void* dzT) {
+    return P % 8 == 0 && C % 8 == 0 && N >= 1 && aligned16(delta) && aligned16(y) && aligned16(pre) && aligned16(dz) && aligned16(dzT) &&
+           ceil_div(C, 64) <= 65535 && N + 4096 <= 65535;
+}
+// dz (may be NULL for the identity: dz is delta), dzT, the bias gradient (if dbias != NULL) and, if wout != NULL, the filter
+// repacked for the input-gradient kernel
+static int conv_dz_cwhn_pack(hipStream_t s, int act, const ConvGeom& g, const bf16_t* delta, const bf16_t* y, const bf16_t* pre,
+                             bf16_t* dz, bf16_t* dzT, float* partial, bf16_t* dbias, const bf16_t* w, bf16_t* wout) {
+    const int P = g.OW * g.OH, C = g.Cout, N = g.N;
+    const int chunk = dz_cwhn_chunk(P, C, N);
+    const int64_t gx = ceil_div(ceil_div(P, 64), chunk), gy = ceil_div(C, 64);
+    const int64_t pack_blocks = wout != nullptr ? ceil_div((int64_t)g.kW * g.kH * g.Cin_g * g.Cout, 256) : 0;
+    const int64_t gz = N + ceil_div(pack_blocks, gx * gy);
+    LUX_UNSUPPORTED_IF(gz > 65535, "conv: filter too large for the combined layout pass");
+    float* const part = dbias != nullptr ? partial : nullptr;
+    const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)gz);
+#define LAUNCH_DZC(A) conv_dz_cwhn_pack_kernel<A><<<grid, 256, 0, s>>>(delta, y, pre, dz, dzT, part, P, C, N, chunk, w, wout, g)
+    {
+        ProfScope ps("conv_dz_cwhn_pack_kernel", s);
+        LUX_DISPATCH_ACT(act, LAUNCH_DZC);
+    }
+#undef LAUNCH_DZC
+    LUX_CHECK_LAUNCH();
+    if (dbias != nullptr) {
+        ProfScope ps2("conv_dbias_finalize_kernel", s);
+        conv_dbias_finalize_kernel<<<(unsigned)C, 256, 0, s>>>(partial, dbias, C, (int)(gx * N));
+        LUX_CHECK_LAUNCH();
+    }
     return LUXHIP_OK;
 }
 
@@ -504,26 +639,45 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
     const size_t yb = align256((size_t)g.OW * g.OH * g.Cout * g.N * sizeof(T));
     const size_t wb = align256((size_t)g.kW * g.kH * g.Cin_g * g.Cout * sizeof(T));
     const size_t pb = wgrad_partial_bytes<T>(g);
+    // bf16: dz, its channel-contiguous copy and the bias gradient in one pass, when both a pass over delta and a
+    // transposing copy would run
+    bool one_pass = false;
+    if constexpr (sizeof(T) == 2)
+        one_pass = (act != LUXHIP_ACT_IDENTITY || dbias != nullptr) && (dw != nullptr || dx != nullptr) &&
+                   dz_cwhn_ok(g.OW * g.OH, g.Cout, g.N, delta, y, pre, dz, nullptr);
+    const size_t bb = one_pass && dbias != nullptr ? dz_cwhn_partial_bytes(g.OW * g.OH, g.Cout, g.N) : 0;
     // reserve everything up front: the bias-gradient pass below uses the start of the same
     // workspace, and the buffer must not be reallocated while pointers into it are live
     Workspace ws;
-    int rc = get_workspace(s, xb + yb + wb + pb, &ws);
+    int rc = get_workspace(s, xb + yb + wb + pb + bb, &ws);
     if (rc != LUXHIP_OK) return rc;
-    const T* dzp = delta;
-    if (act != LUXHIP_ACT_IDENTITY || dbias != nullptr) {
-        T* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : dz;
-        rc = bias_act_bwd_dispatch(s, dtype, act, (int64_t)g.OW * g.OH, g.Cout, g.N, delta, y, pre, dz_out, dbias);
-        if (rc != LUXHIP_OK) return rc;
-        if (dz_out) dzp = dz_out;
-    }
-    if (dw == nullptr && dx == nullptr) return LUXHIP_OK;
     const T* xT = xt_kept ? xt_kept : reinterpret_cast<const T*>(ws.data);
     T* dzT = reinterpret_cast<T*>(ws.data + xb);
     T* wD = reinterpret_cast<T*>(ws.data + xb + yb);
     float* partial = reinterpret_cast<float*>(ws.data + xb + yb + wb);
-    if (dx != nullptr) rc = transpose_and_pack<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N, w, wD, g, 1);
-    else rc = transpose_to_cwhn<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N);
-    if (rc != LUXHIP_OK) return rc;
+    const T* dzp = delta;
+    if (one_pass) {
+        if constexpr (sizeof(T) == 2) {
+            bf16_t* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : reinterpret_cast<bf16_t*>(dz);
+            rc = conv_dz_cwhn_pack(s, act, g, reinterpret_cast<const bf16_t*>(delta), reinterpret_cast<const bf16_t*>(y),
+                                   reinterpret_cast<const bf16_t*>(pre), dz_out, reinterpret_cast<bf16_t*>(dzT),
+                                   reinterpret_cast<float*>(ws.data + xb + yb + wb + pb), reinterpret_cast<bf16_t*>(dbias),
+                                   reinterpret_cast<const bf16_t*>(w), dx != nullptr ? reinterpret_cast<bf16_t*>(wD) : nullptr);
+            if (rc != LUXHIP_OK) return rc;
+            if (dz_out) dzp = dz;
+        }
+    } else {
+        if (act != LUXHIP_ACT_IDENTITY || dbias != nullptr) {
+            T* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : dz;
+            rc = bias_act_bwd_dispatch(s, dtype, act, (int64_t)g.OW * g.OH, g.Cout, g.N, delta, y, pre, dz_out, dbias);
+            if (rc != LUXHIP_OK) return rc;
+            if (dz_out) dzp = dz_out;
+        }
+        if (dw == nullptr && dx == nullptr) return LUXHIP_OK;
+        if (dx != nullptr) rc = transpose_and_pack<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N, w, wD, g, 1);
+        else rc = transpose_to_cwhn<T>(s, dzp, dzT, g.OW * g.OH, g.Cout, g.N);
+        if (rc != LUXHIP_OK) return rc;
+    }
     if (dx != nullptr) {
         if ((rc = run_conv_gemm<T>(s, g, true, dzT, wD, nullptr, dx, nullptr, LUXHIP_ACT_IDENTITY, ws.zeros)) != LUXHIP_OK) return rc;
     }
