@@ -642,9 +642,9 @@ static int bn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         uint64_t* words = reinterpret_cast<uint64_t*>(ws.flags);
         const uint32_t spin = (uint32_t)option_bn_spin_limit();
         dim3 grid((unsigned)S, (unsigned)C);
-#define LAUNCH_RES(A) bn_fwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(x, y, words, ws.epoch, spin, prm, g)
+#define LAUNCH_RES(A) launch_exact(ps, bn_fwd_resident_kernel<T, A>, dim3(grid), dim3(kResThreads), 0, s, x, y, words, ws.epoch, spin, prm, g)
         {
-            ProfScope ps("bn_fwd_resident_kernel", s);
+            ProfScope ps("bn_fwd_resident_kernel", s, true);
             LUX_DISPATCH_ACT(act, LAUNCH_RES);
         }
 #undef LAUNCH_RES
@@ -718,10 +718,10 @@ static int bn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t N, 
         const uint32_t spin = (uint32_t)option_bn_spin_limit();
         dim3 grid((unsigned)S, (unsigned)C);
 #define LAUNCH_RES(A)                                                                                               \
-    bn_bwd_resident_kernel<T, A><<<grid, kResThreads, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, \
+    launch_exact(ps, bn_bwd_resident_kernel<T, A>, dim3(grid), dim3(kResThreads), 0, s, delta, x, gamma, beta, save_mean, save_invstd, dx, dgamma, dbeta, \
                                                               words, ws.epoch, spin, inv_count, stats_from_batch, g)
         {
-            ProfScope ps("bn_bwd_resident_kernel", s);
+            ProfScope ps("bn_bwd_resident_kernel", s, true);
             LUX_DISPATCH_ACT(act, LAUNCH_RES);
         }
 #undef LAUNCH_RES

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <mutex>
@@ -72,9 +73,22 @@ struct ProfScope {
     const char* name;
     hipStream_t stream;
     bool active;
-    ProfScope(const char* n, hipStream_t s);
+    // exact scopes (one launch through launch_exact): two events that the dispatch itself signals at its begin
+    // and at its end, so the time is the kernel's alone, without the gap between dependent launches; null while
+    // the profile is off
+    hipEvent_t start = nullptr, stop = nullptr;
+    ProfScope(const char* n, hipStream_t s, bool exact = false);
     ~ProfScope();
 };
+
+// kernel<<<grid, block, lds, s>>>(args...) of an exact scope
+template <typename... KArgs, typename... Args>
+inline void launch_exact(const ProfScope& ps, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s, Args&&... args) {
+    if (ps.start != nullptr)
+        hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, s, ps.start, ps.stop, 0, static_cast<KArgs>(args)...);
+    else
+        kernel<<<grid, block, lds, s>>>(static_cast<KArgs>(args)...);
+}
 
 #define LUX_CHECK_HIP(expr)                                                                     \
     do {                                                                                        \

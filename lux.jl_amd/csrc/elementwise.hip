@@ -324,13 +324,13 @@ static int bias_act_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
             const uint32_t tv = (uint32_t)(total / V);                                                             \
             const FastDiv rowdiv((uint32_t)(I / V));                                                               \
             if (bias && pre)                                                                                       \
-                bias_act_fwd_kernel<T, A, V, true, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, V, true, true>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
             else if (bias)                                                                                         \
-                bias_act_fwd_kernel<T, A, V, true, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, V, true, false>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
             else if (pre)                                                                                          \
-                bias_act_fwd_kernel<T, A, V, false, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, V, false, true>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
             else                                                                                                   \
-                bias_act_fwd_kernel<T, A, V, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, V, false, false>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
         } else if (ptr_ok && bias && total % V == 0) {                                                             \
             const uint32_t tv = (uint32_t)(total / V);                                                             \
             const FastDiv idiv((uint32_t)I);                                                                       \
@@ -341,24 +341,24 @@ static int bias_act_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
         } else if (ptr_ok && !bias && total % V == 0) {                                                            \
             const uint32_t tv = (uint32_t)(total / V);                                                             \
             if (pre)                                                                                               \
-                bias_act_fwd_kernel<T, A, V, false, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, cdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, V, false, true>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, cdiv, cdiv, (uint32_t)C); \
             else                                                                                                   \
-                bias_act_fwd_kernel<T, A, V, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, cdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, V, false, false>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, cdiv, cdiv, (uint32_t)C); \
         } else {                                                                                                   \
             const uint32_t tv = (uint32_t)total;                                                                   \
             const FastDiv rowdiv((uint32_t)I);                                                                     \
             if (bias && pre)                                                                                       \
-                bias_act_fwd_kernel<T, A, 1, true, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, 1, true, true>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
             else if (bias)                                                                                         \
-                bias_act_fwd_kernel<T, A, 1, true, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, 1, true, false>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
             else if (pre)                                                                                          \
-                bias_act_fwd_kernel<T, A, 1, false, true><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, 1, false, true>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
             else                                                                                                   \
-                bias_act_fwd_kernel<T, A, 1, false, false><<<grid_for(tv), kThreads, 0, s>>>(x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
+                launch_exact(ps, bias_act_fwd_kernel<T, A, 1, false, false>, dim3(grid_for(tv)), dim3(kThreads), 0, s, x, bias, y, pre, tv, rowdiv, cdiv, (uint32_t)C); \
         }                                                                                                          \
     } while (0)
     {
-        ProfScope ps("bias_act_fwd_kernel", s);
+        ProfScope ps("bias_act_fwd_kernel", s, true);
         LUX_DISPATCH_ACT(act, LAUNCH_FWD);
     }
 #undef LAUNCH_FWD
@@ -436,12 +436,12 @@ static int bias_act_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64
 #define LAUNCH_CH(A)                                                                                               \
     do {                                                                                                           \
         if (vec)                                                                                                   \
-            bias_act_bwd_channel_kernel<T, A, V><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, counters, counter_stride(C), nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+            launch_exact(ps, bias_act_bwd_channel_kernel<T, A, V>, dim3(grid), dim3(kThreads), 0, s, delta, out, pre, dx, dbias, partial, counters, counter_stride(C), nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
         else                                                                                                       \
-            bias_act_bwd_channel_kernel<T, A, 1><<<grid, kThreads, 0, s>>>(delta, out, pre, dx, dbias, partial, counters, counter_stride(C), nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
+            launch_exact(ps, bias_act_bwd_channel_kernel<T, A, 1>, dim3(grid), dim3(kThreads), 0, s, delta, out, pre, dx, dbias, partial, counters, counter_stride(C), nq, chunk, rowdiv, (uint32_t)(I / vv), (uint32_t)C); \
     } while (0)
         {
-            ProfScope ps("bias_act_bwd_channel_kernel", s);
+            ProfScope ps("bias_act_bwd_channel_kernel", s, true);
             LUX_DISPATCH_ACT(act, LAUNCH_CH);
         }
 #undef LAUNCH_CH

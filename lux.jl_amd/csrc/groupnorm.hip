@@ -588,13 +588,13 @@ static int gn_fwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
         rs.cstride = counter_stride(C);
         rs.N = (uint32_t)N;
     }
-    ProfScope ps("gn_fwd_kernel", s);
+    ProfScope ps("gn_fwd_kernel", s, true);
 #define GN_FWD(A)                                                                                                     \
     do {                                                                                                              \
-        if (L.vec && L.cached) gn_fwd_kernel<T, A, V, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);   \
-        else if (L.vec) gn_fwd_kernel<T, A, V, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);        \
-        else if (L.cached) gn_fwd_kernel<T, A, 1, true><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);      \
-        else gn_fwd_kernel<T, A, 1, false><<<L.blocks, L.threads, 0, s>>>(x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);                   \
+        if (L.vec && L.cached) launch_exact(ps, gn_fwd_kernel<T, A, V, true>, dim3(L.blocks), dim3(L.threads), 0, s, x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);   \
+        else if (L.vec) launch_exact(ps, gn_fwd_kernel<T, A, V, false>, dim3(L.blocks), dim3(L.threads), 0, s, x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);        \
+        else if (L.cached) launch_exact(ps, gn_fwd_kernel<T, A, 1, true>, dim3(L.blocks), dim3(L.threads), 0, s, x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);      \
+        else launch_exact(ps, gn_fwd_kernel<T, A, 1, false>, dim3(L.blocks), dim3(L.threads), 0, s, x, gamma, beta, y, save_mean, save_invstd, L.g, eps, rs);                   \
     } while (0)
     LUX_DISPATCH_ACT(act, GN_FWD);
 #undef GN_FWD
@@ -642,11 +642,11 @@ static int gn_bwd_impl(hipStream_t s, int act, int64_t I, int64_t C, int64_t G, 
         counters = ws.counters;
     }
     {
-        ProfScope ps("gn_bwd_kernel", s);
+        ProfScope ps("gn_bwd_kernel", s, true);
 #define GN_BWD_A(A, VV, CA)                                                                                           \
     do {                                                                                                              \
-        if (affine) gn_bwd_kernel<T, A, VV, CA, true><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g, ex); \
-        else gn_bwd_kernel<T, A, VV, CA, false><<<L.blocks, L.threads, lds_bytes, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g, ex);       \
+        if (affine) launch_exact(ps, gn_bwd_kernel<T, A, VV, CA, true>, dim3(L.blocks), dim3(L.threads), lds_bytes, s, delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g, ex); \
+        else launch_exact(ps, gn_bwd_kernel<T, A, VV, CA, false>, dim3(L.blocks), dim3(L.threads), lds_bytes, s, delta, x, gamma, beta, save_mean, save_invstd, dx, pdg, pdb, dgamma, dbeta, counters, cstride, (uint32_t)N, L.g, ex);       \
     } while (0)
 #define GN_BWD(A)                                                                                                     \
     do {                                                                                                              \

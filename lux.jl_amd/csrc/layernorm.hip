@@ -498,12 +498,12 @@ static int ln_check(int dtype, int act, int64_t L, int64_t R) {
 
 #define LN_VARIANTS(KERNEL, A, ...)                                                                     \
     do {                                                                                                \
-        if (p.vec && p.wave) KERNEL<T, A, V, true, true><<<p.blocks, p.threads, 0, s>>>(__VA_ARGS__);   \
-        else if (p.vec && p.cached) KERNEL<T, A, V, false, true><<<p.blocks, p.threads, 0, s>>>(__VA_ARGS__);  \
-        else if (p.vec) KERNEL<T, A, V, false, false><<<p.blocks, p.threads, 0, s>>>(__VA_ARGS__);      \
-        else if (p.wave) KERNEL<T, A, 1, true, true><<<p.blocks, p.threads, 0, s>>>(__VA_ARGS__);       \
-        else if (p.cached) KERNEL<T, A, 1, false, true><<<p.blocks, p.threads, 0, s>>>(__VA_ARGS__);    \
-        else KERNEL<T, A, 1, false, false><<<p.blocks, p.threads, 0, s>>>(__VA_ARGS__);                 \
+        if (p.vec && p.wave) launch_exact(ps, KERNEL<T, A, V, true, true>, dim3(p.blocks), dim3(p.threads), 0, s, __VA_ARGS__);   \
+        else if (p.vec && p.cached) launch_exact(ps, KERNEL<T, A, V, false, true>, dim3(p.blocks), dim3(p.threads), 0, s, __VA_ARGS__);  \
+        else if (p.vec) launch_exact(ps, KERNEL<T, A, V, false, false>, dim3(p.blocks), dim3(p.threads), 0, s, __VA_ARGS__);      \
+        else if (p.wave) launch_exact(ps, KERNEL<T, A, 1, true, true>, dim3(p.blocks), dim3(p.threads), 0, s, __VA_ARGS__);       \
+        else if (p.cached) launch_exact(ps, KERNEL<T, A, 1, false, true>, dim3(p.blocks), dim3(p.threads), 0, s, __VA_ARGS__);    \
+        else launch_exact(ps, KERNEL<T, A, 1, false, false>, dim3(p.blocks), dim3(p.threads), 0, s, __VA_ARGS__);                 \
     } while (0)
 
 template <typename T>
@@ -513,7 +513,7 @@ static int ln_fwd_impl(hipStream_t s, int act, int64_t L, int64_t R, const T* x,
     const bool ptr_ok = aligned16(x) && aligned16(y) && (gamma == nullptr || (aligned16(gamma) && aligned16(beta)));
     LnPlan p = ln_plan<T>(L, R, ptr_ok);
     const float inv_L = 1.0f / (float)L;
-    ProfScope ps("ln_fwd_kernel", s);
+    ProfScope ps("ln_fwd_kernel", s, true);
 #define LN_FWD(A) LN_VARIANTS(ln_fwd_kernel, A, x, gamma, beta, y, save_mean, save_invstd, p.nvec, (uint32_t)R, inv_L, eps)
     LUX_DISPATCH_ACT(act, LN_FWD);
 #undef LN_FWD
@@ -538,8 +538,8 @@ static int ln_bwd_impl(hipStream_t s, int act, int64_t L, int64_t R, const T* de
         float* pg = reinterpret_cast<float*>(ws.data);
         float* pb = pg + (size_t)blocks * L;
         {
-            ProfScope ps("ln_bwd_fused_kernel", s);
-#define LN_FUSED(A) ln_bwd_fused_kernel<T, A, V><<<(unsigned)blocks, 256, 0, s>>>(delta, x, gamma, beta, save_mean, save_invstd, dx, pg, pb, p.nvec, (uint32_t)R, inv_L)
+            ProfScope ps("ln_bwd_fused_kernel", s, true);
+#define LN_FUSED(A) launch_exact(ps, ln_bwd_fused_kernel<T, A, V>, dim3((unsigned)blocks), dim3(256), 0, s, delta, x, gamma, beta, save_mean, save_invstd, dx, pg, pb, p.nvec, (uint32_t)R, inv_L)
             LUX_DISPATCH_ACT(act, LN_FUSED);
 #undef LN_FUSED
         }
@@ -550,7 +550,7 @@ static int ln_bwd_impl(hipStream_t s, int act, int64_t L, int64_t R, const T* de
         return LUXHIP_OK;
     }
     {
-        ProfScope ps("ln_bwd_dx_kernel", s);
+        ProfScope ps("ln_bwd_dx_kernel", s, true);
 #define LN_BWD(A) LN_VARIANTS(ln_bwd_dx_kernel, A, delta, x, gamma, beta, save_mean, save_invstd, dx, p.nvec, (uint32_t)R, inv_L)
         LUX_DISPATCH_ACT(act, LN_BWD);
 #undef LN_BWD

@@ -49,7 +49,9 @@ std::vector<void*> g_pinned;        // pinned blocks of destroyed streams (a gra
 
 // One event is recorded after every profiled launch; a launch that directly follows another
 // profiled launch on the same stream takes that event as its start, so a launch costs one event
-// record and its time runs from the end of its predecessor to its own end.
+// record and its time runs from the end of its predecessor to its own end (the kernel plus the gap
+// between dependent launches).  Exact scopes hand two events to the dispatch itself instead
+// (hipExtLaunchKernelGGL): the time between them is the kernel's alone, what a kernel trace reports.
 struct ProfEntry {
     const char* name;
     hipStream_t stream;
@@ -73,9 +75,20 @@ static int prof_record(hipStream_t s) {   // g_mu held
     g_prof_events.push_back(e);
     return (int)g_prof_events.size() - 1;
 }
-ProfScope::ProfScope(const char* n, hipStream_t s) : name(n), stream(s), active(g_prof) {
+ProfScope::ProfScope(const char* n, hipStream_t s, bool exact) : name(n), stream(s), active(g_prof) {
     if (!active) return;
     std::lock_guard<std::mutex> lk(g_mu);
+    if (exact) {
+        hipEvent_t a = nullptr, b = nullptr;
+        if (hipEventCreate(&a) != hipSuccess) { active = false; return; }
+        if (hipEventCreate(&b) != hipSuccess) { (void)hipEventDestroy(a); active = false; return; }
+        g_prof_events.push_back(a);
+        g_prof_events.push_back(b);
+        g_prof_entries.push_back(ProfEntry{n, s, (int)g_prof_events.size() - 2, (int)g_prof_events.size() - 1});
+        start = a;
+        stop = b;
+        return;
+    }
     int a = -1;
     if (!g_prof_entries.empty() && g_prof_entries.back().stream == s && g_prof_entries.back().b >= 0)
         a = g_prof_entries.back().b;
@@ -85,7 +98,7 @@ ProfScope::ProfScope(const char* n, hipStream_t s) : name(n), stream(s), active(
     g_prof_entries.push_back(ProfEntry{n, s, a, -1});
 }
 ProfScope::~ProfScope() {
-    if (!active) return;
+    if (!active || start != nullptr) return;
     std::lock_guard<std::mutex> lk(g_mu);
     // the matching entry is the last one with this name still open
     for (auto it = g_prof_entries.rbegin(); it != g_prof_entries.rend(); ++it)
