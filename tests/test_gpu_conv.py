@@ -328,3 +328,48 @@ def test_window_kernels_random_shapes(gpu, case):
     for tile in (1, 2, 0):
         assert_close(out[tile][0], f64(out[84][0]), "bf16", tag + f"y, conv_tile {tile}")
         assert_close(out[tile][1], f64(out[84][1]), "bf16", tag + f"dgrad, conv_tile {tile}")
+
+
+# Shapes of the bf16 pullback's single pass over delta (dz as it lies, its channel-contiguous copy, the bias gradient's
+# partial sums, the repacked filter): positions and channels in multiples of 8.  Chosen for its special cases.
+ONE_PASS_CASES = [
+    # x shape, w shape, stride, pad, groups
+    ((24, 20, 16, 3), (3, 3, 16, 72), 1, 1, 1),        # 480 positions: a partial last tile; 72 channels: a partial second channel tile
+    ((8, 8, 8, 2), (1, 1, 8, 8), 1, 0, 1),             # one partial tile in both directions
+    ((32, 30, 32, 9), (3, 3, 16, 64), 1, 1, 2),        # 960 positions: fifteen tiles; groups
+    ((64, 64, 8, 16), (3, 3, 8, 128), 1, 1, 1),        # 2048 tiles: a workgroup walks two of them and keeps the channel sums in registers
+    ((16, 16, 8, 2), (2, 2, 8, 200), 2, 0, 1),         # 64 positions, four channel tiles (the last with 8 channels), strided
+]
+
+
+@pytest.mark.parametrize("case", range(len(ONE_PASS_CASES)))
+@pytest.mark.parametrize("act", ["relu", "gelu", "identity"])
+def test_pullback_single_pass_over_delta(gpu, case, act):
+    """with and without a bias (the partial sums), with the identity (dz is delta itself) and with activations that
+    take their derivative from the output (relu) or from the pre-activation (gelu)"""
+    xs, ws, stride, pad, groups = ONE_PASS_CASES[case]
+    rng = np.random.default_rng(stable_seed("one pass", case, act))
+    gd, od = cdims(gpu, xs, ws, stride=stride, padding=pad, groups=groups)
+    assert (od.y_shape()[0] * od.y_shape()[1]) % 8 == 0 and ws[3] % 8 == 0
+    fan_in = ws[0] * ws[1] * ws[2]
+    for with_bias in (True, False):
+        x, w, b, delta = host_inputs("bf16", rng.normal(size=xs), rng.normal(size=ws) * np.sqrt(2.0 / fan_in),
+                                     rng.normal(size=ws[3]) * 0.1 if with_bias else None, rng.normal(size=od.y_shape()))
+        tag = f"bf16 {act} one-pass case {case} bias={with_bias}"
+        y, back = gpu.pullback(gpu.fused_conv_bias_activation, act, dev(gpu, w, "bf16"), dev(gpu, x, "bf16"), dev(gpu, b, "bf16"), gd)
+        wy, _, _, _ = O.fused_conv_pullback(act, f64(w), f64(x), f64(b), od, f64(delta))
+        gw, gx, gb = back(dev(gpu, delta, "bf16"))
+        # y, the pre-activation and dz are stored in bf16 between the passes
+        pre = O.bias_add(O.conv(f64(x), f64(w), od), f64(b))
+        yq, preq = (f64(O.round_to_bf16(a.astype(np.float32))) for a in (wy, pre))
+        dzx = O.grad_activation(f64(delta), yq, act, preq)
+        dz = f64(O.round_to_bf16(dzx.astype(np.float32)))
+        dzr = rms(delta)
+        assert_close(gw.to_numpy(), O.conv_filter_grad(f64(x), dz, od), "bf16", tag + " dw",
+                     scale=np.sqrt(np.prod(od.y_shape()) / ws[3]) * dzr * rms(x) * 0.5)
+        assert_close(gx.to_numpy(), O.conv_data_grad(dz, f64(w), od), "bf16", tag + " dx",
+                     scale=np.sqrt(ws[0] * ws[1] * ws[3] / groups) * dzr * rms(w) * 0.5)
+        if with_bias:
+            assert_close(gb.to_numpy(), O.grad_bias_add(b, dzx), "bf16", tag + " db")
+        else:
+            assert gb is None
