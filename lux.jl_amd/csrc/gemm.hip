@@ -202,6 +202,48 @@ __global__ __launch_bounds__(256) void attn_rowdot_kernel(const T* __restrict__ 
     for (int o = 32; o >= 1; o >>= 1) acc += __shfl_xor(acc, o);
     if (lane == 0) d[col] = acc;
 }
+// Columns whose length, leading dimension and strides are multiples of 4 elements (aligned accordingly): sixteen lanes per
+// column (four columns per wave), four consecutive elements per lane and trip, so that a wave's loads are 8- or 16-byte
+// vectors that cover whole cache lines of four columns.
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void attn_rowdot_quad_kernel(const T* __restrict__ dO, const TO* __restrict__ O, float* __restrict__ d, int E,
+                                                               int N, int64_t ldo, int bd0, int bd1, int64_t s0, int64_t s1, int64_t s2,
+                                                               int64_t cols) {
+    const int64_t col = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int sub = threadIdx.x & 15;
+    float acc = 0.0f;
+    if (col < cols) {
+        const int64_t b = col / N;
+        const int n = (int)(col - b * N);
+        const int i0 = (int)(b % bd0), i1 = (int)((b / bd0) % bd1);
+        const int64_t i2 = b / ((int64_t)bd0 * bd1);
+        const int64_t off = i0 * s0 + i1 * s1 + i2 * s2 + (int64_t)n * ldo;
+        for (int e = sub * 4; e < E; e += 64) {
+            float a[4], o[4];
+            if constexpr (sizeof(T) == 2) {
+                const uint2 w = *reinterpret_cast<const uint2*>(dO + off + e);
+                a[0] = __uint_as_float(w.x << 16); a[1] = __uint_as_float(w.x & 0xffff0000u);
+                a[2] = __uint_as_float(w.y << 16); a[3] = __uint_as_float(w.y & 0xffff0000u);
+            } else {
+                const float4 w = *reinterpret_cast<const float4*>(dO + off + e);
+                a[0] = w.x; a[1] = w.y; a[2] = w.z; a[3] = w.w;
+            }
+            if constexpr (sizeof(TO) == 2) {
+                const uint2 w = *reinterpret_cast<const uint2*>(O + off + e);
+                o[0] = __uint_as_float(w.x << 16); o[1] = __uint_as_float(w.x & 0xffff0000u);
+                o[2] = __uint_as_float(w.y << 16); o[3] = __uint_as_float(w.y & 0xffff0000u);
+            } else {
+                const float4 w = *reinterpret_cast<const float4*>(O + off + e);
+                o[0] = w.x; o[1] = w.y; o[2] = w.z; o[3] = w.w;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = fmaf(a[i], o[i], acc);
+        }
+    }
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) acc += __shfl_xor(acc, o);      // within the sixteen lanes of a column
+    if (sub == 0 && col < cols) d[col] = acc;
+}
 
 static int gemm_check(int dtype, int act, int64_t M, int64_t N, int64_t K) {
     LUX_UNSUPPORTED_IF(dtype != LUXHIP_F32 && dtype != LUXHIP_BF16, "unsupported dtype %d", dtype);
@@ -294,18 +336,23 @@ int luxhip_attention_weights_pullback(luxhip_stream_t s, int dtype, int64_t S, i
     float* d = reinterpret_cast<float*>(ws.data);
     {
         ProfScope ps("attn_rowdot_kernel", (hipStream_t)s);
-        const unsigned grid = (unsigned)ceil_div(cols, 4);
         const int b0 = (int)batch_dims[0], b1 = (int)batch_dims[1];
-        const int64_t *so = strides_o;
-        if (dtype == LUXHIP_F32)
-            attn_rowdot_kernel<float, float><<<grid, 256, 0, (hipStream_t)s>>>((const float*)d_out, (const float*)out, d, (int)Ev, (int)L, ldo,
-                                                                               b0, b1, so[0], so[1], so[2], cols);
-        else if (wide)
-            attn_rowdot_kernel<bf16_t, float><<<grid, 256, 0, (hipStream_t)s>>>((const bf16_t*)d_out, (const float*)out, d, (int)Ev, (int)L,
-                                                                                ldo, b0, b1, so[0], so[1], so[2], cols);
-        else
-            attn_rowdot_kernel<bf16_t, bf16_t><<<grid, 256, 0, (hipStream_t)s>>>((const bf16_t*)d_out, (const bf16_t*)out, d, (int)Ev, (int)L,
-                                                                                 ldo, b0, b1, so[0], so[1], so[2], cols);
+        const int64_t* so = strides_o;
+        const size_t eo = dtype == LUXHIP_F32 || wide ? 4 : 2, ed = dtype == LUXHIP_F32 ? 4 : 2;      // element sizes of out and d_out
+        const bool quad = Ev % 4 == 0 && ldo % 4 == 0 && so[0] % 4 == 0 && so[1] % 4 == 0 && so[2] % 4 == 0 &&
+                          reinterpret_cast<uintptr_t>(d_out) % (4 * ed) == 0 && reinterpret_cast<uintptr_t>(out) % (4 * eo) == 0;
+        const unsigned grid = (unsigned)ceil_div(cols, quad ? 16 : 4);
+#define ROWDOT(T, TO)                                                                                                                   \
+    do {                                                                                                                                \
+        if (quad) attn_rowdot_quad_kernel<T, TO><<<grid, 256, 0, (hipStream_t)s>>>((const T*)d_out, (const TO*)out, d, (int)Ev, (int)L, ldo, \
+                                                                                   b0, b1, so[0], so[1], so[2], cols);                  \
+        else attn_rowdot_kernel<T, TO><<<grid, 256, 0, (hipStream_t)s>>>((const T*)d_out, (const TO*)out, d, (int)Ev, (int)L, ldo, b0, b1, \
+                                                                         so[0], so[1], so[2], cols);                                   \
+    } while (0)
+        if (dtype == LUXHIP_F32) ROWDOT(float, float);
+        else if (wide) ROWDOT(bf16_t, float);
+        else ROWDOT(bf16_t, bf16_t);
+#undef ROWDOT
         LUX_CHECK_LAUNCH();
     }
     // dprobs (S x L) = v' (S x Ev) * d_out (Ev x L), with the softmax rule as its epilogue
