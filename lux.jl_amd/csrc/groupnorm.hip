@@ -222,6 +222,10 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
     const uint32_t qbeg = part * g.pvec, qend = CACHED ? qbeg + g.pvec : g.nvec;   // this workgroup's vectors of the slice
     const size_t base = (size_t)slice * g.nvec * VEC;
     const float mean = save_mean[slice], invstd = save_invstd[slice];
+    // the normalised value: with 16-bit storage one fused multiply-add (x carries 8 bits, so the rounding of mean * invstd
+    // does not show); fp32 storage subtracts first, which keeps every bit when x is close to the mean
+    const float nmean = -mean * invstd;
+    auto xhat = [&](float xe) { return sizeof(T) == 2 ? fmaf(xe, invstd, nmean) : (xe - mean) * invstd; };
     if constexpr (AFFINE) {
         for (uint32_t i = threadIdx.x; i < 2 * nw * g.Cg; i += T_) lds[16 + i] = 0.0f;
         __syncthreads();
@@ -293,7 +297,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                 const float pre = fmaf(xv[e], sc, sh);
                 dy *= Act<ACT>::d(Act<ACT>::f(pre), pre);
             }
-            const float xh = (xv[e] - mean) * invstd;
+            const float xh = xhat(xv[e]);
             gv[e] = dy * gm;
             a = fmaf(dy, xh, a);
             b += dy;
@@ -339,7 +343,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                     grad_terms(q, d[0], v[0], gv, a, b);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        const float xh = (v[0][e] - mean) * invstd;
+                        const float xh = xhat(v[0][e]);
                         s1 += gv[e];
                         s2 = fmaf(gv[e], xh, s2);
                     }
@@ -379,7 +383,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                 grad_terms(q, d[0], v[0], gv, a, b);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    const float xh = (v[0][e] - mean) * invstd;
+                    const float xh = xhat(v[0][e]);
                     s1 += gv[e];
                     s2 = fmaf(gv[e], xh, s2);
                 }
@@ -409,7 +413,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         t1 += gv[e];
-                        t2 = fmaf(gv[e], (v[0][e] - mean) * invstd, t2);
+                        t2 = fmaf(gv[e], xhat(v[0][e]), t2);
                     }
                 }
                 t1 = block_sum(t1, sm);
@@ -469,7 +473,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
         grad_terms(q, dv, xv, gv, a, b);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            const float xh = (xv[e] - mean) * invstd;
+            const float xh = xhat(xv[e]);
             o[e] = invstd * (gv[e] - s1 - xh * s2);
         }
         gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
@@ -494,7 +498,7 @@ __global__ void gn_bwd_kernel(const T* __restrict__ delta, const T* __restrict__
                     float o[VEC];
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        const float xh = (v[0][e] - mean) * invstd;
+                        const float xh = xhat(v[0][e]);
                         o[e] = fmaf(xh, k2, fmaf(d[0][e], kg, k1));
                     }
                     gn_store<T, VEC>(dx, base + (size_t)q * VEC, o);
