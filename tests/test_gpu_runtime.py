@@ -288,3 +288,21 @@ def test_a_recorded_graph_keeps_its_workspace_block_after_growth(gpu):
             hip.hipGraphDestroy(graph)
         gpu.set_stream(main)
         gpu._lib.call("luxhip_stream_destroy", stream)
+
+
+@pytest.mark.parametrize("n,offset", [(4096, 0), (4099, 0), (8 * 1000 + 8, 1), (7, 0), (8 * 70000, 0)])
+def test_storage_conversion_every_access_path(gpu, n, offset):
+    """fp32 -> bf16 (round to nearest even) and back: lengths that are and are not multiples of the eight elements a
+    thread converts at once, and a source that starts one element into its allocation (the element-wise kernel)."""
+    rng = np.random.default_rng(n + offset)
+    h = (rng.normal(size=n + offset) * 10.0 ** rng.integers(-3, 4, n + offset)).astype(np.float32)
+    base = gpu.DeviceArray.from_numpy(h, "f32")
+    src = gpu.DeviceArray((n,), "f32", ptr=base.ptr + offset * 4, base=base) if offset else base
+    lo = gpu.DeviceArray((n,), "bf16")
+    gpu._lib.call("luxhip_convert", gpu.current_stream(), src.code, lo.code, n, src.ptr, lo.ptr)
+    want = O.round_to_bf16(h[offset:])
+    got = lo.to_numpy()
+    assert np.array_equal(np.asarray(got, np.float32), np.asarray(want, np.float32))
+    back = gpu.DeviceArray((n,), "f32")
+    gpu._lib.call("luxhip_convert", gpu.current_stream(), lo.code, back.code, n, lo.ptr, back.ptr)
+    assert np.array_equal(back.to_numpy(), np.asarray(want, np.float32))
