@@ -672,15 +672,23 @@ def timed(lux, fn, steps, warmup):
 
 
 REGIONS = 3
+SETTLE_S = 0.3          # untimed run-in of every workload before its timed regions (at least the warm-up steps)
 
 
 def timed_regions(lux, fn, steps, warmup):
     """The warm-up, then REGIONS timed regions of `steps` steps each, back to back.  Returns the region with the
     median time (device events, host clock) and the per-step times of all regions: one sample cannot tell a slow
     box from a clock that has not settled."""
+    t_warm = time.perf_counter()
     for _ in range(warmup):
         fn()
     lux.synchronize()
+    # the device's clock needs a few hundred milliseconds of the workload before it settles (it is power-managed);
+    # short workloads therefore keep running, untimed, until SETTLE_S have passed since the warm-up began
+    while time.perf_counter() - t_warm < SETTLE_S:
+        for _ in range(max(warmup, 10)):
+            fn()
+        lux.synchronize()
     samples = []
     for _ in range(REGIONS):
         e0, e1 = lux.Event(), lux.Event()
@@ -852,7 +860,8 @@ def measure(lux, name, args):
         "workload": wl.name, "description": wl.description, "dtype": wl.dtype, "bound": wl.bound, "value": round(value, 2), "unit": unit,
         "steps": steps, "warmup": warmup, "ms_per_step": round(ms_head, 5), "frac_of_peak": round(value / peak, 4),
         "ms_per_step_gpu_events": round(ms_gpu_head, 5), "ms_per_step_host_clock": round(ms_wall_head, 5),
-        "timing": f"median of {REGIONS} timed regions of {steps} steps each, after {warmup} warm-up steps", "spread": spread,
+        "timing": f"median of {REGIONS} timed regions of {steps} steps each, after {warmup} warm-up steps and an untimed run-in "
+                  f"that lasts until {SETTLE_S} s have passed since the warm-up began", "spread": spread,
         "roofline": roofline, "kernels": kernels,
     }
     if cold is not None:

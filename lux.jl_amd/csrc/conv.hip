@@ -209,9 +209,15 @@ __global__ __launch_bounds__(256) void conv_dz_cwhn_pack_kernel(const bf16_t* __
 
 // dbias[c] = sum over slices of partial[slice][c]: one workgroup per channel, thread t adds slices t, t + 256, ...;
 // the threads' sums are added in a fixed order (within a wave, then the four waves in turn).
-__global__ __launch_bounds__(256) void conv_dbias_finalize_kernel(const float* __restrict__ partial, bf16_t* dbias, int C, int S) {
+// What is left of the bias gradient after conv_dz_cwhn_pack_kernel: `slices` partial sums per channel.  Either a launch of
+// its own or extra workgroups of the launch that adds up the filter gradient's partial sums (both are a few microseconds).
+struct BiasPartials {
+    const float* partial = nullptr;
+    bf16_t* dbias = nullptr;
+    int C = 0, slices = 0;
+};
+__device__ __forceinline__ void conv_dbias_finalize_channel(const float* __restrict__ partial, bf16_t* dbias, int C, int S, int c) {
     __shared__ float sw[4];
-    const int c = blockIdx.x;
     float t = 0.0f;
     for (int sl = threadIdx.x; sl < S; sl += 256) t += partial[(size_t)sl * C + c];
     t = wave_sum(t);
@@ -219,13 +225,20 @@ __global__ __launch_bounds__(256) void conv_dbias_finalize_kernel(const float* _
     __syncthreads();
     if (threadIdx.x == 0) st(dbias + c, ((sw[0] + sw[1]) + sw[2]) + sw[3]);
 }
+__global__ __launch_bounds__(256) void conv_dbias_finalize_kernel(const float* __restrict__ partial, bf16_t* dbias, int C, int S) {
+    conv_dbias_finalize_channel(partial, dbias, C, S, (int)blockIdx.x);
+}
 
 // dw[a, b, ci, g*Cout_g + col] = sum over slices of partial[slice][m' = t*Cin_g + ci][col].
 // A thread owns 4 consecutive m' (one 16-byte load per slice, eight slices in flight); slices are
 // added in order.
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw, ConvGeom g,
-                                                           int grp, int slices) {
+                                                           int grp, int slices, int reduce_blocks, BiasPartials bp) {
+    if ((int)blockIdx.x >= reduce_blocks) {       // workgroups behind the reduction: one channel of the bias gradient each
+        conv_dbias_finalize_channel(bp.partial, bp.dbias, bp.C, bp.slices, (int)blockIdx.x - reduce_blocks);
+        return;
+    }
     const int Mrows = g.kW * g.kH * g.Cin_g;
     const int total = Mrows * g.Cout_g;
     const int idx = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
@@ -353,7 +366,7 @@ static bool dz_cwhn_ok(int P, int C, int N, const void* delta, const void* y, co
 // dz (may be NULL for the identity: dz is delta), dzT, the bias gradient (if dbias != NULL) and, if wout != NULL, the filter
 // repacked for the input-gradient kernel
 static int conv_dz_cwhn_pack(hipStream_t s, int act, const ConvGeom& g, const bf16_t* delta, const bf16_t* y, const bf16_t* pre,
-                             bf16_t* dz, bf16_t* dzT, float* partial, bf16_t* dbias, const bf16_t* w, bf16_t* wout) {
+                             bf16_t* dz, bf16_t* dzT, float* partial, bf16_t* dbias, const bf16_t* w, bf16_t* wout, BiasPartials* later) {
     const int P = g.OW * g.OH, C = g.Cout, N = g.N;
     const int chunk = dz_cwhn_chunk(P, C, N);
     const int64_t gx = ceil_div(ceil_div(P, 64), chunk), gy = ceil_div(C, 64);
@@ -370,6 +383,10 @@ static int conv_dz_cwhn_pack(hipStream_t s, int act, const ConvGeom& g, const bf
 #undef LAUNCH_DZC
     LUX_CHECK_LAUNCH();
     if (dbias != nullptr) {
+        if (later != nullptr) {           // the caller adds the channels' sums to a later launch
+            later->partial = partial; later->dbias = dbias; later->C = C; later->slices = (int)(gx * N);
+            return LUXHIP_OK;
+        }
         ProfScope ps2("conv_dbias_finalize_kernel", s);
         conv_dbias_finalize_kernel<<<(unsigned)C, 256, 0, s>>>(partial, dbias, C, (int)(gx * N));
         LUX_CHECK_LAUNCH();
@@ -522,7 +539,7 @@ static bool wgrad_direct_ok(const ConvGeom& g, const void* xT, const void* dy) {
 // the general kernel; may be NULL when wgrad_direct_ok).
 template <typename T>
 static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy, const T* dyT, float* partial, T* dw,
-                     const void* zeros) {
+                     const void* zeros, const BiasPartials* bias = nullptr) {
     constexpr int V = GemmTraits<T>::VEC;
     int slices, kslice;
     bool small;
@@ -579,7 +596,10 @@ static int run_wgrad(hipStream_t s, const ConvGeom& g, const T* xT, const T* dy,
         if (rc != LUXHIP_OK) return rc;
         ProfScope ps("wgrad_reduce_kernel", s);
         const int total = Mrows * g.Cout_g;
-        wgrad_reduce_kernel<T><<<(unsigned)ceil_div(total, 1024), 256, 0, s>>>(partial, dw, g, grp, slices);
+        const int reduce_blocks = (int)ceil_div(total, 1024);
+        BiasPartials bp;
+        if (bias != nullptr && grp == g.groups - 1) bp = *bias;       // the bias gradient's channels ride on the last group's launch
+        wgrad_reduce_kernel<T><<<(unsigned)(reduce_blocks + bp.C), 256, 0, s>>>(partial, dw, g, grp, slices, reduce_blocks, bp);
         LUX_CHECK_LAUNCH();
     }
     return LUXHIP_OK;
@@ -656,13 +676,15 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
     T* wD = reinterpret_cast<T*>(ws.data + xb + yb);
     float* partial = reinterpret_cast<float*>(ws.data + xb + yb + wb);
     const T* dzp = delta;
+    BiasPartials bias_later;              // set by the single pass when the filter gradient's reduction will finish the bias gradient
     if (one_pass) {
         if constexpr (sizeof(T) == 2) {
             bf16_t* dz_out = act == LUXHIP_ACT_IDENTITY ? nullptr : reinterpret_cast<bf16_t*>(dz);
             rc = conv_dz_cwhn_pack(s, act, g, reinterpret_cast<const bf16_t*>(delta), reinterpret_cast<const bf16_t*>(y),
                                    reinterpret_cast<const bf16_t*>(pre), dz_out, reinterpret_cast<bf16_t*>(dzT),
                                    reinterpret_cast<float*>(ws.data + xb + yb + wb + pb), reinterpret_cast<bf16_t*>(dbias),
-                                   reinterpret_cast<const bf16_t*>(w), dx != nullptr ? reinterpret_cast<bf16_t*>(wD) : nullptr);
+                                   reinterpret_cast<const bf16_t*>(w), dx != nullptr ? reinterpret_cast<bf16_t*>(wD) : nullptr,
+                                   dw != nullptr ? &bias_later : nullptr);
             if (rc != LUXHIP_OK) return rc;
             if (dz_out) dzp = dz;
         }
@@ -684,7 +706,8 @@ static int fused_conv_bwd_t(hipStream_t s, int dtype, int act, const ConvGeom& g
     if (dw != nullptr) {
         if (!xt_kept && (rc = transpose_to_cwhn<T>(s, x, reinterpret_cast<T*>(ws.data), g.W * g.H, g.Cin, g.N)) != LUXHIP_OK)
             return rc;
-        if ((rc = run_wgrad<T>(s, g, xT, dzp, dzT, partial, dw, ws.zeros)) != LUXHIP_OK) return rc;
+        if ((rc = run_wgrad<T>(s, g, xT, dzp, dzT, partial, dw, ws.zeros, bias_later.dbias != nullptr ? &bias_later : nullptr)) != LUXHIP_OK)
+            return rc;
     }
     return LUXHIP_OK;
 }
