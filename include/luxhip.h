@@ -96,8 +96,11 @@ int luxhip_event_elapsed_ms(float* ms, luxhip_event_t start, luxhip_event_t stop
 int luxhip_event_destroy(luxhip_event_t e);
 
 /* Per-kernel timing (no counterpart in the reference, which has no tracing for its native GPU
- * path): while enabled, every kernel launch is bracketed by HIP events on its own stream.
- * luxhip_profile_report synchronises, writes a JSON array of {kernel, count, total_ms, min_ms,
+ * path): while enabled, every kernel launch is timed with HIP events on its own stream.  The
+ * streaming kernels (bias_activation, batchnorm, groupnorm, layernorm) hand two events to their
+ * dispatch, which signals them at the begin and at the end of the kernel itself: the duration a
+ * kernel trace reports.  The other launches are bracketed by events recorded around them (the
+ * kernel plus the gap to the launch before it).  luxhip_profile_report synchronises, writes a JSON array of {kernel, count, total_ms, min_ms,
  * max_ms} into buf and clears the log. */
 int luxhip_profile_enable(int on);
 /* Tuning switches (no counterpart in LuxLib; tests use them to reach every code path):
